@@ -1,0 +1,48 @@
+// Picks the matrix-core prefill attention unit built for the head size at hand.  Each unit
+// (attention_mfma.hip compiled with RLIS_HEAD_DIM = 32, 64, ... 256) serves head sizes up to
+// its own, padding the rest with zeros.
+#include "common.h"
+
+#define DECL(D)                                                                               \
+  extern "C" int rlis_attn_prefill_mfma_d##D(                                                 \
+      const void* q, long long q_stride, void* out, long long out_stride, const void* k_pages, \
+      const void* v_pages, const int* block_tables, int max_pages, const int* cu_seqlens,     \
+      const int* start_pos, const int* tile_map, int num_tiles, int nh, int nkv, int d,       \
+      int page_size, int window, float scale, hipStream_t stream);
+DECL(32) DECL(64) DECL(96) DECL(128) DECL(160) DECL(192) DECL(224) DECL(256)
+#undef DECL
+
+RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out,
+                                    long long out_stride, const void* k_pages,
+                                    const void* v_pages, const int* block_tables, int max_pages,
+                                    const int* cu_seqlens, const int* start_pos,
+                                    const int* tile_map, int num_tiles, int nh, int nkv, int d,
+                                    int page_size, int window, float scale, int reserved,
+                                    hipStream_t stream) {
+  (void)reserved;
+  RLIS_REQUIRE(num_tiles >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0,
+               "attn_prefill_mfma: bad sizes");
+  RLIS_REQUIRE(nh % nkv == 0, "attn_prefill_mfma: %d query heads are not a multiple of %d KV heads",
+               nh, nkv);
+  RLIS_REQUIRE(d % 16 == 0 && d <= 256,
+               "attn_prefill_mfma: head_dim %d must be a multiple of 16 and at most 256", d);
+  RLIS_REQUIRE(page_size % 8 == 0, "attn_prefill_mfma: page size %d must be a multiple of 8",
+               page_size);
+  RLIS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)k_pages % 16) == 0 &&
+                   ((uintptr_t)v_pages % 16) == 0,
+               "attn_prefill_mfma: operands must be 16-byte aligned with row strides in steps of 8");
+  RLIS_REQUIRE(nh <= 65535, "attn_prefill_mfma: too many heads");
+#define CALL(D)                                                                                 \
+  return rlis_attn_prefill_mfma_d##D(q, q_stride, out, out_stride, k_pages, v_pages,            \
+                                     block_tables, max_pages, cu_seqlens, start_pos, tile_map,  \
+                                     num_tiles, nh, nkv, d, page_size, window, scale, stream)
+  if (d <= 32) CALL(32);
+  if (d <= 64) CALL(64);
+  if (d <= 96) CALL(96);
+  if (d <= 128) CALL(128);
+  if (d <= 160) CALL(160);
+  if (d <= 192) CALL(192);
+  if (d <= 224) CALL(224);
+  CALL(256);
+#undef CALL
+}

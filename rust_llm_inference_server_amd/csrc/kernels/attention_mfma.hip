@@ -1,0 +1,243 @@
+// Prefill attention over the paged cache on the matrix cores (bfloat16 operands, float32
+// accumulation and softmax), one compile unit per padded head size RLIS_HEAD_DIM.
+//
+// A workgroup of four waves serves 64 consecutive new tokens of one sequence for one query
+// head; each wave owns 16 of them.  Keys are walked in tiles of BN positions aligned to BN,
+// read through the block table: the K tile [key][dim] and the V tile [dim][key] (the cache
+// keeps V transposed inside a page, so both are copied as they lie) go to LDS once per
+// workgroup.  S = Q K^T and O += P V use v_mfma_f32_16x16x32_bf16; the accumulator of a
+// 16 x 16 block holds, in lane l and register r, row (l / 16) * 4 + r and column l % 16, so the
+// softmax statistics of a row sit in the same lanes for S and for O.
+//
+// The mask is the reference's causal mask offset by the cached length (crates/model/src/
+// attention.rs:225-233): the new token at index i of a sequence with P cached positions sees
+// keys at positions <= P + i, and > P + i - window when a window is given.  Scores are scaled
+// in float32 after the product; probabilities are rounded to bfloat16 only as the operand of
+// the PV product (the row sums use the float32 values).
+#include "common.h"
+
+#include <math.h>
+
+#ifndef RLIS_HEAD_DIM
+#error "RLIS_HEAD_DIM must be defined (padded head size, a multiple of 32)"
+#endif
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+union Frag8 {
+  uint4 u;
+  bf16x8 v;
+  bf16_t e[8];
+};
+
+#define RLIS_CAT2(a, b) a##b
+#define RLIS_CAT(a, b) RLIS_CAT2(a, b)
+#define KERNEL_NAME RLIS_CAT(rlis_attn_prefill_mfma_kernel_d, RLIS_HEAD_DIM)
+
+namespace {
+
+constexpr int D = RLIS_HEAD_DIM;
+constexpr int BN = D <= 128 ? 64 : 32;
+constexpr int KS = D + 8;     // K tile row stride (bf16 elements)
+constexpr int VS = BN + 8;    // V tile row stride
+constexpr int PS = BN + 8;    // P tile row stride
+constexpr int BM = 64;
+
+}  // namespace
+
+__global__ __launch_bounds__(256) void KERNEL_NAME(
+    const bf16_t* __restrict__ q, long long q_stride, bf16_t* __restrict__ out,
+    long long out_stride, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ start_pos, const int* __restrict__ tile_map, int nh, int nkv, int d,
+    int page_size, float scale, int window) {
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[BN * KS];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[D * VS];
+  __shared__ __attribute__((aligned(16))) bf16_t Ps[4 * 16 * PS];
+
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int l16 = lane % 16, lq = lane / 16;
+  const int tile = blockIdx.x, h = blockIdx.y;
+  const int seq = tile_map[2 * tile], qb = tile_map[2 * tile + 1];
+  const int tok_begin = cu_seqlens[seq];
+  const int n_new = cu_seqlens[seq + 1] - tok_begin;
+  const int P = start_pos[seq];
+  const int kvh = h / (nh / nkv);
+  const int* table = block_tables + (long long)seq * max_pages;
+
+  // Query fragments of this wave: row l16 -> new-token index qb + wave * 16 + l16.
+  const int my_qi = qb + wave * 16 + l16;
+  Frag8 qf[D / 32];
+#pragma unroll
+  for (int ks = 0; ks < D / 32; ++ks) {
+    const int dim = ks * 32 + lq * 8;
+    if (my_qi < n_new && dim < d)
+      qf[ks].u = *(const uint4*)(q + (long long)(tok_begin + my_qi) * q_stride + h * d + dim);
+    else
+      qf[ks].u = make_uint4(0, 0, 0, 0);
+  }
+
+  // Rows of the accumulators held by this lane: new-token index qb + wave * 16 + lq * 4 + r.
+  float m[4], l[4];
+  f32x4 o_acc[D / 16];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    m[r] = -INFINITY;
+    l[r] = 0.f;
+  }
+#pragma unroll
+  for (int db = 0; db < D / 16; ++db) o_acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  const int q_last = min(n_new, qb + BM) - 1;           // last new-token index of the tile
+  const int khi = P + q_last + 1;                        // keys [klo, khi) matter to the tile
+  int klo = 0;
+  if (window > 0) klo = max(0, P + qb - window + 1);
+  const int kt0 = (klo / BN) * BN;
+  const int wave_q_first = qb + wave * 16;
+  const int wave_q_last = min(n_new - 1, wave_q_first + 15);
+  bf16_t* my_ps = Ps + wave * 16 * PS;
+
+  for (int k0 = kt0; k0 < khi; k0 += BN) {
+    // ---- stage K [BN][D] and V^T [d][BN] ---------------------------------------------
+    for (int c = tid; c < BN * (D / 8); c += 256) {
+      const int key = c / (D / 8), dc = c % (D / 8);
+      const int kpos = k0 + key;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (kpos < khi && dc * 8 < d) {
+        const long long page = table[kpos / page_size];
+        const int off = kpos % page_size;
+        v = *(const uint4*)(k_pages + ((page * nkv + kvh) * page_size + off) * d + dc * 8);
+      }
+      *(uint4*)(Ks + key * KS + dc * 8) = v;
+    }
+    for (int c = tid; c < d * (BN / 8); c += 256) {
+      const int dim = c / (BN / 8), kg = c % (BN / 8);
+      const int kpos = k0 + kg * 8;
+      Frag8 v;
+      v.u = make_uint4(0, 0, 0, 0);
+      if (kpos < khi) {
+        const long long page = table[kpos / page_size];
+        const int off = kpos % page_size;
+        v.u = *(const uint4*)(v_pages + ((page * nkv + kvh) * (long long)d + dim) * page_size + off);
+        if (kpos + 8 > khi) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (kpos + e >= khi) v.e[e] = 0;
+        }
+      }
+      *(uint4*)(Vs + dim * VS + kg * 8) = v.u;
+    }
+    __syncthreads();
+
+    // Tiles wholly after this wave's last query contribute nothing to it.
+    const bool wave_active = (wave_q_first < n_new) && (k0 <= P + wave_q_last);
+    if (wave_active) {
+      // ---- S = Q K^T -------------------------------------------------------------------
+      f32x4 s_acc[BN / 16];
+#pragma unroll
+      for (int nb = 0; nb < BN / 16; ++nb) {
+        s_acc[nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < D / 32; ++ks) {
+          Frag8 kf;
+          kf.u = *(const uint4*)(Ks + (nb * 16 + l16) * KS + ks * 32 + lq * 8);
+          s_acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks].v, kf.v, s_acc[nb], 0, 0, 0);
+        }
+      }
+      // ---- mask, scale, online softmax ---------------------------------------------------
+      float corr[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int qi = wave_q_first + lq * 4 + r;
+        const int qpos = P + qi;
+        float row_max = -INFINITY;
+#pragma unroll
+        for (int nb = 0; nb < BN / 16; ++nb) {
+          const int kpos = k0 + nb * 16 + l16;
+          const bool ok = (qi < n_new) && (kpos <= qpos) && (window <= 0 || kpos > qpos - window);
+          const float sv = ok ? s_acc[nb][r] * scale : -INFINITY;
+          s_acc[nb][r] = sv;
+          row_max = fmaxf(row_max, sv);
+        }
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) row_max = fmaxf(row_max, __shfl_xor(row_max, o, kWave));
+        const float m_new = fmaxf(m[r], row_max);
+        float row_sum = 0.f;
+#pragma unroll
+        for (int nb = 0; nb < BN / 16; ++nb) {
+          const float sv = s_acc[nb][r];
+          const float p = (sv == -INFINITY) ? 0.f : expf(sv - m_new);
+          s_acc[nb][r] = p;
+          row_sum += p;
+        }
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) row_sum += __shfl_xor(row_sum, o, kWave);
+        corr[r] = (m[r] == -INFINITY) ? 0.f : expf(m[r] - m_new);
+        l[r] = l[r] * corr[r] + row_sum;
+        m[r] = m_new;
+      }
+      // ---- P to LDS (row-major per wave), O rescale ---------------------------------------
+#pragma unroll
+      for (int nb = 0; nb < BN / 16; ++nb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          my_ps[(lq * 4 + r) * PS + nb * 16 + l16] = f32_to_bf16(s_acc[nb][r]);
+#pragma unroll
+      for (int db = 0; db < D / 16; ++db)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o_acc[db][r] *= corr[r];
+    }
+    // The P tile is private to the wave, but the barrier also orders it for the reads below.
+    __syncthreads();
+    if (wave_active) {
+      // ---- O += P V ----------------------------------------------------------------------
+      Frag8 pf[BN / 32];
+#pragma unroll
+      for (int ks = 0; ks < BN / 32; ++ks)
+        pf[ks].u = *(const uint4*)(my_ps + l16 * PS + ks * 32 + lq * 8);
+#pragma unroll
+      for (int db = 0; db < D / 16; ++db) {
+        if (db * 16 < d) {
+#pragma unroll
+          for (int ks = 0; ks < BN / 32; ++ks) {
+            Frag8 vf;
+            vf.u = *(const uint4*)(Vs + (db * 16 + l16) * VS + ks * 32 + lq * 8);
+            o_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[ks].v, vf.v, o_acc[db], 0, 0, 0);
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- normalise and store ------------------------------------------------------------
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int qi = wave_q_first + lq * 4 + r;
+    if (qi >= n_new) continue;
+    const float inv_l = 1.0f / l[r];
+    bf16_t* orow = out + (long long)(tok_begin + qi) * out_stride + h * d;
+#pragma unroll
+    for (int db = 0; db < D / 16; ++db) {
+      const int dim = db * 16 + l16;
+      if (dim < d) orow[dim] = f32_to_bf16(o_acc[db][r] * inv_l);
+    }
+  }
+}
+
+// tile_map holds num_tiles pairs (sequence, first new-token index of a 64-token tile).
+RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
+    const void* q, long long q_stride, void* out, long long out_stride, const void* k_pages,
+    const void* v_pages, const int* block_tables, int max_pages, const int* cu_seqlens,
+    const int* start_pos, const int* tile_map, int num_tiles, int nh, int nkv, int d,
+    int page_size, int window, float scale, hipStream_t stream) {
+  if (num_tiles == 0) return 0;
+  dim3 grid(num_tiles, nh);
+  KERNEL_NAME<<<grid, 256, 0, stream>>>(
+      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,
+      (const bf16_t*)v_pages, block_tables, max_pages, cu_seqlens, start_pos, tile_map, nh, nkv, d,
+      page_size, scale, window);
+  RLIS_LAUNCH_CHECK("attn_prefill_mfma");
+  return 0;
+}

@@ -1,0 +1,84 @@
+// Shared helpers for the gfx950 kernels: bf16 <-> f32 conversion, wave64 reductions and the
+// error channel of the C entry points.  Every entry point returns 0 on success and nonzero
+// after storing a message that rlis_last_error() returns; launches go to the stream the
+// caller passes, nothing is allocated and nothing synchronises.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#define RLIS_API extern "C" __attribute__((visibility("default")))
+
+typedef uint16_t bf16_t;
+
+enum { RLIS_F32 = 0, RLIS_BF16 = 1 };
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+  return __uint_as_float(((uint32_t)v) << 16);
+}
+
+// Round to nearest, ties to even; NaN stays NaN.
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float ld(const float* p) { return *p; }
+__device__ __forceinline__ float ld(const bf16_t* p) { return bf16_to_f32(*p); }
+__device__ __forceinline__ void st(float* p, float v) { *p = v; }
+__device__ __forceinline__ void st(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+
+// Sum over a block of NT threads (NT a multiple of 64); every thread gets the result.  The
+// order of the additions is fixed by NT alone.
+template <int NT>
+__device__ __forceinline__ float block_sum(float v, float* smem /* NT/64 floats */) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  __syncthreads();
+  if (lane == 0) smem[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+#pragma unroll
+  for (int i = 0; i < NT / kWave; ++i) t += smem[i];
+  return t;
+}
+
+// ------------------------------------------------------------------ error channel
+void rlis_set_error(const char* fmt, ...);
+
+#define RLIS_REQUIRE(cond, ...)            \
+  do {                                     \
+    if (!(cond)) {                         \
+      rlis_set_error(__VA_ARGS__);         \
+      return 1;                            \
+    }                                      \
+  } while (0)
+
+#define RLIS_LAUNCH_CHECK(name)                                              \
+  do {                                                                       \
+    hipError_t e_ = hipGetLastError();                                       \
+    if (e_ != hipSuccess) {                                                  \
+      rlis_set_error("%s: launch failed: %s", name, hipGetErrorString(e_));  \
+      return 1;                                                              \
+    }                                                                        \
+  } while (0)
+
+static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+static inline long long ceil_div_ll(long long a, long long b) { return (a + b - 1) / b; }

@@ -1,0 +1,289 @@
+// Row-wise and element-wise kernels of the decoder step: embedding gather, residual add fused
+// with RMSNorm, SwiGLU, rotary position encoding fused with the write of K and V into cache
+// pages, and page copies.  All arithmetic is float32; storage is float32 or bfloat16.
+//
+// Formulas follow the reference: RMSNorm y = x * rsqrt(mean(x^2) + eps) * w
+// (crates/model/src/layers.rs:141-146), SwiGLU silu(gate) * up (layers.rs:179-186), rotate-half
+// rotation with per-position cos/sin rows (crates/model/src/rope.rs:111-117), K and V written
+// at slot = table[pos / page] * page + pos % page before attention reads them
+// (crates/model/src/paged.rs:258-263, 324-337).
+#include "common.h"
+
+static thread_local char g_err[512] = "";
+
+void rlis_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+RLIS_API const char* rlis_last_error() { return g_err; }
+
+// ------------------------------------------------------------------------ embedding
+template <typename TW>
+__global__ void embed_kernel(float* __restrict__ out, const TW* __restrict__ table,
+                             const int* __restrict__ ids, int H) {
+  const int t = blockIdx.x;
+  const long long row = ids[t];
+  const TW* src = table + row * H;
+  float* dst = out + (long long)t * H;
+  for (int j = threadIdx.x; j < H; j += blockDim.x) dst[j] = ld(src + j);
+}
+
+// out (T,H) f32 <- table[ids] ; ids are checked against V on the host before the call.
+RLIS_API int rlis_embed(float* out, const void* table, int table_dtype, const int* ids, int T,
+                        int H, hipStream_t stream) {
+  RLIS_REQUIRE(T >= 0 && H > 0, "embed: bad sizes T=%d H=%d", T, H);
+  if (T == 0) return 0;
+  if (table_dtype == RLIS_F32)
+    embed_kernel<float><<<T, 256, 0, stream>>>(out, (const float*)table, ids, H);
+  else if (table_dtype == RLIS_BF16)
+    embed_kernel<bf16_t><<<T, 256, 0, stream>>>(out, (const bf16_t*)table, ids, H);
+  else
+    RLIS_REQUIRE(false, "embed: unknown table dtype %d", table_dtype);
+  RLIS_LAUNCH_CHECK("embed");
+  return 0;
+}
+
+// ------------------------------------------------------------------- residual add
+template <typename TD>
+__global__ void add_residual_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
+                                    long long n) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) resid[i] += ld(delta + i);
+}
+
+RLIS_API int rlis_add_residual(float* resid, const void* delta, int delta_dtype, long long n,
+                               hipStream_t stream) {
+  if (n <= 0) return 0;
+  const int blocks = (int)(ceil_div_ll(n, 256) < 4096 ? ceil_div_ll(n, 256) : 4096);
+  if (delta_dtype == RLIS_F32)
+    add_residual_kernel<float><<<blocks, 256, 0, stream>>>(resid, (const float*)delta, n);
+  else if (delta_dtype == RLIS_BF16)
+    add_residual_kernel<bf16_t><<<blocks, 256, 0, stream>>>(resid, (const bf16_t*)delta, n);
+  else
+    RLIS_REQUIRE(false, "add_residual: unknown dtype %d", delta_dtype);
+  RLIS_LAUNCH_CHECK("add_residual");
+  return 0;
+}
+
+// ------------------------------------------------------- residual add + RMSNorm
+// One block per output row r; the source row is rows[r] when rows is given.  The residual is
+// float32; delta (may be null) is added first and, when write_resid is set, the sum is stored
+// back.  Sum of squares, rsqrt and both multiplies are float32; one rounding at the store.
+template <typename TD, typename TW, typename TO, int NT>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
+                                   const TW* __restrict__ weight, TO* __restrict__ out,
+                                   const int* __restrict__ rows, int H, float eps,
+                                   int write_resid) {
+  __shared__ float red[NT / kWave];
+  const int r = blockIdx.x;
+  const long long src = rows ? (long long)rows[r] : (long long)r;
+  float* x = resid + src * H;
+  const TD* d = delta ? delta + src * H : nullptr;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < H; j += NT) {
+    float v = x[j];
+    if (d) {
+      v += ld(d + j);
+      if (write_resid) x[j] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum<NT>(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+  TO* o = out + (long long)r * H;
+  const bool reread_sum = d && !write_resid;
+  for (int j = threadIdx.x; j < H; j += NT) {
+    float v = x[j];
+    if (reread_sum) v += ld(d + j);
+    st(o + j, v * inv * ld(weight + j));
+  }
+}
+
+template <typename TD, typename TW, typename TO>
+static void launch_add_rmsnorm(float* resid, const void* delta, const void* weight, void* out,
+                               const int* rows, int R, int H, float eps, int write_resid,
+                               hipStream_t stream) {
+  add_rmsnorm_kernel<TD, TW, TO, 256><<<R, 256, 0, stream>>>(
+      resid, (const TD*)delta, (const TW*)weight, (TO*)out, rows, H, eps, write_resid);
+}
+
+RLIS_API int rlis_add_rmsnorm(float* resid, const void* delta, int delta_dtype,
+                              const void* weight, int weight_dtype, void* out, int out_dtype,
+                              const int* rows, int R, int H, float eps, int write_resid,
+                              hipStream_t stream) {
+  RLIS_REQUIRE(R >= 0 && H > 0, "add_rmsnorm: bad sizes R=%d H=%d", R, H);
+  RLIS_REQUIRE(!(rows && write_resid && delta),
+               "add_rmsnorm: writing the residual back needs all rows, not a selection");
+  if (R == 0) return 0;
+  const int key = (delta ? delta_dtype : out_dtype) * 4 + weight_dtype * 2 + out_dtype;
+#define CASE(k, TD, TW, TO)                                                                  \
+  case k:                                                                                    \
+    launch_add_rmsnorm<TD, TW, TO>(resid, delta, weight, out, rows, R, H, eps, write_resid,  \
+                                   stream);                                                  \
+    break;
+  switch (key) {
+    CASE(0, float, float, float)
+    CASE(1, float, float, bf16_t)
+    CASE(2, float, bf16_t, float)
+    CASE(3, float, bf16_t, bf16_t)
+    CASE(4, bf16_t, float, float)
+    CASE(5, bf16_t, float, bf16_t)
+    CASE(6, bf16_t, bf16_t, float)
+    CASE(7, bf16_t, bf16_t, bf16_t)
+    default:
+      RLIS_REQUIRE(false, "add_rmsnorm: unknown dtypes %d %d %d", delta_dtype, weight_dtype,
+                   out_dtype);
+  }
+#undef CASE
+  RLIS_LAUNCH_CHECK("add_rmsnorm");
+  return 0;
+}
+
+// -------------------------------------------------------------------------- SwiGLU
+// gu (T, 2I): columns [0, I) are the gate projection, [I, 2I) the up projection.
+template <typename TX>
+__global__ void swiglu_kernel(TX* __restrict__ out, const TX* __restrict__ gu, int I,
+                              long long total) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (; i < total; i += stride) {
+    const long long t = i / I;
+    const int c = (int)(i - t * I);
+    const float g = ld(gu + t * 2 * I + c);
+    const float u = ld(gu + t * 2 * I + I + c);
+    const float s = g / (1.0f + expf(-g));
+    st(out + i, s * u);
+  }
+}
+
+RLIS_API int rlis_swiglu(void* out, const void* gu, int dtype, int T, int I, hipStream_t stream) {
+  RLIS_REQUIRE(T >= 0 && I > 0, "swiglu: bad sizes T=%d I=%d", T, I);
+  const long long total = (long long)T * I;
+  if (total == 0) return 0;
+  const int blocks = (int)(ceil_div_ll(total, 256) < 8192 ? ceil_div_ll(total, 256) : 8192);
+  if (dtype == RLIS_F32)
+    swiglu_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gu, I, total);
+  else if (dtype == RLIS_BF16)
+    swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, I, total);
+  else
+    RLIS_REQUIRE(false, "swiglu: unknown dtype %d", dtype);
+  RLIS_LAUNCH_CHECK("swiglu");
+  return 0;
+}
+
+// ------------------------------------------------ rotary encoding + K/V page write
+// qkv (T, row_stride): q heads at columns [0, nh*d), k heads at [k_off, k_off + nkv*d), v heads
+// at [v_off, v_off + nkv*d).  The first rot_dim dims of every q and k head are rotated
+// (rotate-half: dim j pairs with j + rot_dim/2), the rest pass through.  q is rotated in
+// place.  When write_kv is set, rotated k goes to k_pages[page][kv head][offset][d] and v to
+// v_pages[page][kv head][d][offset] (v is stored transposed inside a page), with
+// page = slot / page_size, offset = slot % page_size; rotated k is not stored back to qkv.
+template <typename TX>
+__global__ void rope_kv_write_kernel(TX* __restrict__ qkv, long long row_stride, int k_off,
+                                     int v_off, int nh, int nkv, int d, int rot_dim,
+                                     const float* __restrict__ cos_t,
+                                     const float* __restrict__ sin_t,
+                                     const int* __restrict__ positions,
+                                     const int* __restrict__ slots, TX* __restrict__ k_pages,
+                                     TX* __restrict__ v_pages, int page_size, int write_kv) {
+  const int t = blockIdx.x;
+  TX* row = qkv + (long long)t * row_stride;
+  const int pos = positions[t];
+  const int half = rot_dim / 2;
+  const float* c = cos_t + (long long)pos * half;
+  const float* s = sin_t + (long long)pos * half;
+  // q heads: rotate in place.
+  for (int i = threadIdx.x; i < nh * half; i += blockDim.x) {
+    const int h = i / half, j = i - h * half;
+    TX* p = row + h * d;
+    const float x1 = ld(p + j), x2 = ld(p + j + half);
+    const float cc = c[j], sn = s[j];
+    st(p + j, x1 * cc - x2 * sn);
+    st(p + j + half, x2 * cc + x1 * sn);
+  }
+  if (!write_kv) return;
+  const int slot = slots[t];
+  if (slot < 0) return;
+  const long long page = slot / page_size;
+  const int off = slot - (int)page * page_size;
+  // k heads: rotate and store to the page.
+  for (int i = threadIdx.x; i < nkv * half; i += blockDim.x) {
+    const int h = i / half, j = i - h * half;
+    const TX* p = row + k_off + h * d;
+    const float x1 = ld(p + j), x2 = ld(p + j + half);
+    const float cc = c[j], sn = s[j];
+    TX* dst = k_pages + ((page * nkv + h) * page_size + off) * d;
+    st(dst + j, x1 * cc - x2 * sn);
+    st(dst + j + half, x2 * cc + x1 * sn);
+  }
+  const int tail = d - rot_dim;
+  for (int i = threadIdx.x; i < nkv * tail; i += blockDim.x) {
+    const int h = i / tail, j = rot_dim + (i - h * tail);
+    TX* dst = k_pages + ((page * nkv + h) * page_size + off) * d;
+    dst[j] = row[k_off + h * d + j];
+  }
+  // v heads: store transposed.
+  for (int i = threadIdx.x; i < nkv * d; i += blockDim.x) {
+    const int h = i / d, j = i - h * d;
+    v_pages[((page * nkv + h) * d + j) * page_size + off] = row[v_off + h * d + j];
+  }
+}
+
+RLIS_API int rlis_rope_kv_write(void* qkv, int dtype, long long row_stride, int k_off, int v_off,
+                                int T, int nh, int nkv, int d, int rot_dim, const float* cos_t,
+                                const float* sin_t, const int* positions, const int* slots,
+                                void* k_pages, void* v_pages, int page_size, int write_kv,
+                                hipStream_t stream) {
+  RLIS_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && d > 0, "rope_kv_write: bad sizes");
+  RLIS_REQUIRE(rot_dim >= 0 && rot_dim <= d && rot_dim % 2 == 0,
+               "rope_kv_write: rot_dim %d must be even and at most head_dim %d", rot_dim, d);
+  RLIS_REQUIRE(!write_kv || (page_size > 0 && k_pages && v_pages && slots),
+               "rope_kv_write: cache write asked for without pages");
+  if (T == 0) return 0;
+  if (dtype == RLIS_F32)
+    rope_kv_write_kernel<float><<<T, 256, 0, stream>>>(
+        (float*)qkv, row_stride, k_off, v_off, nh, nkv, d, rot_dim, cos_t, sin_t, positions,
+        slots, (float*)k_pages, (float*)v_pages, page_size, write_kv);
+  else if (dtype == RLIS_BF16)
+    rope_kv_write_kernel<bf16_t><<<T, 256, 0, stream>>>(
+        (bf16_t*)qkv, row_stride, k_off, v_off, nh, nkv, d, rot_dim, cos_t, sin_t, positions,
+        slots, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, write_kv);
+  else
+    RLIS_REQUIRE(false, "rope_kv_write: unknown dtype %d", dtype);
+  RLIS_LAUNCH_CHECK("rope_kv_write");
+  return 0;
+}
+
+// ---------------------------------------------------------------------- page copies
+// pages (num_layers, num_pages, page_elems): copy page src[i] to dst[i] in every layer.
+template <typename TX>
+__global__ void copy_pages_kernel(TX* __restrict__ pages, long long layer_stride,
+                                  long long page_elems, const int* __restrict__ src,
+                                  const int* __restrict__ dst) {
+  const int pair = blockIdx.x, layer = blockIdx.y;
+  const TX* s = pages + layer * layer_stride + (long long)src[pair] * page_elems;
+  TX* d = pages + layer * layer_stride + (long long)dst[pair] * page_elems;
+  for (long long i = threadIdx.x; i < page_elems; i += blockDim.x) d[i] = s[i];
+}
+
+RLIS_API int rlis_copy_pages(void* pages, int dtype, int num_layers, long long num_pages,
+                             long long page_elems, const int* src, const int* dst, int num_pairs,
+                             hipStream_t stream) {
+  RLIS_REQUIRE(num_layers > 0 && num_pages > 0 && page_elems > 0, "copy_pages: bad sizes");
+  if (num_pairs <= 0) return 0;
+  dim3 grid(num_pairs, num_layers);
+  if (dtype == RLIS_F32)
+    copy_pages_kernel<float><<<grid, 256, 0, stream>>>((float*)pages, num_pages * page_elems,
+                                                       page_elems, src, dst);
+  else if (dtype == RLIS_BF16)
+    copy_pages_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)pages, num_pages * page_elems,
+                                                        page_elems, src, dst);
+  else
+    RLIS_REQUIRE(false, "copy_pages: unknown dtype %d", dtype);
+  RLIS_LAUNCH_CHECK("copy_pages");
+  return 0;
+}

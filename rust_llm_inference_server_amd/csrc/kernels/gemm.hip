@@ -1,0 +1,342 @@
+// Matrix products y = x * W^T for the projections (weights are (out, in) row-major, as the
+// reference's Linear holds them: crates/model/src/layers.rs:17-19, 65-69, 82).
+//
+//  * gemm_plain: any sizes, float32 accumulation with ordinary FMAs (no matrix-core
+//    shortcut), operands float32 or bfloat16.  This is the product of the true 32-bit path.
+//  * gemm_bf16_mfma: bfloat16 operands on the matrix cores (v_mfma_f32_32x32x16_bf16),
+//    float32 accumulation, output bfloat16 or float32.  K must be a multiple of 8.
+//  * gemm_bf16_skinny: the decode shape, up to 64 rows of x.  Each weight row is read once
+//    for all rows of x; a wave owns 16 weight rows and a slice of K, the four waves of a
+//    workgroup are summed in a fixed order.  K must be a multiple of 8.
+//
+// In every kernel an output element is a sum over k in an order that depends only on the
+// kernel and K, never on which other rows are in the batch.
+#include "common.h"
+
+// ============================================================== plain FMA product
+template <typename TA, typename TB, typename TC>
+__global__ __launch_bounds__(256) void gemm_plain_kernel(const TA* __restrict__ A,
+                                                         const TB* __restrict__ B,
+                                                         TC* __restrict__ C, int M, int N, int K,
+                                                         long long lda, long long ldb,
+                                                         long long ldc) {
+  constexpr int BM = 64, BN = 64, BK = 16;
+  __shared__ float As[BK][BM + 4];
+  __shared__ float Bs[BK][BN + 4];
+  const int tid = threadIdx.x;
+  const int tx = tid % 16, ty = tid / 16;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+  for (int k0 = 0; k0 < K; k0 += BK) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = tid + i * 256;
+      const int r = idx / BK, kk = idx % BK;
+      const int gm = m0 + r, gn = n0 + r, gk = k0 + kk;
+      As[kk][r] = (gm < M && gk < K) ? ld(A + (long long)gm * lda + gk) : 0.f;
+      Bs[kk][r] = (gn < N && gk < K) ? ld(B + (long long)gn * ldb + gk) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK; ++kk) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = Bs[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int gm = m0 + ty * 4 + i;
+    if (gm >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int gn = n0 + tx * 4 + j;
+      if (gn < N) st(C + (long long)gm * ldc + gn, acc[i][j]);
+    }
+  }
+}
+
+template <typename TA, typename TB, typename TC>
+static void launch_plain(const void* A, const void* B, void* C, int M, int N, int K,
+                         long long lda, long long ldb, long long ldc, hipStream_t stream) {
+  dim3 grid(ceil_div(N, 64), ceil_div(M, 64));
+  gemm_plain_kernel<TA, TB, TC><<<grid, 256, 0, stream>>>((const TA*)A, (const TB*)B, (TC*)C, M,
+                                                          N, K, lda, ldb, ldc);
+}
+
+// C (M,N) = A (M,K) * B (N,K)^T with row strides lda/ldb/ldc in elements.
+RLIS_API int rlis_gemm_plain(const void* A, int a_dtype, const void* B, int b_dtype, void* C,
+                             int c_dtype, int M, int N, int K, long long lda, long long ldb,
+                             long long ldc, hipStream_t stream) {
+  RLIS_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_plain: bad sizes M=%d N=%d K=%d", M, N, K);
+  RLIS_REQUIRE(lda >= K && ldb >= K && ldc >= N, "gemm_plain: row strides shorter than rows");
+  RLIS_REQUIRE(ceil_div(M, 64) <= 65535, "gemm_plain: M=%d is too large", M);
+  if (M == 0) return 0;
+  const int key = a_dtype * 4 + b_dtype * 2 + c_dtype;
+#define CASE(k, TA, TB, TC)                                                    \
+  case k:                                                                      \
+    launch_plain<TA, TB, TC>(A, B, C, M, N, K, lda, ldb, ldc, stream);         \
+    break;
+  switch (key) {
+    CASE(0, float, float, float)
+    CASE(1, float, float, bf16_t)
+    CASE(2, float, bf16_t, float)
+    CASE(3, float, bf16_t, bf16_t)
+    CASE(4, bf16_t, float, float)
+    CASE(5, bf16_t, float, bf16_t)
+    CASE(6, bf16_t, bf16_t, float)
+    CASE(7, bf16_t, bf16_t, bf16_t)
+    default:
+      RLIS_REQUIRE(false, "gemm_plain: unknown dtypes %d %d %d", a_dtype, b_dtype, c_dtype);
+  }
+#undef CASE
+  RLIS_LAUNCH_CHECK("gemm_plain");
+  return 0;
+}
+
+// ================================================================ MFMA bf16 product
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+union Frag8 {
+  uint4 u;
+  bf16x8 v;
+};
+
+// Tile 128 x 128 x 64, four waves in a 2 x 2 arrangement, each wave 64 x 64 as 2 x 2 blocks of
+// v_mfma_f32_32x32x16_bf16.  Operand fragments: lane l holds row (or column) l % 32 and the 8
+// consecutive k at (l / 32) * 8; the accumulator holds column l % 32 and rows
+// (r / 4) * 8 + (l / 32) * 4 + r % 4 for register r.
+template <typename TC>
+__global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __restrict__ A,
+                                                             const bf16_t* __restrict__ B,
+                                                             TC* __restrict__ C, int M, int N,
+                                                             int K, long long lda, long long ldb,
+                                                             long long ldc, int tiles_n) {
+  constexpr int BM = 128, BN = 128, BK = 64, LDS_STRIDE = BK + 8;  // in bf16 elements
+  __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS_STRIDE];
+  __shared__ __attribute__((aligned(16))) bf16_t Bs[BN * LDS_STRIDE];
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int wm = wave / 2, wn = wave % 2;
+  const int tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // Each thread moves 4 chunks of 8 bf16 per operand per tile: chunk c covers row c / 8,
+  // k offset (c % 8) * 8.
+  uint4 ra[4], rb[4];
+  auto load_global = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = tid + i * 256;
+      const int r = c / 8, kc = (c % 8) * 8;
+      const int gk = k0 + kc;
+      const int gm = m0 + r, gn = n0 + r;
+      ra[i] = (gm < M && gk < K) ? *(const uint4*)(A + (long long)gm * lda + gk)
+                                 : make_uint4(0, 0, 0, 0);
+      rb[i] = (gn < N && gk < K) ? *(const uint4*)(B + (long long)gn * ldb + gk)
+                                 : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto store_lds = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = tid + i * 256;
+      const int r = c / 8, kc = (c % 8) * 8;
+      *(uint4*)(As + r * LDS_STRIDE + kc) = ra[i];
+      *(uint4*)(Bs + r * LDS_STRIDE + kc) = rb[i];
+    }
+  };
+
+  const int num_k = (K + BK - 1) / BK;
+  load_global(0);
+  store_lds();
+  __syncthreads();
+  for (int kt = 0; kt < num_k; ++kt) {
+    if (kt + 1 < num_k) load_global((kt + 1) * BK);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      Frag8 a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int row = wm * 64 + i * 32 + (lane % 32);
+        a[i].u = *(const uint4*)(As + row * LDS_STRIDE + ks * 16 + (lane / 32) * 8);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int row = wn * 64 + j * 32 + (lane % 32);
+        b[j].u = *(const uint4*)(Bs + row * LDS_STRIDE + ks * 16 + (lane / 32) * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i].v, b[j].v, acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+    if (kt + 1 < num_k) {
+      store_lds();
+      __syncthreads();
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int gn = n0 + wn * 64 + j * 32 + (lane % 32);
+      if (gn >= N) continue;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int gm = m0 + wm * 64 + i * 32 + (r / 4) * 8 + (lane / 32) * 4 + (r % 4);
+        if (gm < M) st(C + (long long)gm * ldc + gn, acc[i][j][r]);
+      }
+    }
+}
+
+RLIS_API int rlis_gemm_bf16_mfma(const void* A, const void* B, void* C, int c_dtype, int M, int N,
+                                 int K, long long lda, long long ldb, long long ldc,
+                                 hipStream_t stream) {
+  RLIS_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16_mfma: bad sizes M=%d N=%d K=%d", M, N, K);
+  RLIS_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0,
+               "gemm_bf16_mfma: K=%d and the row strides must be multiples of 8", K);
+  RLIS_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)B % 16) == 0,
+               "gemm_bf16_mfma: operands must be 16-byte aligned");
+  RLIS_REQUIRE(lda >= K && ldb >= K && ldc >= N, "gemm_bf16_mfma: row strides shorter than rows");
+  if (M == 0) return 0;
+  const int tiles_m = ceil_div(M, 128), tiles_n = ceil_div(N, 128);
+  const long long blocks = (long long)tiles_m * tiles_n;
+  RLIS_REQUIRE(blocks < (1ll << 31), "gemm_bf16_mfma: too many tiles");
+  if (c_dtype == RLIS_F32)
+    gemm_bf16_mfma_kernel<float><<<(int)blocks, 256, 0, stream>>>(
+        (const bf16_t*)A, (const bf16_t*)B, (float*)C, M, N, K, lda, ldb, ldc, tiles_n);
+  else if (c_dtype == RLIS_BF16)
+    gemm_bf16_mfma_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>(
+        (const bf16_t*)A, (const bf16_t*)B, (bf16_t*)C, M, N, K, lda, ldb, ldc, tiles_n);
+  else
+    RLIS_REQUIRE(false, "gemm_bf16_mfma: unknown output dtype %d", c_dtype);
+  RLIS_LAUNCH_CHECK("gemm_bf16_mfma");
+  return 0;
+}
+
+// ============================================================ skinny (decode) product
+// y (T, N) = x (T, K) * W (N, K)^T for T <= 16 * NT.  Workgroup = 4 waves; it owns 16 weight
+// rows, wave w owns the k range [w * kslice, (w + 1) * kslice).  v_mfma_f32_16x16x32_bf16 with
+// the weight rows as the M side and the tokens as the N side: lane l holds weight row l % 16
+// (A) or token l % 16 (B) and the 8 consecutive k at (l / 16) * 8; the accumulator holds
+// token l % 16 and weight rows (l / 16) * 4 + r.
+template <typename TC, int NT>
+__global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ X,
+                                                               const bf16_t* __restrict__ W,
+                                                               TC* __restrict__ Y, int T, int N,
+                                                               int K, long long ldx,
+                                                               long long ldw, long long ldy,
+                                                               int kslice) {
+  __shared__ float red[4][NT][4][64];
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int n0 = blockIdx.x * 16;
+  const int wrow = n0 + (lane % 16);
+  const int kq = (lane / 16) * 8;
+  const bool wvalid = wrow < N;
+  const bf16_t* wp = W + (long long)(wvalid ? wrow : 0) * ldw;
+  const bf16_t* xp[NT];
+  bool xvalid[NT];
+#pragma unroll
+  for (int tt = 0; tt < NT; ++tt) {
+    const int tok = tt * 16 + (lane % 16);
+    xvalid[tt] = tok < T;
+    xp[tt] = X + (long long)(xvalid[tt] ? tok : 0) * ldx;
+  }
+  f32x4 acc[NT];
+#pragma unroll
+  for (int tt = 0; tt < NT; ++tt) acc[tt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  const int kbeg = wave * kslice;
+  const int kend = min(K, kbeg + kslice);
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  for (int k = kbeg; k < kend; k += 32) {
+    const int gk = k + kq;
+    const bool kin = gk < kend;  // kslice is a multiple of 32 and K of 8: whole chunks only
+    Frag8 a;
+    a.u = (wvalid && kin) ? *(const uint4*)(wp + gk) : zero;
+#pragma unroll
+    for (int tt = 0; tt < NT; ++tt) {
+      Frag8 b;
+      b.u = (xvalid[tt] && kin) ? *(const uint4*)(xp[tt] + gk) : zero;
+      acc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[tt], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int tt = 0; tt < NT; ++tt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][tt][r][lane] = acc[tt][r];
+  __syncthreads();
+  // 16 * NT tokens x 16 rows results, summed over the four waves in order.
+  for (int i = tid; i < NT * 256; i += 256) {
+    const int tt = i / 256, rem = i % 256;
+    const int r = rem / 64, l = rem % 64;
+    const float s = ((red[0][tt][r][l] + red[1][tt][r][l]) + red[2][tt][r][l]) + red[3][tt][r][l];
+    const int tok = tt * 16 + (l % 16);
+    const int row = n0 + (l / 16) * 4 + r;
+    if (tok < T && row < N) st(Y + (long long)tok * ldy + row, s);
+  }
+}
+
+RLIS_API int rlis_gemm_bf16_skinny(const void* X, const void* W, void* Y, int y_dtype, int T,
+                                   int N, int K, long long ldx, long long ldw, long long ldy,
+                                   hipStream_t stream) {
+  RLIS_REQUIRE(T >= 0 && T <= 64, "gemm_bf16_skinny: T=%d rows, at most 64", T);
+  RLIS_REQUIRE(N > 0 && K > 0, "gemm_bf16_skinny: bad sizes N=%d K=%d", N, K);
+  RLIS_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0,
+               "gemm_bf16_skinny: K=%d and the row strides must be multiples of 8", K);
+  RLIS_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0,
+               "gemm_bf16_skinny: operands must be 16-byte aligned");
+  RLIS_REQUIRE(ldx >= K && ldw >= K && ldy >= N, "gemm_bf16_skinny: row strides shorter than rows");
+  if (T == 0) return 0;
+  const int kslice = ceil_div(ceil_div(K, 4), 32) * 32;
+  const int blocks = ceil_div(N, 16);
+  const int nt = ceil_div(T, 16);
+#define LAUNCH(TC, NT)                                                                        \
+  gemm_bf16_skinny_kernel<TC, NT><<<blocks, 256, 0, stream>>>(                                \
+      (const bf16_t*)X, (const bf16_t*)W, (TC*)Y, T, N, K, ldx, ldw, ldy, kslice)
+  if (y_dtype == RLIS_F32) {
+    switch (nt) {
+      case 1: LAUNCH(float, 1); break;
+      case 2: LAUNCH(float, 2); break;
+      case 3: LAUNCH(float, 3); break;
+      default: LAUNCH(float, 4); break;
+    }
+  } else if (y_dtype == RLIS_BF16) {
+    switch (nt) {
+      case 1: LAUNCH(bf16_t, 1); break;
+      case 2: LAUNCH(bf16_t, 2); break;
+      case 3: LAUNCH(bf16_t, 3); break;
+      default: LAUNCH(bf16_t, 4); break;
+    }
+  } else {
+    RLIS_REQUIRE(false, "gemm_bf16_skinny: unknown output dtype %d", y_dtype);
+  }
+#undef LAUNCH
+  RLIS_LAUNCH_CHECK("gemm_bf16_skinny");
+  return 0;
+}

@@ -1,0 +1,191 @@
+// C entry points of the host runtime (page manager and scheduler) for the Python binding.
+// Handles are opaque pointers; functions return a negative value and keep a message for
+// rlis_rt_last_error() when an argument is wrong or an internal check fails.
+#include <cstring>
+#include <exception>
+#include <string>
+
+#include "cache_manager.h"
+#include "scheduler.h"
+
+#define RT_API extern "C" __attribute__((visibility("default")))
+
+using rlis::CacheManager;
+using rlis::Scheduler;
+
+static thread_local std::string g_error;
+
+RT_API const char* rlis_rt_last_error() { return g_error.c_str(); }
+
+#define GUARD(expr)                     \
+  try {                                 \
+    expr;                               \
+  } catch (const std::exception& e) {   \
+    g_error = e.what();                 \
+    return -1;                          \
+  }
+
+static int copy_message(const std::string& msg, char* buf, int cap) {
+  if (buf && cap > 0) {
+    std::strncpy(buf, msg.c_str(), cap - 1);
+    buf[cap - 1] = 0;
+  }
+  return msg.empty() ? 0 : 1;
+}
+
+// ------------------------------------------------------------------------ cache
+RT_API void* rlis_cache_create(int page_size, int num_groups, const int* windows,
+                               const int* num_pages, int num_state_slots) {
+  try {
+    std::vector<rlis::GroupSpec> groups;
+    for (int g = 0; g < num_groups; ++g) groups.push_back({windows[g], num_pages[g]});
+    return new CacheManager(page_size, groups, num_state_slots);
+  } catch (const std::exception& e) {
+    g_error = e.what();
+    return nullptr;
+  }
+}
+
+RT_API void rlis_cache_destroy(void* h) { delete static_cast<CacheManager*>(h); }
+
+// Returns 0 reserved, 1 out of pages, 2 out of state slots.  Copies come back as triples
+// (group, src, dst); more than `cap` of them is an error.
+RT_API int rlis_cache_reserve(void* h, long long seq, int total, int* copies, int cap, int* n_copies) {
+  auto* m = static_cast<CacheManager*>(h);
+  std::vector<rlis::PageCopy> out;
+  int rc = 0;
+  GUARD(rc = m->reserve(seq, total, &out));
+  if ((int)out.size() > cap) {
+    g_error = "copy list does not fit";
+    return -1;
+  }
+  for (size_t i = 0; i < out.size(); ++i) {
+    copies[3 * i] = out[i].group;
+    copies[3 * i + 1] = out[i].src;
+    copies[3 * i + 2] = out[i].dst;
+  }
+  if (n_copies) *n_copies = (int)out.size();
+  return rc;
+}
+
+RT_API int rlis_cache_advance(void* h, long long seq, int computed) {
+  GUARD(static_cast<CacheManager*>(h)->advance(seq, computed));
+  return 0;
+}
+
+RT_API int rlis_cache_fork(void* h, long long parent, long long child) {
+  GUARD(static_cast<CacheManager*>(h)->fork(parent, child));
+  return 0;
+}
+
+RT_API int rlis_cache_free(void* h, long long seq) {
+  GUARD(static_cast<CacheManager*>(h)->free_seq(seq));
+  return 0;
+}
+
+RT_API int rlis_cache_num_free(void* h, int g) { return static_cast<CacheManager*>(h)->num_free(g); }
+RT_API int rlis_cache_num_pages(void* h, int g) { return static_cast<CacheManager*>(h)->num_pages(g); }
+RT_API int rlis_cache_refcount(void* h, int g, int p) { return static_cast<CacheManager*>(h)->refcount(g, p); }
+RT_API int rlis_cache_num_free_slots(void* h) { return static_cast<CacheManager*>(h)->num_free_slots(); }
+RT_API int rlis_cache_contains(void* h, long long seq) { return static_cast<CacheManager*>(h)->contains(seq); }
+
+RT_API int rlis_cache_pages_needed(void* h, long long seq, int total, int g) {
+  return static_cast<CacheManager*>(h)->pages_needed(seq, total, g);
+}
+
+// Writes the block table of (seq, group) into out (up to cap entries) and returns its
+// length, or -1 for an unknown request.
+RT_API int rlis_cache_table(void* h, long long seq, int g, int* out, int cap) {
+  const rlis::SeqEntry* e = static_cast<CacheManager*>(h)->entry(seq);
+  if (!e) return -1;
+  const auto& pages = e->pages[g];
+  const int n = (int)pages.size() < cap ? (int)pages.size() : cap;
+  for (int i = 0; i < n; ++i) out[i] = pages[i];
+  return (int)pages.size();
+}
+
+// info[0..2] = reserved tokens, computed tokens, state slot; returns -1 for an unknown request.
+RT_API int rlis_cache_info(void* h, long long seq, int* info) {
+  const rlis::SeqEntry* e = static_cast<CacheManager*>(h)->entry(seq);
+  if (!e) return -1;
+  info[0] = e->num_tokens;
+  info[1] = e->num_computed;
+  info[2] = e->state_slot;
+  return 0;
+}
+
+RT_API int rlis_cache_check(void* h, char* buf, int cap) {
+  return copy_message(static_cast<CacheManager*>(h)->check_invariants(), buf, cap);
+}
+
+// -------------------------------------------------------------------- scheduler
+RT_API void* rlis_sched_create(void* cache, int max_num_seqs, int max_batched_tokens,
+                               int watermark_pages, int policy) {
+  try {
+    rlis::SchedulerConfig cfg{max_num_seqs, max_batched_tokens, watermark_pages,
+                              policy == 1 ? rlis::kStatic : rlis::kContinuous};
+    return new Scheduler(cfg, static_cast<CacheManager*>(cache));
+  } catch (const std::exception& e) {
+    g_error = e.what();
+    return nullptr;
+  }
+}
+
+RT_API void rlis_sched_destroy(void* h) { delete static_cast<Scheduler*>(h); }
+
+RT_API int rlis_sched_add(void* h, long long id, int prompt_len) {
+  GUARD(static_cast<Scheduler*>(h)->add(id, prompt_len));
+  return 0;
+}
+
+// seqs: triples (id, start, end) as long long; copies: triples (group, src, dst).
+RT_API int rlis_sched_schedule(void* h, long long* seqs, int seq_cap, int* n_seqs,
+                               long long* preempted, int pre_cap, int* n_pre, int* copies,
+                               int copy_cap, int* n_copies) {
+  rlis::Schedule s;
+  GUARD(s = static_cast<Scheduler*>(h)->schedule());
+  if ((int)s.seqs.size() > seq_cap || (int)s.preempted.size() > pre_cap ||
+      (int)s.copies.size() > copy_cap) {
+    g_error = "schedule does not fit the buffers";
+    return -1;
+  }
+  for (size_t i = 0; i < s.seqs.size(); ++i) {
+    seqs[3 * i] = s.seqs[i].id;
+    seqs[3 * i + 1] = s.seqs[i].start;
+    seqs[3 * i + 2] = s.seqs[i].end;
+  }
+  for (size_t i = 0; i < s.preempted.size(); ++i) preempted[i] = s.preempted[i];
+  for (size_t i = 0; i < s.copies.size(); ++i) {
+    copies[3 * i] = s.copies[i].group;
+    copies[3 * i + 1] = s.copies[i].src;
+    copies[3 * i + 2] = s.copies[i].dst;
+  }
+  *n_seqs = (int)s.seqs.size();
+  *n_pre = (int)s.preempted.size();
+  *n_copies = (int)s.copies.size();
+  return 0;
+}
+
+RT_API int rlis_sched_advance(void* h, long long id, int end) {
+  GUARD(static_cast<Scheduler*>(h)->advance(id, end));
+  return 0;
+}
+RT_API int rlis_sched_append_token(void* h, long long id) {
+  GUARD(static_cast<Scheduler*>(h)->append_token(id));
+  return 0;
+}
+RT_API int rlis_sched_is_caught_up(void* h, long long id) { return static_cast<Scheduler*>(h)->is_caught_up(id); }
+RT_API int rlis_sched_remove(void* h, long long id) {
+  GUARD(static_cast<Scheduler*>(h)->remove(id));
+  return 0;
+}
+RT_API int rlis_sched_has_work(void* h) { return static_cast<Scheduler*>(h)->has_work(); }
+RT_API int rlis_sched_num_running(void* h) { return static_cast<Scheduler*>(h)->num_running(); }
+RT_API int rlis_sched_num_waiting(void* h) { return static_cast<Scheduler*>(h)->num_waiting(); }
+RT_API long long rlis_sched_num_preemptions(void* h) { return static_cast<Scheduler*>(h)->num_preemptions(); }
+RT_API int rlis_sched_max_seq_tokens(void* h) { return static_cast<Scheduler*>(h)->max_seq_tokens(); }
+RT_API int rlis_sched_num_tokens(void* h, long long id) { return static_cast<Scheduler*>(h)->num_tokens(id); }
+RT_API int rlis_sched_num_computed(void* h, long long id) { return static_cast<Scheduler*>(h)->num_computed(id); }
+RT_API int rlis_sched_check(void* h, char* buf, int cap) {
+  return copy_message(static_cast<Scheduler*>(h)->check(), buf, cap);
+}

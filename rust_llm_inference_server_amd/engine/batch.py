@@ -1,0 +1,165 @@
+"""Per-step metadata: what one batch of (request, its next tokens) looks like to the kernels.
+
+The reference builds the same per step in ``PagedBatch::new`` (crates/model/src/paged.rs:
+256-296): positions ``P_i .. P_i + n_i`` of every sequence concatenated in batch order
+(llama.rs:252), the write slot ``table[pos / page] * page + pos % page`` of every new token
+(paged.rs:258-263), zero-padded block tables and context lengths (paged.rs:199-213).  Here one
+slot id per token is enough (the write kernel spreads it over heads and dims), and all of it
+goes to the device in one copy."""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+PREFILL_TILE = 64     # new tokens per workgroup of the matrix-core prefill attention
+
+
+@dataclass
+class StepEntry:
+    """One request's part of a step: its next ``tokens`` (continuing exactly at its cached
+    length) and ``want``, the indices among them whose logits are asked for."""
+    seq_id: int
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class GroupStep:
+    page_size: int
+    window: Optional[int]
+    block_tables: torch.Tensor        # (S, max_pages) int32
+    slots: torch.Tensor               # (T) int32
+
+
+@dataclass
+class StepContext:
+    num_tokens: int
+    num_seqs: int
+    ids: torch.Tensor                 # (T) int32
+    positions: torch.Tensor           # (T) int32, absolute
+    seq_of_token: torch.Tensor        # (T) int32, index into the step's sequences
+    cu_seqlens: torch.Tensor          # (S + 1) int32
+    start_pos: torch.Tensor           # (S) int32: positions cached before the step
+    ctx_lens: torch.Tensor            # (S) int32: positions cached after the step
+    logit_rows: torch.Tensor          # (R) int32: token rows whose logits are wanted
+    num_logit_rows: int
+    state_slots: torch.Tensor         # (S) int32
+    tile_map: torch.Tensor            # (num_tiles, 2) int32: (sequence, first new-token index)
+    num_tiles: int
+    groups: List[GroupStep]
+    max_context: int
+    max_new: int
+    all_decode: bool
+    decode_splits: Optional[int] = None
+    # Host copies, for parts that plan on the host.
+    host_start_pos: List[int] = field(default_factory=list)
+    host_new: List[int] = field(default_factory=list)
+    host_state_slots: List[int] = field(default_factory=list)
+
+
+def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
+               vocab_size: int) -> StepContext:
+    """Lay out a step.  Every entry's request must hold reserved positions for its tokens."""
+    if not entries:
+        raise ValueError("a step needs at least one request")
+    ps = cache.page_size
+    ids: List[int] = []
+    positions: List[int] = []
+    seq_of_token: List[int] = []
+    cu = [0]
+    start_pos: List[int] = []
+    ctx_lens: List[int] = []
+    logit_rows: List[int] = []
+    state_slots: List[int] = []
+    tiles: List[int] = []
+    ng = cache.num_groups
+    tables: List[List[List[int]]] = [[] for _ in range(ng)]
+    slots: List[List[int]] = [[] for _ in range(ng)]
+    seen = set()
+    for s, e in enumerate(entries):
+        n = len(e.tokens)
+        if n == 0:
+            raise ValueError("empty sequence in batch")          # llama.rs:231-233
+        if e.seq_id in seen:
+            raise ValueError(f"request {e.seq_id} appears twice in one step")
+        seen.add(e.seq_id)
+        if not cache.contains(e.seq_id):
+            raise ValueError(f"request {e.seq_id}: position 0 has no page reserved")
+        reserved, computed, slot = cache._get_info(e.seq_id)
+        if computed + n > reserved:
+            # paged.rs:258-263 "position {pos} has no block reserved"
+            raise ValueError(f"request {e.seq_id}: position {reserved} has no page reserved")
+        for t in e.tokens:
+            if not 0 <= int(t) < vocab_size:
+                raise ValueError(f"request {e.seq_id}: token id {t} is outside the vocabulary "
+                                 f"of {vocab_size}")
+        base = len(ids)
+        ids.extend(int(t) for t in e.tokens)
+        positions.extend(range(computed, computed + n))
+        seq_of_token.extend([s] * n)
+        cu.append(base + n)
+        start_pos.append(computed)
+        ctx_lens.append(computed + n)
+        state_slots.append(max(slot, 0))
+        for w in e.want:
+            if not 0 <= int(w) < n:
+                raise ValueError(f"request {e.seq_id}: wanted index {w} is outside its {n} tokens")
+            logit_rows.append(base + int(w))
+        tiles.extend(x for qb in range(0, n, PREFILL_TILE) for x in (s, qb))
+        for g in range(ng):
+            table = cache.table(e.seq_id, g)
+            tables[g].append(table)
+            for p in range(computed, computed + n):
+                page = table[p // ps]
+                if page < 0:
+                    raise ValueError(f"request {e.seq_id}: position {p} has no page reserved")
+                slots[g].append(page * ps + p % ps)
+    T, S = len(ids), len(entries)
+    widths = [max(8, -(-max(len(t) for t in tables[g]) // 8) * 8) for g in range(ng)]
+    flat: List[int] = []
+    offsets = {}
+
+    def put(name, values):
+        offsets[name] = (len(flat), len(values))
+        flat.extend(values)
+        flat.extend([0] * (-len(flat) % 4))     # keep every array 16-byte aligned
+
+    put("ids", ids)
+    put("positions", positions)
+    put("seq_of_token", seq_of_token)
+    put("cu", cu)
+    put("start_pos", start_pos)
+    put("ctx_lens", ctx_lens)
+    put("logit_rows", logit_rows)
+    put("state_slots", state_slots)
+    put("tiles", tiles)
+    for g in range(ng):
+        put(f"slots{g}", slots[g])
+        rows: List[int] = []
+        for t in tables[g]:
+            rows.extend(max(p, 0) for p in t)
+            rows.extend([0] * (widths[g] - len(t)))
+        put(f"tables{g}", rows)
+    host = torch.tensor(flat, dtype=torch.int32)
+    if device.type == "cuda":
+        host = host.pin_memory()
+    dev = host.to(device, non_blocking=True)
+
+    def view(name):
+        o, n = offsets[name]
+        return dev[o:o + n]
+
+    groups = [GroupStep(page_size=ps, window=cache.groups[g].window,
+                        block_tables=view(f"tables{g}").reshape(S, widths[g]),
+                        slots=view(f"slots{g}")) for g in range(ng)]
+    return StepContext(
+        num_tokens=T, num_seqs=S, ids=view("ids"), positions=view("positions"),
+        seq_of_token=view("seq_of_token"), cu_seqlens=view("cu"), start_pos=view("start_pos"),
+        ctx_lens=view("ctx_lens"), logit_rows=view("logit_rows"), num_logit_rows=len(logit_rows),
+        state_slots=view("state_slots"), tile_map=view("tiles"), num_tiles=len(tiles) // 2,
+        groups=groups, max_context=max(ctx_lens), max_new=max(len(e.tokens) for e in entries),
+        all_decode=all(len(e.tokens) == 1 for e in entries),
+        host_start_pos=start_pos, host_new=[len(e.tokens) for e in entries],
+        host_state_slots=state_slots)

@@ -1,0 +1,148 @@
+"""The step function and what it owns: the model's parts, the page manager and the pools.
+
+``ModelRunner.step(entries)`` runs one batch of (request, its next tokens): portions of
+prompts beside single decoded tokens, cut anywhere.  It computes only the tokens it is given,
+reads everything earlier from the cache, writes the new keys and values there, and returns
+float32 logits at the wanted rows.  It is the one forward path: the engine, the replay
+program, the perplexity tool and the benchmark all call it.  Its contract is the reference's
+``Llama::forward_batch`` over a ``PagedBatch`` (crates/model/src/llama.rs:216-286;
+crates/model/src/paged.rs:154-161, 255-296)."""
+from __future__ import annotations
+
+import os
+from typing import Dict, List, Optional, Sequence, Union
+
+import torch
+
+from ..cache.manager import CacheManager, GroupSpec
+from ..cache.pools import CachePools
+from ..models.spec import Model, ModelSpec
+from ..registry import architecture_of, read_config_dict
+from ..weights.loader import load_weights
+from ..weights.random_init import random_weights
+from .batch import StepContext, StepEntry, build_step
+
+DTYPES = {"float32": torch.float32, "fp32": torch.float32, "f32": torch.float32,
+          "bfloat16": torch.bfloat16, "bf16": torch.bfloat16}
+
+
+def parse_dtype(name: Union[str, torch.dtype]) -> torch.dtype:
+    if isinstance(name, torch.dtype):
+        if name not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"dtype {name} is not supported (float32 or bfloat16)")
+        return name
+    try:
+        return DTYPES[name.lower()]
+    except KeyError:
+        raise ValueError(f"dtype '{name}' is not supported (float32 or bfloat16)") from None
+
+
+def default_device() -> torch.device:
+    if not torch.cuda.is_available():
+        raise RuntimeError("no GPU is visible: this engine runs on an AMD GPU only")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def load_model(folder: str, dtype: Union[str, torch.dtype], max_positions: int,
+               device: Optional[torch.device] = None) -> Model:
+    """Build the model a folder holds: the architecture named in ``config.json`` chooses the
+    configuration class and the specification, the safetensors files give the weights."""
+    device = device or default_device()
+    act = parse_dtype(dtype)
+    cfg_dict = read_config_dict(folder)
+    arch = architecture_of(cfg_dict)
+    cfg = arch.parse_config(cfg_dict)
+    spec = arch.build_spec(cfg)
+    weights = load_weights(folder, spec.tensor_specs(), act, device, spec.optional_tensors)
+    limit = getattr(cfg, "max_position_embeddings", max_positions)
+    model = Model(spec, weights, act, device, min(max_positions, limit))
+    model.config = cfg
+    return model
+
+
+def random_model(config: Union[dict, object], seed: int, dtype: Union[str, torch.dtype],
+                 max_positions: int, device: Optional[torch.device] = None,
+                 architecture: str = "LlamaForCausalLM") -> Model:
+    """A model with seeded random weights, built in memory from a configuration."""
+    from ..registry import architecture as lookup
+    device = device or default_device()
+    act = parse_dtype(dtype)
+    if isinstance(config, dict):
+        arch = architecture_of(config) if "architectures" in config else lookup(architecture)
+        cfg = arch.parse_config(config)
+    else:
+        arch, cfg = lookup(getattr(config, "architecture", architecture)), config
+    spec = arch.build_spec(cfg)
+    weights = random_weights(spec.tensor_specs(), seed, act, device)
+    limit = getattr(cfg, "max_position_embeddings", max_positions)
+    model = Model(spec, weights, act, device, min(max_positions, limit))
+    model.config = cfg
+    return model
+
+
+class ModelRunner:
+    """A model with its cache.  ``num_pages`` sizes every page group's pool."""
+
+    def __init__(self, model: Model, num_pages: int, page_size: int = 16,
+                 max_num_seqs: int = 64, max_batched_tokens: Optional[int] = None):
+        self.model = model
+        self.device = model.device
+        self.page_size = page_size
+        self.max_num_seqs = max_num_seqs
+        self.max_batched_tokens = max_batched_tokens
+        groups = [GroupSpec(num_pages, g.request.window) for g in model.cache_groups]
+        if not groups:
+            groups = [GroupSpec(num_pages, None)]      # the manager always has one group
+        self.cache = CacheManager(page_size, groups,
+                                  max_num_seqs if model.state_bytes else 0)
+        self.pools = CachePools(model.cache_groups, [num_pages] * len(model.cache_groups),
+                                page_size, model.act_dtype, model.device,
+                                max_num_seqs if model.state_bytes else 0, model.state_bytes)
+        self.vocab_size = model.spec.vocab_size
+
+    # ------------------------------------------------------------------- pages
+    def reserve(self, seq_id: int, total_tokens: int) -> None:
+        """Make positions ``[0, total_tokens)`` of a request addressable; raises
+        ``OutOfPages`` (and changes nothing) when the pools cannot hold them."""
+        if total_tokens > self.model.max_positions:
+            raise ValueError(f"sequence of {total_tokens} positions exceeds max_seq_len "
+                             f"{self.model.max_positions}")
+        self.apply_copies(self.cache.reserve(seq_id, total_tokens))
+
+    def apply_copies(self, copies) -> None:
+        by_group: Dict[int, List] = {}
+        for c in copies:
+            by_group.setdefault(c.group, []).append(c)
+        for g, cs in by_group.items():
+            if g < len(self.pools.k):
+                self.pools.copy_pages(g, [c.src for c in cs], [c.dst for c in cs])
+
+    def free(self, seq_id: int) -> None:
+        self.cache.free(seq_id)
+
+    def num_computed(self, seq_id: int) -> int:
+        return self.cache.num_computed(seq_id)
+
+    # -------------------------------------------------------------------- step
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run one batch; returns float32 logits ``(wanted rows, vocab)`` in the order of the
+        entries and of their ``want`` lists."""
+        if len(entries) > self.max_num_seqs:
+            raise ValueError(f"{len(entries)} requests in one step, max_num_seqs is "
+                             f"{self.max_num_seqs}")
+        total = sum(len(e.tokens) for e in entries)
+        if self.max_batched_tokens is not None and total > self.max_batched_tokens:
+            raise ValueError(f"{total} tokens in one step, max_batched_tokens is "
+                             f"{self.max_batched_tokens}")
+        step = build_step(entries, self.cache, self.device, self.vocab_size)
+        if step.max_context > self.model.max_positions:
+            raise ValueError(f"sequence of {step.max_context} positions exceeds max_seq_len "
+                             f"{self.model.max_positions}")
+        if self.pools.state is not None:
+            for start, slot in zip(step.host_start_pos, step.host_state_slots):
+                if start == 0:
+                    self.pools.zero_state(slot)      # a fresh (or recomputed) request
+        logits = self.model.forward(step, self.pools)
+        for e, start in zip(entries, step.host_start_pos):
+            self.cache.advance(e.seq_id, start + len(e.tokens))
+        return logits

@@ -1,0 +1,319 @@
+"""The kernels as Python functions over torch tensors on the GPU.
+
+Each function checks on the host that shapes, dtypes, strides and alignment are what its
+kernel and grid assume, then launches on torch's current stream.  Nothing here computes on
+the CPU; without the compiled library or without a GPU the first call raises.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from . import lib
+from .lib import KernelError
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+# bf16 products with at most this many rows of x take the skinny kernel.
+SKINNY_MAX_ROWS = 64
+# "library": bf16 products with more rows and bf16 output go to torch.matmul (hipBLASLt);
+# "own": they take the hand-written matrix-core kernel.
+BF16_GEMM = "library"
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise KernelError(f"unsupported dtype {t.dtype} (float32 and bfloat16 only)") from None
+
+
+def _check(t: torch.Tensor, name: str, dtype=None, ndim: Optional[int] = None) -> None:
+    if not t.is_cuda:
+        raise KernelError(f"{name}: tensor is on {t.device}, kernels run on the GPU only")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: expected {dtype}, got {t.dtype}")
+    if ndim is not None and t.dim() != ndim:
+        raise KernelError(f"{name}: expected {ndim} dimensions, got shape {tuple(t.shape)}")
+
+
+def _rows_contig(t: torch.Tensor, name: str) -> int:
+    """Row stride of a 2-D tensor whose rows are contiguous."""
+    _check(t, name, ndim=2)
+    if t.shape[1] > 1 and t.stride(1) != 1:
+        raise KernelError(f"{name}: rows must be contiguous, strides are {t.stride()}")
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+
+def _i32(t: torch.Tensor, name: str, n: Optional[int] = None) -> int:
+    _check(t, name, torch.int32)
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: must be contiguous")
+    if n is not None and t.numel() < n:
+        raise KernelError(f"{name}: needs {n} entries, has {t.numel()}")
+    return t.data_ptr()
+
+
+# --------------------------------------------------------------------------- rows
+def embed(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """Rows ``table[ids]`` as the float32 residual stream ``(T, H)``."""
+    _check(table, "embed table", ndim=2)
+    T, (V, H) = ids.numel(), table.shape
+    if not table.is_contiguous():
+        raise KernelError("embed table must be contiguous")
+    out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    lib.call("rlis_embed", out.data_ptr(), table.data_ptr(), _dt(table), _i32(ids, "ids", T),
+             T, H, lib.stream_ptr())
+    return out
+
+
+def add_residual(resid: torch.Tensor, delta: torch.Tensor) -> None:
+    """``resid += delta`` with the sum formed in float32."""
+    _check(resid, "residual", torch.float32)
+    _check(delta, "delta")
+    if resid.shape != delta.shape or not (resid.is_contiguous() and delta.is_contiguous()):
+        raise KernelError("add_residual: shapes differ or tensors are not contiguous")
+    lib.call("rlis_add_residual", resid.data_ptr(), delta.data_ptr(), _dt(delta), resid.numel(),
+             lib.stream_ptr())
+
+
+def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
+                eps: float, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
+                write_resid: bool = True) -> torch.Tensor:
+    """``norm(resid + delta) * weight`` row by row.
+
+    With ``rows`` only those rows are produced and the residual is left as it is; otherwise
+    the sum is stored back into ``resid`` when ``write_resid`` is set."""
+    _check(resid, "residual", torch.float32, 2)
+    T, H = resid.shape
+    if not resid.is_contiguous():
+        raise KernelError("add_rmsnorm: residual must be contiguous")
+    if delta is not None:
+        _check(delta, "delta", ndim=2)
+        if delta.shape != resid.shape or not delta.is_contiguous():
+            raise KernelError("add_rmsnorm: delta must match the residual and be contiguous")
+    _check(weight, "norm weight", ndim=1)
+    if weight.numel() != H or not weight.is_contiguous():
+        raise KernelError(f"add_rmsnorm: weight has {weight.numel()} entries, rows have {H}")
+    if rows is not None:
+        R, rows_ptr, write_resid = rows.numel(), _i32(rows, "rows"), False
+    else:
+        R, rows_ptr = T, None
+    out = torch.empty((R, H), dtype=out_dtype, device=resid.device)
+    lib.call("rlis_add_rmsnorm", resid.data_ptr(),
+             None if delta is None else delta.data_ptr(), 0 if delta is None else _dt(delta),
+             weight.data_ptr(), _dt(weight), out.data_ptr(), _DT[out_dtype], rows_ptr, R, H,
+             float(eps), int(bool(write_resid)), lib.stream_ptr())
+    return out
+
+
+def swiglu(gu: torch.Tensor) -> torch.Tensor:
+    """``silu(gu[:, :I]) * gu[:, I:]`` for ``gu`` of shape ``(T, 2 I)``."""
+    _check(gu, "gate/up", ndim=2)
+    T, two_i = gu.shape
+    if two_i % 2 or not gu.is_contiguous():
+        raise KernelError("swiglu: input must be contiguous with an even number of columns")
+    out = torch.empty((T, two_i // 2), dtype=gu.dtype, device=gu.device)
+    lib.call("rlis_swiglu", out.data_ptr(), gu.data_ptr(), _dt(gu), T, two_i // 2,
+             lib.stream_ptr())
+    return out
+
+
+# ----------------------------------------------------------------------- products
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None
+           ) -> torch.Tensor:
+    """``x @ w.T`` for ``x (T, K)`` and ``w (N, K)``, float32 accumulation.
+
+    A float32 weight (or float32 ``x``) takes the plain FMA kernel, the true 32-bit product.
+    bfloat16 operands take the skinny kernel up to 64 rows, else the matrix-core GEMM (ours
+    for float32 output, the library's or ours for bfloat16 output)."""
+    ldx = _rows_contig(x, "linear x")
+    ldw = _rows_contig(w, "linear weight")
+    T, K = x.shape
+    N, K2 = w.shape
+    if K != K2:
+        raise KernelError(f"linear: x has {K} columns, the weight {K2}")
+    out_dtype = out_dtype or x.dtype
+    stream = lib.stream_ptr()
+    bf16 = x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+    aligned = (K % 8 == 0 and ldx % 8 == 0 and ldw % 8 == 0
+               and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+    if bf16 and aligned and T > SKINNY_MAX_ROWS and out_dtype == torch.bfloat16 \
+            and BF16_GEMM == "library":
+        return torch.matmul(x, w.t())
+    y = torch.empty((T, N), dtype=out_dtype, device=x.device)
+    if T == 0:
+        return y
+    if bf16 and aligned:
+        name = "rlis_gemm_bf16_skinny" if T <= SKINNY_MAX_ROWS else "rlis_gemm_bf16_mfma"
+        lib.call(name, x.data_ptr(), w.data_ptr(), y.data_ptr(), _DT[out_dtype], T, N, K, ldx,
+                 ldw, N, stream)
+    else:
+        lib.call("rlis_gemm_plain", x.data_ptr(), _dt(x), w.data_ptr(), _dt(w), y.data_ptr(),
+                 _DT[out_dtype], T, N, K, ldx, ldw, N, stream)
+    return y
+
+
+# ------------------------------------------------------------ rotation + cache write
+def rope_kv_write(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                  cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                  positions: torch.Tensor, slots: Optional[torch.Tensor],
+                  k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor],
+                  page_size: int, write_kv: bool = True) -> None:
+    """Rotate the q and k heads of ``qkv (T, (nh + 2 nkv) d)`` by their positions (q in
+    place) and, when ``write_kv``, store rotated k and v into the pages at ``slots``.
+
+    ``cos``/``sin`` are float32 ``(max_positions, rot_dim / 2)``; None means no rotation.
+    ``k_pages (pages, nkv, page, d)``, ``v_pages (pages, nkv, d, page)``."""
+    stride = _rows_contig(qkv, "qkv")
+    T = qkv.shape[0]
+    nh, nkv, d = num_heads, num_kv_heads, head_dim
+    if qkv.shape[1] != (nh + 2 * nkv) * d:
+        raise KernelError(f"rope_kv_write: qkv has {qkv.shape[1]} columns, expected "
+                          f"{(nh + 2 * nkv) * d}")
+    if cos is None:
+        rot, cos_ptr, sin_ptr = 0, None, None
+    else:
+        _check(cos, "cos", torch.float32, 2)
+        _check(sin, "sin", torch.float32, 2)
+        if cos.shape != sin.shape or not (cos.is_contiguous() and sin.is_contiguous()):
+            raise KernelError("rope_kv_write: cos and sin must match and be contiguous")
+        rot, cos_ptr, sin_ptr = 2 * cos.shape[1], cos.data_ptr(), sin.data_ptr()
+        if rot > d:
+            raise KernelError(f"rope_kv_write: rotation width {rot} exceeds head_dim {d}")
+    kp = vp = sp = None
+    if write_kv:
+        if k_pages is None or v_pages is None or slots is None:
+            raise KernelError("rope_kv_write: a cache write needs pages and slots")
+        for t, name, shape in ((k_pages, "k_pages", (nkv, page_size, d)),
+                               (v_pages, "v_pages", (nkv, d, page_size))):
+            _check(t, name, qkv.dtype, 4)
+            if tuple(t.shape[1:]) != shape or not t.is_contiguous():
+                raise KernelError(f"rope_kv_write: {name} has shape {tuple(t.shape)}, expected "
+                                  f"(pages, {shape[0]}, {shape[1]}, {shape[2]}) contiguous")
+        kp, vp, sp = k_pages.data_ptr(), v_pages.data_ptr(), _i32(slots, "slots", T)
+    lib.call("rlis_rope_kv_write", qkv.data_ptr(), _dt(qkv), stride, nh * d, (nh + nkv) * d, T,
+             nh, nkv, d, rot, cos_ptr, sin_ptr, _i32(positions, "positions", T), sp, kp, vp,
+             page_size, int(bool(write_kv)), lib.stream_ptr())
+
+
+def copy_pages(pages: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
+    """``pages (layers, num_pages, ...)``: copy page ``src[i]`` onto ``dst[i]`` in every layer."""
+    _check(pages, "pages")
+    if pages.dim() < 3 or not pages.is_contiguous():
+        raise KernelError("copy_pages: pages must be (layers, num_pages, ...) contiguous")
+    n = src.numel()
+    if dst.numel() != n:
+        raise KernelError("copy_pages: src and dst differ in length")
+    page_elems = pages[0, 0].numel()
+    lib.call("rlis_copy_pages", pages.data_ptr(), _dt(pages), pages.shape[0], pages.shape[1],
+             page_elems, _i32(src, "src"), _i32(dst, "dst"), n, lib.stream_ptr())
+
+
+# ----------------------------------------------------------------------- attention
+def decode_splits(num_seqs: int, num_kv_heads: int, group: int, max_context: int) -> int:
+    """Partitions per context for the decode kernel: enough workgroups to fill 256 compute
+    units twice, at least 256 positions each (the rule of crates/model/src/
+    paged_attention.rs:21-36, with the target sized for this chip)."""
+    pairs = max(1, num_seqs * num_kv_heads * math.ceil(group / 8))
+    return max(1, min(math.ceil(512 / pairs), math.ceil(max_context / 256)))
+
+
+def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                    k_pages: torch.Tensor, v_pages: torch.Tensor, page_size: int,
+                    block_tables: torch.Tensor, step, scale: float,
+                    window: Optional[int] = None, force: Optional[str] = None) -> torch.Tensor:
+    """Attention of the step's new tokens over the paged cache -> ``(T, nh * d)``.
+
+    ``qkv`` holds the rotated queries in its first ``nh * d`` columns; K and V of the new
+    tokens are already in the pages.  ``step`` is the ``StepContext`` (token and sequence
+    metadata on the device).  The kernel is chosen from the shape of the batch: every
+    sequence brings one token -> decode kernel; bfloat16 with multi-token sequences ->
+    matrix-core prefill kernel; float32, or sizes those kernels refuse -> generic kernel.
+    ``force`` names one of 'generic', 'decode', 'prefill' for tests."""
+    q_stride = _rows_contig(qkv, "qkv")
+    T = qkv.shape[0]
+    nh, nkv, d = num_heads, num_kv_heads, head_dim
+    if nh % nkv:
+        raise KernelError(f"attention: {nh} query heads are not a multiple of {nkv} KV heads")
+    for t, name, shape in ((k_pages, "k_pages", (nkv, page_size, d)),
+                           (v_pages, "v_pages", (nkv, d, page_size))):
+        _check(t, name, qkv.dtype, 4)
+        if tuple(t.shape[1:]) != shape or not t.is_contiguous():
+            raise KernelError(f"attention: {name} has shape {tuple(t.shape)}, expected "
+                              f"(pages, {shape[0]}, {shape[1]}, {shape[2]}) contiguous")
+    _check(block_tables, "block_tables", torch.int32, 2)
+    if block_tables.shape[0] < step.num_seqs or not block_tables.is_contiguous():
+        raise KernelError("attention: block table rows do not cover the step's sequences")
+    max_pages = block_tables.shape[1]
+    need_pages = -(-step.max_context // page_size)
+    if max_pages < need_pages:
+        raise KernelError(f"attention: block tables hold {max_pages} pages per sequence, the "
+                          f"longest context needs {need_pages}")
+    if T != step.num_tokens:
+        raise KernelError(f"attention: qkv has {T} rows, the step {step.num_tokens} tokens")
+    win = int(window) if window else 0
+    out = torch.empty((T, nh * d), dtype=qkv.dtype, device=qkv.device)
+    stream = lib.stream_ptr()
+    kind = force
+    if kind is None:
+        if step.all_decode and d % 8 == 0 and d <= 256 and (nh // nkv) * d <= 2048:
+            kind = "decode"
+        elif (qkv.dtype == torch.bfloat16 and d % 16 == 0 and d <= 256 and page_size % 8 == 0
+              and q_stride % 8 == 0 and not step.all_decode):
+            kind = "prefill"
+        else:
+            kind = "generic"
+    if kind == "decode":
+        if not step.all_decode:
+            raise KernelError("attention: the decode kernel needs one token per sequence")
+        S = step.num_seqs
+        splits = step.decode_splits or decode_splits(S, nkv, nh // nkv, step.max_context)
+        part_ml = part_acc = None
+        if splits > 1:
+            part_ml = torch.empty((S, nh, splits, 2), dtype=torch.float32, device=qkv.device)
+            part_acc = torch.empty((S, nh, splits, d), dtype=torch.float32, device=qkv.device)
+        lib.call("rlis_attn_decode", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(), nh * d,
+                 None if part_ml is None else part_ml.data_ptr(),
+                 None if part_acc is None else part_acc.data_ptr(),
+                 k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,
+                 _i32(step.ctx_lens, "ctx_lens", S), None, S, nh, nkv, d, page_size,
+                 float(scale), win, splits, stream)
+    elif kind == "prefill":
+        if qkv.dtype != torch.bfloat16:
+            raise KernelError("attention: the matrix-core prefill kernel is bfloat16 only")
+        lib.call("rlis_attn_prefill_mfma", qkv.data_ptr(), q_stride, out.data_ptr(), nh * d,
+                 k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,
+                 _i32(step.cu_seqlens, "cu_seqlens", step.num_seqs + 1),
+                 _i32(step.start_pos, "start_pos", step.num_seqs),
+                 _i32(step.tile_map, "tile_map", 2 * step.num_tiles), step.num_tiles, nh, nkv, d,
+                 page_size, win, float(scale), 0, stream)
+    elif kind == "generic":
+        lib.call("rlis_attn_generic", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(), nh * d,
+                 k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,
+                 _i32(step.seq_of_token, "seq_of_token", T), _i32(step.positions, "positions", T),
+                 T, nh, nkv, d, page_size, float(scale), win, stream)
+    else:
+        raise KernelError(f"attention: unknown kernel '{kind}'")
+    return out
+
+
+# ------------------------------------------------------------------------ sampling
+def sample_rows(logits: torch.Tensor, keys: torch.Tensor, inv_temps: torch.Tensor
+                ) -> torch.Tensor:
+    """One token per row of float32 ``logits (R, V)``: argmax where ``inv_temps`` is 0, else
+    Gumbel-max with noise keyed by ``keys`` (int32 bit patterns of the 32-bit row keys)."""
+    stride = _rows_contig(logits, "logits")
+    _check(logits, "logits", torch.float32)
+    R, V = logits.shape
+    _check(inv_temps, "inv_temps", torch.float32)
+    out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    lib.call("rlis_sample_rows", logits.data_ptr(), stride, R, V, _i32(keys, "keys", R),
+             inv_temps.data_ptr(), out.data_ptr(), lib.stream_ptr())
+    return out
+
+
+__all__ = ["KernelError", "add_residual", "add_rmsnorm", "copy_pages", "decode_splits", "embed",
+           "linear", "paged_attention", "rope_kv_write", "sample_rows", "swiglu"]

@@ -1,0 +1,74 @@
+"""Loads the compiled kernel library and declares its C entry points.
+
+There is no fallback: without a GPU, or without the library, every op raises.  The library
+is built on first use when it is absent (``csrc/build.py``)."""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_float, c_int, c_longlong, c_void_p
+from typing import Optional
+
+import torch
+
+_LIB: Optional[ctypes.CDLL] = None
+
+P, I, L, F = c_void_p, c_int, c_longlong, c_float
+
+_SIGNATURES = {
+    "rlis_embed": [P, P, I, P, I, I, P],
+    "rlis_add_residual": [P, P, I, L, P],
+    "rlis_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, P],
+    "rlis_swiglu": [P, P, I, I, I, P],
+    "rlis_rope_kv_write": [P, I, L, I, I, I, I, I, I, I, P, P, P, P, P, P, I, I, P],
+    "rlis_copy_pages": [P, I, I, L, L, P, P, I, P],
+    "rlis_gemm_plain": [P, I, P, I, P, I, I, I, I, L, L, L, P],
+    "rlis_gemm_bf16_mfma": [P, P, P, I, I, I, I, L, L, L, P],
+    "rlis_gemm_bf16_skinny": [P, P, P, I, I, I, I, L, L, L, P],
+    "rlis_attn_generic": [P, I, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
+    "rlis_attn_decode": [P, I, L, P, L, P, P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, P],
+    "rlis_attn_prefill_mfma": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P],
+    "rlis_sample_rows": [P, L, I, I, P, P, P, P],
+}
+
+
+class KernelError(RuntimeError):
+    """A kernel entry point refused its arguments or a launch failed."""
+
+
+def load() -> ctypes.CDLL:
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    if not torch.cuda.is_available():
+        raise RuntimeError(
+            "rust_llm_inference_server_amd needs an AMD GPU (gfx950): torch.cuda.is_available() "
+            "is False and there is no CPU fallback"
+        )
+    from ..csrc import build
+    path = build.ensure("kernels")
+    lib = ctypes.CDLL(path)
+    lib.rlis_last_error.restype = c_char_p
+    lib.rlis_last_error.argtypes = []
+    for name, argtypes in _SIGNATURES.items():
+        fn = getattr(lib, name, None)
+        if fn is None:
+            raise RuntimeError(f"{path} does not export {name}; rebuild the kernels")
+        fn.restype = c_int
+        fn.argtypes = argtypes
+    _LIB = lib
+    return lib
+
+
+def loaded_path() -> Optional[str]:
+    return None if _LIB is None else _LIB._name
+
+
+def call(name: str, *args) -> None:
+    lib = load()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        raise KernelError(lib.rlis_last_error().decode("utf-8", "replace"))
+
+
+def stream_ptr() -> int:
+    return torch.cuda.current_stream().cuda_stream

@@ -1,0 +1,234 @@
+"""The interfaces of the parts a model is put together from, and one registry per kind.
+
+A model is a list of blocks; a block arranges a *mixer* (the part through which a token sees
+earlier tokens), a *feed-forward* and *norms*; a mixer may use a *position encoding*.  Each
+part is built from a ``PartSpec`` (a kind name plus a dict of parameters that carries every
+size and constant), a weight-name prefix and a ``BuildContext``.  No part knows which model
+it is in: what it needs arrives as parameters, per-step data arrives in the ``StepContext``.
+
+The reference builds its layers the same way, with constants passed in:
+``RmsNorm::new(weight, eps)`` (crates/model/src/layers.rs:112-118), ``Attention::new(q, k, v,
+bias, o, cfg)`` (attention.rs:23-41), ``Mlp::new(gate, up, down)`` (layers.rs:165-167),
+``Rope::from_inv_freqs`` (rope.rs:61-78).
+
+Adding a part: subclass the base class of its kind, decorate it with ``@register(kind_name)``
+and name it in a model's specification.  The registries are open; a test may register a part
+of its own without touching this package.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional, Tuple, Type
+
+import torch
+
+
+# --------------------------------------------------------------------------- specs
+@dataclass(frozen=True)
+class TensorSpec:
+    """One checkpoint tensor a part reads: its full name, its shape and how random weights
+    for it are drawn (``normal``: N(0, std); ``ones_normal``: 1 + N(0, std))."""
+
+    name: str
+    shape: Tuple[int, ...]
+    init: str = "normal"
+    std: float = 0.02
+
+
+@dataclass
+class PartSpec:
+    kind: str
+    params: Dict[str, Any] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class CacheRequest:
+    """What a mixer needs from the paged cache: keys and values of ``num_kv_heads`` heads of
+    ``head_dim`` for every earlier position (``window`` None) or for the last ``window``
+    positions only.  Mixers with equal requests share a page group."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+    def group_key(self) -> Tuple[int, int, Optional[int]]:
+        return (self.num_kv_heads, self.head_dim, self.window)
+
+
+@dataclass
+class CacheBinding:
+    """Where one run of a mixer keeps its memory of the past.
+
+    ``k_pages``/``v_pages`` are this run's slices of its group's page pool, ``group`` indexes
+    ``StepContext.groups`` (block tables and slots of that group).  ``writes`` is false when
+    the run reads the cache another run has written in the same step.  ``state`` is the
+    run's slice of the fixed-size per-request state buffer, ``(num_slots, state_bytes)``
+    uint8, or None when the mixer asked for none."""
+
+    group: int = -1
+    k_pages: Optional[torch.Tensor] = None
+    v_pages: Optional[torch.Tensor] = None
+    writes: bool = True
+    state: Optional[torch.Tensor] = None
+
+
+@dataclass
+class BuildContext:
+    """What a part may look at while it is built."""
+
+    device: torch.device
+    act_dtype: torch.dtype                      # torch.float32 or torch.bfloat16
+    weights: Dict[str, torch.Tensor]            # checkpoint name -> device tensor
+    max_positions: int                          # longest sequence the engine will run
+    shared: Dict[Any, Any] = field(default_factory=dict)   # e.g. position tables by parameters
+
+    def take(self, name: str) -> torch.Tensor:
+        try:
+            return self.weights[name]
+        except KeyError:
+            raise KeyError(f"weight '{name}' was not loaded") from None
+
+
+# ---------------------------------------------------------------------- registries
+_REGISTRIES: Dict[str, Dict[str, Type["Part"]]] = {
+    "mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {},
+    "embedding": {}, "head": {},
+}
+
+
+def register(category: str, kind: str) -> Callable[[Type["Part"]], Type["Part"]]:
+    """Class decorator: make ``kind`` buildable as a part of ``category``."""
+    if category not in _REGISTRIES:
+        raise KeyError(f"unknown part category '{category}' (known: {sorted(_REGISTRIES)})")
+
+    def deco(cls: Type["Part"]) -> Type["Part"]:
+        _REGISTRIES[category][kind] = cls
+        cls.category = category
+        cls.kind = kind
+        return cls
+
+    return deco
+
+
+def lookup(category: str, kind: str) -> Type["Part"]:
+    reg = _REGISTRIES[category]
+    if kind not in reg:
+        raise KeyError(f"no {category} of kind '{kind}' is registered (known: {sorted(reg)})")
+    return reg[kind]
+
+
+def create(category: str, spec: PartSpec, prefix: str, ctx: BuildContext) -> "Part":
+    return lookup(category, spec.kind)(spec.params, prefix, ctx)
+
+
+def tensor_specs(category: str, spec: PartSpec, prefix: str) -> List[TensorSpec]:
+    return lookup(category, spec.kind).tensor_specs(spec.params, prefix)
+
+
+def join(prefix: str, name: str) -> str:
+    return f"{prefix}.{name}" if prefix else name
+
+
+# ---------------------------------------------------------------------- base classes
+class Part:
+    category = ""
+    kind = ""
+
+    @classmethod
+    def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
+        """The checkpoint tensors this part reads, by full name."""
+        return []
+
+    def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
+        self.params = params
+        self.prefix = prefix
+
+
+class Norm(Part):
+    """``forward(stream)`` returns the normalised activations ``(T, H)`` in the activation
+    dtype; it first adds the stream's pending delta into the 32-bit residual (one fused pass).
+    ``forward_rows(stream, rows)`` does the same for the selected rows only and leaves the
+    residual untouched."""
+
+    def forward(self, stream: "ResidualStream") -> torch.Tensor:
+        raise NotImplementedError
+
+    def forward_rows(self, stream: "ResidualStream", rows: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Built once per distinct parameter set and shared by the mixers that name it."""
+
+
+class Mixer(Part):
+    """``forward(x, step, binding)`` maps activations ``(T, H)`` to ``(T, H)``.
+
+    ``cache_request()`` says what the mixer keeps in pages (None: nothing);
+    ``state_bytes()`` how many bytes of fixed-size state it keeps per request (0: none).  A
+    mixer with state must leave, after a step, the state as it is after the last token the
+    step brought for that request."""
+
+    def cache_request(self) -> Optional[CacheRequest]:
+        return None
+
+    def state_bytes(self) -> int:
+        return 0
+
+    def forward(self, x: torch.Tensor, step: Any, binding: CacheBinding) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """``forward(x, step)`` maps activations ``(T, H)`` to ``(T, H)``, row by row."""
+
+    def forward(self, x: torch.Tensor, step: Any) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """Arranges a mixer, a feed-forward and their norms around the residual stream."""
+
+    mixer: Mixer
+
+    def forward(self, stream: "ResidualStream", step: Any, binding: CacheBinding) -> None:
+        raise NotImplementedError
+
+
+class Embedding(Part):
+    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+        """Token ids ``(T)`` int32 -> residual stream ``(T, H)`` float32."""
+        raise NotImplementedError
+
+
+class Head(Part):
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """Normalised rows ``(R, H)`` -> logits ``(R, V)`` float32."""
+        raise NotImplementedError
+
+
+class ResidualStream:
+    """The residual sum, kept in 32-bit, plus a delta that has not been added yet.
+
+    A block's output is left *pending* so that the next norm can add it and normalise in one
+    pass over the row; the sum itself is always formed and stored in float32."""
+
+    __slots__ = ("x", "pending")
+
+    def __init__(self, x: torch.Tensor):
+        assert x.dtype == torch.float32
+        self.x = x
+        self.pending: Optional[torch.Tensor] = None
+
+    def add(self, delta: torch.Tensor) -> None:
+        if self.pending is not None:
+            self.flush()
+        self.pending = delta
+
+    def flush(self) -> torch.Tensor:
+        """Fold a pending delta into the residual and return the residual."""
+        if self.pending is not None:
+            from .. import ops
+            ops.add_residual(self.x, self.pending)
+            self.pending = None
+        return self.x

@@ -1,0 +1,34 @@
+"""RMSNorm: ``y = x * rsqrt(mean(x^2) + eps) * w`` over the hidden axis; the weight multiplies
+directly, not as ``1 + w`` (crates/model/src/layers.rs:103-122, 141-146).  The input is the
+32-bit residual stream; statistics and both multiplies are 32-bit, one rounding at the store."""
+from __future__ import annotations
+
+from typing import Any, Dict, List
+
+import torch
+
+from .. import ops
+from .base import BuildContext, Norm, ResidualStream, TensorSpec, join, register
+
+
+@register("norm", "rmsnorm")
+class RMSNorm(Norm):
+    """Parameters: ``size`` (hidden width), ``eps``."""
+
+    @classmethod
+    def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
+        return [TensorSpec(join(prefix, "weight"), (params["size"],), init="ones_normal")]
+
+    def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
+        super().__init__(params, prefix, ctx)
+        self.eps = float(params["eps"])
+        self.weight = ctx.take(join(prefix, "weight"))
+        self.out_dtype = ctx.act_dtype
+
+    def forward(self, stream: ResidualStream) -> torch.Tensor:
+        delta, stream.pending = stream.pending, None
+        return ops.add_rmsnorm(stream.x, delta, self.weight, self.eps, self.out_dtype)
+
+    def forward_rows(self, stream: ResidualStream, rows: torch.Tensor) -> torch.Tensor:
+        return ops.add_rmsnorm(stream.x, stream.pending, self.weight, self.eps, self.out_dtype,
+                               rows=rows)
