@@ -1,0 +1,444 @@
+"""Each kernel alone against a plain float32 PyTorch reference of the same op, at sizes other
+than the engine's test models: widths and vocabularies that are no power of two, head sizes
+in steps of 16, odd head counts and groups, page sizes 8 to 64."""
+import math
+
+import pytest
+import torch
+
+import plain_llama as plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype, f32=1e-4, bf16=2e-2):
+    return dict(atol=f32, rtol=f32) if dtype == torch.float32 else dict(atol=bf16, rtol=bf16)
+
+
+def rnd(*shape, dtype=torch.float32, scale=1.0, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from rust_llm_inference_server_amd import ops
+    from rust_llm_inference_server_amd.ops import lib
+    lib.load()
+    assert lib.loaded_path().endswith("librlis_kernels.so")
+    return ops
+
+
+# ----------------------------------------------------------------------- rows
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("V,H,T", [(331, 100, 7), (1000, 2048, 33), (50, 3, 1)])
+def test_embed(ops, dtype, V, H, T):
+    table = rnd(V, H, dtype=dtype)
+    ids = torch.randint(0, V, (T,), dtype=torch.int32, device=DEV)
+    out = ops.embed(ids, table)
+    assert out.dtype == torch.float32
+    torch.testing.assert_close(out, table[ids.long()].float(), atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("w_dtype", DTYPES)
+@pytest.mark.parametrize("T,H,eps", [(5, 100, 1e-5), (3, 2048, 1e-6), (2, 8192, 1e-5), (1, 7, 0.1)])
+def test_add_rmsnorm(ops, out_dtype, w_dtype, T, H, eps):
+    resid = rnd(T, H, seed=1) * 3
+    delta = rnd(T, H, dtype=out_dtype, seed=2)
+    w = (1 + rnd(H, seed=3) * 0.1).to(w_dtype)
+    want_resid = resid + delta.float()
+    want = plain.rms_norm(want_resid.cpu(), w.float().cpu(), eps)
+    r = resid.clone()
+    out = ops.add_rmsnorm(r, delta, w, eps, out_dtype)
+    torch.testing.assert_close(r, want_resid, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(out.float().cpu(), want, **tol(out_dtype, 2e-5))
+    # no delta: plain norm, residual untouched
+    r2 = resid.clone()
+    out2 = ops.add_rmsnorm(r2, None, w, eps, out_dtype)
+    torch.testing.assert_close(r2, resid, atol=0, rtol=0)
+    torch.testing.assert_close(out2.float().cpu(), plain.rms_norm(resid.cpu(), w.float().cpu(), eps),
+                               **tol(out_dtype, 2e-5))
+    # selected rows with a pending delta: residual untouched, rows in the asked order
+    rows = torch.tensor([T - 1, 0], dtype=torch.int32, device=DEV)
+    r3 = resid.clone()
+    out3 = ops.add_rmsnorm(r3, delta, w, eps, out_dtype, rows=rows)
+    torch.testing.assert_close(r3, resid, atol=0, rtol=0)
+    torch.testing.assert_close(out3.float().cpu(), want[[T - 1, 0]], **tol(out_dtype, 2e-5))
+
+
+def test_rmsnorm_unit_mean_square(ops):
+    # with w = 1 and eps = 0 every row has unit mean square; scaling the input changes nothing
+    x = rnd(4, 300, seed=5) * 7
+    w = torch.ones(300, device=DEV)
+    y = ops.add_rmsnorm(x.clone(), None, w, 0.0, torch.float32)
+    torch.testing.assert_close((y * y).mean(-1), torch.ones(4, device=DEV), atol=1e-5, rtol=1e-5)
+    y2 = ops.add_rmsnorm((x * 5).clone(), None, w, 0.0, torch.float32)
+    torch.testing.assert_close(y, y2, atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_add_residual(ops, dtype):
+    r = rnd(9, 77, seed=1)
+    d = rnd(9, 77, dtype=dtype, seed=2)
+    want = r + d.float()
+    ops.add_residual(r, d)
+    torch.testing.assert_close(r, want, atol=1e-6, rtol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,I", [(3, 172), (17, 8192), (1, 5)])
+def test_swiglu(ops, dtype, T, I):
+    gu = rnd(T, 2 * I, dtype=dtype, scale=2.0)
+    want = torch.nn.functional.silu(gu[:, :I].float()) * gu[:, I:].float()
+    torch.testing.assert_close(ops.swiglu(gu).float(), want, **tol(dtype, 1e-5))
+    z = torch.zeros(1, 2 * I, dtype=dtype, device=DEV)
+    assert ops.swiglu(z).abs().max().item() == 0.0          # silu(0) = 0
+
+
+# ------------------------------------------------------------------- products
+@pytest.mark.parametrize("T,N,K", [(1, 331, 100), (5, 100, 172), (64, 130, 96), (65, 257, 100),
+                                   (200, 3072, 2048), (3, 7, 5)])
+def test_linear_float32(ops, T, N, K):
+    x, w = rnd(T, K, seed=1), rnd(N, K, seed=2, scale=0.05)
+    want = (x.double() @ w.double().t()).float()
+    torch.testing.assert_close(ops.linear(x, w), want, atol=2e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("T,N,K", [(1, 2048, 2048), (1, 331, 104), (8, 3072, 2048), (16, 100, 64),
+                                   (17, 130, 96), (33, 8192, 2048), (64, 2048, 8192),
+                                   (65, 257, 104), (200, 3072, 2048), (300, 331, 2048),
+                                   (128, 128, 64), (5, 100, 100), (70, 100, 172)])
+def test_linear_bfloat16(ops, out_dtype, T, N, K):
+    """Skinny kernel (T <= 64), matrix-core GEMM (float32 output or forced), library GEMM, and
+    the plain kernel for K that is no multiple of 8: all against a float64 product of the same
+    bf16-rounded operands."""
+    x, w = rnd(T, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2, scale=0.05)
+    want = (x.double() @ w.double().t()).float()
+    got = ops.linear(x, w, out_dtype)
+    assert got.dtype == out_dtype
+    scale = want.abs().max().item()
+    if out_dtype == torch.float32:
+        torch.testing.assert_close(got, want, atol=2e-5 * max(1.0, scale) * math.sqrt(K / 64), rtol=1e-4)
+    else:
+        torch.testing.assert_close(got.float(), want, atol=scale / 128, rtol=1e-2)
+    old = ops.BF16_GEMM
+    try:
+        ops.BF16_GEMM = "own"
+        got2 = ops.linear(x, w, out_dtype)
+    finally:
+        ops.BF16_GEMM = old
+    torch.testing.assert_close(got2.float(), got.float(), atol=scale / 128, rtol=1e-2)
+
+
+def test_linear_mixed_dtypes(ops):
+    # a weight stored in 32 bits stays so: bfloat16 activations times a float32 weight
+    x, w = rnd(9, 100, dtype=torch.bfloat16, seed=1), rnd(50, 100, seed=2)
+    want = x.float() @ w.t()
+    torch.testing.assert_close(ops.linear(x, w, torch.bfloat16).float(), want, atol=0.1, rtol=1e-2)
+    torch.testing.assert_close(ops.linear(x, w, torch.float32), want, atol=1e-4, rtol=1e-4)
+
+
+def test_linear_rows_do_not_depend_on_the_batch(ops):
+    """A row's product is the same bits whichever other rows share the call (same kernel)."""
+    for dtype in DTYPES:
+        x, w = rnd(40, 256, dtype=dtype, seed=1), rnd(300, 256, dtype=dtype, seed=2)
+        full = ops.linear(x, w, torch.float32)
+        part = ops.linear(x[5:23].contiguous(), w, torch.float32)
+        torch.testing.assert_close(part, full[5:23], atol=0, rtol=0)
+
+
+# ---------------------------------------------------------- rotation + cache write
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,rot,ps", [(4, 1, 16, 16, 16), (6, 2, 32, 32, 8), (5, 5, 48, 48, 16),
+                                              (3, 1, 80, 40, 32), (32, 8, 64, 64, 16)])
+def test_rope_kv_write(ops, dtype, nh, nkv, d, rot, ps):
+    T, pages = 11, 9
+    inv = plain.inv_freqs(rot, 10000.0, None)
+    positions = torch.tensor([0, 1, 2, 40, 41, 7, 100, 3, 4, 5, 6], dtype=torch.int32)
+    cos_all, sin_all = plain.rope_tables(inv, range(128))
+    qkv = rnd(T, (nh + 2 * nkv) * d, dtype=dtype, seed=4)
+    slots = torch.randperm(pages * ps, generator=torch.Generator().manual_seed(1))[:T].to(torch.int32)
+    k_pages = torch.zeros(pages, nkv, ps, d, dtype=dtype, device=DEV)
+    v_pages = torch.zeros(pages, nkv, d, ps, dtype=dtype, device=DEV)
+    src = qkv.clone()
+    ops.rope_kv_write(qkv, nh, nkv, d, cos_all.to(DEV), sin_all.to(DEV), positions.to(DEV),
+                      slots.to(DEV), k_pages, v_pages, ps)
+    x = src.float().cpu()
+    q = x[:, :nh * d].reshape(T, nh, d)
+    k = x[:, nh * d:(nh + nkv) * d].reshape(T, nkv, d)
+    v = x[:, (nh + nkv) * d:].reshape(T, nkv, d)
+    cos, sin = cos_all[positions.long()], sin_all[positions.long()]
+
+    def rotate(t):          # (T, heads, d): rotate the first `rot` dims, pass the rest
+        r = plain.rope_apply(t[..., :rot].transpose(0, 1), cos, sin).transpose(0, 1)
+        return torch.cat([r, t[..., rot:]], dim=-1)
+
+    t = tol(dtype, 1e-5, 1e-2)
+    torch.testing.assert_close(qkv[:, :nh * d].float().cpu().reshape(T, nh, d), rotate(q), **t)
+    torch.testing.assert_close(qkv[:, nh * d:].cpu(), src[:, nh * d:].cpu(), atol=0, rtol=0)
+    kr = rotate(k)
+    for i in range(T):
+        page, off = int(slots[i]) // ps, int(slots[i]) % ps
+        torch.testing.assert_close(k_pages[page, :, off, :].float().cpu(), kr[i], **t)
+        torch.testing.assert_close(v_pages[page, :, :, off].float().cpu(), v[i], atol=0, rtol=0)
+    # rows that were not written stay zero
+    written = torch.zeros(pages * ps, dtype=torch.bool)
+    written[slots.long()] = True
+    assert k_pages.float().abs().sum(dim=(1, 3)).reshape(-1)[~written].max().item() == 0.0
+
+
+def test_rope_position_zero_is_identity_and_norm_is_kept(ops):
+    nh, nkv, d, ps = 2, 1, 32, 8
+    inv = plain.inv_freqs(d, 10000.0, None)
+    cos, sin = plain.rope_tables(inv, range(64))
+    qkv = rnd(2, (nh + 2 * nkv) * d, seed=3)
+    src = qkv.clone()
+    pos = torch.tensor([0, 37], dtype=torch.int32, device=DEV)
+    ops.rope_kv_write(qkv, nh, nkv, d, cos.to(DEV), sin.to(DEV), pos, None, None, None, ps,
+                      write_kv=False)
+    torch.testing.assert_close(qkv[0], src[0], atol=0, rtol=0)
+    n0 = src[1, :nh * d].reshape(nh, d).norm(dim=-1)
+    n1 = qkv[1, :nh * d].reshape(nh, d).norm(dim=-1)
+    torch.testing.assert_close(n0, n1, atol=1e-5, rtol=1e-5)
+    assert (qkv[1, :nh * d] - src[1, :nh * d]).abs().max().item() > 0.1
+
+
+# ---------------------------------------------------------------------- attention
+class FakeStep:
+    pass
+
+
+def paged_case(lens_cached, lens_new, nh, nkv, d, ps, dtype, seed=0, q_scale=1.0):
+    """A batch of sequences with scattered pages.  Returns (qkv, k_pages, v_pages, tables,
+    step, per-sequence K and V in float32, q in float32)."""
+    S = len(lens_new)
+    g = torch.Generator().manual_seed(seed)
+    totals = [c + n for c, n in zip(lens_cached, lens_new)]
+    pages_per = [-(-t // ps) for t in totals]
+    num_pages = sum(pages_per) + 3
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    tables, it = [], iter(perm)
+    for p in pages_per:
+        tables.append([next(it) for _ in range(p)])
+    width = max(8, max(pages_per))
+    bt = torch.zeros(S, width, dtype=torch.int32)
+    for s, t in enumerate(tables):
+        bt[s, :len(t)] = torch.tensor(t, dtype=torch.int32)
+    k_pages = torch.randn(num_pages, nkv, ps, d, generator=g).to(dtype)   # stale contents
+    v_pages = torch.randn(num_pages, nkv, d, ps, generator=g).to(dtype)
+    ks, vs = [], []
+    for s in range(S):
+        k = torch.randn(totals[s], nkv, d, generator=g).to(dtype)
+        v = torch.randn(totals[s], nkv, d, generator=g).to(dtype)
+        for p in range(totals[s]):
+            k_pages[tables[s][p // ps], :, p % ps, :] = k[p]
+            v_pages[tables[s][p // ps], :, :, p % ps] = v[p]
+        ks.append(k.float())
+        vs.append(v.float())
+    T = sum(lens_new)
+    qkv = (torch.randn(T, (nh + 2 * nkv) * d, generator=g) * q_scale).to(dtype)
+    step = FakeStep()
+    step.num_tokens, step.num_seqs = T, S
+    cu = [0]
+    for n in lens_new:
+        cu.append(cu[-1] + n)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    step.cu_seqlens, step.start_pos = i32(cu), i32(lens_cached)
+    step.ctx_lens = i32(totals)
+    step.positions = i32([c + i for c, n in zip(lens_cached, lens_new) for i in range(n)])
+    step.seq_of_token = i32([s for s, n in enumerate(lens_new) for _ in range(n)])
+    tiles = [x for s, n in enumerate(lens_new) for qb in range(0, n, 64) for x in (s, qb)]
+    step.tile_map, step.num_tiles = i32(tiles), len(tiles) // 2
+    step.max_context, step.max_new = max(totals), max(lens_new)
+    step.all_decode = all(n == 1 for n in lens_new)
+    step.decode_splits = None
+    return (qkv.to(DEV), k_pages.to(DEV), v_pages.to(DEV), bt.to(DEV), step, ks, vs, cu)
+
+
+def reference_attention(qkv, ks, vs, cu, lens_cached, lens_new, nh, nkv, d, scale, window):
+    outs = []
+    q_all = qkv.float().cpu()[:, :nh * d]
+    for s, (c, n) in enumerate(zip(lens_cached, lens_new)):
+        q = q_all[cu[s]:cu[s + 1]].reshape(n, nh, d).transpose(0, 1)
+        k, v = ks[s].transpose(0, 1), vs[s].transpose(0, 1)
+        mask = plain.causal_mask(n, c, window)
+        o = plain.gqa_attention(q, k, v, mask, scale)
+        outs.append(o.transpose(0, 1).reshape(n, nh * d))
+    return torch.cat(outs)
+
+
+LAYOUTS = [(4, 1, 16, 16), (6, 2, 32, 8), (5, 5, 48, 16), (32, 8, 64, 16), (24, 8, 128, 16),
+           (8, 8, 64, 32), (12, 2, 128, 64), (3, 1, 80, 8), (16, 2, 256, 16), (9, 3, 112, 16)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,ps", LAYOUTS)
+@pytest.mark.parametrize("kind", ["generic", "prefill"])
+def test_attention_mixed_batch(ops, dtype, nh, nkv, d, ps, kind):
+    """Portions of prompts (with and without cached positions, across page and tile edges)
+    beside single tokens, in one batch, through scattered block tables."""
+    if kind == "prefill" and dtype != torch.bfloat16:
+        pytest.skip("the matrix-core prefill kernel is bfloat16 only")
+    cached = [0, 5, 40, 0, 63, 130, 17]
+    new = [33, 1, 70, 2, 1, 129, 64]
+    scale = 1.0 / math.sqrt(d)
+    qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=nh)
+    got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, None, force=kind)
+    want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, None)
+    torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind", ["generic", "prefill", "decode"])
+@pytest.mark.parametrize("window", [1, 7, 64, 100])
+def test_attention_window(ops, dtype, kind, window):
+    if kind == "prefill" and dtype != torch.bfloat16:
+        pytest.skip("the matrix-core prefill kernel is bfloat16 only")
+    nh, nkv, d, ps = 6, 2, 32, 8
+    cached, new = ([0, 30, 200, 99], [50, 90, 3, 1]) if kind != "decode" else ([0, 30, 200, 99, 6], [1] * 5)
+    scale = 0.2
+    qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=window)
+    got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window, force=kind)
+    want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, window)
+    torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,ps", LAYOUTS)
+def test_attention_decode(ops, dtype, nh, nkv, d, ps):
+    """One token per sequence, 37 context lengths 1 + (i * 53) % 700 as in the reference's
+    kernel test (crates/model/src/paged_attention.rs:461-527), unsplit and split."""
+    lens = [1 + (i * 53) % 700 for i in range(37)]
+    cached, new = [l - 1 for l in lens], [1] * len(lens)
+    scale = 1.0 / math.sqrt(d)
+    qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=d)
+    want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, None)
+    for splits in (1, 3, 8):
+        step.decode_splits = splits
+        got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, None, force="decode")
+        torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
+    step.decode_splits = None
+    got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, None)
+    torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_decode_long_split(ops, dtype):
+    """Long contexts beside short ones with many partitions, some of them empty
+    (lens [1, 5, 300, 4000, 9000]: paged_attention.rs:503-527)."""
+    nh, nkv, d, ps = 8, 2, 64, 16
+    lens = [1, 5, 300, 4000, 9000]
+    cached, new = [l - 1 for l in lens], [1] * len(lens)
+    scale = 1.0 / math.sqrt(d)
+    qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=9)
+    want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, None)
+    for splits in (None, 36):
+        step.decode_splits = splits
+        got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, None, force="decode")
+        torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind", ["generic", "prefill", "decode"])
+def test_attention_finds_a_far_key(ops, dtype, kind):
+    """One key among hundreds is made to stand out (its key vector equals the scaled query
+    direction); the output must be that key's value, wherever its page lies."""
+    if kind == "prefill" and dtype != torch.bfloat16:
+        pytest.skip("the matrix-core prefill kernel is bfloat16 only")
+    nh, nkv, d, ps = 4, 2, 64, 16
+    total = 777
+    cached, new = ([total - 1], [1]) if kind == "decode" else ([total - 3], [3])
+    qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=5)
+    far = 131                                   # in the middle of a page, far from the end
+    table = bt[0].tolist()
+    qdir = qkv[-1, :d].float()                  # last token, head 0 (KV head 0)
+    kp[table[far // ps], 0, far % ps, :] = (qdir * 50.0 / qdir.norm()).to(dtype)
+    ks[0][far, 0, :] = kp[table[far // ps], 0, far % ps, :].float().cpu()
+    scale = 1.0
+    got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, None, force=kind)
+    want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, None)
+    torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
+    torch.testing.assert_close(got[-1, :d].float().cpu(), vs[0][far, 0, :], **tol(dtype, 1e-4, 2e-2))
+
+
+def test_attention_one_key_returns_its_value(ops):
+    nh, nkv, d, ps = 4, 2, 32, 8
+    for kind in ("generic", "decode"):
+        qkv, kp, vp, bt, step, ks, vs, cu = paged_case([0, 0], [1, 1], nh, nkv, d, ps, torch.float32)
+        got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, 0.3, None, force=kind)
+        for s in range(2):
+            for h in range(nh):
+                torch.testing.assert_close(got[s, h * d:(h + 1) * d].cpu(), vs[s][0, h // 2],
+                                           atol=1e-6, rtol=1e-6)
+
+
+# ------------------------------------------------------------------------ sampling
+def test_sample_rows_greedy_and_ties(ops):
+    # the reference's vector: ties go to the lowest index (crates/model/src/sampling.rs:184-199)
+    logits = torch.tensor([[0.1, 3.0, -1.0, 3.0], [5.0, 1.0, 5.0, 0.0]], device=DEV)
+    zeros_i = torch.zeros(2, dtype=torch.int32, device=DEV)
+    zeros_f = torch.zeros(2, device=DEV)
+    assert ops.sample_rows(logits, zeros_i, zeros_f).tolist() == [1, 0]
+    neg = torch.tensor([[float("-inf"), -5.0]], device=DEV)
+    assert ops.sample_rows(neg, zeros_i[:1], zeros_f[:1]).tolist() == [1]
+    big = rnd(5, 128256, seed=3)
+    got = ops.sample_rows(big, torch.zeros(5, dtype=torch.int32, device=DEV), torch.zeros(5, device=DEV))
+    assert got.tolist() == big.argmax(dim=-1).tolist()
+
+
+def test_sample_rows_temperature_matches_host_reference(ops):
+    V = 50021
+    logits = rnd(6, V, seed=11) * 2
+    keys = [plain.row_key(42 + r, 100 + r) for r in range(6)]
+    inv_t = [1 / 0.7, 1 / 0.8, 0.0, 1 / 1.3, 1 / 0.1, 1.0]
+    kt = torch.tensor([k - (1 << 32) if k >= (1 << 31) else k for k in keys], dtype=torch.int32, device=DEV)
+    got = ops.sample_rows(logits, kt, torch.tensor(inv_t, device=DEV)).tolist()
+    want = [plain.sample_row(logits[r].cpu(), keys[r], inv_t[r]) for r in range(6)]
+    assert got == want
+    # the same key gives the same token whatever the neighbours are
+    again = ops.sample_rows(logits[3:4].contiguous(), kt[3:4].contiguous(),
+                            torch.tensor(inv_t[3:4], device=DEV)).tolist()
+    assert again == got[3:4]
+
+
+def test_sample_rows_frequencies_follow_softmax(ops):
+    # crates/model/src/sampling.rs:216-241: l = [0, 1, 2, -1], T = 0.7, 20,000 keys, within 0.015
+    n = 20000
+    l = torch.tensor([0.0, 1.0, 2.0, -1.0])
+    logits = l.repeat(n, 1).to(DEV)
+    keys = [plain.row_key(42, i) for i in range(n)]
+    kt = torch.tensor([k - (1 << 32) if k >= (1 << 31) else k for k in keys], dtype=torch.int32, device=DEV)
+    got = ops.sample_rows(logits, kt, torch.full((n,), 1 / 0.7, device=DEV))
+    freq = torch.bincount(got.long().cpu(), minlength=4).float() / n
+    want = torch.softmax(l / 0.7, dim=0)
+    assert (freq - want).abs().max().item() < 0.015
+
+
+# ---------------------------------------------------------------------- page copies
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_copy_pages(ops, dtype):
+    pages = rnd(3, 10, 2, 8, 16, dtype=dtype)
+    src = torch.tensor([1, 7], dtype=torch.int32, device=DEV)
+    dst = torch.tensor([4, 0], dtype=torch.int32, device=DEV)
+    want = pages.clone()
+    want[:, 4], want[:, 0] = pages[:, 1], pages[:, 7]
+    ops.copy_pages(pages, src, dst)
+    torch.testing.assert_close(pages, want, atol=0, rtol=0)
+
+
+# ----------------------------------------------------------------- refusals
+def test_kernels_refuse_what_they_cannot_do(ops):
+    with pytest.raises(ops.KernelError):
+        ops.linear(rnd(2, 8), rnd(3, 9))
+    with pytest.raises(ops.KernelError):
+        ops.swiglu(rnd(2, 7))
+    with pytest.raises(ops.KernelError):
+        ops.embed(torch.zeros(2, dtype=torch.int32), torch.zeros(4, 4))       # CPU tensors
+    qkv, kp, vp, bt, step, *_ = paged_case([0], [4], 2, 1, 24, 8, torch.bfloat16)
+    with pytest.raises(ops.KernelError):           # head_dim 24 is no multiple of 16
+        ops.paged_attention(qkv, 2, 1, 24, kp, vp, 8, bt, step, 1.0, None, force="prefill")
