@@ -1,0 +1,64 @@
+"""The host side of the engine (batch layout, block tables, page manager, run order) under
+every way of cutting the work, with the kernels replaced by a slow torch double on the CPU.
+The kernels themselves are tested on the GPU (test_kernels_gpu.py, test_replay_gpu.py)."""
+import pytest
+import torch
+
+import plain_llama as plain
+import traces
+from conftest import TINY
+
+
+@pytest.fixture(scope="module")
+def ref_a(tiny_folders):
+    folder = tiny_folders["a"]
+    w, c = plain.read_weights(folder), plain.read_config(folder)
+    reqs = traces.random_requests(c["vocab_size"], [5, 17, 33, 70, 1, 2, 64, 90], seed=3)
+    return folder, reqs, {k: plain.forward(w, c, t) for k, t in reqs.items()}
+
+
+@pytest.mark.parametrize("family", ["whole", "tail", "portions", "mixed"])
+def test_replay_families_cpu(cpu_ops, ref_a, family):
+    from rust_llm_inference_server_amd.engine import ModelRunner, load_model
+    folder, reqs, ref = ref_a
+    build = {"whole": traces.trace_whole, "tail": traces.trace_tail,
+             "portions": traces.trace_portions, "mixed": traces.trace_mixed}[family]
+    steps, max_tokens = build(reqs)
+    model = load_model(folder, "float32", max_positions=128, device=torch.device("cpu"))
+    runner = ModelRunner(model, num_pages=max_tokens // 16, page_size=16, max_num_seqs=8)
+    outputs = traces.replay_in_process(runner, steps)
+    got = traces.collect(steps, outputs, TINY["a"]["vocab_size"])
+    for k, tokens in reqs.items():
+        mine = torch.stack([got[k][p] for p in range(len(tokens))])
+        assert (mine - ref[k]).abs().max().item() < 1e-4
+    assert runner.cache.num_free_pages(0) == runner.cache.num_pages(0)
+
+
+def test_step_errors(cpu_ops, tiny_folders):
+    """The step's refusals (crates/model/src/llama.rs:218-240; paged.rs:258-263)."""
+    from rust_llm_inference_server_amd.engine import ModelRunner, StepEntry, load_model
+    model = load_model(tiny_folders["a"], "float32", max_positions=64, device=torch.device("cpu"))
+    runner = ModelRunner(model, num_pages=8, page_size=16, max_num_seqs=2)
+    with pytest.raises(ValueError, match="at least one request"):
+        runner.step([])
+    runner.reserve(1, 4)
+    with pytest.raises(ValueError, match="empty sequence"):
+        runner.step([StepEntry(1, [], [])])
+    with pytest.raises(ValueError, match="no page reserved"):
+        runner.step([StepEntry(1, [1, 2, 3, 4, 5], [])])
+    with pytest.raises(ValueError, match="no page reserved"):
+        runner.step([StepEntry(9, [1], [])])
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        runner.step([StepEntry(1, [256], [])])
+    with pytest.raises(ValueError, match="wanted index"):
+        runner.step([StepEntry(1, [1, 2], [2])])
+    with pytest.raises(ValueError, match="appears twice"):
+        runner.step([StepEntry(1, [1], []), StepEntry(1, [2], [])])
+    with pytest.raises(ValueError, match="exceeds max_seq_len"):
+        runner.reserve(1, 65)
+    runner.reserve(2, 1)
+    with pytest.raises(ValueError, match="max_num_seqs"):
+        runner.step([StepEntry(1, [1], []), StepEntry(2, [1], []), StepEntry(3, [1], [])])
+    out = runner.step([StepEntry(1, [1, 2], [1]), StepEntry(2, [3], [])])
+    assert out.shape == (1, 256)
+    assert runner.num_computed(1) == 2 and runner.num_computed(2) == 1
