@@ -1,0 +1,258 @@
+"""The request loop: admit, schedule, step, sample, finish, free.
+
+What the reference's engine thread does each iteration (crates/engine/src/engine.rs:500-531,
+617-726), without the thread and the channels: ``add_request`` validates and queues a request,
+``step`` runs one scheduled batch through the model and samples a token for every request
+whose tokens are all computed, ``generate`` loops until its requests are finished.
+
+Finishing follows ``Sequence::accept`` (engine.rs:404-429): an EOS token (unless
+``ignore_eos``) ends the request with reason ``stop`` and is not appended; reaching
+``max_tokens`` ends it with reason ``length``.  When pages run out the scheduler preempts the
+newest request, which later recomputes its prompt and its generated tokens in one prefill and,
+its sampling being keyed by position, continues with the same tokens (engine.rs tests
+157-194)."""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Dict, Iterable, List, Optional, Sequence, Tuple, Union
+
+import torch
+
+from ..config.engine import EngineConfig
+from ..models.spec import Model
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler, sample_on_device
+from .batch import StepEntry
+from .runner import ModelRunner, load_model
+from .scheduler import Scheduler
+
+
+@dataclass
+class Completion:
+    """What a finished request returns (engine.rs:139-158 ``Finish``)."""
+    request_id: int
+    token_ids: List[int]
+    finish_reason: str                 # "stop" or "length"
+    prompt_tokens: int
+    ttft: float                        # seconds from arrival to the first token
+    decode_time: float                 # seconds from the first token to the last
+
+    @property
+    def completion_tokens(self) -> int:
+        return len(self.token_ids)
+
+    @property
+    def decode_tokens_per_sec(self) -> float:
+        """(completion - 1) / decode_time (engine.rs:150-157)."""
+        if self.completion_tokens < 2 or self.decode_time <= 0:
+            return 0.0
+        return (self.completion_tokens - 1) / self.decode_time
+
+
+@dataclass
+class EngineStats:
+    steps: int = 0
+    prefill_tokens: int = 0
+    generated_tokens: int = 0
+    preemptions: int = 0
+    running: int = 0
+    waiting: int = 0
+    pages_used: int = 0
+    pages_total: int = 0
+
+
+class _Sequence:
+    def __init__(self, seq_id: int, prompt: Sequence[int], params: SamplingParams):
+        self.id = seq_id
+        self.tokens = [int(t) for t in prompt]
+        self.prompt_len = len(self.tokens)
+        self.params = params
+        self.sampler = Sampler(params)
+        self.arrived = time.perf_counter()
+        self.first_token_at: Optional[float] = None
+        self.last_token_at: Optional[float] = None
+        self.finish_reason: Optional[str] = None
+
+    @property
+    def output_len(self) -> int:
+        return len(self.tokens) - self.prompt_len
+
+
+class Engine:
+    """``Engine(model, config)`` where ``model`` is a built ``Model`` or a model folder."""
+
+    def __init__(self, model: Union[Model, str], config: Optional[EngineConfig] = None,
+                 dtype: str = "bfloat16", eos_token_ids: Optional[Iterable[int]] = None):
+        self.config = config or EngineConfig()
+        self.config.validate()
+        cfg = self.config
+        if isinstance(model, str):
+            model = load_model(model, dtype, max_positions=cfg.max_seq_len)
+        self.model = model
+        elem = 2 if model.act_dtype == torch.bfloat16 else 4
+        if cfg.num_pages is not None:
+            num_pages = cfg.num_pages
+        else:
+            # engine.rs:252-262: pool bytes / (bytes of K and V per token * block size)
+            per_token = sum(2 * len(g.writer_runs) * g.request.num_kv_heads * g.request.head_dim
+                            for g in model.cache_groups) * elem
+            num_pages = int(cfg.kv_cache_gb * (1 << 30)) // max(1, per_token * cfg.block_size)
+        if num_pages < 2:
+            raise ValueError(f"the cache pool holds {num_pages} pages; at least 2 are needed")
+        watermark = cfg.watermark_pages
+        if watermark is None:
+            watermark = max(1, num_pages // 100)            # engine.rs:263-271
+        self.runner = ModelRunner(model, num_pages=num_pages, page_size=cfg.block_size,
+                                  max_num_seqs=cfg.max_num_seqs,
+                                  max_batched_tokens=max(cfg.max_batched_tokens, cfg.max_num_seqs))
+        self.scheduler = Scheduler(self.runner.cache, cfg.max_num_seqs,
+                                   max(cfg.max_batched_tokens, cfg.max_num_seqs),
+                                   watermark_pages=watermark, policy=cfg.scheduler)
+        # engine.rs:280: the longest request is bounded by the rope table and by the pool
+        self.max_seq_len = min(model.max_positions, self.scheduler.max_seq_tokens)
+        if eos_token_ids is None:
+            eos_token_ids = getattr(getattr(model, "config", None), "eos_token_ids", ())
+        self.eos_token_ids = set(int(t) for t in eos_token_ids)
+        self._seqs: Dict[int, _Sequence] = {}
+        self._finished: Dict[int, Completion] = {}
+        self._next_id = 0
+        self.stats_ = EngineStats(pages_total=num_pages)
+
+    # ----------------------------------------------------------------- requests
+    def add_request(self, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None
+                    ) -> int:
+        """Queue a request; refuses what could never run (engine.rs:332-356)."""
+        params = params or SamplingParams()
+        params.validate()
+        if len(prompt_ids) == 0 or params.max_tokens == 0:
+            raise ValueError("empty prompt or max_tokens of 0")
+        total = len(prompt_ids) + params.max_tokens
+        if total > self.max_seq_len:
+            raise ValueError(f"{total} tokens exceeds max_seq_len {self.max_seq_len}")
+        vocab = self.model.spec.vocab_size
+        for t in prompt_ids:
+            if not 0 <= int(t) < vocab:
+                raise ValueError(f"token id {t} is outside the vocabulary of {vocab}")
+        seq_id = self._next_id
+        self._next_id += 1
+        self._seqs[seq_id] = _Sequence(seq_id, prompt_ids, params)
+        self.scheduler.add(seq_id, len(prompt_ids))
+        return seq_id
+
+    def cancel(self, seq_id: int) -> None:
+        """Drop a request wherever it is; its pages are free at once (engine.rs:562-573)."""
+        if seq_id in self._seqs:
+            self.scheduler.remove(seq_id)
+            del self._seqs[seq_id]
+
+    def has_work(self) -> bool:
+        return self.scheduler.has_work()
+
+    # --------------------------------------------------------------------- step
+    def step(self) -> List[Tuple[int, Optional[int], bool]]:
+        """One scheduled batch.  Returns ``(request id, token or None, finished)`` for every
+        request that produced a token (``None`` with ``finished``: it stopped at an EOS)."""
+        sched = self.scheduler.schedule()
+        self.stats_.preemptions = self.scheduler.num_preemptions
+        if not sched.seqs:
+            if self.scheduler.has_work():
+                # engine.rs:516-522: a schedule without sequences while work exists is a bug
+                for seq_id in list(self._seqs):
+                    self.cancel(seq_id)
+                raise RuntimeError("scheduler made no progress")
+            return []
+        self.runner.apply_copies(sched.copies)
+        entries, final = [], []
+        for seq_id, start, end in sched.seqs:
+            seq = self._seqs[seq_id]
+            last = end == len(seq.tokens)
+            entries.append(StepEntry(seq_id, seq.tokens[start:end],
+                                     [end - start - 1] if last else []))
+            final.append(last)
+        logits = self.runner.step(entries)
+        self.stats_.steps += 1
+        # Rows that yield a token, split between the device kernel and the host sampler.
+        device_rows, device_modes, host_rows = [], [], []
+        row = 0
+        for (seq_id, start, end), last in zip(sched.seqs, final):
+            self.scheduler.advance(seq_id, end)
+            if not last:
+                self.stats_.prefill_tokens += end - start
+                continue
+            seq = self._seqs[seq_id]
+            mode = seq.sampler.device_mode(len(seq.tokens))
+            if mode is not None:
+                device_rows.append((row, seq_id))
+                device_modes.append(mode)
+            else:
+                host_rows.append((row, seq_id))
+            row += 1
+        picked: Dict[int, int] = {}
+        if device_rows:
+            idx = [r for r, _ in device_rows]
+            sub = logits if len(idx) == logits.shape[0] else logits[
+                torch.tensor(idx, device=logits.device)].contiguous()
+            for (_, seq_id), tok in zip(device_rows, sample_on_device(sub, device_modes)):
+                picked[seq_id] = tok
+        if host_rows:
+            idx = torch.tensor([r for r, _ in host_rows], device=logits.device)
+            host_logits = logits[idx].cpu().numpy()
+            for (_, seq_id), lrow in zip(host_rows, host_logits):
+                seq = self._seqs[seq_id]
+                picked[seq_id] = seq.sampler.sample(lrow, seq.tokens, len(seq.tokens))
+        out = []
+        for (seq_id, _, _), last in zip(sched.seqs, final):
+            if last:
+                out.append(self._accept(self._seqs[seq_id], picked[seq_id]))
+        self.stats_.running = self.scheduler.num_running
+        self.stats_.waiting = self.scheduler.num_waiting
+        self.stats_.pages_used = self.stats_.pages_total - self.runner.cache.num_free_pages(0)
+        return out
+
+    def _accept(self, seq: _Sequence, token: int) -> Tuple[int, Optional[int], bool]:
+        now = time.perf_counter()
+        if seq.first_token_at is None:
+            seq.first_token_at = now
+        seq.last_token_at = now
+        stops = (not seq.params.ignore_eos and token in self.eos_token_ids) \
+            or token in seq.params.stop_token_ids
+        if stops:
+            self._finish(seq, "stop")
+            return (seq.id, None, True)
+        seq.tokens.append(token)
+        self.stats_.generated_tokens += 1
+        if seq.output_len >= seq.params.max_tokens:
+            self._finish(seq, "length")
+            return (seq.id, token, True)
+        self.scheduler.append_token(seq.id)
+        return (seq.id, token, False)
+
+    def _finish(self, seq: _Sequence, reason: str) -> None:
+        seq.finish_reason = reason
+        self.scheduler.remove(seq.id)
+        del self._seqs[seq.id]
+        self._finished[seq.id] = Completion(
+            request_id=seq.id, token_ids=seq.tokens[seq.prompt_len:], finish_reason=reason,
+            prompt_tokens=seq.prompt_len, ttft=(seq.first_token_at or seq.arrived) - seq.arrived,
+            decode_time=(seq.last_token_at or 0.0) - (seq.first_token_at or 0.0))
+
+    # ----------------------------------------------------------------- generate
+    def generate(self, prompts: Sequence[Sequence[int]],
+                 params: Union[SamplingParams, Sequence[SamplingParams], None] = None
+                 ) -> List[Completion]:
+        """Run the prompts to completion under continuous batching; results in their order."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params or SamplingParams()] * len(prompts)
+        if len(params) != len(prompts):
+            raise ValueError("one SamplingParams per prompt, or one for all")
+        ids = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
+        while any(i in self._seqs for i in ids):
+            self.step()
+        return [self._finished.pop(i) for i in ids]
+
+    def pop_finished(self, seq_id: int) -> Optional[Completion]:
+        return self._finished.pop(seq_id, None)
+
+    def stats(self) -> EngineStats:
+        return self.stats_

@@ -21,6 +21,9 @@ SKINNY_MAX_ROWS = 64
 # "library": bf16 products with more rows and bf16 output go to torch.matmul (hipBLASLt);
 # "own": they take the hand-written matrix-core kernel.
 BF16_GEMM = "library"
+# None: attention kernels are chosen from the batch; "generic": the generic kernel always
+# (what the command line's --attention v1 asks for).
+FORCE_ATTENTION: Optional[str] = None
 
 
 def _dt(t: torch.Tensor) -> int:
@@ -257,7 +260,7 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     win = int(window) if window else 0
     out = torch.empty((T, nh * d), dtype=qkv.dtype, device=qkv.device)
     stream = lib.stream_ptr()
-    kind = force
+    kind = force or FORCE_ATTENTION
     if kind is None:
         if step.all_decode and d % 8 == 0 and d <= 256 and (nh // nkv) * d <= 2048:
             kind = "decode"
