@@ -53,7 +53,7 @@ def main() -> int:
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
-    cfg["max_position_embeddings"] = min(cfg["max_position_embeddings"], max(args.context, 4096))
+    cfg["max_position_embeddings"] = min(cfg["max_position_embeddings"], max(args.context, 4096) + 64)
     page = 16
     K, W = args.steps, args.warmup
     elem = 2 if args.dtype == "bfloat16" else 4
@@ -78,7 +78,7 @@ def main() -> int:
         pages = batch * (-(-context // page) + 1) + 8
         engine = Engine(model, EngineConfig(max_num_seqs=max(batch, 1), max_batched_tokens=2048,
                                             num_pages=pages, block_size=page,
-                                            max_seq_len=context + 1, watermark_pages=0))
+                                            max_seq_len=context + 8, watermark_pages=0))
         sp = SamplingParams(max_tokens=steps + warmup + 1, ignore_eos=True)
         for p in prompts(batch, prompt_len):
             engine.add_request(p, sp)
