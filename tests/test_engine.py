@@ -1,0 +1,143 @@
+"""The request loop end to end on tiny random models, as the reference's engine tests do
+(crates/engine/tests/engine.rs:58-275): every case runs on the GPU (``-m gpu``) and, with the
+kernels replaced by the slow torch double, on the CPU, where it tests the host logic alone."""
+import pytest
+import torch
+
+import plain_llama as plain
+from conftest import TINY
+from rust_llm_inference_server_amd.config import EngineConfig
+from rust_llm_inference_server_amd.sampling import SamplingParams
+
+BACKENDS = ["double", pytest.param("gpu", marks=pytest.mark.gpu)]
+
+
+@pytest.fixture(params=BACKENDS)
+def backend(request):
+    if request.param == "double":
+        import cpu_ops
+        cpu_ops.install(request.getfixturevalue("monkeypatch"))
+        return torch.device("cpu")
+    return torch.device("cuda", 0)
+
+
+def load(folder, device, dtype="float32", max_positions=256):
+    from rust_llm_inference_server_amd.engine import load_model
+    return load_model(folder, dtype, max_positions, device)
+
+
+def engine_for(model, **kw):
+    from rust_llm_inference_server_amd.engine import Engine
+    cfg = dict(max_num_seqs=8, max_batched_tokens=64, num_pages=64, block_size=8,
+               max_seq_len=256, watermark_pages=1)
+    cfg.update(kw)
+    return Engine(model, EngineConfig(**cfg))
+
+
+def prompts_for(vocab, lengths, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, vocab, (n,), generator=g).tolist() for n in lengths]
+
+
+def test_greedy_generation_matches_the_plain_implementation(backend, tiny_folders):
+    """BASELINE workload 0/1 in small: prompts 5/17/33 (and 1/9/40), 8 greedy tokens each."""
+    for name, lengths in (("a", [5, 17, 33]), ("b", [1, 9, 40])):
+        folder = tiny_folders[name]
+        w, c = plain.read_weights(folder), plain.read_config(folder)
+        prompts = prompts_for(c["vocab_size"], lengths, seed=1)
+        engine = engine_for(load(folder, backend), max_batched_tokens=24)
+        outs = engine.generate(prompts, SamplingParams.greedy(8))
+        for p, o in zip(prompts, outs):
+            assert o.token_ids == plain.greedy_generate(w, c, p, 8)
+            assert o.finish_reason == "length" and o.prompt_tokens == len(p)
+        assert engine.runner.cache.num_free_pages() == 64
+
+
+def test_batched_equals_solo_and_chunked_equals_single_shot(backend, tiny_folders):
+    model = load(tiny_folders["b"], backend)
+    prompts = prompts_for(384, [30, 3, 57, 12], seed=2)
+    sp = SamplingParams.greedy(6)
+    together = [o.token_ids for o in engine_for(model).generate(prompts, sp)]
+    solo = [engine_for(model).generate([p], sp)[0].token_ids for p in prompts]
+    assert together == solo
+    chunked = [o.token_ids for o in engine_for(model, max_batched_tokens=16).generate(prompts, sp)]
+    assert chunked == together                      # engine.rs tests: budget 16 == single shot
+    static = [o.token_ids for o in engine_for(model, scheduler="static").generate(prompts, sp)]
+    assert static == together
+
+
+def test_preemption_and_recompute_do_not_change_the_output(backend, tiny_folders):
+    """So few pages that running requests are preempted (engine.rs tests 157-194): the victims
+    recompute prompt and generated tokens and continue with the same tokens."""
+    model = load(tiny_folders["a"], backend, max_positions=128)
+    prompts = prompts_for(256, [9] * 6, seed=3)
+    for sp in (SamplingParams.greedy(24), SamplingParams(temperature=0.8, seed=11, max_tokens=24)):
+        roomy = engine_for(model, num_pages=64)
+        want = [o.token_ids for o in roomy.generate(prompts, sp)]
+        assert roomy.stats().preemptions == 0
+        tight = engine_for(model, num_pages=12, watermark_pages=0)
+        got = [o.token_ids for o in tight.generate(prompts, sp)]
+        assert tight.stats().preemptions > 0
+        assert got == want
+        assert tight.runner.cache.num_free_pages() == 12
+        tight.runner.cache.check_invariants()
+
+
+def test_seeded_temperature_ignores_the_neighbours(backend, tiny_folders):
+    model = load(tiny_folders["b"], backend)
+    prompts = prompts_for(384, [1, 9, 40, 100], seed=4)
+    sp = SamplingParams(temperature=0.8, seed=1234, max_tokens=12)
+    among = [o.token_ids for o in engine_for(model, max_batched_tokens=24).generate(prompts, sp)]
+    alone = [engine_for(model).generate([p], sp)[0].token_ids for p in prompts]
+    assert among == alone
+    again = [o.token_ids for o in engine_for(model).generate(prompts, sp)]
+    assert again == among                            # same seed, same tokens
+    other = engine_for(model).generate(prompts[2:3], SamplingParams(temperature=0.8, seed=5, max_tokens=12))
+    assert other[0].token_ids != among[2]
+    assert len(set(among[3])) > 1
+
+
+def test_host_sampler_modes_run_and_are_reproducible(backend, tiny_folders):
+    model = load(tiny_folders["b"], backend)
+    prompts = prompts_for(384, [7, 21], seed=5)
+    one = SamplingParams(temperature=0.9, top_k=1, seed=3, max_tokens=6)
+    greedy = [o.token_ids for o in engine_for(model).generate(prompts, SamplingParams.greedy(6))]
+    assert [o.token_ids for o in engine_for(model).generate(prompts, one)] == greedy
+    sp = SamplingParams(temperature=1.2, top_k=20, top_p=0.9, repetition_penalty=1.3, seed=3, max_tokens=6)
+    a = [o.token_ids for o in engine_for(model).generate(prompts, sp)]
+    b = [o.token_ids for o in engine_for(model).generate(prompts[::-1], sp)][::-1]
+    assert a == b
+
+
+def test_eos_and_limits(backend, tiny_folders):
+    model = load(tiny_folders["a"], backend, max_positions=128)
+    prompt = prompts_for(256, [6], seed=6)[0]
+    from rust_llm_inference_server_amd.engine import Engine
+    first = engine_for(model).generate([prompt], SamplingParams.greedy(3))[0].token_ids[0]
+    cfg = EngineConfig(max_num_seqs=2, max_batched_tokens=64, num_pages=16, block_size=8, max_seq_len=128)
+    stops = Engine(model, cfg, eos_token_ids=[first])
+    out = stops.generate([prompt], SamplingParams.greedy(5))[0]
+    assert (out.finish_reason, out.token_ids) == ("stop", [])       # EOS is not appended
+    out = stops.generate([prompt], SamplingParams(max_tokens=5, ignore_eos=True))[0]
+    assert out.finish_reason == "length" and len(out.token_ids) == 5
+    with pytest.raises(ValueError, match="empty prompt or max_tokens of 0"):
+        stops.add_request([], SamplingParams())
+    with pytest.raises(ValueError, match="empty prompt or max_tokens of 0"):
+        stops.add_request([1], SamplingParams(max_tokens=0))
+    with pytest.raises(ValueError, match="exceeds max_seq_len"):
+        stops.add_request([1] * 100, SamplingParams(max_tokens=100))
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        stops.add_request([256], SamplingParams())
+
+
+def test_cancel_returns_the_pages(backend, tiny_folders):
+    model = load(tiny_folders["a"], backend, max_positions=128)
+    engine = engine_for(model, num_pages=16)
+    a = engine.add_request(prompts_for(256, [20])[0], SamplingParams.greedy(50))
+    b = engine.add_request(prompts_for(256, [5])[0], SamplingParams.greedy(4))
+    engine.step()
+    engine.cancel(a)
+    while engine.has_work():
+        engine.step()
+    assert engine.pop_finished(b).finish_reason == "length" and engine.pop_finished(a) is None
+    assert engine.runner.cache.num_free_pages() == 16

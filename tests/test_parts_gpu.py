@@ -1,0 +1,343 @@
+"""The parts alone, and models put together from them in ways the Llama decoder does not use:
+a layer with a window beside layers without, a layer named twice in the run order, a layer
+that reads another layer's cache, and a toy mixer with state of its own that the test defines
+and registers without touching the package.  Everything runs on the GPU against plain code."""
+import json
+import math
+import os
+
+import pytest
+import torch
+
+import plain_llama as plain
+import traces
+from conftest import TINY_B
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda", 0)
+
+
+def ctx_for(weights, dtype=torch.float32, max_positions=256):
+    from rust_llm_inference_server_amd.parts import BuildContext
+    return BuildContext(device=DEV, act_dtype=dtype, max_positions=max_positions,
+                        weights={k: v.to(DEV) for k, v in weights.items()})
+
+
+# --------------------------------------------------------------- each part alone
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    from rust_llm_inference_server_amd.parts import PartSpec, ResidualStream, create
+    w = {"n.weight": 1 + 0.1 * torch.randn(100)}
+    norm = create("norm", PartSpec("rmsnorm", {"size": 100, "eps": 1e-6}), "n", ctx_for(w, dtype))
+    x, d = torch.randn(6, 100), torch.randn(6, 100).to(dtype)
+    stream = ResidualStream(x.to(DEV).clone())
+    stream.add(d.to(DEV))
+    y = norm.forward(stream)
+    assert stream.pending is None and y.dtype == dtype
+    want_x = x + d.float()
+    torch.testing.assert_close(stream.x.cpu(), want_x, atol=1e-6, rtol=1e-6)   # 32-bit residual
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    torch.testing.assert_close(y.float().cpu(), plain.rms_norm(want_x, w["n.weight"], 1e-6),
+                               atol=tol, rtol=tol)
+    rows = torch.tensor([4, 1], dtype=torch.int32, device=DEV)
+    stream.add(d.to(DEV))
+    y2 = norm.forward_rows(stream, rows)
+    want2 = plain.rms_norm((want_x + d.float())[[4, 1]], w["n.weight"], 1e-6)
+    torch.testing.assert_close(y2.float().cpu(), want2, atol=tol, rtol=tol)
+
+
+def test_position_part_tables():
+    from rust_llm_inference_server_amd.parts import PartSpec, create
+    sc = TINY_B["rope_scaling"]
+    rope = create("position", PartSpec("rope", {"rot_dim": 32, "theta": 500000.0, "scaling": sc}),
+                  "", ctx_for({}, max_positions=200))
+    cos, sin = plain.rope_tables(plain.inv_freqs(32, 500000.0, sc), range(200))
+    assert rope.cos.dtype == torch.float32 and rope.cos.shape == (200, 16)
+    torch.testing.assert_close(rope.cos.cpu(), cos, atol=1e-6, rtol=0)
+    torch.testing.assert_close(rope.sin.cpu(), sin, atol=1e-6, rtol=0)
+    with pytest.raises(ValueError, match="unknown scaling"):
+        create("position", PartSpec("rope", {"rot_dim": 32, "theta": 1e4,
+                                             "scaling": {"rope_type": "yarn"}}), "", ctx_for({}))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feed_forward_embedding_and_head_parts(dtype):
+    from rust_llm_inference_server_amd.parts import PartSpec, create
+    H, I, V = 72, 200, 131
+    w = {"m.gate_proj.weight": torch.randn(I, H) * 0.1, "m.up_proj.weight": torch.randn(I, H) * 0.1,
+         "m.down_proj.weight": torch.randn(H, I) * 0.1, "e.weight": torch.randn(V, H),
+         "h.weight": torch.randn(V, H) * 0.1}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    ctx = ctx_for(w, dtype)
+    mlp = create("feed_forward", PartSpec("swiglu", {"hidden_size": H, "intermediate_size": I}), "m", ctx)
+    x = torch.randn(9, H).to(dtype)
+    wf = {k: v.float() for k, v in w.items()}
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
+    torch.testing.assert_close(mlp.forward(x.to(DEV), None).float().cpu(),
+                               plain.swiglu_mlp(x.float(), wf, "m"), atol=tol, rtol=tol)
+    emb = create("embedding", PartSpec("token", {"vocab_size": V, "hidden_size": H}), "e", ctx)
+    ids = [5, 130, 0, 5]
+    out = emb.forward(torch.tensor(ids, dtype=torch.int32, device=DEV))
+    assert out.dtype == torch.float32
+    torch.testing.assert_close(out.cpu(), plain.embedding(wf["e.weight"], ids), atol=0, rtol=0)
+    for tied in (None, "e.weight"):
+        head = create("head", PartSpec("linear", {"vocab_size": V, "hidden_size": H, "tied_to": tied}),
+                      "h", ctx)
+        logits = head.forward(x.to(DEV))
+        assert logits.dtype == torch.float32
+        torch.testing.assert_close(logits.cpu(), plain.linear(x.float(), wf[tied or "h.weight"]),
+                                   atol=tol * 10, rtol=tol)
+
+
+# --------------------------------------------------- models built from a ModelSpec
+def layer_spec(H, nh, nkv, d, I, eps, theta, window, mixer="attention", extra=None):
+    from rust_llm_inference_server_amd.parts import PartSpec
+    norm = PartSpec("rmsnorm", {"size": H, "eps": eps})
+    mixer_params = {"hidden_size": H, "num_heads": nh, "num_kv_heads": nkv, "head_dim": d,
+                    "scale": 1 / math.sqrt(d), "window": window,
+                    "position": PartSpec("rope", {"rot_dim": d, "theta": theta, "scaling": None})}
+    if extra:
+        mixer_params = extra
+    return PartSpec("prenorm", {
+        "mixer": PartSpec(mixer, mixer_params),
+        "feed_forward": PartSpec("swiglu", {"hidden_size": H, "intermediate_size": I}),
+        "mixer_norm": norm, "ffn_norm": norm,
+        "names": {"mixer_norm": "input_layernorm", "mixer": "self_attn",
+                  "ffn_norm": "post_attention_layernorm", "feed_forward": "mlp"}})
+
+
+def toy_spec(blocks, run_order=None, H=64, V=97):
+    from rust_llm_inference_server_amd.models import LayerSpec, ModelSpec
+    from rust_llm_inference_server_amd.parts import PartSpec
+    return ModelSpec(
+        hidden_size=H, vocab_size=V,
+        embedding=PartSpec("token", {"vocab_size": V, "hidden_size": H}),
+        embedding_prefix="model.embed_tokens",
+        layers=[LayerSpec(b, f"model.layers.{i}") for i, b in enumerate(blocks)],
+        final_norm=PartSpec("rmsnorm", {"size": H, "eps": 1e-5}), final_norm_prefix="model.norm",
+        head=PartSpec("linear", {"vocab_size": V, "hidden_size": H, "tied_to": None}),
+        head_prefix="lm_head", run_order=run_order)
+
+
+def plain_toy_forward(w, ids, layers, runs, H=64, eps=1e-5, theta=1e4):
+    """Whole-sequence forward of the toy models: ``layers`` is a list of dicts
+    (nh, nkv, d, window), ``runs`` a list of (layer, cache_of) like the run order."""
+    x = plain.embedding(w["model.embed_tokens.weight"], ids)
+    T = len(ids)
+    kv_of_run = {}
+    for r, (li, cache_of) in enumerate(runs):
+        L, p = layers[li], f"model.layers.{li}"
+        h = plain.rms_norm(x, w[f"{p}.input_layernorm.weight"], eps)
+        nh, nkv, d = L["nh"], L["nkv"], L["d"]
+        inv = plain.inv_freqs(d, theta, None)
+        cos, sin = plain.rope_tables(inv, range(T))
+        q = plain.linear(h, w[f"{p}.self_attn.q_proj.weight"]).reshape(T, nh, d).transpose(0, 1)
+        q = plain.rope_apply(q, cos, sin)
+        if cache_of is None:
+            k = plain.linear(h, w[f"{p}.self_attn.k_proj.weight"]).reshape(T, nkv, d).transpose(0, 1)
+            v = plain.linear(h, w[f"{p}.self_attn.v_proj.weight"]).reshape(T, nkv, d).transpose(0, 1)
+            kv_of_run[r] = (plain.rope_apply(k, cos, sin), v)
+        k, v = kv_of_run[r if cache_of is None else cache_of]
+        o = plain.gqa_attention(q, k, v, plain.causal_mask(T, 0, L["window"]))
+        x = x + plain.linear(o.transpose(0, 1).reshape(T, nh * d), w[f"{p}.self_attn.o_proj.weight"])
+        h = plain.rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], eps)
+        x = x + plain.swiglu_mlp(h, w, f"{p}.mlp")
+    return plain.linear(plain.rms_norm(x, w["model.norm.weight"], eps), w["lm_head.weight"])
+
+
+def run_families(spec, weights, dtype, reqs, ref, tol, page_size=8, check_window_pages=False):
+    from rust_llm_inference_server_amd.engine import ModelRunner
+    from rust_llm_inference_server_amd.models import Model
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    for build in (traces.trace_whole, traces.trace_tail, traces.trace_portions, traces.trace_mixed):
+        steps, max_tokens = build(reqs)
+        model = Model(spec, {k: v.to(tdt).to(DEV) for k, v in weights.items()}, tdt, DEV, 256)
+        runner = ModelRunner(model, num_pages=max_tokens // page_size, page_size=page_size,
+                             max_num_seqs=8)
+        outputs = traces.replay_in_process(runner, steps)
+        got = traces.collect(steps, outputs, spec.vocab_size)
+        for k, tokens in reqs.items():
+            mine = torch.stack([got[k][p] for p in range(len(tokens))])
+            diff = (mine - ref[k]).abs().max(dim=-1).values
+            bad = (diff > tol).nonzero()
+            assert bad.numel() == 0, (f"{build.__name__} request {k}: first wrong position "
+                                      f"{int(bad[0])} (|diff| {diff[bad[0]].item():.3e})")
+        for g in range(runner.cache.num_groups):
+            assert runner.cache.num_free_pages(g) == runner.cache.num_pages(g)
+    return runner
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
+def test_window_layers_beside_full_layers(dtype, tol):
+    """Layer 0 sees every earlier position, layer 1 only the last 24, layer 2 the last 5 (less
+    than a page): three page groups; windowed groups give pages back while a request runs."""
+    from rust_llm_inference_server_amd.weights import random_weights
+    layers = [dict(nh=4, nkv=2, d=16, window=None), dict(nh=4, nkv=2, d=16, window=24),
+              dict(nh=2, nkv=1, d=32, window=5)]
+    spec = toy_spec([layer_spec(64, L["nh"], L["nkv"], L["d"], 96, 1e-5, 1e4, L["window"]) for L in layers])
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    w = {k: v.to(tdt).float() for k, v in random_weights(spec.tensor_specs(), 3, torch.float32).items()}
+    # sharpen attention so that a key just outside a window would be seen if it leaked in
+    for i in range(3):
+        w[f"model.layers.{i}.self_attn.q_proj.weight"] *= 8
+        w[f"model.layers.{i}.self_attn.k_proj.weight"] *= 8
+    w = {k: v.to(tdt).float() for k, v in w.items()}
+    reqs = traces.random_requests(97, [70, 9, 130, 33, 2, 64], seed=5)
+    runs = [(0, None), (1, None), (2, None)]
+    ref = {k: plain_toy_forward(w, t, layers, runs) for k, t in reqs.items()}
+    runner = run_families(spec, w, dtype, reqs, ref, tol)
+    assert [g.window for g in runner.cache.groups] == [None, 24, 5]
+    # pages of the windowed groups return while the request is alive
+    runner.reserve(0, 100)
+    from rust_llm_inference_server_amd.engine import StepEntry
+    runner.step([StepEntry(0, reqs["r2"][:100], [])])
+    free = [runner.cache.num_free_pages(g) for g in range(3)]
+    assert free[0] < free[1] < free[2]
+    runner.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
+def test_run_order_names_a_layer_twice_and_shares_a_cache(dtype, tol):
+    """Run order: layer 0, layer 1, layer 0 again (a second cache of its own), then layer 1
+    reading the cache its first run wrote (it writes nothing)."""
+    from rust_llm_inference_server_amd.models import RunEntry
+    from rust_llm_inference_server_amd.weights import random_weights
+    layers = [dict(nh=4, nkv=1, d=16, window=None), dict(nh=3, nkv=3, d=16, window=None)]
+    order = [RunEntry(0), RunEntry(1), RunEntry(0), RunEntry(1, cache_of=1)]
+    spec = toy_spec([layer_spec(64, L["nh"], L["nkv"], L["d"], 80, 1e-5, 1e4, None) for L in layers],
+                    run_order=order)
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    w = {k: v.to(tdt).float() for k, v in random_weights(spec.tensor_specs(), 4, torch.float32).items()}
+    reqs = traces.random_requests(97, [40, 5, 90, 17], seed=6)
+    runs = [(0, None), (1, None), (0, None), (1, 1)]
+    ref = {k: plain_toy_forward(w, t, layers, runs) for k, t in reqs.items()}
+    from rust_llm_inference_server_amd.models import Model
+    model = Model(spec, {k: v.to(DEV) for k, v in w.items()}, torch.float32, DEV, 256)
+    assert [len(g.writer_runs) for g in model.cache_groups] == [2, 1]
+    assert [(b.group, b.slot, b.writes) for b in model.bindings] == \
+        [(0, 0, True), (1, 0, True), (0, 1, True), (1, 0, False)]
+    run_families(spec, w, dtype, reqs, ref, tol)
+    from rust_llm_inference_server_amd.models import ModelSpec
+    bad = toy_spec([layer_spec(64, 4, 1, 16, 80, 1e-5, 1e4, None)] * 2,
+                   run_order=[RunEntry(0, cache_of=1), RunEntry(1)])
+    with pytest.raises(ValueError, match="does not run before"):
+        bad.validate()
+
+
+# ------------------------------------------------ a toy mixer with state of its own
+def register_toy():
+    """Defined and registered here, in the test: a mixer whose memory of the past is one
+    vector per request, the running sum of its inputs (kept in the request's state slot)."""
+    from rust_llm_inference_server_amd.parts import Mixer, TensorSpec, register
+    from rust_llm_inference_server_amd.parts.base import join
+
+    @register("mixer", "toy_running_sum")
+    class RunningSum(Mixer):
+        @classmethod
+        def tensor_specs(cls, params, prefix):
+            return [TensorSpec(join(prefix, "mix.weight"), (params["hidden_size"],) * 2)]
+
+        def __init__(self, params, prefix, ctx):
+            super().__init__(params, prefix, ctx)
+            self.size = params["hidden_size"]
+            self.weight = ctx.take(join(prefix, "mix.weight")).float()
+            self.decay = float(params["decay"])
+            self.act_dtype = ctx.act_dtype
+
+        def state_bytes(self):
+            return 4 * self.size
+
+        def forward(self, x, step, binding):
+            out = torch.empty_like(x, dtype=torch.float32)
+            begin = 0
+            for n, slot in zip(step.host_new, step.host_state_slots):
+                state = binding.state[slot].view(torch.float32)
+                for t in range(begin, begin + n):            # in order, token by token
+                    state.mul_(self.decay).add_(x[t].float())
+                    out[t] = state
+                begin += n
+            return (out @ self.weight.t()).to(self.act_dtype)
+
+    return RunningSum
+
+
+def plain_running_sum_model(w, ids, layers, H=48, eps=1e-5, decay=0.9):
+    x = plain.embedding(w["model.embed_tokens.weight"], ids)
+    T = len(ids)
+    for li, kind in enumerate(layers):
+        p = f"model.layers.{li}"
+        h = plain.rms_norm(x, w[f"{p}.input_layernorm.weight"], eps)
+        if kind == "toy":
+            s, rows = torch.zeros(H), []
+            for t in range(T):
+                s = s * decay + h[t]
+                rows.append(s)
+            x = x + torch.stack(rows) @ w[f"{p}.self_attn.mix.weight"].t()
+        else:
+            cfg = {"num_attention_heads": 3, "num_key_value_heads": 1, "head_dim": 16}
+            x = x + plain.attention_layer(h, w, f"{p}.self_attn", cfg, plain.inv_freqs(16, 1e4, None))
+        h = plain.rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], eps)
+        x = x + plain.swiglu_mlp(h, w, f"{p}.mlp")
+    return plain.linear(plain.rms_norm(x, w["model.norm.weight"], eps), w["lm_head.weight"])
+
+
+def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
+    """A new mixer kind and a new architecture name, both registered from the test; the model
+    folder is loaded through the ordinary loader and replayed in every way of cutting, with
+    fewer state slots than requests so that slots (and their stale contents) are used again."""
+    from rust_llm_inference_server_amd.engine import ModelRunner, load_model
+    from rust_llm_inference_server_amd.registry import Architecture, register_architecture
+    from rust_llm_inference_server_amd.weights import write_model_folder
+    register_toy()
+    H = 48
+    kinds = ["toy", "attention", "toy"]
+
+    def build_spec(cfg):
+        blocks = []
+        for kind in cfg["mixers"]:
+            if kind == "toy":
+                blocks.append(layer_spec(H, 0, 0, 0, 64, 1e-5, 1e4, None, mixer="toy_running_sum",
+                                         extra={"hidden_size": H, "decay": 0.9}))
+            else:
+                blocks.append(layer_spec(H, 3, 1, 16, 64, 1e-5, 1e4, None))
+        return toy_spec(blocks, H=H, V=cfg["vocab_size"])
+
+    register_architecture(Architecture("ToyForCausalLM", parse_config=lambda d: d,
+                                       build_spec=build_spec, config_to_dict=lambda c: c))
+    config = {"architectures": ["ToyForCausalLM"], "vocab_size": 97, "mixers": kinds}
+    spec = build_spec(config)
+    folder = str(tmp_path / "toy")
+    write_model_folder(folder, config, spec.tensor_specs(), seed=9)
+    w = plain.read_weights(folder)
+    reqs = traces.random_requests(97, [30, 4, 70, 11, 45, 2], seed=8)
+    ref = {k: plain_running_sum_model(w, t, kinds) for k, t in reqs.items()}
+    for build in (traces.trace_whole, traces.trace_tail, traces.trace_portions, traces.trace_mixed):
+        steps, max_tokens = build(reqs)
+        model = load_model(folder, "float32", max_positions=128)
+        assert model.state_bytes == 2 * 4 * H and len(model.cache_groups) == 1
+        runner = ModelRunner(model, num_pages=max_tokens // 16, page_size=16, max_num_seqs=4)
+        assert runner.cache.num_state_slots == 4          # 6 requests share 4 slots over time
+        got = traces.collect(steps, traces.replay_in_process(runner, steps), 97)
+        for k, tokens in reqs.items():
+            mine = torch.stack([got[k][p] for p in range(len(tokens))])
+            assert (mine - ref[k]).abs().max().item() < 2e-4, f"{build.__name__} request {k}"
+        assert runner.cache.num_free_slots() == 4
+
+
+def test_long_decoding_stays_on_the_plain_path(tiny_folders):
+    """A short prompt, then 230 tokens one by one (teacher-forced), across many page edges."""
+    from rust_llm_inference_server_amd.engine import ModelRunner, StepEntry, load_model
+    folder = tiny_folders["b"]
+    w, c = plain.read_weights(folder), plain.read_config(folder)
+    ids = traces.random_requests(c["vocab_size"], [240], seed=12)["r0"]
+    ref = plain.forward(w, c, ids)
+    for dtype, tol in (("float32", 1e-4), ("bfloat16", 3e-2)):
+        model = load_model(folder, dtype, max_positions=256)
+        runner = ModelRunner(model, num_pages=32, page_size=8, max_num_seqs=2)
+        runner.reserve(0, 10)
+        rows = [runner.step([StepEntry(0, ids[:10], list(range(10)))]).cpu()]
+        for p in range(10, len(ids)):
+            runner.reserve(0, p + 1)
+            rows.append(runner.step([StepEntry(0, [ids[p]], [0])]).cpu())
+        diff = (torch.cat(rows) - ref).abs().max(dim=-1).values
+        assert diff.max().item() < tol, f"{dtype}: first wrong position {int((diff >= tol).nonzero()[0])}"
