@@ -296,7 +296,7 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
         blocks = []
         for kind in cfg["mixers"]:
             if kind == "toy":
-                blocks.append(layer_spec(H, 0, 0, 0, 64, 1e-5, 1e4, None, mixer="toy_running_sum",
+                blocks.append(layer_spec(H, 1, 1, 16, 64, 1e-5, 1e4, None, mixer="toy_running_sum",
                                          extra={"hidden_size": H, "decay": 0.9}))
             else:
                 blocks.append(layer_spec(H, 3, 1, 16, 64, 1e-5, 1e4, None))
