@@ -40,6 +40,8 @@ def runtime() -> ctypes.CDLL:
             "rlis_cache_table": (c_int, [c_void_p, c_longlong, c_int, PI, c_int]),
             "rlis_cache_info": (c_int, [c_void_p, c_longlong, PI]),
             "rlis_cache_check": (c_int, [c_void_p, c_char_p, c_int]),
+            "rlis_cache_decode_batch": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p,
+                                                c_void_p, c_void_p, c_void_p]),
             "rlis_sched_create": (c_void_p, [c_void_p, c_int, c_int, c_int, c_int]),
             "rlis_sched_destroy": (None, [c_void_p]),
             "rlis_sched_add": (c_int, [c_void_p, c_longlong, c_int]),
@@ -185,6 +187,15 @@ class CacheManager:
     def free(self, seq: int) -> None:
         if runtime().rlis_cache_free(self._h, seq) != 0:
             raise RuntimeError(rt_error())
+
+    def decode_batch(self, seqs_ptr: int, n: int, width: int, positions_ptr: int,
+                     state_slots_ptr: int, tables_ptrs, slots_ptrs) -> None:
+        """Fill the metadata of a step of one token per request straight into caller-owned
+        int32 buffers (see ``rlis_cache_decode_batch``); ``tables_ptrs`` and ``slots_ptrs``
+        are ctypes arrays of one pointer per group."""
+        if runtime().rlis_cache_decode_batch(self._h, seqs_ptr, n, width, positions_ptr,
+                                             state_slots_ptr, tables_ptrs, slots_ptrs) != 0:
+            raise ValueError(rt_error())
 
     def check_invariants(self) -> None:
         buf = ctypes.create_string_buffer(512)

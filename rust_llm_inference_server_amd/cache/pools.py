@@ -23,11 +23,15 @@ class CachePools:
         self.dtype = dtype
         self.k: List[torch.Tensor] = []
         self.v: List[torch.Tensor] = []
+        # One page beyond the manager's is scratch: padding rows of a captured decode step
+        # read and write it, so they touch nothing a request owns.
+        self.scratch_page = max(num_pages) if len(num_pages) else 0
         for layout, pages in zip(cache_groups, num_pages):
             r, n = layout.request, max(1, len(layout.writer_runs))
-            self.k.append(torch.zeros((n, pages, r.num_kv_heads, page_size, r.head_dim),
+            total = self.scratch_page + 1
+            self.k.append(torch.zeros((n, total, r.num_kv_heads, page_size, r.head_dim),
                                       dtype=dtype, device=device))
-            self.v.append(torch.zeros((n, pages, r.num_kv_heads, r.head_dim, page_size),
+            self.v.append(torch.zeros((n, total, r.num_kv_heads, r.head_dim, page_size),
                                       dtype=dtype, device=device))
         self.state: Optional[torch.Tensor] = None
         if state_bytes > 0 and num_state_slots > 0:

@@ -98,37 +98,72 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
   const int wave_q_last = min(n_new - 1, wave_q_first + 15);
   bf16_t* my_ps = Ps + wave * 16 * PS;
 
-  for (int k0 = kt0; k0 < khi; k0 += BN) {
-    // ---- stage K [BN][D] and V^T [d][BN] ---------------------------------------------
-    for (int c = tid; c < BN * (D / 8); c += 256) {
+  // Staging registers: the next tile's K and V^T chunks travel global -> registers while the
+  // current tile is computed from LDS, then registers -> LDS.
+  constexpr int K_CHUNKS = BN * (D / 8);
+  constexpr int KCH = (K_CHUNKS + 255) / 256;
+  constexpr int VCH = (D * (BN / 8) + 255) / 256;
+  uint4 kreg[KCH], vreg[VCH];
+  const int v_chunks = d * (BN / 8);
+  auto load_tile = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      const int c = tid + i * 256;
       const int key = c / (D / 8), dc = c % (D / 8);
       const int kpos = k0 + key;
       uint4 v = make_uint4(0, 0, 0, 0);
-      if (kpos < khi && dc * 8 < d) {
+      if (c < K_CHUNKS && kpos < khi && dc * 8 < d) {
         const long long page = table[kpos / page_size];
         const int off = kpos % page_size;
         v = *(const uint4*)(k_pages + ((page * nkv + kvh) * page_size + off) * d + dc * 8);
       }
-      *(uint4*)(Ks + key * KS + dc * 8) = v;
+      kreg[i] = v;
     }
-    for (int c = tid; c < d * (BN / 8); c += 256) {
-      const int dim = c / (BN / 8), kg = c % (BN / 8);
-      const int kpos = k0 + kg * 8;
+#pragma unroll
+    for (int i = 0; i < VCH; ++i) {
+      const int c = tid + i * 256;
       Frag8 v;
       v.u = make_uint4(0, 0, 0, 0);
-      if (kpos < khi) {
-        const long long page = table[kpos / page_size];
-        const int off = kpos % page_size;
-        v.u = *(const uint4*)(v_pages + ((page * nkv + kvh) * (long long)d + dim) * page_size + off);
-        if (kpos + 8 > khi) {
+      if (c < v_chunks) {
+        const int dim = c / (BN / 8), kg = c % (BN / 8);
+        const int kpos = k0 + kg * 8;
+        if (kpos < khi) {
+          const long long page = table[kpos / page_size];
+          const int off = kpos % page_size;
+          v.u = *(const uint4*)(v_pages + ((page * nkv + kvh) * (long long)d + dim) * page_size + off);
+          if (kpos + 8 > khi) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (kpos + e >= khi) v.e[e] = 0;
+            for (int e = 0; e < 8; ++e)
+              if (kpos + e >= khi) v.e[e] = 0;
+          }
         }
       }
-      *(uint4*)(Vs + dim * VS + kg * 8) = v.u;
+      vreg[i] = v.u;
     }
-    __syncthreads();
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      const int c = tid + i * 256;
+      if (c < K_CHUNKS) *(uint4*)(Ks + (c / (D / 8)) * KS + (c % (D / 8)) * 8) = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < VCH; ++i) {
+      const int c = tid + i * 256;
+      if (c < v_chunks) *(uint4*)(Vs + (c / (BN / 8)) * VS + (c % (BN / 8)) * 8) = vreg[i];
+    }
+  };
+
+  // Scores are kept in the base-2 domain: s * scale * log2(e), so that e^x is one v_exp_f32.
+  const float scale2 = scale * 1.4426950408889634f;
+  if (kt0 < khi) {
+    load_tile(kt0);
+    store_tile();
+  }
+  __syncthreads();
+  for (int k0 = kt0; k0 < khi; k0 += BN) {
+    const bool more = k0 + BN < khi;
+    if (more) load_tile(k0 + BN);
 
     // Tiles wholly after this wave's last query contribute nothing to it.
     const bool wave_active = (wave_q_first < n_new) && (k0 <= P + wave_q_last);
@@ -156,7 +191,7 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
         for (int nb = 0; nb < BN / 16; ++nb) {
           const int kpos = k0 + nb * 16 + l16;
           const bool ok = (qi < n_new) && (kpos <= qpos) && (window <= 0 || kpos > qpos - window);
-          const float sv = ok ? s_acc[nb][r] * scale : -INFINITY;
+          const float sv = ok ? s_acc[nb][r] * scale2 : -INFINITY;
           s_acc[nb][r] = sv;
           row_max = fmaxf(row_max, sv);
         }
@@ -167,13 +202,13 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
 #pragma unroll
         for (int nb = 0; nb < BN / 16; ++nb) {
           const float sv = s_acc[nb][r];
-          const float p = (sv == -INFINITY) ? 0.f : expf(sv - m_new);
+          const float p = (sv == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(sv - m_new);
           s_acc[nb][r] = p;
           row_sum += p;
         }
 #pragma unroll
         for (int o = 1; o < 16; o <<= 1) row_sum += __shfl_xor(row_sum, o, kWave);
-        corr[r] = (m[r] == -INFINITY) ? 0.f : expf(m[r] - m_new);
+        corr[r] = (m[r] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m[r] - m_new);
         l[r] = l[r] * corr[r] + row_sum;
         m[r] = m_new;
       }
@@ -209,6 +244,10 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
       }
     }
     __syncthreads();
+    if (more) {
+      store_tile();
+      __syncthreads();
+    }
   }
 
   // ---- normalise and store ------------------------------------------------------------

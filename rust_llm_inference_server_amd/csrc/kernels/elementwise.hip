@@ -103,12 +103,61 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
   }
 }
 
+// The same for rows of at most NT * VPT elements, which stay in registers between the sum
+// of squares and the store: one read of every input, no second pass.
+template <typename TD, typename TW, typename TO, int NT, int VPT>
+__global__ __launch_bounds__(NT) void add_rmsnorm_small_kernel(
+    float* __restrict__ resid, const TD* __restrict__ delta, const TW* __restrict__ weight,
+    TO* __restrict__ out, const int* __restrict__ rows, int H, float eps, int write_resid) {
+  __shared__ float red[NT / kWave];
+  const int r = blockIdx.x;
+  const long long src = rows ? (long long)rows[r] : (long long)r;
+  float* x = resid + src * H;
+  const TD* d = delta ? delta + src * H : nullptr;
+  float v[VPT], w[VPT];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int j = threadIdx.x + i * NT;
+    v[i] = 0.f;
+    w[i] = 0.f;
+    if (j < H) {
+      v[i] = x[j];
+      if (d) v[i] += ld(d + j);
+      w[i] = ld(weight + j);
+    }
+    ss += v[i] * v[i];
+  }
+  if (d && write_resid) {
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int j = threadIdx.x + i * NT;
+      if (j < H) x[j] = v[i];
+    }
+  }
+  ss = block_sum<NT>(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+  TO* o = out + (long long)r * H;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int j = threadIdx.x + i * NT;
+    if (j < H) st(o + j, v[i] * inv * w[i]);
+  }
+}
+
 template <typename TD, typename TW, typename TO>
 static void launch_add_rmsnorm(float* resid, const void* delta, const void* weight, void* out,
                                const int* rows, int R, int H, float eps, int write_resid,
                                hipStream_t stream) {
-  add_rmsnorm_kernel<TD, TW, TO, 256><<<R, 256, 0, stream>>>(
-      resid, (const TD*)delta, (const TW*)weight, (TO*)out, rows, H, eps, write_resid);
+  if (H <= 256 * 4)
+    add_rmsnorm_small_kernel<TD, TW, TO, 256, 4><<<R, 256, 0, stream>>>(
+        resid, (const TD*)delta, (const TW*)weight, (TO*)out, rows, H, eps, write_resid);
+  else if (H <= 256 * 16)
+    add_rmsnorm_small_kernel<TD, TW, TO, 256, 16><<<R, 256, 0, stream>>>(
+        resid, (const TD*)delta, (const TW*)weight, (TO*)out, rows, H, eps, write_resid);
+  else
+    add_rmsnorm_kernel<TD, TW, TO, 256><<<R, 256, 0, stream>>>(
+        resid, (const TD*)delta, (const TW*)weight, (TO*)out, rows, H, eps, write_resid);
 }
 
 RLIS_API int rlis_add_rmsnorm(float* resid, const void* delta, int delta_dtype,

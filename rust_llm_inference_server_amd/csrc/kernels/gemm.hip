@@ -6,8 +6,9 @@
 //  * gemm_bf16_mfma: bfloat16 operands on the matrix cores (v_mfma_f32_32x32x16_bf16),
 //    float32 accumulation, output bfloat16 or float32.  K must be a multiple of 8.
 //  * gemm_bf16_skinny: the decode shape, up to 64 rows of x.  Each weight row is read once
-//    for all rows of x; a wave owns 16 weight rows and a slice of K, the four waves of a
-//    workgroup are summed in a fixed order.  K must be a multiple of 8.
+//    for all rows of x; a wave owns 16 (or 32) weight rows and a slice of K, the eight waves of
+//    a workgroup are summed in a fixed order.  K must be a multiple of 8.  A gated variant
+//    fuses the SwiGLU of the feed-forward into the gate/up product.
 //
 // In every kernel an output element is a sum over k in an order that depends only on the
 // kernel and K, never on which other rows are in the batch.
@@ -240,103 +241,180 @@ RLIS_API int rlis_gemm_bf16_mfma(const void* A, const void* B, void* C, int c_dt
 }
 
 // ============================================================ skinny (decode) product
-// y (T, N) = x (T, K) * W (N, K)^T for T <= 16 * NT.  Workgroup = 4 waves; it owns 16 weight
-// rows, wave w owns the k range [w * kslice, (w + 1) * kslice).  v_mfma_f32_16x16x32_bf16 with
-// the weight rows as the M side and the tokens as the N side: lane l holds weight row l % 16
-// (A) or token l % 16 (B) and the 8 consecutive k at (l / 16) * 8; the accumulator holds
-// token l % 16 and weight rows (l / 16) * 4 + r.
-template <typename TC, int NT>
-__global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ X,
+// y (T, N) = x (T, K) * W (N, K)^T for T <= 64 (NT = ceil(T / 16) token tiles).  A workgroup of
+// eight waves owns 16 * RB weight rows; wave w owns the k range [w * kslice, (w + 1) * kslice)
+// and walks it in chunks of 32 * U, issuing all loads of a chunk before its products so that
+// U * RB 16-byte weight loads per lane are in flight.  v_mfma_f32_16x16x32_bf16 with the weight
+// rows as the M side and the tokens as the N side: lane l holds weight row l % 16 (A) or token
+// l % 16 (B) and the 8 consecutive k at (l / 16) * 8; the accumulator holds token l % 16 and
+// weight rows (l / 16) * 4 + r.  The eight waves are summed through LDS in wave order.
+//
+// GATED: W holds gate rows [0, N) and up rows [N, 2N); the workgroup computes both for its
+// columns and stores silu(gate) * up (the SwiGLU of crates/model/src/layers.rs:179-186), so
+// the (T, 2N) intermediate never exists.
+constexpr int kSkinnyWaves = 8;
+
+template <typename TC, int NT, int RB, bool GATED>
+__global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ X,
                                                                const bf16_t* __restrict__ W,
                                                                TC* __restrict__ Y, int T, int N,
                                                                int K, long long ldx,
                                                                long long ldw, long long ldy,
                                                                int kslice) {
-  __shared__ float red[4][NT][4][64];
+  constexpr int RBT = GATED ? 2 * RB : RB;                 // row blocks of 16 weight rows
+  constexpr int U = (NT * RBT <= 1) ? 8 : ((NT * RBT <= 4) ? 4 : 2);
+  __shared__ float red[kSkinnyWaves][NT][256];
+  __shared__ float fin[RBT][NT][256];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-  const int n0 = blockIdx.x * 16;
-  const int wrow = n0 + (lane % 16);
-  const int kq = (lane / 16) * 8;
-  const bool wvalid = wrow < N;
-  const bf16_t* wp = W + (long long)(wvalid ? wrow : 0) * ldw;
+  const int m = lane % 16, kq = (lane / 16) * 8;
+  const int n0 = blockIdx.x * 16 * RB;
+
+  const bf16_t* wp[RBT];
+  bool wvalid[RBT];
+#pragma unroll
+  for (int rb = 0; rb < RBT; ++rb) {
+    const int col = n0 + (rb % RB) * 16 + m;               // output column
+    wvalid[rb] = col < N;
+    const long long row = (GATED && rb >= RB) ? (long long)N + col : col;
+    wp[rb] = W + (wvalid[rb] ? row : 0) * ldw;
+  }
   const bf16_t* xp[NT];
   bool xvalid[NT];
 #pragma unroll
   for (int tt = 0; tt < NT; ++tt) {
-    const int tok = tt * 16 + (lane % 16);
+    const int tok = tt * 16 + m;
     xvalid[tt] = tok < T;
     xp[tt] = X + (long long)(xvalid[tt] ? tok : 0) * ldx;
   }
-  f32x4 acc[NT];
+  f32x4 acc[RBT][NT];
 #pragma unroll
-  for (int tt = 0; tt < NT; ++tt) acc[tt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int rb = 0; rb < RBT; ++rb)
+#pragma unroll
+    for (int tt = 0; tt < NT; ++tt) acc[rb][tt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
   const int kbeg = wave * kslice;
   const int kend = min(K, kbeg + kslice);
   const uint4 zero = make_uint4(0, 0, 0, 0);
-  for (int k = kbeg; k < kend; k += 32) {
-    const int gk = k + kq;
-    const bool kin = gk < kend;  // kslice is a multiple of 32 and K of 8: whole chunks only
-    Frag8 a;
-    a.u = (wvalid && kin) ? *(const uint4*)(wp + gk) : zero;
+  for (int k = kbeg; k < kend; k += 32 * U) {
+    Frag8 a[RBT][U], b[NT][U];
 #pragma unroll
-    for (int tt = 0; tt < NT; ++tt) {
-      Frag8 b;
-      b.u = (xvalid[tt] && kin) ? *(const uint4*)(xp[tt] + gk) : zero;
-      acc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[tt], 0, 0, 0);
+    for (int u = 0; u < U; ++u) {
+      const int gk = k + u * 32 + kq;
+      const bool kin = gk < kend;     // kslice is a multiple of 32 and K of 8: whole chunks only
+#pragma unroll
+      for (int rb = 0; rb < RBT; ++rb)
+        a[rb][u].u = (wvalid[rb] && kin) ? *(const uint4*)(wp[rb] + gk) : zero;
+#pragma unroll
+      for (int tt = 0; tt < NT; ++tt)
+        b[tt][u].u = (xvalid[tt] && kin) ? *(const uint4*)(xp[tt] + gk) : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int rb = 0; rb < RBT; ++rb)
+#pragma unroll
+        for (int tt = 0; tt < NT; ++tt)
+          acc[rb][tt] =
+              __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rb][u].v, b[tt][u].v, acc[rb][tt], 0, 0, 0);
+  }
+
+  // Sum the eight waves, one row block at a time: fin[rb][tt][r * 64 + l] is the product for
+  // token tt * 16 + l % 16 and weight row (l / 16) * 4 + r of block rb.
+#pragma unroll
+  for (int rb = 0; rb < RBT; ++rb) {
+    if (rb > 0) __syncthreads();
+#pragma unroll
+    for (int tt = 0; tt < NT; ++tt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[wave][tt][r * 64 + lane] = acc[rb][tt][r];
+    __syncthreads();
+    for (int i = tid; i < NT * 256; i += 512) {
+      const int tt = i / 256, e = i % 256;
+      float s = red[0][tt][e];
+#pragma unroll
+      for (int w = 1; w < kSkinnyWaves; ++w) s += red[w][tt][e];
+      fin[rb][tt][e] = s;
     }
   }
-#pragma unroll
-  for (int tt = 0; tt < NT; ++tt)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave][tt][r][lane] = acc[tt][r];
   __syncthreads();
-  // 16 * NT tokens x 16 rows results, summed over the four waves in order.
-  for (int i = tid; i < NT * 256; i += 256) {
-    const int tt = i / 256, rem = i % 256;
-    const int r = rem / 64, l = rem % 64;
-    const float s = ((red[0][tt][r][l] + red[1][tt][r][l]) + red[2][tt][r][l]) + red[3][tt][r][l];
+  for (int i = tid; i < RB * NT * 256; i += 512) {
+    const int rb = i / (NT * 256), tt = (i / 256) % NT, e = i % 256;
+    const int r = e / 64, l = e % 64;
     const int tok = tt * 16 + (l % 16);
-    const int row = n0 + (l / 16) * 4 + r;
-    if (tok < T && row < N) st(Y + (long long)tok * ldy + row, s);
+    const int col = n0 + rb * 16 + (l / 16) * 4 + r;
+    if (tok >= T || col >= N) continue;
+    float v = fin[rb][tt][e];
+    if (GATED) {
+      const float up = fin[RB + rb][tt][e];
+      v = v / (1.0f + expf(-v)) * up;
+    }
+    st(Y + (long long)tok * ldy + col, v);
   }
+}
+
+template <typename TC, int NT, int RB, bool GATED>
+static void launch_skinny(const void* X, const void* W, void* Y, int T, int N, int K,
+                          long long ldx, long long ldw, long long ldy, hipStream_t stream) {
+  const int kslice = ceil_div(ceil_div(K, kSkinnyWaves), 32) * 32;
+  const int blocks = ceil_div(N, 16 * RB);
+  gemm_bf16_skinny_kernel<TC, NT, RB, GATED><<<blocks, 512, 0, stream>>>(
+      (const bf16_t*)X, (const bf16_t*)W, (TC*)Y, T, N, K, ldx, ldw, ldy, kslice);
+}
+
+template <typename TC, bool GATED>
+static void dispatch_skinny(const void* X, const void* W, void* Y, int T, int N, int K,
+                            long long ldx, long long ldw, long long ldy, hipStream_t stream) {
+  const int nt = ceil_div(T, 16);
+  // Two row blocks per workgroup when that still leaves every compute unit a workgroup or two.
+  const bool wide = !GATED && N >= 8192;
+#define GO(NT)                                                                         \
+  do {                                                                                 \
+    if (wide) launch_skinny<TC, NT, 2, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream); \
+    else launch_skinny<TC, NT, 1, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);     \
+  } while (0)
+  switch (nt) {
+    case 1: GO(1); break;
+    case 2: GO(2); break;
+    case 3: GO(3); break;
+    default: GO(4); break;
+  }
+#undef GO
+}
+
+static int check_skinny(const char* name, const void* X, const void* W, int T, int N, int K,
+                        long long ldx, long long ldw, long long ldy) {
+  RLIS_REQUIRE(T >= 0 && T <= 64, "%s: T=%d rows, at most 64", name, T);
+  RLIS_REQUIRE(N > 0 && K > 0, "%s: bad sizes N=%d K=%d", name, N, K);
+  RLIS_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0,
+               "%s: K=%d and the row strides must be multiples of 8", name, K);
+  RLIS_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0,
+               "%s: operands must be 16-byte aligned", name);
+  RLIS_REQUIRE(ldx >= K && ldw >= K && ldy >= N, "%s: row strides shorter than rows", name);
+  return 0;
 }
 
 RLIS_API int rlis_gemm_bf16_skinny(const void* X, const void* W, void* Y, int y_dtype, int T,
                                    int N, int K, long long ldx, long long ldw, long long ldy,
                                    hipStream_t stream) {
-  RLIS_REQUIRE(T >= 0 && T <= 64, "gemm_bf16_skinny: T=%d rows, at most 64", T);
-  RLIS_REQUIRE(N > 0 && K > 0, "gemm_bf16_skinny: bad sizes N=%d K=%d", N, K);
-  RLIS_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0,
-               "gemm_bf16_skinny: K=%d and the row strides must be multiples of 8", K);
-  RLIS_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0,
-               "gemm_bf16_skinny: operands must be 16-byte aligned");
-  RLIS_REQUIRE(ldx >= K && ldw >= K && ldy >= N, "gemm_bf16_skinny: row strides shorter than rows");
+  if (check_skinny("gemm_bf16_skinny", X, W, T, N, K, ldx, ldw, ldy)) return 1;
   if (T == 0) return 0;
-  const int kslice = ceil_div(ceil_div(K, 4), 32) * 32;
-  const int blocks = ceil_div(N, 16);
-  const int nt = ceil_div(T, 16);
-#define LAUNCH(TC, NT)                                                                        \
-  gemm_bf16_skinny_kernel<TC, NT><<<blocks, 256, 0, stream>>>(                                \
-      (const bf16_t*)X, (const bf16_t*)W, (TC*)Y, T, N, K, ldx, ldw, ldy, kslice)
-  if (y_dtype == RLIS_F32) {
-    switch (nt) {
-      case 1: LAUNCH(float, 1); break;
-      case 2: LAUNCH(float, 2); break;
-      case 3: LAUNCH(float, 3); break;
-      default: LAUNCH(float, 4); break;
-    }
-  } else if (y_dtype == RLIS_BF16) {
-    switch (nt) {
-      case 1: LAUNCH(bf16_t, 1); break;
-      case 2: LAUNCH(bf16_t, 2); break;
-      case 3: LAUNCH(bf16_t, 3); break;
-      default: LAUNCH(bf16_t, 4); break;
-    }
-  } else {
+  if (y_dtype == RLIS_F32)
+    dispatch_skinny<float, false>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
+  else if (y_dtype == RLIS_BF16)
+    dispatch_skinny<bf16_t, false>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
+  else
     RLIS_REQUIRE(false, "gemm_bf16_skinny: unknown output dtype %d", y_dtype);
-  }
-#undef LAUNCH
   RLIS_LAUNCH_CHECK("gemm_bf16_skinny");
+  return 0;
+}
+
+// y (T, N) = silu(x Wg^T) * (x Wu^T) with W = [Wg; Wu] of shape (2N, K), bfloat16 throughout.
+RLIS_API int rlis_gemm_bf16_skinny_swiglu(const void* X, const void* W, void* Y, int T, int N,
+                                          int K, long long ldx, long long ldw, long long ldy,
+                                          hipStream_t stream) {
+  if (check_skinny("gemm_bf16_skinny_swiglu", X, W, T, N, K, ldx, ldw, ldy)) return 1;
+  if (T == 0) return 0;
+  dispatch_skinny<bf16_t, true>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
+  RLIS_LAUNCH_CHECK("gemm_bf16_skinny_swiglu");
   return 0;
 }

@@ -114,6 +114,46 @@ RT_API int rlis_cache_info(void* h, long long seq, int* info) {
   return 0;
 }
 
+// One decode token per request, for n requests at once: for request i writes the cached
+// length (the new token's position) to positions[i], its state slot to state_slots[i], and for
+// every group g its block table into tables[g][i * width ...] (missing pages as 0, the rest
+// of the row untouched) and the new token's write slot into slots[g][i].  tables and slots
+// are arrays of one pointer per group.  Returns 0, or -1 with a message when a request is
+// unknown, has no position reserved for the token, or a table is wider than `width`.
+RT_API int rlis_cache_decode_batch(void* h, const long long* seqs, int n, int width,
+                                   int* positions, int* state_slots, int** tables, int** slots) {
+  auto* m = static_cast<CacheManager*>(h);
+  const int ps = m->page_size();
+  for (int i = 0; i < n; ++i) {
+    const rlis::SeqEntry* e = m->entry(seqs[i]);
+    if (!e || e->num_computed + 1 > e->num_tokens) {
+      g_error = "request " + std::to_string(seqs[i]) + ": position " +
+                std::to_string(e ? e->num_tokens : 0) + " has no page reserved";
+      return -1;
+    }
+    const int pos = e->num_computed;
+    positions[i] = pos;
+    state_slots[i] = e->state_slot < 0 ? 0 : e->state_slot;
+    for (int g = 0; g < m->num_groups(); ++g) {
+      const auto& pages = e->pages[g];
+      if ((int)pages.size() > width) {
+        g_error = "block table of request " + std::to_string(seqs[i]) + " is wider than the buffer";
+        return -1;
+      }
+      int* row = tables[g] + (long long)i * width;
+      for (size_t p = 0; p < pages.size(); ++p) row[p] = pages[p] < 0 ? 0 : pages[p];
+      const int page = pages[pos / ps];
+      if (page < 0) {
+        g_error = "request " + std::to_string(seqs[i]) + ": position " + std::to_string(pos) +
+                  " has no page reserved";
+        return -1;
+      }
+      slots[g][i] = page * ps + pos % ps;
+    }
+  }
+  return 0;
+}
+
 RT_API int rlis_cache_check(void* h, char* buf, int cap) {
   return copy_message(static_cast<CacheManager*>(h)->check_invariants(), buf, cap);
 }

@@ -105,7 +105,8 @@ class Engine:
             watermark = max(1, num_pages // 100)            # engine.rs:263-271
         self.runner = ModelRunner(model, num_pages=num_pages, page_size=cfg.block_size,
                                   max_num_seqs=cfg.max_num_seqs,
-                                  max_batched_tokens=max(cfg.max_batched_tokens, cfg.max_num_seqs))
+                                  max_batched_tokens=max(cfg.max_batched_tokens, cfg.max_num_seqs),
+                                  use_graphs=cfg.use_graphs)
         self.scheduler = Scheduler(self.runner.cache, cfg.max_num_seqs,
                                    max(cfg.max_batched_tokens, cfg.max_num_seqs),
                                    watermark_pages=watermark, policy=cfg.scheduler)

@@ -84,8 +84,11 @@ class ModelRunner:
     """A model with its cache.  ``num_pages`` sizes every page group's pool."""
 
     def __init__(self, model: Model, num_pages: int, page_size: int = 16,
-                 max_num_seqs: int = 64, max_batched_tokens: Optional[int] = None):
+                 max_num_seqs: int = 64, max_batched_tokens: Optional[int] = None,
+                 use_graphs: bool = True):
         self.model = model
+        self.use_graphs = use_graphs and model.device.type == "cuda" and model.graph_safe
+        self._graphs: Dict[int, object] = {}
         self.device = model.device
         self.page_size = page_size
         self.max_num_seqs = max_num_seqs
@@ -131,6 +134,8 @@ class ModelRunner:
             raise ValueError(f"{len(entries)} requests in one step, max_num_seqs is "
                              f"{self.max_num_seqs}")
         total = sum(len(e.tokens) for e in entries)
+        if self.use_graphs and total == len(entries) and total > 0:
+            return self._decode_step(entries)
         if self.max_batched_tokens is not None and total > self.max_batched_tokens:
             raise ValueError(f"{total} tokens in one step, max_batched_tokens is "
                              f"{self.max_batched_tokens}")
@@ -146,3 +151,39 @@ class ModelRunner:
         for e, start in zip(entries, step.host_start_pos):
             self.cache.advance(e.seq_id, start + len(e.tokens))
         return logits
+
+    def _decode_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """A step of one token per request, replayed from the HIP graph of its batch-size
+        bucket (captured at first use).  Same kernels, same results as the eager step."""
+        from .graph import DecodeGraph, bucket_for
+        S = len(entries)
+        seq_ids = [e.seq_id for e in entries]
+        if len(set(seq_ids)) != S:
+            raise ValueError("a request appears twice in one step")
+        tokens = [int(e.tokens[0]) for e in entries]
+        if min(tokens) < 0 or max(tokens) >= self.vocab_size:
+            raise ValueError(f"a token id is outside the vocabulary of {self.vocab_size}")
+        rows: List[int] = []
+        for i, e in enumerate(entries):
+            for w in e.want:
+                if int(w) != 0:
+                    raise ValueError(f"request {e.seq_id}: wanted index {w} is outside its 1 tokens")
+                rows.append(i)
+        bucket = bucket_for(S, self.max_num_seqs)
+        graph = self._graphs.get(bucket)
+        if graph is None:
+            graph = self._graphs[bucket] = DecodeGraph(self, bucket)
+        logits = graph.run(seq_ids, tokens)
+        positions = graph.h["positions"]
+        if int(positions[:S].max()) + 1 > self.model.max_positions:
+            raise ValueError(f"sequence of {int(positions[:S].max()) + 1} positions exceeds "
+                             f"max_seq_len {self.model.max_positions}")
+        if self.pools.state is not None:
+            pass                                   # graph-safe mixers keep no state slots
+        for i, seq in enumerate(seq_ids):
+            self.cache.advance(seq, int(positions[i]) + 1)
+        if rows == list(range(S)):
+            return logits
+        if not rows:
+            return logits[:0]
+        return logits[torch.tensor(rows, device=logits.device)]

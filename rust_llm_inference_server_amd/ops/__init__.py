@@ -159,6 +159,29 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     return y
 
 
+def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+    """``silu(x @ Wg.T) * (x @ Wu.T)`` for ``w_gate_up = [Wg; Wu]`` of shape ``(2 I, K)``.
+
+    Up to 64 rows of bfloat16 take one kernel that never stores the ``(T, 2 I)`` intermediate;
+    everything else is the product followed by the SwiGLU kernel."""
+    T, K = x.shape
+    two_i = w_gate_up.shape[0]
+    if two_i % 2:
+        raise KernelError("linear_swiglu: the fused weight needs an even number of rows")
+    ldx = _rows_contig(x, "linear_swiglu x")
+    ldw = _rows_contig(w_gate_up, "linear_swiglu weight")
+    fused = (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
+             and 0 < T <= SKINNY_MAX_ROWS and K == w_gate_up.shape[1] and K % 8 == 0
+             and ldx % 8 == 0 and ldw % 8 == 0 and x.data_ptr() % 16 == 0
+             and w_gate_up.data_ptr() % 16 == 0)
+    if not fused:
+        return swiglu(linear(x, w_gate_up, x.dtype))
+    y = torch.empty((T, two_i // 2), dtype=torch.bfloat16, device=x.device)
+    lib.call("rlis_gemm_bf16_skinny_swiglu", x.data_ptr(), w_gate_up.data_ptr(), y.data_ptr(), T,
+             two_i // 2, K, ldx, ldw, two_i // 2, lib.stream_ptr())
+    return y
+
+
 # ------------------------------------------------------------ rotation + cache write
 def rope_kv_write(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                   cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
@@ -319,4 +342,4 @@ def sample_rows(logits: torch.Tensor, keys: torch.Tensor, inv_temps: torch.Tenso
 
 
 __all__ = ["KernelError", "add_residual", "add_rmsnorm", "copy_pages", "decode_splits", "embed",
-           "linear", "paged_attention", "rope_kv_write", "sample_rows", "swiglu"]
+           "linear", "linear_swiglu", "paged_attention", "rope_kv_write", "sample_rows", "swiglu"]

@@ -24,6 +24,8 @@ class PagedAttention(Mixer):
     """Parameters: ``hidden_size``, ``num_heads``, ``num_kv_heads``, ``head_dim``, ``scale``,
     ``window`` (None: all earlier positions), ``position`` (a PartSpec)."""
 
+    graph_safe = True
+
     @classmethod
     def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
         H, nh, nkv, d = (params[k] for k in ("hidden_size", "num_heads", "num_kv_heads",

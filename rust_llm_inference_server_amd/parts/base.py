@@ -169,6 +169,10 @@ class Mixer(Part):
     mixer with state must leave, after a step, the state as it is after the last token the
     step brought for that request."""
 
+    # True when forward launches only device work that reads the step's device tensors, so
+    # that a decode step may be captured into a HIP graph and replayed with new metadata.
+    graph_safe = False
+
     def cache_request(self) -> Optional[CacheRequest]:
         return None
 

@@ -135,6 +135,26 @@ def test_linear_bfloat16(ops, out_dtype, T, N, K):
     torch.testing.assert_close(got2.float(), got.float(), atol=scale / 128, rtol=1e-2)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,I,K", [(1, 8192, 2048), (8, 172, 104), (16, 320, 192), (33, 1000, 256),
+                                   (64, 8192, 2048), (65, 172, 104), (5, 100, 100)])
+def test_linear_swiglu(ops, dtype, T, I, K):
+    """The gated product (one kernel up to 64 bfloat16 rows, two kernels otherwise) against
+    silu(x Wg^T) * (x Wu^T) in float64."""
+    x = rnd(T, K, dtype=dtype, seed=1)
+    w = rnd(2 * I, K, dtype=dtype, seed=2, scale=0.05)
+    g = x.double() @ w[:I].double().t()
+    u = x.double() @ w[I:].double().t()
+    want = (torch.nn.functional.silu(g) * u).float()
+    got = ops.linear_swiglu(x, w)
+    assert got.dtype == dtype and got.shape == (T, I)
+    scale = max(1.0, want.abs().max().item())
+    if dtype == torch.float32:
+        torch.testing.assert_close(got, want, atol=1e-4 * scale, rtol=1e-4)
+    else:
+        torch.testing.assert_close(got.float(), want, atol=scale / 64, rtol=2e-2)
+
+
 def test_linear_mixed_dtypes(ops):
     # a weight stored in 32 bits stays so: bfloat16 activations times a float32 weight
     x, w = rnd(9, 100, dtype=torch.bfloat16, seed=1), rnd(50, 100, seed=2)

@@ -38,11 +38,11 @@ def case(request, tmp_path_factory):
     return name, cfg, out
 
 
-def make_runner(folder, dtype, max_tokens, page_size=16):
+def make_runner(folder, dtype, max_tokens, page_size=16, use_graphs=True):
     from rust_llm_inference_server_amd.engine import ModelRunner, load_model
     model = load_model(folder, dtype, max_positions=max(64, max_tokens))
     return ModelRunner(model, num_pages=-(-max_tokens // page_size), page_size=page_size,
-                       max_num_seqs=16)
+                       max_num_seqs=16, use_graphs=use_graphs)
 
 
 def check(steps, outputs, reqs, ref, vocab, tol):
@@ -73,6 +73,27 @@ def test_replay_families(case, dtype, family):
     print(f"{name} {dtype} {family}: worst |diff| {worst:.3e}")
     # every page came back
     assert runner.cache.num_free_pages(0) == runner.cache.num_pages(0)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_decode_steps_match_eager_ones(case, dtype):
+    """Steps of one token per request run from a captured HIP graph.  Replayed many times with
+    eager steps (prefill portions, page copies, host synchronisation) in between, every replay
+    must give what the eager step gives."""
+    name, cfg, per_dtype = case
+    folder, reqs, ref = per_dtype[dtype]
+    page = 8 if name == "b" else 16
+    for build in (traces.trace_tail, traces.trace_mixed):
+        steps, max_tokens = build(reqs)
+        eager = make_runner(folder, dtype, max_tokens, page, use_graphs=False)
+        graphed = make_runner(folder, dtype, max_tokens, page, use_graphs=True)
+        assert graphed.use_graphs and not eager.use_graphs
+        out_e = traces.replay_in_process(eager, steps)
+        out_g = traces.replay_in_process(graphed, steps)
+        assert graphed._graphs, "no decode step took the graph path"
+        check(steps, out_g, reqs, ref, cfg["vocab_size"], TOL[dtype])
+        for k in out_e:
+            torch.testing.assert_close(out_g[k], out_e[k], atol=TOL[dtype] / 4, rtol=0)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
