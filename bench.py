@@ -36,6 +36,9 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--points-context", type=int, default=512)
     ap.add_argument("--skip-points", action="store_true")
+    ap.add_argument("--skip-prefill", action="store_true")
+    ap.add_argument("--max-batched-tokens", type=int, default=8192,
+                    help="token budget of the engine steps that prefill the decode runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (single-GPU engine)")
@@ -76,7 +79,8 @@ def main() -> int:
         """tokens/s and ms/step of `steps` decode steps whose last one reaches `context`."""
         prompt_len = context - (steps + warmup)
         pages = batch * (-(-context // page) + 1) + 8
-        engine = Engine(model, EngineConfig(max_num_seqs=max(batch, 1), max_batched_tokens=2048,
+        engine = Engine(model, EngineConfig(max_num_seqs=max(batch, 1),
+                                            max_batched_tokens=max(args.max_batched_tokens, batch),
                                             num_pages=pages, block_size=page,
                                             max_seq_len=context + 8, watermark_pages=0))
         sp = SamplingParams(max_tokens=steps + warmup + 1, ignore_eos=True)
@@ -100,7 +104,7 @@ def main() -> int:
     runner = ModelRunner(model, num_pages=-(-T // page) + 1, page_size=page, max_num_seqs=1)
     prompt = prompts(1, T)[0]
     times = []
-    for i in range(4):
+    for i in range(1 if args.skip_prefill else 4):
         runner.reserve(0, T)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -108,7 +112,7 @@ def main() -> int:
         torch.cuda.synchronize()
         times.append(time.perf_counter() - t0)
         runner.free(0)
-    prefill_s = min(times[1:])
+    prefill_s = min(times[1:] or times)
     linear_flops = 2.0 * T * L * (layer_params - 2 * H)
     attn_flops = 4.0 * L * nh * d * T * (T + 1) / 2
     head_flops = 2.0 * V * H

@@ -8,7 +8,7 @@
       const void* q, long long q_stride, void* out, long long out_stride, const void* k_pages, \
       const void* v_pages, const int* block_tables, int max_pages, const int* cu_seqlens,     \
       const int* start_pos, const int* tile_map, int num_tiles, int nh, int nkv, int d,       \
-      int page_size, int window, float scale, hipStream_t stream);
+      int page_shift, int window, float scale, hipStream_t stream);
 DECL(32) DECL(64) DECL(96) DECL(128) DECL(160) DECL(192) DECL(224) DECL(256)
 #undef DECL
 
@@ -26,8 +26,10 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
                nh, nkv);
   RLIS_REQUIRE(d % 16 == 0 && d <= 256,
                "attn_prefill_mfma: head_dim %d must be a multiple of 16 and at most 256", d);
-  RLIS_REQUIRE(page_size % 8 == 0, "attn_prefill_mfma: page size %d must be a multiple of 8",
-               page_size);
+  RLIS_REQUIRE(page_size >= 8 && (page_size & (page_size - 1)) == 0,
+               "attn_prefill_mfma: page size %d must be a power of two, at least 8", page_size);
+  int page_shift = 0;
+  while ((1 << page_shift) < page_size) ++page_shift;
   RLIS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)k_pages % 16) == 0 &&
                    ((uintptr_t)v_pages % 16) == 0,
                "attn_prefill_mfma: operands must be 16-byte aligned with row strides in steps of 8");
@@ -35,7 +37,7 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
 #define CALL(D)                                                                                 \
   return rlis_attn_prefill_mfma_d##D(q, q_stride, out, out_stride, k_pages, v_pages,            \
                                      block_tables, max_pages, cu_seqlens, start_pos, tile_map,  \
-                                     num_tiles, nh, nkv, d, page_size, window, scale, stream)
+                                     num_tiles, nh, nkv, d, page_shift, window, scale, stream)
   if (d <= 32) CALL(32);
   if (d <= 64) CALL(64);
   if (d <= 96) CALL(96);

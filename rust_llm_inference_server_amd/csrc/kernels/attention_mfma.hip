@@ -5,15 +5,24 @@
 // head; each wave owns 16 of them.  Keys are walked in tiles of BN positions aligned to BN,
 // read through the block table: the K tile [key][dim] and the V tile [dim][key] (the cache
 // keeps V transposed inside a page, so both are copied as they lie) go to LDS once per
-// workgroup.  S = Q K^T and O += P V use v_mfma_f32_16x16x32_bf16; the accumulator of a
-// 16 x 16 block holds, in lane l and register r, row (l / 16) * 4 + r and column l % 16, so the
-// softmax statistics of a row sit in the same lanes for S and for O.
+// workgroup, the next tile travelling global -> registers while the current one is computed.
+//
+// Both products are computed transposed with v_mfma_f32_16x16x32_bf16, whose 16 x 16 result
+// holds, in lane l and register r, row (l / 16) * 4 + r and column l % 16:
+//   S^T = K Q^T   (rows: keys, columns: queries)
+//   O^T = V^T P^T (rows: dims, columns: queries)
+// so a lane only ever holds values of ONE query, column l % 16: its running maximum,
+// denominator and rescaling factor are plain per-lane scalars, the row reductions need two
+// lane exchanges, and the probabilities a lane holds after the softmax are exactly the
+// B-operand fragment of the second product (the k slots of a step of 32 keys are mapped to
+// keys {16 * 2s + 4 q + j} and {16 * (2s + 1) + 4 q + j}), so P never leaves the registers.
 //
 // The mask is the reference's causal mask offset by the cached length (crates/model/src/
 // attention.rs:225-233): the new token at index i of a sequence with P cached positions sees
 // keys at positions <= P + i, and > P + i - window when a window is given.  Scores are scaled
-// in float32 after the product; probabilities are rounded to bfloat16 only as the operand of
-// the PV product (the row sums use the float32 values).
+// in float32 after the product (kept in the base-2 domain so that e^x is one v_exp_f32);
+// probabilities are rounded to bfloat16 only as the operand of the second product (the row
+// sums use the float32 values).
 #include "common.h"
 
 #include <math.h>
@@ -27,6 +36,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 union Frag8 {
   uint4 u;
+  uint2 h[2];
   bf16x8 v;
   bf16_t e[8];
 };
@@ -41,7 +51,6 @@ constexpr int D = RLIS_HEAD_DIM;
 constexpr int BN = D <= 128 ? 64 : 32;
 constexpr int KS = D + 8;     // K tile row stride (bf16 elements)
 constexpr int VS = BN + 8;    // V tile row stride
-constexpr int PS = BN + 8;    // P tile row stride
 constexpr int BM = 64;
 
 }  // namespace
@@ -51,10 +60,9 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
     long long out_stride, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_seqlens,
     const int* __restrict__ start_pos, const int* __restrict__ tile_map, int nh, int nkv, int d,
-    int page_size, float scale, int window) {
+    int page_shift, float scale, int window) {
   __shared__ __attribute__((aligned(16))) bf16_t Ks[BN * KS];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[D * VS];
-  __shared__ __attribute__((aligned(16))) bf16_t Ps[4 * 16 * PS];
 
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int l16 = lane % 16, lq = lane / 16;
@@ -65,9 +73,13 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
   const int P = start_pos[seq];
   const int kvh = h / (nh / nkv);
   const int* table = block_tables + (long long)seq * max_pages;
+  const int page_mask = (1 << page_shift) - 1;
 
-  // Query fragments of this wave: row l16 -> new-token index qb + wave * 16 + l16.
-  const int my_qi = qb + wave * 16 + l16;
+  // This lane's query: new-token index qb + wave * 16 + l16.  Its fragments serve as the
+  // B operand (column l16) of S^T = K Q^T.
+  const int wave_q_first = qb + wave * 16;
+  const int my_qi = wave_q_first + l16;
+  const int my_qpos = P + my_qi;
   Frag8 qf[D / 32];
 #pragma unroll
   for (int ks = 0; ks < D / 32; ++ks) {
@@ -78,14 +90,8 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
       qf[ks].u = make_uint4(0, 0, 0, 0);
   }
 
-  // Rows of the accumulators held by this lane: new-token index qb + wave * 16 + lq * 4 + r.
-  float m[4], l[4];
-  f32x4 o_acc[D / 16];
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    m[r] = -INFINITY;
-    l[r] = 0.f;
-  }
+  float m_run = -INFINITY, l_run = 0.f;
+  f32x4 o_acc[D / 16];      // O^T: rows are dims db * 16 + lq * 4 + r, the column is this query
 #pragma unroll
   for (int db = 0; db < D / 16; ++db) o_acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
@@ -94,12 +100,9 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
   int klo = 0;
   if (window > 0) klo = max(0, P + qb - window + 1);
   const int kt0 = (klo / BN) * BN;
-  const int wave_q_first = qb + wave * 16;
   const int wave_q_last = min(n_new - 1, wave_q_first + 15);
-  bf16_t* my_ps = Ps + wave * 16 * PS;
 
-  // Staging registers: the next tile's K and V^T chunks travel global -> registers while the
-  // current tile is computed from LDS, then registers -> LDS.
+  // Staging registers for the next tile.
   constexpr int K_CHUNKS = BN * (D / 8);
   constexpr int KCH = (K_CHUNKS + 255) / 256;
   constexpr int VCH = (D * (BN / 8) + 255) / 256;
@@ -113,9 +116,9 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
       const int kpos = k0 + key;
       uint4 v = make_uint4(0, 0, 0, 0);
       if (c < K_CHUNKS && kpos < khi && dc * 8 < d) {
-        const long long page = table[kpos / page_size];
-        const int off = kpos % page_size;
-        v = *(const uint4*)(k_pages + ((page * nkv + kvh) * page_size + off) * d + dc * 8);
+        const long long page = table[kpos >> page_shift];
+        const int off = kpos & page_mask;
+        v = *(const uint4*)(k_pages + (((page * nkv + kvh) << page_shift) + off) * d + dc * 8);
       }
       kreg[i] = v;
     }
@@ -128,9 +131,10 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
         const int dim = c / (BN / 8), kg = c % (BN / 8);
         const int kpos = k0 + kg * 8;
         if (kpos < khi) {
-          const long long page = table[kpos / page_size];
-          const int off = kpos % page_size;
-          v.u = *(const uint4*)(v_pages + ((page * nkv + kvh) * (long long)d + dim) * page_size + off);
+          const long long page = table[kpos >> page_shift];
+          const int off = kpos & page_mask;
+          v.u = *(const uint4*)(v_pages +
+                                (((page * nkv + kvh) * (long long)d + dim) << page_shift) + off);
           if (kpos + 8 > khi) {
 #pragma unroll
             for (int e = 0; e < 8; ++e)
@@ -154,8 +158,7 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
     }
   };
 
-  // Scores are kept in the base-2 domain: s * scale * log2(e), so that e^x is one v_exp_f32.
-  const float scale2 = scale * 1.4426950408889634f;
+  const float scale2 = scale * 1.4426950408889634f;      // scores in the base-2 domain
   if (kt0 < khi) {
     load_tile(kt0);
     store_tile();
@@ -168,77 +171,81 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
     // Tiles wholly after this wave's last query contribute nothing to it.
     const bool wave_active = (wave_q_first < n_new) && (k0 <= P + wave_q_last);
     if (wave_active) {
-      // ---- S = Q K^T -------------------------------------------------------------------
-      f32x4 s_acc[BN / 16];
+      // ---- S^T = K Q^T: block nb holds keys k0 + nb * 16 + lq * 4 + r for query l16 --------
+      f32x4 s[BN / 16];
 #pragma unroll
       for (int nb = 0; nb < BN / 16; ++nb) {
-        s_acc[nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        s[nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < D / 32; ++ks) {
           Frag8 kf;
           kf.u = *(const uint4*)(Ks + (nb * 16 + l16) * KS + ks * 32 + lq * 8);
-          s_acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks].v, kf.v, s_acc[nb], 0, 0, 0);
+          s[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[ks].v, s[nb], 0, 0, 0);
         }
       }
-      // ---- mask, scale, online softmax ---------------------------------------------------
-      float corr[4];
+      // ---- scale, mask (only where a tile meets the diagonal, the window or the end) -----
+      const bool plain_tile = (k0 + BN - 1 <= P + wave_q_first) &&
+                              (window <= 0 || k0 > P + wave_q_first + 15 - window);
+      float mx = -INFINITY;
+      if (plain_tile) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int qi = wave_q_first + lq * 4 + r;
-        const int qpos = P + qi;
-        float row_max = -INFINITY;
+        for (int nb = 0; nb < BN / 16; ++nb)
 #pragma unroll
-        for (int nb = 0; nb < BN / 16; ++nb) {
-          const int kpos = k0 + nb * 16 + l16;
-          const bool ok = (qi < n_new) && (kpos <= qpos) && (window <= 0 || kpos > qpos - window);
-          const float sv = ok ? s_acc[nb][r] * scale2 : -INFINITY;
-          s_acc[nb][r] = sv;
-          row_max = fmaxf(row_max, sv);
-        }
+          for (int r = 0; r < 4; ++r) {
+            s[nb][r] *= scale2;
+            mx = fmaxf(mx, s[nb][r]);
+          }
+      } else {
 #pragma unroll
-        for (int o = 1; o < 16; o <<= 1) row_max = fmaxf(row_max, __shfl_xor(row_max, o, kWave));
-        const float m_new = fmaxf(m[r], row_max);
-        float row_sum = 0.f;
+        for (int nb = 0; nb < BN / 16; ++nb)
 #pragma unroll
-        for (int nb = 0; nb < BN / 16; ++nb) {
-          const float sv = s_acc[nb][r];
-          const float p = (sv == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(sv - m_new);
-          s_acc[nb][r] = p;
-          row_sum += p;
-        }
-#pragma unroll
-        for (int o = 1; o < 16; o <<= 1) row_sum += __shfl_xor(row_sum, o, kWave);
-        corr[r] = (m[r] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m[r] - m_new);
-        l[r] = l[r] * corr[r] + row_sum;
-        m[r] = m_new;
+          for (int r = 0; r < 4; ++r) {
+            const int kpos = k0 + nb * 16 + lq * 4 + r;
+            const bool ok = (kpos <= my_qpos) && (window <= 0 || kpos > my_qpos - window);
+            const float sv = ok ? s[nb][r] * scale2 : -INFINITY;
+            s[nb][r] = sv;
+            mx = fmaxf(mx, sv);
+          }
       }
-      // ---- P to LDS (row-major per wave), O rescale ---------------------------------------
+      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      const float m_new = fmaxf(m_run, mx);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;   // a query with no key yet
+      const float corr = __builtin_amdgcn_exp2f(m_run - m_safe);  // 0 when m_run is -inf
+      float sum = 0.f;
 #pragma unroll
       for (int nb = 0; nb < BN / 16; ++nb)
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          my_ps[(lq * 4 + r) * PS + nb * 16 + l16] = f32_to_bf16(s_acc[nb][r]);
+        for (int r = 0; r < 4; ++r) {
+          const float p = __builtin_amdgcn_exp2f(s[nb][r] - m_safe);   // exp2(-inf) = 0
+          s[nb][r] = p;
+          sum += p;
+        }
+      sum += __shfl_xor(sum, 16, kWave);
+      sum += __shfl_xor(sum, 32, kWave);
+      l_run = l_run * corr + sum;
+      m_run = m_new;
 #pragma unroll
       for (int db = 0; db < D / 16; ++db)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) o_acc[db][r] *= corr[r];
-    }
-    // The P tile is private to the wave, but the barrier also orders it for the reads below.
-    __syncthreads();
-    if (wave_active) {
-      // ---- O += P V ----------------------------------------------------------------------
-      Frag8 pf[BN / 32];
+        for (int r = 0; r < 4; ++r) o_acc[db][r] *= corr;
+      // ---- O^T += V^T P^T: P^T fragments come straight from the registers ----------------
 #pragma unroll
-      for (int ks = 0; ks < BN / 32; ++ks)
-        pf[ks].u = *(const uint4*)(my_ps + l16 * PS + ks * 32 + lq * 8);
+      for (int st = 0; st < BN / 32; ++st) {
+        bf16x8 pf;
 #pragma unroll
-      for (int db = 0; db < D / 16; ++db) {
-        if (db * 16 < d) {
+        for (int j = 0; j < 4; ++j) {
+          pf[j] = (__bf16)s[2 * st][j];
+          pf[4 + j] = (__bf16)s[2 * st + 1][j];
+        }
 #pragma unroll
-          for (int ks = 0; ks < BN / 32; ++ks) {
+        for (int db = 0; db < D / 16; ++db) {
+          if (db * 16 < d) {
             Frag8 vf;
-            vf.u = *(const uint4*)(Vs + (db * 16 + l16) * VS + ks * 32 + lq * 8);
-            o_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[ks].v, vf.v, o_acc[db], 0, 0, 0);
+            const bf16_t* vrow = Vs + (db * 16 + l16) * VS + st * 32 + lq * 4;
+            vf.h[0] = *(const uint2*)(vrow);
+            vf.h[1] = *(const uint2*)(vrow + 16);
+            o_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf, o_acc[db], 0, 0, 0);
           }
         }
       }
@@ -250,17 +257,19 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
     }
   }
 
-  // ---- normalise and store ------------------------------------------------------------
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int qi = wave_q_first + lq * 4 + r;
-    if (qi >= n_new) continue;
-    const float inv_l = 1.0f / l[r];
-    bf16_t* orow = out + (long long)(tok_begin + qi) * out_stride + h * d;
+  // ---- normalise and store: this lane holds dims db * 16 + lq * 4 + [0, 4) of its query ----
+  if (my_qi < n_new) {
+    const float inv_l = 1.0f / l_run;
+    bf16_t* orow = out + (long long)(tok_begin + my_qi) * out_stride + h * d;
 #pragma unroll
     for (int db = 0; db < D / 16; ++db) {
-      const int dim = db * 16 + l16;
-      if (dim < d) orow[dim] = f32_to_bf16(o_acc[db][r] * inv_l);
+      const int dim = db * 16 + lq * 4;
+      if (dim < d) {
+        union { uint2 u; bf16_t e[4]; } o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o.e[r] = f32_to_bf16(o_acc[db][r] * inv_l);
+        *(uint2*)(orow + dim) = o.u;
+      }
     }
   }
 }
@@ -270,13 +279,13 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
     const void* q, long long q_stride, void* out, long long out_stride, const void* k_pages,
     const void* v_pages, const int* block_tables, int max_pages, const int* cu_seqlens,
     const int* start_pos, const int* tile_map, int num_tiles, int nh, int nkv, int d,
-    int page_size, int window, float scale, hipStream_t stream) {
+    int page_shift, int window, float scale, hipStream_t stream) {
   if (num_tiles == 0) return 0;
   dim3 grid(num_tiles, nh);
   KERNEL_NAME<<<grid, 256, 0, stream>>>(
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,
       (const bf16_t*)v_pages, block_tables, max_pages, cu_seqlens, start_pos, tile_map, nh, nkv, d,
-      page_size, scale, window);
+      page_shift, scale, window);
   RLIS_LAUNCH_CHECK("attn_prefill_mfma");
   return 0;
 }

@@ -418,3 +418,187 @@ RLIS_API int rlis_gemm_bf16_skinny_swiglu(const void* X, const void* W, void* Y,
   RLIS_LAUNCH_CHECK("gemm_bf16_skinny_swiglu");
   return 0;
 }
+
+// =================================================== row-streaming product (T <= 8)
+// y (T, N) = x (T, K) * W (N, K)^T for up to 8 rows of x, the shape of decode at small batch,
+// where nothing matters but reading W at full memory speed.  A wave streams whole weight rows:
+// one load instruction brings 1 KiB of ONE row, lane l holding the 8 weights at k = kc + 8 l.
+// To reduce over k on the matrix cores the 64 chunks of such a kilobyte are laid out as the
+// operands of v_mfma_f32_16x16x32_bf16: chunk l is row l % 16, k-group l / 16 of A, and the
+// same chunk of a row of x is column l % 16, k-group l / 16 of B.  The product's diagonal
+// C[m][m] is then the dot product of the chunks m, 16 + m, 32 + m, 48 + m of both, and the
+// trace of C, accumulated over the row, is the whole dot product.  The off-diagonal terms are
+// waste the matrix cores have room for: the kernel is bound by memory.
+//
+// x is staged in LDS once per workgroup (and per k-chunk when T * K does not fit); a wave
+// keeps R = 2 rows in flight (gate and up of one column in the gated form) and walks its
+// share of the rows.  Sums run over k in an order fixed by K alone.
+template <typename TC, int TT, bool GATED, int R, int U>
+__global__ __launch_bounds__(256) void gemv_bf16_rows_kernel(const bf16_t* __restrict__ X,
+                                                             const bf16_t* __restrict__ W,
+                                                             TC* __restrict__ Y, int T, int N,
+                                                             int K, long long ldx, long long ldw,
+                                                             long long ldy, int kc_len,
+                                                             int groups_per_wave) {
+  extern __shared__ __attribute__((aligned(16))) bf16_t x_s[];      // TT * kc_len
+  static_assert(!GATED || R % 2 == 0, "gated rows come in gate/up pairs");
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  constexpr int CPG = GATED ? R / 2 : R;                 // output columns per row group
+  const int num_groups = (N + CPG - 1) / CPG;
+  // Waves take row groups in turn (group = round * waves + wave), so that at any moment the
+  // waves of the grid read neighbouring rows and the traffic spreads over all memory channels.
+  const long long my_wave = (long long)blockIdx.x * 4 + wave;
+  const long long num_waves = (long long)gridDim.x * 4;
+  const bool is_diag = ((lane % 16) / 4) == (lane / 16);
+  const int diag_r = lane % 4;
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  const int num_chunks = (K + kc_len - 1) / kc_len;      // > 1 only with groups_per_wave == 1
+
+  f32x4 acc[R][TT];
+  for (int gi = 0; gi < groups_per_wave; ++gi) {
+    const long long g = gi * num_waves + my_wave;
+    const bool g_valid = g < num_groups;
+    long long rows[R];
+    bool rvalid[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      // gated: rows 0 .. CPG-1 are gate rows of the group's columns, CPG .. R-1 their up rows
+      const long long col = g * CPG + (i % CPG);
+      rows[i] = (GATED && i >= CPG) ? col + N : col;
+      rvalid[i] = g_valid && col < N;
+    }
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+#pragma unroll
+      for (int t = 0; t < TT; ++t) acc[i][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    for (int ch = 0; ch < num_chunks; ++ch) {
+      const int kbase = ch * kc_len;
+      const int klen = min(kc_len, K - kbase);
+      if (gi == 0 || num_chunks > 1) {
+        // Stage x[:, kbase : kbase + klen] (zero rows beyond T, zero tail up to 512).
+        if (num_chunks > 1 || gi > 0) __syncthreads();
+        const int kpad = ((klen + 511) / 512) * 512;
+        for (int c = tid; c < TT * (kpad / 8); c += 256) {
+          const int t = c / (kpad / 8), kk = (c % (kpad / 8)) * 8;
+          uint4 v = zero;
+          if (t < T && kk < klen) v = *(const uint4*)(X + (long long)t * ldx + kbase + kk);
+          *(uint4*)(x_s + t * kc_len + kk) = v;
+        }
+        __syncthreads();
+      }
+      for (int kk = 0; kk < klen; kk += 512 * U) {
+        Frag8 a[R][U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int k = kk + u * 512 + lane * 8;
+#pragma unroll
+          for (int i = 0; i < R; ++i)
+            a[i][u].u = (rvalid[i] && k < klen) ? *(const uint4*)(W + rows[i] * ldw + kbase + k) : zero;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int k = kk + u * 512 + lane * 8;
+          if (kk + u * 512 < klen) {
+#pragma unroll
+            for (int t = 0; t < TT; ++t) {
+              Frag8 b;
+              b.u = *(const uint4*)(x_s + t * kc_len + k);
+#pragma unroll
+              for (int i = 0; i < R; ++i)
+                acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i][u].v, b.v, acc[i][t], 0, 0, 0);
+            }
+          }
+        }
+      }
+    }
+    // Trace of every accumulator -> the dot products of this row group.
+    float sums[R][TT];
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+#pragma unroll
+      for (int t = 0; t < TT; ++t) {
+        const f32x4 c = acc[i][t];
+        float v = diag_r == 0 ? c[0] : (diag_r == 1 ? c[1] : (diag_r == 2 ? c[2] : c[3]));
+        sums[i][t] = wave_sum(is_diag ? v : 0.f);
+      }
+    if (lane == 0 && g_valid) {
+#pragma unroll
+      for (int t = 0; t < TT; ++t) {
+        if (t >= T) break;
+        if (GATED) {
+#pragma unroll
+          for (int i = 0; i < CPG; ++i)
+            if (rvalid[i]) {
+              const float gate = sums[i][t];
+              st(Y + (long long)t * ldy + rows[i], gate / (1.0f + expf(-gate)) * sums[CPG + i][t]);
+            }
+        } else {
+#pragma unroll
+          for (int i = 0; i < R; ++i)
+            if (rvalid[i]) st(Y + (long long)t * ldy + rows[i], sums[i][t]);
+        }
+      }
+    }
+  }
+}
+
+template <typename TC, int TT, bool GATED>
+static int launch_gemv_rows(const void* X, const void* W, void* Y, int T, int N, int K,
+                            long long ldx, long long ldw, long long ldy, hipStream_t stream) {
+  // x in LDS: whole K when TT * K * 2 bytes fit into 48 KiB, else k-chunks of a multiple of 512.
+  const int kpad = ceil_div(K, 512) * 512;
+  int kc_len = kpad;
+  const int fit = (48 * 1024 / (TT * 2)) / 512 * 512;
+  if (kc_len > fit) kc_len = fit;
+  const int num_chunks = ceil_div(K, kc_len);
+  constexpr int R = TT <= 2 ? 4 : 2;
+  constexpr int U = TT <= 4 ? 2 : 1;
+  constexpr int CPG = GATED ? R / 2 : R;
+  const long long groups = ceil_div(N, CPG);
+  long long blocks;
+  int groups_per_wave;
+  if (num_chunks > 1) {
+    groups_per_wave = 1;
+    blocks = ceil_div_ll(groups, 4);
+  } else {
+    blocks = ceil_div_ll(groups, 4);
+    if (blocks > 2048) blocks = 2048;
+    groups_per_wave = (int)ceil_div_ll(groups, blocks * 4);
+    blocks = ceil_div_ll(groups, (long long)groups_per_wave * 4);
+  }
+  const size_t smem = (size_t)TT * kc_len * sizeof(bf16_t);
+  gemv_bf16_rows_kernel<TC, TT, GATED, R, U><<<(int)blocks, 256, smem, stream>>>(
+      (const bf16_t*)X, (const bf16_t*)W, (TC*)Y, T, N, K, ldx, ldw, ldy, kc_len, groups_per_wave);
+  return 0;
+}
+
+template <typename TC, bool GATED>
+static int dispatch_gemv_rows(const void* X, const void* W, void* Y, int T, int N, int K,
+                              long long ldx, long long ldw, long long ldy, hipStream_t stream) {
+  if (T <= 1) return launch_gemv_rows<TC, 1, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
+  if (T <= 2) return launch_gemv_rows<TC, 2, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
+  if (T <= 4) return launch_gemv_rows<TC, 4, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
+  return launch_gemv_rows<TC, 8, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
+}
+
+// gated == 0: y (T, N) = x W^T.  gated != 0: W is (2N, K) = [Wg; Wu] and
+// y (T, N) = silu(x Wg^T) * (x Wu^T).  T <= 8, bfloat16 operands, K a multiple of 8.
+RLIS_API int rlis_gemv_bf16_rows(const void* X, const void* W, void* Y, int y_dtype, int T, int N,
+                                 int K, long long ldx, long long ldw, long long ldy, int gated,
+                                 hipStream_t stream) {
+  if (check_skinny("gemv_bf16_rows", X, W, T, N, K, ldx, ldw, ldy)) return 1;
+  RLIS_REQUIRE(T <= 8, "gemv_bf16_rows: T=%d rows, at most 8", T);
+  RLIS_REQUIRE(!gated || y_dtype == RLIS_BF16, "gemv_bf16_rows: the gated form stores bfloat16");
+  if (T == 0) return 0;
+  if (gated)
+    dispatch_gemv_rows<bf16_t, true>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
+  else if (y_dtype == RLIS_F32)
+    dispatch_gemv_rows<float, false>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
+  else if (y_dtype == RLIS_BF16)
+    dispatch_gemv_rows<bf16_t, false>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
+  else
+    RLIS_REQUIRE(false, "gemv_bf16_rows: unknown output dtype %d", y_dtype);
+  RLIS_LAUNCH_CHECK("gemv_bf16_rows");
+  return 0;
+}

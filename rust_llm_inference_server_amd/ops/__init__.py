@@ -18,6 +18,8 @@ _DT = {torch.float32: 0, torch.bfloat16: 1}
 
 # bf16 products with at most this many rows of x take the skinny kernel.
 SKINNY_MAX_ROWS = 64
+# ... and with at most this many rows the row-streaming kernel.
+GEMV_MAX_ROWS = 8
 # "library": bf16 products with more rows and bf16 output go to torch.matmul (hipBLASLt);
 # "own": they take the hand-written matrix-core kernel.
 BF16_GEMM = "library"
@@ -149,7 +151,10 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     y = torch.empty((T, N), dtype=out_dtype, device=x.device)
     if T == 0:
         return y
-    if bf16 and aligned:
+    if bf16 and aligned and T <= GEMV_MAX_ROWS:
+        lib.call("rlis_gemv_bf16_rows", x.data_ptr(), w.data_ptr(), y.data_ptr(), _DT[out_dtype],
+                 T, N, K, ldx, ldw, N, 0, stream)
+    elif bf16 and aligned:
         name = "rlis_gemm_bf16_skinny" if T <= SKINNY_MAX_ROWS else "rlis_gemm_bf16_mfma"
         lib.call(name, x.data_ptr(), w.data_ptr(), y.data_ptr(), _DT[out_dtype], T, N, K, ldx,
                  ldw, N, stream)
@@ -177,8 +182,12 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
     if not fused:
         return swiglu(linear(x, w_gate_up, x.dtype))
     y = torch.empty((T, two_i // 2), dtype=torch.bfloat16, device=x.device)
-    lib.call("rlis_gemm_bf16_skinny_swiglu", x.data_ptr(), w_gate_up.data_ptr(), y.data_ptr(), T,
-             two_i // 2, K, ldx, ldw, two_i // 2, lib.stream_ptr())
+    if T <= GEMV_MAX_ROWS:
+        lib.call("rlis_gemv_bf16_rows", x.data_ptr(), w_gate_up.data_ptr(), y.data_ptr(), 1, T,
+                 two_i // 2, K, ldx, ldw, two_i // 2, 1, lib.stream_ptr())
+    else:
+        lib.call("rlis_gemm_bf16_skinny_swiglu", x.data_ptr(), w_gate_up.data_ptr(), y.data_ptr(),
+                 T, two_i // 2, K, ldx, ldw, two_i // 2, lib.stream_ptr())
     return y
 
 
@@ -287,8 +296,9 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     if kind is None:
         if step.all_decode and d % 8 == 0 and d <= 256 and (nh // nkv) * d <= 2048:
             kind = "decode"
-        elif (qkv.dtype == torch.bfloat16 and d % 16 == 0 and d <= 256 and page_size % 8 == 0
-              and q_stride % 8 == 0 and not step.all_decode):
+        elif (qkv.dtype == torch.bfloat16 and d % 16 == 0 and d <= 256 and page_size >= 8
+              and page_size & (page_size - 1) == 0 and q_stride % 8 == 0
+              and not step.all_decode):
             kind = "prefill"
         else:
             kind = "generic"

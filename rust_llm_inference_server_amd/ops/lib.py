@@ -25,6 +25,7 @@ _SIGNATURES = {
     "rlis_gemm_bf16_mfma": [P, P, P, I, I, I, I, L, L, L, P],
     "rlis_gemm_bf16_skinny": [P, P, P, I, I, I, I, L, L, L, P],
     "rlis_gemm_bf16_skinny_swiglu": [P, P, P, I, I, I, L, L, L, P],
+    "rlis_gemv_bf16_rows": [P, P, P, I, I, I, I, L, L, L, I, P],
     "rlis_attn_generic": [P, I, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
     "rlis_attn_decode": [P, I, L, P, L, P, P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, P],
     "rlis_attn_prefill_mfma": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P],

@@ -110,6 +110,7 @@ def test_linear_float32(ops, T, N, K):
 
 @pytest.mark.parametrize("out_dtype", DTYPES)
 @pytest.mark.parametrize("T,N,K", [(1, 2048, 2048), (1, 331, 104), (8, 3072, 2048), (16, 100, 64),
+                                   (2, 2048, 8192), (7, 2049, 14336), (3, 128256, 2048), (4, 7, 520),
                                    (17, 130, 96), (33, 8192, 2048), (64, 2048, 8192),
                                    (65, 257, 104), (200, 3072, 2048), (300, 331, 2048),
                                    (128, 128, 64), (5, 100, 100), (70, 100, 172)])
@@ -137,6 +138,7 @@ def test_linear_bfloat16(ops, out_dtype, T, N, K):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,I,K", [(1, 8192, 2048), (8, 172, 104), (16, 320, 192), (33, 1000, 256),
+                                   (8, 8192, 2048), (3, 1001, 4608), (8, 77, 14336),
                                    (64, 8192, 2048), (65, 172, 104), (5, 100, 100)])
 def test_linear_swiglu(ops, dtype, T, I, K):
     """The gated product (one kernel up to 64 bfloat16 rows, two kernels otherwise) against
