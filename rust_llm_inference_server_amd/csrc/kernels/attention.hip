@@ -338,6 +338,19 @@ __global__ void attn_reduce_kernel(TX* __restrict__ out, long long out_stride,
   }
 }
 
+// Launches the merge of `splits` partitions for S sequences of bfloat16 output (used by the
+// matrix-core decode kernel, which lives in another unit).
+int rlis_launch_attn_reduce_bf16(void* out, long long out_stride, const float* part_ml,
+                                 const float* part_acc, int S, int nh, int d, int splits,
+                                 hipStream_t stream) {
+  dim3 grid(nh, S);
+  const int threads = d <= 64 ? 64 : (d <= 128 ? 128 : 256);
+  attn_reduce_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)out, out_stride, part_ml,
+                                                           part_acc, nullptr, nh, d, splits);
+  RLIS_LAUNCH_CHECK("attn_reduce");
+  return 0;
+}
+
 template <typename TX, int G>
 static int launch_decode(const void* q, long long q_stride, void* out, long long out_stride,
                          float* part_ml, float* part_acc, const void* k_pages,

@@ -12,6 +12,19 @@
 DECL(32) DECL(64) DECL(96) DECL(128) DECL(160) DECL(192) DECL(224) DECL(256)
 #undef DECL
 
+#define DECL(D)                                                                                \
+  extern "C" int rlis_attn_decode_mfma_d##D(                                                   \
+      const void* q, long long q_stride, void* out, long long out_stride, float* part_ml,      \
+      float* part_acc, const void* k_pages, const void* v_pages, const int* block_tables,      \
+      int max_pages, const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift,       \
+      int window, float scale, int splits, hipStream_t stream);
+DECL(32) DECL(64) DECL(96) DECL(128) DECL(160) DECL(192) DECL(224) DECL(256)
+#undef DECL
+
+int rlis_launch_attn_reduce_bf16(void* out, long long out_stride, const float* part_ml,
+                                 const float* part_acc, int S, int nh, int d, int splits,
+                                 hipStream_t stream);
+
 RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out,
                                     long long out_stride, const void* k_pages,
                                     const void* v_pages, const int* block_tables, int max_pages,
@@ -33,7 +46,6 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
   RLIS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)k_pages % 16) == 0 &&
                    ((uintptr_t)v_pages % 16) == 0,
                "attn_prefill_mfma: operands must be 16-byte aligned with row strides in steps of 8");
-  RLIS_REQUIRE(nh <= 65535, "attn_prefill_mfma: too many heads");
 #define CALL(D)                                                                                 \
   return rlis_attn_prefill_mfma_d##D(q, q_stride, out, out_stride, k_pages, v_pages,            \
                                      block_tables, max_pages, cu_seqlens, start_pos, tile_map,  \
@@ -47,4 +59,50 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
   if (d <= 224) CALL(224);
   CALL(256);
 #undef CALL
+}
+
+// One query token per sequence (bfloat16): q rows are the sequences themselves.  Needs at most
+// 16 query heads per KV head; part_ml (S, nh, splits, 2) and part_acc (S, nh, splits, d) float32
+// when splits > 1.
+RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
+                                   long long out_stride, float* part_ml, float* part_acc,
+                                   const void* k_pages, const void* v_pages,
+                                   const int* block_tables, int max_pages, const int* ctx_lens,
+                                   int S, int nh, int nkv, int d, int page_size, int window,
+                                   float scale, int splits, hipStream_t stream) {
+  RLIS_REQUIRE(S >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0, "attn_decode_mfma: bad sizes");
+  RLIS_REQUIRE(nh % nkv == 0 && nh / nkv <= 16,
+               "attn_decode_mfma: %d query heads per KV head, at most 16", nkv ? nh / nkv : 0);
+  RLIS_REQUIRE(d % 16 == 0 && d <= 256,
+               "attn_decode_mfma: head_dim %d must be a multiple of 16 and at most 256", d);
+  RLIS_REQUIRE((long long)(nh / nkv) * (d + 2) * 32 <= 64 * 1024,
+               "attn_decode_mfma: group of %d heads of size %d does not fit the merge buffer",
+               nh / nkv, d);
+  RLIS_REQUIRE(page_size >= 8 && (page_size & (page_size - 1)) == 0,
+               "attn_decode_mfma: page size %d must be a power of two, at least 8", page_size);
+  RLIS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)k_pages % 16) == 0 &&
+                   ((uintptr_t)v_pages % 16) == 0,
+               "attn_decode_mfma: operands must be 16-byte aligned with row strides in steps of 8");
+  RLIS_REQUIRE(splits >= 1 && splits <= 65535 && S <= 65535, "attn_decode_mfma: bad grid");
+  RLIS_REQUIRE(splits == 1 || (part_ml && part_acc), "attn_decode_mfma: partitions need a workspace");
+  int page_shift = 0;
+  while ((1 << page_shift) < page_size) ++page_shift;
+  int rc;
+#define CALL(D)                                                                                 \
+  rc = rlis_attn_decode_mfma_d##D(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,     \
+                                  v_pages, block_tables, max_pages, ctx_lens, S, nh, nkv, d,    \
+                                  page_shift, window, scale, splits, stream)
+  if (d <= 32) CALL(32);
+  else if (d <= 64) CALL(64);
+  else if (d <= 96) CALL(96);
+  else if (d <= 128) CALL(128);
+  else if (d <= 160) CALL(160);
+  else if (d <= 192) CALL(192);
+  else if (d <= 224) CALL(224);
+  else CALL(256);
+#undef CALL
+  if (rc) return rc;
+  if (splits > 1 && S > 0)
+    return rlis_launch_attn_reduce_bf16(out, out_stride, part_ml, part_acc, S, nh, d, splits, stream);
+  return 0;
 }

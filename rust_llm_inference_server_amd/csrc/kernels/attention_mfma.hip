@@ -60,13 +60,23 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
     long long out_stride, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_seqlens,
     const int* __restrict__ start_pos, const int* __restrict__ tile_map, int nh, int nkv, int d,
-    int page_shift, float scale, int window) {
+    int page_shift, float scale, int window, int num_tiles, int tiles_per_round) {
   __shared__ __attribute__((aligned(16))) bf16_t Ks[BN * KS];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[D * VS];
 
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int l16 = lane % 16, lq = lane / 16;
-  const int tile = blockIdx.x, h = blockIdx.y;
+  // Blocks are numbered heads-fastest over the tiles, which arrive sorted by falling work.
+  // One round of blocks (tiles_per_round tiles x all heads) fills the compute units once; every
+  // other round walks its tiles backwards, so that a unit that drew a long tile in one round
+  // draws a short one in the next.
+  const int h = blockIdx.x % nh;
+  int tile = blockIdx.x / nh;
+  if (tiles_per_round > 0) {
+    const int round = tile / tiles_per_round, within = tile % tiles_per_round;
+    const bool whole = (round + 1) * tiles_per_round <= num_tiles;
+    if ((round & 1) && whole) tile = round * tiles_per_round + (tiles_per_round - 1 - within);
+  }
   const int seq = tile_map[2 * tile], qb = tile_map[2 * tile + 1];
   const int tok_begin = cu_seqlens[seq];
   const int n_new = cu_seqlens[seq + 1] - tok_begin;
@@ -225,10 +235,13 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
       sum += __shfl_xor(sum, 32, kWave);
       l_run = l_run * corr + sum;
       m_run = m_new;
+      // The accumulator needs rescaling only when some query's maximum moved.
+      if (__any(corr != 1.0f)) {
 #pragma unroll
-      for (int db = 0; db < D / 16; ++db)
+        for (int db = 0; db < D / 16; ++db)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) o_acc[db][r] *= corr;
+          for (int r = 0; r < 4; ++r) o_acc[db][r] *= corr;
+      }
       // ---- O^T += V^T P^T: P^T fragments come straight from the registers ----------------
 #pragma unroll
       for (int st = 0; st < BN / 32; ++st) {
@@ -274,18 +287,251 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
   }
 }
 
-// tile_map holds num_tiles pairs (sequence, first new-token index of a 64-token tile).
+// tile_map holds num_tiles pairs (sequence, first new-token index of a 64-token tile), sorted
+// by falling number of keys the tile walks.
 RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
     const void* q, long long q_stride, void* out, long long out_stride, const void* k_pages,
     const void* v_pages, const int* block_tables, int max_pages, const int* cu_seqlens,
     const int* start_pos, const int* tile_map, int num_tiles, int nh, int nkv, int d,
     int page_shift, int window, float scale, hipStream_t stream) {
   if (num_tiles == 0) return 0;
-  dim3 grid(num_tiles, nh);
-  KERNEL_NAME<<<grid, 256, 0, stream>>>(
+  const long long blocks = (long long)num_tiles * nh;
+  if (blocks >= (1ll << 31)) {
+    rlis_set_error("attn_prefill_mfma: too many tiles");
+    return 1;
+  }
+  // 256 compute units: a round is the tiles whose blocks fill them once.
+  const int tiles_per_round = (nh <= 256 && 256 % nh == 0) ? 256 / nh : 0;
+  KERNEL_NAME<<<(int)blocks, 256, 0, stream>>>(
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,
       (const bf16_t*)v_pages, block_tables, max_pages, cu_seqlens, start_pos, tile_map, nh, nkv, d,
-      page_shift, scale, window);
+      page_shift, scale, window, num_tiles, tiles_per_round);
   RLIS_LAUNCH_CHECK("attn_prefill_mfma");
+  return 0;
+}
+
+// ===================================================================== decode kernel
+// One query token per sequence.  A workgroup serves one (KV head, sequence, partition): its
+// eight waves walk the partition in chunks of 32 keys (wave w takes chunks w, w + 8, ...) and
+// are merged at the end; partitions are merged by attn_reduce (attention.hip).  The g query
+// heads of the KV head take the place of the 16 queries of the prefill kernel: column l % 16
+// of S^T = K Q^T and O^T = V^T P^T is head l % 16 of the group (columns beyond g are zero
+// queries, never stored).  Nothing goes through LDS on the way in: lanes load K rows and V^T
+// rows from the pages directly in operand layout, 16 keys x 64 bytes and 16 dims x 32 bytes per
+// instruction, the next chunk while the current one is computed.
+//
+// Partitions are laid over key positions aligned to 32: with lo the first visible key and
+// lo32 = lo rounded down to 32, partition s covers [lo32 + s * part, lo32 + (s + 1) * part)
+// cut to [lo, ctx), part = ceil((ctx - lo32) / splits) rounded up to 256.  Page ids of a chunk
+// are fetched one chunk ahead of its keys and values, which are fetched one chunk ahead of use.
+#define DECODE_KERNEL_NAME RLIS_CAT(rlis_attn_decode_mfma_kernel_d, RLIS_HEAD_DIM)
+
+constexpr int kDecodeWaves = 8;
+
+__global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
+    const bf16_t* __restrict__ q, long long q_stride, bf16_t* __restrict__ out,
+    long long out_stride, float* __restrict__ part_ml, float* __restrict__ part_acc,
+    const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const int* __restrict__ block_tables, int max_pages, const int* __restrict__ ctx_lens,
+    int nh, int nkv, int d, int page_shift, float scale, int window, int splits) {
+  extern __shared__ float dsm[];           // ml: waves * g * 2 ; acc: waves * g * d
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int l16 = lane % 16, lq = lane / 16;
+  const int kvh = blockIdx.x, seq = blockIdx.y, split = blockIdx.z;
+  const int g = nh / nkv;
+  const int ctx = ctx_lens[seq];
+  const int* table = block_tables + (long long)seq * max_pages;
+  const int page_mask = (1 << page_shift) - 1;
+  const int lo = (window > 0 && ctx - window > 0) ? ctx - window : 0;
+  const int lo32 = lo & ~31;
+  int part = (ctx - lo32 + splits - 1) / splits;
+  constexpr int kStride = 32 * kDecodeWaves;       // keys between two chunks of one wave
+  part = ((part + kStride - 1) / kStride) * kStride;
+  const int kbeg = lo32 + split * part;
+  const int kend = min(ctx, kbeg + part);
+
+  Frag8 qf[D / 32];
+#pragma unroll
+  for (int ks = 0; ks < D / 32; ++ks) {
+    const int dim = ks * 32 + lq * 8;
+    if (l16 < g && dim < d)
+      qf[ks].u = *(const uint4*)(q + (long long)seq * q_stride + (kvh * g + l16) * d + dim);
+    else
+      qf[ks].u = make_uint4(0, 0, 0, 0);
+  }
+  float m_run = -INFINITY, l_run = 0.f;
+  f32x4 o_acc[D / 16];
+#pragma unroll
+  for (int db = 0; db < D / 16; ++db) o_acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  const float scale2 = scale * 1.4426950408889634f;
+
+  struct Chunk {
+    Frag8 k[2][D / 32];
+    Frag8 v[D / 16];
+  };
+  struct Pages {            // page of this lane's K row (two row blocks) and V keys (two halves)
+    int k[2], v[2];
+  };
+  auto load_pages = [&](int c0, Pages& pg) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int key = c0 + i * 16 + l16, key4 = c0 + i * 16 + lq * 4;
+      pg.k[i] = key < kend ? table[key >> page_shift] : 0;
+      pg.v[i] = key4 < kend ? table[key4 >> page_shift] : 0;
+    }
+  };
+  auto load_chunk = [&](int c0, const Pages& pg, Chunk& ch) {
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      const int key = c0 + nb * 16 + l16;
+      const bool ok = key < kend;
+      const bf16_t* kp =
+          k_pages + ((((long long)pg.k[nb] * nkv + kvh) << page_shift) + (key & page_mask)) * d;
+#pragma unroll
+      for (int ks = 0; ks < D / 32; ++ks) {
+        const int dim = ks * 32 + lq * 8;
+        ch.k[nb][ks].u = (ok && dim < d) ? *(const uint4*)(kp + dim) : make_uint4(0, 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int key4 = c0 + half * 16 + lq * 4;        // four keys, inside one page
+      const bool ok = key4 < kend;
+      const int off = key4 & page_mask;
+#pragma unroll
+      for (int db = 0; db < D / 16; ++db) {
+        const int dim = db * 16 + l16;
+        ch.v[db].h[half] = (ok && dim < d)
+            ? *(const uint2*)(v_pages + ((((long long)pg.v[half] * nkv + kvh) * d + dim) << page_shift) + off)
+            : make_uint2(0, 0);
+      }
+    }
+  };
+
+  int c0 = kbeg + wave * 32;
+  Chunk cur;
+  Pages pg_next;
+  if (c0 < kend) {
+    Pages pg;
+    load_pages(c0, pg);
+    load_chunk(c0, pg, cur);
+    load_pages(c0 + kStride, pg_next);
+  }
+  for (; c0 < kend; c0 += kStride) {
+    Chunk nxt;
+    const bool more = c0 + kStride < kend;
+    if (more) {
+      load_chunk(c0 + kStride, pg_next, nxt);
+      load_pages(c0 + 2 * kStride, pg_next);
+    }
+    f32x4 s[2];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      s[nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < D / 32; ++ks)
+        s[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[nb][ks].v, qf[ks].v, s[nb], 0, 0, 0);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int key = c0 + nb * 16 + lq * 4 + r;
+        const float sv = (key >= lo && key < kend) ? s[nb][r] * scale2 : -INFINITY;
+        s[nb][r] = sv;
+        mx = fmaxf(mx, sv);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float corr = __builtin_amdgcn_exp2f(m_run - m_safe);
+    float sum = 0.f;
+    bf16x8 pf;
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float p = __builtin_amdgcn_exp2f(s[nb][r] - m_safe);
+        sum += p;
+        pf[nb * 4 + r] = (__bf16)p;
+      }
+    sum += __shfl_xor(sum, 16, kWave);
+    sum += __shfl_xor(sum, 32, kWave);
+    l_run = l_run * corr + sum;
+    m_run = m_new;
+#pragma unroll
+    for (int db = 0; db < D / 16; ++db) {
+      if (db * 16 < d) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o_acc[db][r] *= corr;
+        // keys whose values were never loaded (beyond kend) have p = 0 and zero fragments
+        o_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.v[db].v, pf, o_acc[db], 0, 0, 0);
+      }
+    }
+    if (more) cur = nxt;
+  }
+
+  // ---- merge the waves (in wave order), then store the partition ------------------
+  float* ml_s = dsm;                       // [wave][head][2]
+  float* acc_s = dsm + kDecodeWaves * g * 2;   // [wave][head][d]
+  if (l16 < g) {
+    if (lq == 0) {
+      ml_s[(wave * g + l16) * 2] = m_run;
+      ml_s[(wave * g + l16) * 2 + 1] = l_run;
+    }
+#pragma unroll
+    for (int db = 0; db < D / 16; ++db)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int dim = db * 16 + lq * 4 + r;
+        if (dim < d) acc_s[(wave * g + l16) * d + dim] = o_acc[db][r];
+      }
+  }
+  __syncthreads();
+  for (int i = tid; i < g * d; i += 64 * kDecodeWaves) {
+    const int hh = i / d, j = i % d;
+    float big = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kDecodeWaves; ++w) big = fmaxf(big, ml_s[(w * g + hh) * 2]);
+    float lsum = 0.f, a = 0.f;
+#pragma unroll
+    for (int w = 0; w < kDecodeWaves; ++w) {
+      const float mw = ml_s[(w * g + hh) * 2];
+      if (mw == -INFINITY) continue;
+      const float e = __builtin_amdgcn_exp2f(mw - big);
+      lsum += ml_s[(w * g + hh) * 2 + 1] * e;
+      a += acc_s[(w * g + hh) * d + j] * e;
+    }
+    const int h = kvh * g + hh;
+    if (splits == 1) {
+      out[(long long)seq * out_stride + h * d + j] = f32_to_bf16(a / lsum);
+    } else {
+      const long long idx = ((long long)seq * nh + h) * splits + split;
+      part_acc[idx * d + j] = a;
+      if (j == 0) {
+        // attn_reduce works with natural-log maxima: m * ln 2
+        part_ml[idx * 2] = big * 0.6931471805599453f;
+        part_ml[idx * 2 + 1] = lsum;
+      }
+    }
+  }
+}
+
+RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
+    const void* q, long long q_stride, void* out, long long out_stride, float* part_ml,
+    float* part_acc, const void* k_pages, const void* v_pages, const int* block_tables,
+    int max_pages, const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift, int window,
+    float scale, int splits, hipStream_t stream) {
+  if (S == 0) return 0;
+  const int g = nh / nkv;
+  dim3 grid(nkv, S, splits);
+  const size_t smem = (size_t)kDecodeWaves * g * (2 + d) * sizeof(float);
+  DECODE_KERNEL_NAME<<<grid, 64 * kDecodeWaves, smem, stream>>>(
+      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, part_ml, part_acc,
+      (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, max_pages, ctx_lens, nh, nkv, d,
+      page_shift, scale, window, splits);
+  RLIS_LAUNCH_CHECK("attn_decode_mfma");
   return 0;
 }

@@ -543,7 +543,7 @@ __global__ __launch_bounds__(256) void gemv_bf16_rows_kernel(const bf16_t* __res
   }
 }
 
-template <typename TC, int TT, bool GATED>
+template <typename TC, int TT, bool GATED, int R, int U>
 static int launch_gemv_rows(const void* X, const void* W, void* Y, int T, int N, int K,
                             long long ldx, long long ldw, long long ldy, hipStream_t stream) {
   // x in LDS: whole K when TT * K * 2 bytes fit into 48 KiB, else k-chunks of a multiple of 512.
@@ -552,19 +552,12 @@ static int launch_gemv_rows(const void* X, const void* W, void* Y, int T, int N,
   const int fit = (48 * 1024 / (TT * 2)) / 512 * 512;
   if (kc_len > fit) kc_len = fit;
   const int num_chunks = ceil_div(K, kc_len);
-  constexpr int R = TT <= 2 ? 4 : 2;
-  constexpr int U = TT <= 4 ? 2 : 1;
   constexpr int CPG = GATED ? R / 2 : R;
   const long long groups = ceil_div(N, CPG);
-  long long blocks;
-  int groups_per_wave;
-  if (num_chunks > 1) {
-    groups_per_wave = 1;
-    blocks = ceil_div_ll(groups, 4);
-  } else {
-    blocks = ceil_div_ll(groups, 4);
-    if (blocks > 2048) blocks = 2048;
-    groups_per_wave = (int)ceil_div_ll(groups, blocks * 4);
+  long long blocks = ceil_div_ll(groups, 4);
+  int groups_per_wave = 1;
+  if (num_chunks == 1 && blocks > 2048) {
+    groups_per_wave = (int)ceil_div_ll(groups, 2048 * 4);
     blocks = ceil_div_ll(groups, (long long)groups_per_wave * 4);
   }
   const size_t smem = (size_t)TT * kc_len * sizeof(bf16_t);
@@ -573,13 +566,25 @@ static int launch_gemv_rows(const void* X, const void* W, void* Y, int T, int N,
   return 0;
 }
 
+// Rows in flight per wave: four (two k-chunks each) when that still leaves every compute
+// unit several waves, else two.
+template <typename TC, int TT, bool GATED>
+static int pick_gemv_rows(const void* X, const void* W, void* Y, int T, int N, int K,
+                          long long ldx, long long ldw, long long ldy, hipStream_t stream) {
+  constexpr int U = TT <= 4 ? 2 : 1;
+  const long long rows_total = GATED ? 2ll * N : N;
+  if (TT <= 2 && rows_total >= 16384)
+    return launch_gemv_rows<TC, TT, GATED, 4, U>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
+  return launch_gemv_rows<TC, TT, GATED, 2, U>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
+}
+
 template <typename TC, bool GATED>
 static int dispatch_gemv_rows(const void* X, const void* W, void* Y, int T, int N, int K,
                               long long ldx, long long ldw, long long ldy, hipStream_t stream) {
-  if (T <= 1) return launch_gemv_rows<TC, 1, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
-  if (T <= 2) return launch_gemv_rows<TC, 2, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
-  if (T <= 4) return launch_gemv_rows<TC, 4, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
-  return launch_gemv_rows<TC, 8, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
+  if (T <= 1) return pick_gemv_rows<TC, 1, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
+  if (T <= 2) return pick_gemv_rows<TC, 2, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
+  if (T <= 4) return pick_gemv_rows<TC, 4, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
+  return pick_gemv_rows<TC, 8, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
 }
 
 // gated == 0: y (T, N) = x W^T.  gated != 0: W is (2N, K) = [Wg; Wu] and

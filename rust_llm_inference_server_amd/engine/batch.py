@@ -73,7 +73,7 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
     ctx_lens: List[int] = []
     logit_rows: List[int] = []
     state_slots: List[int] = []
-    tiles: List[int] = []
+    tiles: List[Tuple[int, int, int]] = []      # (keys the tile walks, sequence, first index)
     ng = cache.num_groups
     tables: List[List[List[int]]] = [[] for _ in range(ng)]
     slots: List[List[int]] = [[] for _ in range(ng)]
@@ -107,7 +107,8 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
             if not 0 <= int(w) < n:
                 raise ValueError(f"request {e.seq_id}: wanted index {w} is outside its {n} tokens")
             logit_rows.append(base + int(w))
-        tiles.extend(x for qb in range(0, n, PREFILL_TILE) for x in (s, qb))
+        tiles.extend((computed + min(n, qb + PREFILL_TILE), s, qb)
+                     for qb in range(0, n, PREFILL_TILE))
         for g in range(ng):
             table = cache.table(e.seq_id, g)
             tables[g].append(table)
@@ -134,7 +135,9 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
     put("ctx_lens", ctx_lens)
     put("logit_rows", logit_rows)
     put("state_slots", state_slots)
-    put("tiles", tiles)
+    # Longest tiles first: the prefill attention kernel hands them out in this order.
+    tiles.sort(key=lambda t: -t[0])
+    put("tiles", [x for _, s_, qb in tiles for x in (s_, qb)])
     for g in range(ng):
         put(f"slots{g}", slots[g])
         rows: List[int] = []
@@ -158,7 +161,7 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
         num_tokens=T, num_seqs=S, ids=view("ids"), positions=view("positions"),
         seq_of_token=view("seq_of_token"), cu_seqlens=view("cu"), start_pos=view("start_pos"),
         ctx_lens=view("ctx_lens"), logit_rows=view("logit_rows"), num_logit_rows=len(logit_rows),
-        state_slots=view("state_slots"), tile_map=view("tiles"), num_tiles=len(tiles) // 2,
+        state_slots=view("state_slots"), tile_map=view("tiles"), num_tiles=len(tiles),
         groups=groups, max_context=max(ctx_lens), max_new=max(len(e.tokens) for e in entries),
         all_decode=all(len(e.tokens) == 1 for e in entries),
         host_start_pos=start_pos, host_new=[len(e.tokens) for e in entries],

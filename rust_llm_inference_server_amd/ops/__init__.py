@@ -19,13 +19,19 @@ _DT = {torch.float32: 0, torch.bfloat16: 1}
 # bf16 products with at most this many rows of x take the skinny kernel.
 SKINNY_MAX_ROWS = 64
 # ... and with at most this many rows the row-streaming kernel.
-GEMV_MAX_ROWS = 8
+GEMV_MAX_ROWS = 2
+# ... or this many rows when the weight has at least GEMV_WIDE_N rows (the output head).
+GEMV_MAX_ROWS_WIDE = 4
+GEMV_WIDE_N = 32768
 # "library": bf16 products with more rows and bf16 output go to torch.matmul (hipBLASLt);
 # "own": they take the hand-written matrix-core kernel.
 BF16_GEMM = "library"
 # None: attention kernels are chosen from the batch; "generic": the generic kernel always
 # (what the command line's --attention v1 asks for).
 FORCE_ATTENTION: Optional[str] = None
+# "matrix": bfloat16 decode attention on the matrix cores where it applies; "vector": always
+# the vector-unit decode kernel (tests compare the two).
+DECODE_ATTENTION = "matrix"
 
 
 def _dt(t: torch.Tensor) -> int:
@@ -151,7 +157,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     y = torch.empty((T, N), dtype=out_dtype, device=x.device)
     if T == 0:
         return y
-    if bf16 and aligned and T <= GEMV_MAX_ROWS:
+    if bf16 and aligned and (T <= GEMV_MAX_ROWS
+                             or (T <= GEMV_MAX_ROWS_WIDE and N >= GEMV_WIDE_N)):
         lib.call("rlis_gemv_bf16_rows", x.data_ptr(), w.data_ptr(), y.data_ptr(), _DT[out_dtype],
                  T, N, K, ldx, ldw, N, 0, stream)
     elif bf16 and aligned:
@@ -311,12 +318,23 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
         if splits > 1:
             part_ml = torch.empty((S, nh, splits, 2), dtype=torch.float32, device=qkv.device)
             part_acc = torch.empty((S, nh, splits, d), dtype=torch.float32, device=qkv.device)
-        lib.call("rlis_attn_decode", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(), nh * d,
-                 None if part_ml is None else part_ml.data_ptr(),
-                 None if part_acc is None else part_acc.data_ptr(),
-                 k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,
-                 _i32(step.ctx_lens, "ctx_lens", S), None, S, nh, nkv, d, page_size,
-                 float(scale), win, splits, stream)
+        g = nh // nkv
+        mfma = (qkv.dtype == torch.bfloat16 and d % 16 == 0 and g <= 16
+                and g * (d + 2) * 32 <= 65536
+                and page_size >= 8 and page_size & (page_size - 1) == 0 and q_stride % 8 == 0
+                and DECODE_ATTENTION != "vector")
+        ml_ptr = None if part_ml is None else part_ml.data_ptr()
+        acc_ptr = None if part_acc is None else part_acc.data_ptr()
+        if mfma:
+            lib.call("rlis_attn_decode_mfma", qkv.data_ptr(), q_stride, out.data_ptr(), nh * d,
+                     ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
+                     block_tables.data_ptr(), max_pages, _i32(step.ctx_lens, "ctx_lens", S), S,
+                     nh, nkv, d, page_size, win, float(scale), splits, stream)
+        else:
+            lib.call("rlis_attn_decode", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(),
+                     nh * d, ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
+                     block_tables.data_ptr(), max_pages, _i32(step.ctx_lens, "ctx_lens", S), None,
+                     S, nh, nkv, d, page_size, float(scale), win, splits, stream)
     elif kind == "prefill":
         if qkv.dtype != torch.bfloat16:
             raise KernelError("attention: the matrix-core prefill kernel is bfloat16 only")

@@ -23,6 +23,16 @@ def rnd(*shape, dtype=torch.float32, scale=1.0, seed=0):
     return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
 
 
+@pytest.fixture(params=["matrix", "vector"])
+def decode_kind(request):
+    """Both decode attention kernels: on the matrix cores (bfloat16) and on the vector units."""
+    from rust_llm_inference_server_amd import ops
+    old = ops.DECODE_ATTENTION
+    ops.DECODE_ATTENTION = request.param
+    yield request.param
+    ops.DECODE_ATTENTION = old
+
+
 @pytest.fixture(scope="module")
 def ops():
     from rust_llm_inference_server_amd import ops
@@ -127,12 +137,13 @@ def test_linear_bfloat16(ops, out_dtype, T, N, K):
         torch.testing.assert_close(got, want, atol=2e-5 * max(1.0, scale) * math.sqrt(K / 64), rtol=1e-4)
     else:
         torch.testing.assert_close(got.float(), want, atol=scale / 128, rtol=1e-2)
-    old = ops.BF16_GEMM
+    old = ops.BF16_GEMM, ops.GEMV_MAX_ROWS
     try:
         ops.BF16_GEMM = "own"
+        ops.GEMV_MAX_ROWS = 0 if T <= old[1] else 8       # the other kernel for this many rows
         got2 = ops.linear(x, w, out_dtype)
     finally:
-        ops.BF16_GEMM = old
+        ops.BF16_GEMM, ops.GEMV_MAX_ROWS = old
     torch.testing.assert_close(got2.float(), got.float(), atol=scale / 128, rtol=1e-2)
 
 
@@ -150,6 +161,13 @@ def test_linear_swiglu(ops, dtype, T, I, K):
     want = (torch.nn.functional.silu(g) * u).float()
     got = ops.linear_swiglu(x, w)
     assert got.dtype == dtype and got.shape == (T, I)
+    old = ops.GEMV_MAX_ROWS
+    try:
+        ops.GEMV_MAX_ROWS = 0 if T <= old else 8              # the other kernel for this many rows
+        other = ops.linear_swiglu(x, w)
+    finally:
+        ops.GEMV_MAX_ROWS = old
+    torch.testing.assert_close(other.float(), got.float(), atol=0.05, rtol=2e-2)
     scale = max(1.0, want.abs().max().item())
     if dtype == torch.float32:
         torch.testing.assert_close(got, want, atol=1e-4 * scale, rtol=1e-4)
@@ -318,7 +336,7 @@ def test_attention_mixed_batch(ops, dtype, nh, nkv, d, ps, kind):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("kind", ["generic", "prefill", "decode"])
 @pytest.mark.parametrize("window", [1, 7, 64, 100])
-def test_attention_window(ops, dtype, kind, window):
+def test_attention_window(ops, dtype, kind, window, decode_kind):
     if kind == "prefill" and dtype != torch.bfloat16:
         pytest.skip("the matrix-core prefill kernel is bfloat16 only")
     nh, nkv, d, ps = 6, 2, 32, 8
@@ -332,7 +350,7 @@ def test_attention_window(ops, dtype, kind, window):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,d,ps", LAYOUTS)
-def test_attention_decode(ops, dtype, nh, nkv, d, ps):
+def test_attention_decode(ops, dtype, nh, nkv, d, ps, decode_kind):
     """One token per sequence, 37 context lengths 1 + (i * 53) % 700 as in the reference's
     kernel test (crates/model/src/paged_attention.rs:461-527), unsplit and split."""
     lens = [1 + (i * 53) % 700 for i in range(37)]
@@ -350,7 +368,7 @@ def test_attention_decode(ops, dtype, nh, nkv, d, ps):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_attention_decode_long_split(ops, dtype):
+def test_attention_decode_long_split(ops, dtype, decode_kind):
     """Long contexts beside short ones with many partitions, some of them empty
     (lens [1, 5, 300, 4000, 9000]: paged_attention.rs:503-527)."""
     nh, nkv, d, ps = 8, 2, 64, 16
@@ -367,7 +385,7 @@ def test_attention_decode_long_split(ops, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("kind", ["generic", "prefill", "decode"])
-def test_attention_finds_a_far_key(ops, dtype, kind):
+def test_attention_finds_a_far_key(ops, dtype, kind, decode_kind):
     """One key among hundreds is made to stand out (its key vector equals the scaled query
     direction); the output must be that key's value, wherever its page lies."""
     if kind == "prefill" and dtype != torch.bfloat16:
