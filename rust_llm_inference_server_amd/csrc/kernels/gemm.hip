@@ -294,19 +294,27 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(const bf16_t* __r
 
   const int kbeg = wave * kslice;
   const int kend = min(K, kbeg + kslice);
-  const uint4 zero = make_uint4(0, 0, 0, 0);
   for (int k = kbeg; k < kend; k += 32 * U) {
     Frag8 a[RBT][U], b[NT][U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int gk = k + u * 32 + kq;
       const bool kin = gk < kend;     // kslice is a multiple of 32 and K of 8: whole chunks only
+      // Loads are never predicated off (the compiler would turn that into flat loads of a
+      // zero kept in scratch): out-of-range lanes read a safe address and are zeroed after.
+      const int sk = kin ? gk : k;
 #pragma unroll
-      for (int rb = 0; rb < RBT; ++rb)
-        a[rb][u].u = (wvalid[rb] && kin) ? *(const uint4*)(wp[rb] + gk) : zero;
+      for (int rb = 0; rb < RBT; ++rb) {
+        const uint4 v = *(const uint4*)(wp[rb] + sk);
+        const bool ok = wvalid[rb] && kin;
+        a[rb][u].u = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+      }
 #pragma unroll
-      for (int tt = 0; tt < NT; ++tt)
-        b[tt][u].u = (xvalid[tt] && kin) ? *(const uint4*)(xp[tt] + gk) : zero;
+      for (int tt = 0; tt < NT; ++tt) {
+        const uint4 v = *(const uint4*)(xp[tt] + sk);
+        const bool ok = xvalid[tt] && kin;
+        b[tt][u].u = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+      }
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -605,5 +613,244 @@ RLIS_API int rlis_gemv_bf16_rows(const void* X, const void* W, void* Y, int y_dt
   else
     RLIS_REQUIRE(false, "gemv_bf16_rows: unknown output dtype %d", y_dtype);
   RLIS_LAUNCH_CHECK("gemv_bf16_rows");
+  return 0;
+}
+
+// ============================================================ streaming skinny product
+// y (T <= 16, N) = x W^T at the speed of the weight stream.
+//
+// Work is cut into tiles of 16 (or 8) weight rows times a k slice of up to 16 items of 256; a
+// workgroup has one wave per item and walks over tiles (persistent, its slice fixed), so the
+// rows of x that a wave needs are loaded once, straight into operand layout, and stay in
+// registers.  An item's weights are loaded row by row, 512 contiguous bytes per half wave,
+// which keeps the memory system at its streaming rate, one tile ahead of the arithmetic.  The
+// matrix-core operand wants lane l to hold row l % 16 instead, so the item goes through an
+// LDS tile private to the wave (chunks XOR-swizzled by row, so both directions are free of
+// bank conflicts).  One v_mfma_f32_16x16x32_bf16 accumulator per wave; the waves of a
+// workgroup are summed in LDS in wave order.  With more than one slice (K > 4096) every slice
+// stores its own float32 partial result, which the consumer adds in slice order: the order
+// of a sum depends on K alone.  The gated form pairs gate rows with their up rows in one
+// tile and applies the SwiGLU before the store.
+constexpr int kStreamItem = 256;                        // k per item
+constexpr int kStreamTileBytes = 16 * kStreamItem * 2;  // one wave's tile in LDS
+constexpr int kStreamMaxWaves = 16;
+
+__device__ __forceinline__ void wave_lds_fence() {
+  // LDS operations of one wave execute in order; this only stops the compiler from moving
+  // reads of other lanes' data above the writes.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+struct StreamShape {
+  int T, N, K;
+  long long ldx, ldw, ldy, part_stride;   // part_stride: elements between partial results
+  int num_tiles, num_slices;
+};
+
+template <typename TC, bool GATED, int TR /* weight rows per tile: 16 or 8 */>
+__global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __restrict__ X,
+                                                                const bf16_t* __restrict__ W,
+                                                                TC* __restrict__ Y,
+                                                                const StreamShape sh) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char stream_smem[];
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, nwaves = blockDim.x / 64;
+  unsigned char* tile_s = stream_smem + wave * kStreamTileBytes;
+  float* red = (float*)(stream_smem + nwaves * kStreamTileBytes);      // [2][nwaves][256]
+  const int half = lane / 32, l32 = lane % 32;          // loading: row parity, 16-byte chunk
+  const int oi = lane % 16, og = lane / 16;             // operand: row (or token), k group
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  const int T = sh.T, N = sh.N, K = sh.K;
+  const int slice = blockIdx.x % sh.num_slices;
+  const int tile_step = gridDim.x / sh.num_slices;
+  const int nitems = (K + kStreamItem - 1) / kStreamItem;
+  const int item = slice * nwaves + wave;
+  const bool has_item = item < nitems;
+  const int kb = item * kStreamItem;
+  const int ka = kb + l32 * 8;                          // this lane's k when loading weights
+  const bool a_ok = has_item && ka < K;
+
+  Frag8 b[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int k = kb + (4 * j + og) * 8;
+    const bool ok = has_item && oi < T && k < K;
+    const uint4 v = *(const uint4*)(X + (ok ? (long long)oi * sh.ldx + k : 0));
+    b[j].u = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+  }
+
+  // Tile row r = 2 p + half of tile `tile` is weight row tile * rows + r; gated, the first
+  // half of a tile's rows are the gate rows of consecutive columns and the second half their
+  // up rows, N further down.  Everything but `half` and the lane's k is uniform over the wave.
+  constexpr int cols_per_tile = GATED ? TR / 2 : TR;
+  // Loads are never predicated off (that would cost registers for the zeros): a row past the
+  // end reads row 0 instead and is not stored; a k past the end reads k = 0 and is zeroed.
+  const int ka_safe = a_ok ? ka : 0;
+  const bf16_t* w_lane = W + (long long)half * sh.ldw + ka_safe;
+#define RLIS_STREAM_LOAD_TILE(a, tile_)                                                         \
+  {                                                                                             \
+    const int tl_ = (tile_);                                                                    \
+    if (tl_ < sh.num_tiles) {                                                                   \
+      const bf16_t* w_tile = w_lane + (long long)tl_ * cols_per_tile * sh.ldw;                  \
+      const int col0 = tl_ * cols_per_tile + half;                                              \
+      _Pragma("unroll") for (int p = 0; p < TR / 2; ++p) {                                      \
+        {                                                                                       \
+          const int c = GATED ? (2 * p) % cols_per_tile : 2 * p; /* column within the tile */   \
+          const long long up = (GATED && 2 * p >= cols_per_tile) ? (long long)N * sh.ldw : 0;   \
+          const bf16_t* ptr = col0 + c < N ? w_tile + (long long)c * sh.ldw + up : W + ka_safe; \
+          const uint4 v_ = *(const uint4*)ptr;                                                  \
+          a[p].x = a_ok ? v_.x : 0u;                                                            \
+          a[p].y = a_ok ? v_.y : 0u;                                                            \
+          a[p].z = a_ok ? v_.z : 0u;                                                            \
+          a[p].w = a_ok ? v_.w : 0u;                                                            \
+        }                                                                                       \
+      }                                                                                         \
+    }                                                                                           \
+  }
+
+  uint4 a[TR / 2];
+  int tile = blockIdx.x / sh.num_slices;
+  RLIS_STREAM_LOAD_TILE(a, tile);
+  int par = 0;
+  for (; tile < sh.num_tiles; tile += tile_step) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    if (has_item) {
+#pragma unroll
+      for (int p = 0; p < TR / 2; ++p) {
+        const int r = 2 * p + half;
+        *(uint4*)(tile_s + r * (kStreamItem * 2) + ((l32 ^ r) * 16)) = a[p];
+      }
+    }
+    RLIS_STREAM_LOAD_TILE(a, tile + tile_step);  // on its way during the arithmetic
+    if (has_item) {
+      wave_lds_fence();
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        Frag8 af;
+        af.u = *(const uint4*)(tile_s + oi * (kStreamItem * 2) + (((4 * j + og) ^ oi) * 16));
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af.v, b[j].v, acc, 0, 0, 0);
+      }
+      wave_lds_fence();
+    }
+    // acc: token oi, tile rows og * 4 + r.  red[par][wave][token][row]; the buffer of the
+    // tile before is still being read by slower waves, the one before that is free again
+    // after this tile's barrier.
+    float* red_p = red + par * nwaves * 256;
+    *(float4*)(red_p + wave * 256 + oi * 16 + og * 4) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    __syncthreads();
+    if (tid < 256) {
+      const int t = tid / 16, i = tid % 16;
+      TC* y = Y + (long long)slice * sh.part_stride + (long long)t * sh.ldy;
+      if (GATED) {
+        constexpr int h = TR / 2;
+        const long long c = (long long)tile * h + i;
+        if (i < h && t < T && c < N) {
+          float gate = 0.f, up = 0.f;
+          for (int w = 0; w < nwaves; ++w) {
+            gate += red_p[w * 256 + t * 16 + i];
+            up += red_p[w * 256 + t * 16 + h + i];
+          }
+          st(y + c, gate / (1.0f + expf(-gate)) * up);
+        }
+      } else {
+        const long long n = (long long)tile * TR + i;
+        if (i < TR && t < T && n < N) {
+          float sum = 0.f;
+          for (int w = 0; w < nwaves; ++w) sum += red_p[w * 256 + t * 16 + i];
+          st(y + n, sum);
+        }
+      }
+    }
+    par ^= 1;
+  }
+#undef RLIS_STREAM_LOAD_TILE
+}
+
+// Number of k slices a product over K is cut into (a function of K alone).
+static int stream_slices(int K) {
+  return ceil_div(ceil_div(K, kStreamItem), kStreamMaxWaves);
+}
+
+template <typename TC, bool GATED, int TR>
+static int launch_stream_tiles(const void* X, const void* W, void* Y, StreamShape sh, int nwaves,
+                               int num_cus, hipStream_t stream) {
+  static bool lds_raised = false;
+  if (!lds_raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_stream_kernel<TC, GATED, TR>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       kStreamMaxWaves * (kStreamTileBytes + 2048));
+    RLIS_REQUIRE(e == hipSuccess, "gemm_bf16_stream: cannot raise the LDS limit: %s",
+                 hipGetErrorString(e));
+    lds_raised = true;
+  }
+  const size_t smem = (size_t)nwaves * (kStreamTileBytes + 2048);
+  const int per_cu = max(1, (int)((160 * 1024) / smem));
+  const long long tiles = ceil_div_ll(sh.N, GATED ? TR / 2 : TR);
+  RLIS_REQUIRE(tiles <= 0x3fffffffll, "gemm_bf16_stream: N=%d is too large", sh.N);
+  sh.num_tiles = (int)tiles;
+  long long groups = tiles;                                // workgroups per slice
+  const long long cap = max(1, num_cus * per_cu / sh.num_slices);
+  if (groups > cap) groups = cap;
+  gemm_bf16_stream_kernel<TC, GATED, TR><<<(int)(groups * sh.num_slices), nwaves * 64, smem, stream>>>(
+      (const bf16_t*)X, (const bf16_t*)W, (TC*)Y, sh);
+  return 0;
+}
+
+template <typename TC, bool GATED>
+static int launch_stream(const void* X, const void* W, void* Y, int T, int N, int K, long long ldx,
+                         long long ldw, long long ldy, long long part_stride,
+                         hipStream_t stream) {
+  const int nitems = ceil_div(K, kStreamItem);
+  const int slices = stream_slices(K);
+  const int nwaves = max(4, ceil_div(nitems, slices));
+  static int num_cus = 0;
+  if (num_cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    RLIS_REQUIRE(hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess,
+                 "gemm_bf16_stream: cannot read the device properties");
+    num_cus = prop.multiProcessorCount;
+  }
+  StreamShape sh;
+  sh.T = T; sh.N = N; sh.K = K; sh.ldx = ldx; sh.ldw = ldw; sh.ldy = ldy;
+  sh.part_stride = part_stride;
+  sh.num_slices = slices;
+  sh.num_tiles = 0;
+  // Tiles of 8 rows when 16-row tiles would leave compute units without work: a unit draws
+  // only its share of the memory bandwidth, however much it has in flight.
+  if ((long long)ceil_div(N, GATED ? 8 : 16) * slices < num_cus)
+    return launch_stream_tiles<TC, GATED, 8>(X, W, Y, sh, nwaves, num_cus, stream);
+  return launch_stream_tiles<TC, GATED, 16>(X, W, Y, sh, nwaves, num_cus, stream);
+}
+
+// Slices that rlis_gemm_bf16_stream cuts K into; with more than one, Y receives that many
+// float32 partial results, part_stride elements apart, to be added in order.
+RLIS_API int rlis_gemm_bf16_stream_slices(int K) { return stream_slices(K); }
+
+// gated == 0: y (T, N) = x W^T.  gated != 0: W is (2N, K) = [Wg; Wu] and
+// y (T, N) = silu(x Wg^T) * (x Wu^T), K <= 4096.  T <= 16, bfloat16 operands, K a multiple of 8.
+RLIS_API int rlis_gemm_bf16_stream(const void* X, const void* W, void* Y, int y_dtype, int T,
+                                   int N, int K, long long ldx, long long ldw, long long ldy,
+                                   long long part_stride, int gated, hipStream_t stream) {
+  if (check_skinny("gemm_bf16_stream", X, W, T, N, K, ldx, ldw, ldy)) return 1;
+  RLIS_REQUIRE(T <= 16, "gemm_bf16_stream: T=%d rows, at most 16", T);
+  const int slices = stream_slices(K);
+  RLIS_REQUIRE(slices == 1 || (!gated && y_dtype == RLIS_F32 && part_stride >= (long long)T * ldy),
+               "gemm_bf16_stream: K=%d takes %d slices, which need float32 partial results and "
+               "no gate", K, slices);
+  RLIS_REQUIRE(!gated || y_dtype == RLIS_BF16, "gemm_bf16_stream: the gated form stores bfloat16");
+  if (T == 0) return 0;
+  int rc;
+  if (gated)
+    rc = launch_stream<bf16_t, true>(X, W, Y, T, N, K, ldx, ldw, ldy, part_stride, stream);
+  else if (y_dtype == RLIS_F32)
+    rc = launch_stream<float, false>(X, W, Y, T, N, K, ldx, ldw, ldy, part_stride, stream);
+  else if (y_dtype == RLIS_BF16)
+    rc = launch_stream<bf16_t, false>(X, W, Y, T, N, K, ldx, ldw, ldy, part_stride, stream);
+  else
+    RLIS_REQUIRE(false, "gemm_bf16_stream: unknown output dtype %d", y_dtype);
+  if (rc) return rc;
+  RLIS_LAUNCH_CHECK("gemm_bf16_stream");
   return 0;
 }

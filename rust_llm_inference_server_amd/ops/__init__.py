@@ -18,6 +18,8 @@ _DT = {torch.float32: 0, torch.bfloat16: 1}
 
 # bf16 products with at most this many rows of x take the skinny kernel.
 SKINNY_MAX_ROWS = 64
+# ... with at most this many rows the streaming kernel (16 at most; 0 switches it off),
+STREAM_MAX_ROWS = 16
 # ... and with at most this many rows the row-streaming kernel.
 GEMV_MAX_ROWS = 2
 # ... or this many rows when the weight has at least GEMV_WIDE_N rows (the output head).
@@ -80,14 +82,29 @@ def embed(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def _delta_parts(resid: torch.Tensor, delta: torch.Tensor, what: str) -> int:
+    """A delta is shaped like the residual, or is a stack ``(S, T, H)`` of float32 partial sums
+    (what ``linear(..., partials=True)`` returns) that are added in order."""
+    _check(delta, "delta")
+    if not delta.is_contiguous():
+        raise KernelError(f"{what}: delta must be contiguous")
+    if delta.shape == resid.shape:
+        return 1
+    if delta.dim() == resid.dim() + 1 and delta.shape[1:] == resid.shape \
+            and delta.dtype == torch.float32 and delta.shape[0] >= 1:
+        return delta.shape[0]
+    raise KernelError(f"{what}: delta of shape {tuple(delta.shape)} does not match the residual "
+                      f"{tuple(resid.shape)}")
+
+
 def add_residual(resid: torch.Tensor, delta: torch.Tensor) -> None:
     """``resid += delta`` with the sum formed in float32."""
     _check(resid, "residual", torch.float32)
-    _check(delta, "delta")
-    if resid.shape != delta.shape or not (resid.is_contiguous() and delta.is_contiguous()):
-        raise KernelError("add_residual: shapes differ or tensors are not contiguous")
+    if not resid.is_contiguous():
+        raise KernelError("add_residual: residual must be contiguous")
+    parts = _delta_parts(resid, delta, "add_residual")
     lib.call("rlis_add_residual", resid.data_ptr(), delta.data_ptr(), _dt(delta), resid.numel(),
-             lib.stream_ptr())
+             parts, lib.stream_ptr())
 
 
 def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
@@ -101,10 +118,7 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
     T, H = resid.shape
     if not resid.is_contiguous():
         raise KernelError("add_rmsnorm: residual must be contiguous")
-    if delta is not None:
-        _check(delta, "delta", ndim=2)
-        if delta.shape != resid.shape or not delta.is_contiguous():
-            raise KernelError("add_rmsnorm: delta must match the residual and be contiguous")
+    parts = 1 if delta is None else _delta_parts(resid, delta, "add_rmsnorm")
     _check(weight, "norm weight", ndim=1)
     if weight.numel() != H or not weight.is_contiguous():
         raise KernelError(f"add_rmsnorm: weight has {weight.numel()} entries, rows have {H}")
@@ -116,7 +130,7 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
     lib.call("rlis_add_rmsnorm", resid.data_ptr(),
              None if delta is None else delta.data_ptr(), 0 if delta is None else _dt(delta),
              weight.data_ptr(), _dt(weight), out.data_ptr(), _DT[out_dtype], rows_ptr, R, H,
-             float(eps), int(bool(write_resid)), lib.stream_ptr())
+             float(eps), int(bool(write_resid)), parts, T * H, lib.stream_ptr())
     return out
 
 
@@ -133,13 +147,22 @@ def swiglu(gu: torch.Tensor) -> torch.Tensor:
 
 
 # ----------------------------------------------------------------------- products
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None
-           ) -> torch.Tensor:
+def stream_slices(K: int) -> int:
+    """Number of k slices the streaming kernel cuts a product over ``K`` into."""
+    return lib.load().rlis_gemm_bf16_stream_slices(K)
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+           partials: bool = False) -> torch.Tensor:
     """``x @ w.T`` for ``x (T, K)`` and ``w (N, K)``, float32 accumulation.
 
     A float32 weight (or float32 ``x``) takes the plain FMA kernel, the true 32-bit product.
-    bfloat16 operands take the skinny kernel up to 64 rows, else the matrix-core GEMM (ours
-    for float32 output, the library's or ours for bfloat16 output)."""
+    bfloat16 operands take the streaming kernel up to 16 rows, the skinny kernel up to 64, else
+    the matrix-core GEMM (ours for float32 output, the library's or ours for bfloat16 output).
+
+    ``partials``: the caller hands the result to the residual stream and takes it as a stack
+    ``(S, T, N)`` of float32 partial sums too (one per k slice of the streaming kernel, added in
+    order by ``add_rmsnorm`` / ``add_residual``) where that saves a pass."""
     ldx = _rows_contig(x, "linear x")
     ldw = _rows_contig(w, "linear weight")
     T, K = x.shape
@@ -154,6 +177,16 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     if bf16 and aligned and T > SKINNY_MAX_ROWS and out_dtype == torch.bfloat16 \
             and BF16_GEMM == "library":
         return torch.matmul(x, w.t())
+    if bf16 and aligned and 0 < T <= STREAM_MAX_ROWS:
+        slices = stream_slices(K)
+        if slices == 1 or partials:
+            if slices == 1:
+                y = torch.empty((T, N), dtype=out_dtype, device=x.device)
+            else:
+                y = torch.empty((slices, T, N), dtype=torch.float32, device=x.device)
+            lib.call("rlis_gemm_bf16_stream", x.data_ptr(), w.data_ptr(), y.data_ptr(),
+                     _DT[y.dtype], T, N, K, ldx, ldw, N, T * N, 0, stream)
+            return y
     y = torch.empty((T, N), dtype=out_dtype, device=x.device)
     if T == 0:
         return y
@@ -189,7 +222,10 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
     if not fused:
         return swiglu(linear(x, w_gate_up, x.dtype))
     y = torch.empty((T, two_i // 2), dtype=torch.bfloat16, device=x.device)
-    if T <= GEMV_MAX_ROWS:
+    if T <= STREAM_MAX_ROWS and stream_slices(K) == 1:
+        lib.call("rlis_gemm_bf16_stream", x.data_ptr(), w_gate_up.data_ptr(), y.data_ptr(), 1, T,
+                 two_i // 2, K, ldx, ldw, two_i // 2, 0, 1, lib.stream_ptr())
+    elif T <= GEMV_MAX_ROWS:
         lib.call("rlis_gemv_bf16_rows", x.data_ptr(), w_gate_up.data_ptr(), y.data_ptr(), 1, T,
                  two_i // 2, K, ldx, ldw, two_i // 2, 1, lib.stream_ptr())
     else:

@@ -16,8 +16,8 @@ P, I, L, F = c_void_p, c_int, c_longlong, c_float
 
 _SIGNATURES = {
     "rlis_embed": [P, P, I, P, I, I, P],
-    "rlis_add_residual": [P, P, I, L, P],
-    "rlis_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, P],
+    "rlis_add_residual": [P, P, I, L, I, P],
+    "rlis_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, I, L, P],
     "rlis_swiglu": [P, P, I, I, I, P],
     "rlis_rope_kv_write": [P, I, L, I, I, I, I, I, I, I, P, P, P, P, P, P, I, I, P],
     "rlis_copy_pages": [P, I, I, L, L, P, P, I, P],
@@ -26,6 +26,7 @@ _SIGNATURES = {
     "rlis_gemm_bf16_skinny": [P, P, P, I, I, I, I, L, L, L, P],
     "rlis_gemm_bf16_skinny_swiglu": [P, P, P, I, I, I, L, L, L, P],
     "rlis_gemv_bf16_rows": [P, P, P, I, I, I, I, L, L, L, I, P],
+    "rlis_gemm_bf16_stream": [P, P, P, I, I, I, I, L, L, L, L, I, P],
     "rlis_attn_generic": [P, I, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
     "rlis_attn_decode": [P, I, L, P, L, P, P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, P],
     "rlis_attn_decode_mfma": [P, L, P, L, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, P],
@@ -58,6 +59,8 @@ def load() -> ctypes.CDLL:
             raise RuntimeError(f"{path} does not export {name}; rebuild the kernels")
         fn.restype = c_int
         fn.argtypes = argtypes
+    lib.rlis_gemm_bf16_stream_slices.restype = c_int
+    lib.rlis_gemm_bf16_stream_slices.argtypes = [I]
     _LIB = lib
     return lib
 

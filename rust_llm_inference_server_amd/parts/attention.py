@@ -73,4 +73,4 @@ class PagedAttention(Mixer):
         out = ops.paged_attention(qkv, self.num_heads, self.num_kv_heads, self.head_dim,
                                   binding.k_pages, binding.v_pages, group.page_size,
                                   group.block_tables, step, self.scale, self.window)
-        return ops.linear(out, self.w_o, self.act_dtype)
+        return ops.linear(out, self.w_o, self.act_dtype, partials=True)

@@ -162,7 +162,9 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    """``forward(x, step, binding)`` maps activations ``(T, H)`` to ``(T, H)``.
+    """``forward(x, step, binding)`` maps activations ``(T, H)`` to ``(T, H)``.  The result goes
+    to the residual stream, so it may also be a stack ``(S, T, H)`` of float32 partial sums
+    (what ``ops.linear(..., partials=True)`` returns), which the stream adds in order.
 
     ``cache_request()`` says what the mixer keeps in pages (None: nothing);
     ``state_bytes()`` how many bytes of fixed-size state it keeps per request (0: none).  A
@@ -184,7 +186,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    """``forward(x, step)`` maps activations ``(T, H)`` to ``(T, H)``, row by row."""
+    """``forward(x, step)`` maps activations ``(T, H)`` to ``(T, H)``, row by row (or to a
+    stack of float32 partial sums of that, as a mixer may)."""
 
     def forward(self, x: torch.Tensor, step: Any) -> torch.Tensor:
         raise NotImplementedError

@@ -34,4 +34,5 @@ class SwiGLU(FeedForward):
         self.act_dtype = ctx.act_dtype
 
     def forward(self, x: torch.Tensor, step: Any) -> torch.Tensor:
-        return ops.linear(ops.linear_swiglu(x, self.w_gate_up), self.w_down, self.act_dtype)
+        return ops.linear(ops.linear_swiglu(x, self.w_gate_up), self.w_down, self.act_dtype,
+                          partials=True)

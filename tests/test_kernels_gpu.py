@@ -147,6 +147,42 @@ def test_linear_bfloat16(ops, out_dtype, T, N, K):
     torch.testing.assert_close(got2.float(), got.float(), atol=scale / 128, rtol=1e-2)
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16], ids=["f32out", "bf16out"])
+@pytest.mark.parametrize("T,N,K", [(1, 2048, 2048), (8, 2048, 8192), (16, 3072, 2048), (3, 130, 96),
+                                   (16, 331, 104), (7, 17, 14336), (5, 1001, 4608), (9, 16, 8),
+                                   (2, 128256, 256)])
+def test_linear_streaming_kernel(ops, out_dtype, T, N, K):
+    """The streaming kernel for up to 16 rows (weights through LDS into operand layout), plain and
+    gated, against float64 products of the same bf16-rounded operands; sizes that end inside a
+    k item, inside a row tile, and with more k items than a workgroup has waves."""
+    x, w = rnd(T, K, dtype=torch.bfloat16, seed=3), rnd(N, K, dtype=torch.bfloat16, seed=4, scale=0.05)
+    want = (x.double() @ w.double().t()).float()
+    old = ops.STREAM_MAX_ROWS
+    try:
+        ops.STREAM_MAX_ROWS = 16
+        if ops.stream_slices(K) > 1:       # one float32 partial result per k slice
+            parts = ops.linear(x, w, partials=True)
+            assert parts.shape == (ops.stream_slices(K), T, N)
+            got = parts.sum(dim=0).to(out_dtype)
+        else:
+            got = ops.linear(x, w, out_dtype)
+        gated = None
+        if N % 2 == 0 and out_dtype == torch.bfloat16 and ops.stream_slices(K) == 1:
+            gated = ops.linear_swiglu(x, w)
+    finally:
+        ops.STREAM_MAX_ROWS = old
+    scale = max(1.0, want.abs().max().item())
+    if out_dtype == torch.float32:
+        torch.testing.assert_close(got, want, atol=2e-5 * scale * math.sqrt(K / 64), rtol=1e-4)
+    else:
+        torch.testing.assert_close(got.float(), want, atol=scale / 128, rtol=1e-2)
+    if gated is not None:
+        g, u = want[:, :N // 2].double(), want[:, N // 2:].double()
+        want_g = (torch.nn.functional.silu(g) * u).float()
+        torch.testing.assert_close(gated.float(), want_g, atol=max(1.0, want_g.abs().max().item()) / 64,
+                                   rtol=2e-2)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,I,K", [(1, 8192, 2048), (8, 172, 104), (16, 320, 192), (33, 1000, 256),
                                    (8, 8192, 2048), (3, 1001, 4608), (8, 77, 14336),
