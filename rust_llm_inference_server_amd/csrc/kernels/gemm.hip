@@ -9,6 +9,8 @@
 //    for all rows of x; a wave owns 16 (or 32) weight rows and a slice of K, the eight waves of
 //    a workgroup are summed in a fixed order.  K must be a multiple of 8.  A gated variant
 //    fuses the SwiGLU of the feed-forward into the gate/up product.
+//  * gemm_bf16_stream: up to 16 rows of x at the streaming rate of the memory: weights are
+//    loaded row-contiguously and turned into operand layout in LDS.  Plain and gated.
 //
 // In every kernel an output element is a sum over k in an order that depends only on the
 // kernel and K, never on which other rows are in the batch.
@@ -427,195 +429,6 @@ RLIS_API int rlis_gemm_bf16_skinny_swiglu(const void* X, const void* W, void* Y,
   return 0;
 }
 
-// =================================================== row-streaming product (T <= 8)
-// y (T, N) = x (T, K) * W (N, K)^T for up to 8 rows of x, the shape of decode at small batch,
-// where nothing matters but reading W at full memory speed.  A wave streams whole weight rows:
-// one load instruction brings 1 KiB of ONE row, lane l holding the 8 weights at k = kc + 8 l.
-// To reduce over k on the matrix cores the 64 chunks of such a kilobyte are laid out as the
-// operands of v_mfma_f32_16x16x32_bf16: chunk l is row l % 16, k-group l / 16 of A, and the
-// same chunk of a row of x is column l % 16, k-group l / 16 of B.  The product's diagonal
-// C[m][m] is then the dot product of the chunks m, 16 + m, 32 + m, 48 + m of both, and the
-// trace of C, accumulated over the row, is the whole dot product.  The off-diagonal terms are
-// waste the matrix cores have room for: the kernel is bound by memory.
-//
-// x is staged in LDS once per workgroup (and per k-chunk when T * K does not fit); a wave
-// keeps R = 2 rows in flight (gate and up of one column in the gated form) and walks its
-// share of the rows.  Sums run over k in an order fixed by K alone.
-template <typename TC, int TT, bool GATED, int R, int U>
-__global__ __launch_bounds__(256) void gemv_bf16_rows_kernel(const bf16_t* __restrict__ X,
-                                                             const bf16_t* __restrict__ W,
-                                                             TC* __restrict__ Y, int T, int N,
-                                                             int K, long long ldx, long long ldw,
-                                                             long long ldy, int kc_len,
-                                                             int groups_per_wave) {
-  extern __shared__ __attribute__((aligned(16))) bf16_t x_s[];      // TT * kc_len
-  static_assert(!GATED || R % 2 == 0, "gated rows come in gate/up pairs");
-  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-  constexpr int CPG = GATED ? R / 2 : R;                 // output columns per row group
-  const int num_groups = (N + CPG - 1) / CPG;
-  // Waves take row groups in turn (group = round * waves + wave), so that at any moment the
-  // waves of the grid read neighbouring rows and the traffic spreads over all memory channels.
-  const long long my_wave = (long long)blockIdx.x * 4 + wave;
-  const long long num_waves = (long long)gridDim.x * 4;
-  const bool is_diag = ((lane % 16) / 4) == (lane / 16);
-  const int diag_r = lane % 4;
-  const uint4 zero = make_uint4(0, 0, 0, 0);
-  const int num_chunks = (K + kc_len - 1) / kc_len;      // > 1 only with groups_per_wave == 1
-
-  f32x4 acc[R][TT];
-  for (int gi = 0; gi < groups_per_wave; ++gi) {
-    const long long g = gi * num_waves + my_wave;
-    const bool g_valid = g < num_groups;
-    long long rows[R];
-    bool rvalid[R];
-#pragma unroll
-    for (int i = 0; i < R; ++i) {
-      // gated: rows 0 .. CPG-1 are gate rows of the group's columns, CPG .. R-1 their up rows
-      const long long col = g * CPG + (i % CPG);
-      rows[i] = (GATED && i >= CPG) ? col + N : col;
-      rvalid[i] = g_valid && col < N;
-    }
-#pragma unroll
-    for (int i = 0; i < R; ++i)
-#pragma unroll
-      for (int t = 0; t < TT; ++t) acc[i][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
-    for (int ch = 0; ch < num_chunks; ++ch) {
-      const int kbase = ch * kc_len;
-      const int klen = min(kc_len, K - kbase);
-      if (gi == 0 || num_chunks > 1) {
-        // Stage x[:, kbase : kbase + klen] (zero rows beyond T, zero tail up to 512).
-        if (num_chunks > 1 || gi > 0) __syncthreads();
-        const int kpad = ((klen + 511) / 512) * 512;
-        for (int c = tid; c < TT * (kpad / 8); c += 256) {
-          const int t = c / (kpad / 8), kk = (c % (kpad / 8)) * 8;
-          uint4 v = zero;
-          if (t < T && kk < klen) v = *(const uint4*)(X + (long long)t * ldx + kbase + kk);
-          *(uint4*)(x_s + t * kc_len + kk) = v;
-        }
-        __syncthreads();
-      }
-      for (int kk = 0; kk < klen; kk += 512 * U) {
-        Frag8 a[R][U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int k = kk + u * 512 + lane * 8;
-#pragma unroll
-          for (int i = 0; i < R; ++i)
-            a[i][u].u = (rvalid[i] && k < klen) ? *(const uint4*)(W + rows[i] * ldw + kbase + k) : zero;
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int k = kk + u * 512 + lane * 8;
-          if (kk + u * 512 < klen) {
-#pragma unroll
-            for (int t = 0; t < TT; ++t) {
-              Frag8 b;
-              b.u = *(const uint4*)(x_s + t * kc_len + k);
-#pragma unroll
-              for (int i = 0; i < R; ++i)
-                acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i][u].v, b.v, acc[i][t], 0, 0, 0);
-            }
-          }
-        }
-      }
-    }
-    // Trace of every accumulator -> the dot products of this row group.
-    float sums[R][TT];
-#pragma unroll
-    for (int i = 0; i < R; ++i)
-#pragma unroll
-      for (int t = 0; t < TT; ++t) {
-        const f32x4 c = acc[i][t];
-        float v = diag_r == 0 ? c[0] : (diag_r == 1 ? c[1] : (diag_r == 2 ? c[2] : c[3]));
-        sums[i][t] = wave_sum(is_diag ? v : 0.f);
-      }
-    if (lane == 0 && g_valid) {
-#pragma unroll
-      for (int t = 0; t < TT; ++t) {
-        if (t >= T) break;
-        if (GATED) {
-#pragma unroll
-          for (int i = 0; i < CPG; ++i)
-            if (rvalid[i]) {
-              const float gate = sums[i][t];
-              st(Y + (long long)t * ldy + rows[i], gate / (1.0f + expf(-gate)) * sums[CPG + i][t]);
-            }
-        } else {
-#pragma unroll
-          for (int i = 0; i < R; ++i)
-            if (rvalid[i]) st(Y + (long long)t * ldy + rows[i], sums[i][t]);
-        }
-      }
-    }
-  }
-}
-
-template <typename TC, int TT, bool GATED, int R, int U>
-static int launch_gemv_rows(const void* X, const void* W, void* Y, int T, int N, int K,
-                            long long ldx, long long ldw, long long ldy, hipStream_t stream) {
-  // x in LDS: whole K when TT * K * 2 bytes fit into 48 KiB, else k-chunks of a multiple of 512.
-  const int kpad = ceil_div(K, 512) * 512;
-  int kc_len = kpad;
-  const int fit = (48 * 1024 / (TT * 2)) / 512 * 512;
-  if (kc_len > fit) kc_len = fit;
-  const int num_chunks = ceil_div(K, kc_len);
-  constexpr int CPG = GATED ? R / 2 : R;
-  const long long groups = ceil_div(N, CPG);
-  long long blocks = ceil_div_ll(groups, 4);
-  int groups_per_wave = 1;
-  if (num_chunks == 1 && blocks > 2048) {
-    groups_per_wave = (int)ceil_div_ll(groups, 2048 * 4);
-    blocks = ceil_div_ll(groups, (long long)groups_per_wave * 4);
-  }
-  const size_t smem = (size_t)TT * kc_len * sizeof(bf16_t);
-  gemv_bf16_rows_kernel<TC, TT, GATED, R, U><<<(int)blocks, 256, smem, stream>>>(
-      (const bf16_t*)X, (const bf16_t*)W, (TC*)Y, T, N, K, ldx, ldw, ldy, kc_len, groups_per_wave);
-  return 0;
-}
-
-// Rows in flight per wave: four (two k-chunks each) when that still leaves every compute
-// unit several waves, else two.
-template <typename TC, int TT, bool GATED>
-static int pick_gemv_rows(const void* X, const void* W, void* Y, int T, int N, int K,
-                          long long ldx, long long ldw, long long ldy, hipStream_t stream) {
-  constexpr int U = TT <= 4 ? 2 : 1;
-  const long long rows_total = GATED ? 2ll * N : N;
-  if (TT <= 2 && rows_total >= 16384)
-    return launch_gemv_rows<TC, TT, GATED, 4, U>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
-  return launch_gemv_rows<TC, TT, GATED, 2, U>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
-}
-
-template <typename TC, bool GATED>
-static int dispatch_gemv_rows(const void* X, const void* W, void* Y, int T, int N, int K,
-                              long long ldx, long long ldw, long long ldy, hipStream_t stream) {
-  if (T <= 1) return pick_gemv_rows<TC, 1, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
-  if (T <= 2) return pick_gemv_rows<TC, 2, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
-  if (T <= 4) return pick_gemv_rows<TC, 4, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
-  return pick_gemv_rows<TC, 8, GATED>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
-}
-
-// gated == 0: y (T, N) = x W^T.  gated != 0: W is (2N, K) = [Wg; Wu] and
-// y (T, N) = silu(x Wg^T) * (x Wu^T).  T <= 8, bfloat16 operands, K a multiple of 8.
-RLIS_API int rlis_gemv_bf16_rows(const void* X, const void* W, void* Y, int y_dtype, int T, int N,
-                                 int K, long long ldx, long long ldw, long long ldy, int gated,
-                                 hipStream_t stream) {
-  if (check_skinny("gemv_bf16_rows", X, W, T, N, K, ldx, ldw, ldy)) return 1;
-  RLIS_REQUIRE(T <= 8, "gemv_bf16_rows: T=%d rows, at most 8", T);
-  RLIS_REQUIRE(!gated || y_dtype == RLIS_BF16, "gemv_bf16_rows: the gated form stores bfloat16");
-  if (T == 0) return 0;
-  if (gated)
-    dispatch_gemv_rows<bf16_t, true>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
-  else if (y_dtype == RLIS_F32)
-    dispatch_gemv_rows<float, false>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
-  else if (y_dtype == RLIS_BF16)
-    dispatch_gemv_rows<bf16_t, false>(X, W, Y, T, N, K, ldx, ldw, ldy, stream);
-  else
-    RLIS_REQUIRE(false, "gemv_bf16_rows: unknown output dtype %d", y_dtype);
-  RLIS_LAUNCH_CHECK("gemv_bf16_rows");
-  return 0;
-}
-
 // ============================================================ streaming skinny product
 // y (T <= 16, N) = x W^T at the speed of the weight stream.
 //
@@ -649,11 +462,43 @@ struct StreamShape {
   int num_tiles, num_slices;
 };
 
-template <typename TC, bool GATED, int TR /* weight rows per tile: 16 or 8 */>
+// NORM: x is not given but made on the fly as (resid + delta) * norm_weight, and the products
+// are scaled by rsqrt(mean((resid + delta)^2) + eps) of their row at the end, which is the
+// RMSNorm of crates/model/src/layers.rs:103-122 in front of the projection (the scale is one
+// number per row and commutes with the product).  Needs all of K in one slice, so that the
+// workgroup sees whole rows.  Workgroup 0 also stores resid + delta to resid_out.
+struct StreamNorm {
+  const float* resid;        // (rows, K) float32
+  const void* delta;         // null, or `parts` arrays (rows, K), part_stride elements apart
+  int delta_f32, parts;
+  long long part_stride;
+  const void* weight;        // (K)
+  int weight_f32;
+  float eps;
+  const int* rows;           // null, or the row of resid/delta that token t reads
+  float* resid_out;          // null, or where resid + delta goes (not resid itself)
+};
+
+__device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
+  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
+  const uint4 u = *(const uint4*)p;
+  const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = __uint_as_float(w[i] << 16);
+    v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+
+template <typename TC, bool GATED, int TR /* weight rows per tile: 16 or 8 */, bool NORM>
 __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __restrict__ X,
                                                                 const bf16_t* __restrict__ W,
                                                                 TC* __restrict__ Y,
-                                                                const StreamShape sh) {
+                                                                const StreamShape sh,
+                                                                const StreamNorm nm) {
   extern __shared__ __attribute__((aligned(16))) unsigned char stream_smem[];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, nwaves = blockDim.x / 64;
   unsigned char* tile_s = stream_smem + wave * kStreamTileBytes;
@@ -670,15 +515,6 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
   const int kb = item * kStreamItem;
   const int ka = kb + l32 * 8;                          // this lane's k when loading weights
   const bool a_ok = has_item && ka < K;
-
-  Frag8 b[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int k = kb + (4 * j + og) * 8;
-    const bool ok = has_item && oi < T && k < K;
-    const uint4 v = *(const uint4*)(X + (ok ? (long long)oi * sh.ldx + k : 0));
-    b[j].u = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
-  }
 
   // Tile row r = 2 p + half of tile `tile` is weight row tile * rows + r; gated, the first
   // half of a tile's rows are the gate rows of consecutive columns and the second half their
@@ -711,7 +547,86 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
 
   uint4 a[TR / 2];
   int tile = blockIdx.x / sh.num_slices;
-  RLIS_STREAM_LOAD_TILE(a, tile);
+  RLIS_STREAM_LOAD_TILE(a, tile);        // the first tile is on its way during the prologue
+
+  // The rows of x in operand layout: token oi, k = kb + (4 j + og) * 8 .. + 8 for step j.
+  Frag8 b[8];
+  float inv_rms = 1.f;                   // NORM: of token tid / 16, in the threads that store
+  if (!NORM) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int k = kb + (4 * j + og) * 8;
+      const bool ok = has_item && oi < T && k < K;
+      const uint4 v = *(const uint4*)(X + (ok ? (long long)oi * sh.ldx + k : 0));
+      b[j].u = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+    }
+  } else {
+    // Each wave makes its own 16 x 256 item of x: (resid + delta) * norm_weight, rounded to
+    // bfloat16, written to its LDS tile (which the weights use only afterwards) in units of
+    // one token and 8 k, a half wave per token so that the reads are contiguous; then every
+    // lane picks its operand chunks from there.  Sums of squares go per (wave, token) to the
+    // second half of `red`, which the tiles use only after their first barrier.
+    const bool store_sum = nm.resid_out != nullptr && blockIdx.x == 0;
+    float* ss_s = red + nwaves * 256;
+    if (!has_item) {
+      if (lane < 16) ss_s[wave * 16 + lane] = 0.f;
+    } else {
+      for (int u = lane; u < T * 32; u += 64) {
+        const int t = u / 32, c = u % 32;
+        const int k = kb + c * 8;
+        const bool ok = k < K;
+        const long long src = nm.rows ? (long long)nm.rows[t] : (long long)t;
+        const long long at = src * K + (ok ? k : 0);
+        float v[8], d[8], w[8];
+        load8(nm.resid + at, v);
+        if (nm.delta) {
+          for (int s = 0; s < nm.parts; ++s) {
+            if (nm.delta_f32)
+              load8((const float*)nm.delta + s * nm.part_stride + at, d);
+            else
+              load8((const bf16_t*)nm.delta + s * nm.part_stride + at, d);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] += d[e];
+          }
+          if (store_sum && ok) {
+            *(float4*)(nm.resid_out + at) = make_float4(v[0], v[1], v[2], v[3]);
+            *(float4*)(nm.resid_out + at + 4) = make_float4(v[4], v[5], v[6], v[7]);
+          }
+        }
+        if (nm.weight_f32)
+          load8((const float*)nm.weight + (ok ? k : 0), w);
+        else
+          load8((const bf16_t*)nm.weight + (ok ? k : 0), w);
+        float ss = 0.f;
+        Frag8 xw;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float x = ok ? v[e] : 0.f;
+          ss += x * x;
+          xw.v[e] = (__bf16)(x * w[e]);
+        }
+        *(uint4*)(tile_s + t * (kStreamItem * 2) + ((c ^ t) * 16)) = xw.u;
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) ss += __shfl_xor(ss, o, kWave);
+        if (l32 == 0) ss_s[wave * 16 + t] = ss;
+      }
+      wave_lds_fence();
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint4 v = *(const uint4*)(tile_s + oi * (kStreamItem * 2) + (((4 * j + og) ^ oi) * 16));
+        const bool ok = oi < T;
+        b[j].u = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+      }
+      wave_lds_fence();
+    }
+    __syncthreads();
+    if (tid < 256) {
+      float tot = 0.f;
+      for (int w = 0; w < nwaves; ++w) tot += ss_s[w * 16 + tid / 16];
+      inv_rms = 1.0f / sqrtf(tot / (float)K + nm.eps);
+    }
+  }
+
   int par = 0;
   for (; tile < sh.num_tiles; tile += tile_step) {
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -751,6 +666,8 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
             gate += red_p[w * 256 + t * 16 + i];
             up += red_p[w * 256 + t * 16 + h + i];
           }
+          gate *= inv_rms;
+          up *= inv_rms;
           st(y + c, gate / (1.0f + expf(-gate)) * up);
         }
       } else {
@@ -758,7 +675,7 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
         if (i < TR && t < T && n < N) {
           float sum = 0.f;
           for (int w = 0; w < nwaves; ++w) sum += red_p[w * 256 + t * 16 + i];
-          st(y + n, sum);
+          st(y + n, sum * inv_rms);
         }
       }
     }
@@ -772,12 +689,13 @@ static int stream_slices(int K) {
   return ceil_div(ceil_div(K, kStreamItem), kStreamMaxWaves);
 }
 
-template <typename TC, bool GATED, int TR>
-static int launch_stream_tiles(const void* X, const void* W, void* Y, StreamShape sh, int nwaves,
-                               int num_cus, hipStream_t stream) {
+template <typename TC, bool GATED, int TR, bool NORM>
+static int launch_stream_tiles(const void* X, const void* W, void* Y, StreamShape sh,
+                               const StreamNorm& nm, int nwaves, int num_cus,
+                               hipStream_t stream) {
   static bool lds_raised = false;
   if (!lds_raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_stream_kernel<TC, GATED, TR>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_stream_kernel<TC, GATED, TR, NORM>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize,
                                        kStreamMaxWaves * (kStreamTileBytes + 2048));
     RLIS_REQUIRE(e == hipSuccess, "gemm_bf16_stream: cannot raise the LDS limit: %s",
@@ -792,15 +710,16 @@ static int launch_stream_tiles(const void* X, const void* W, void* Y, StreamShap
   long long groups = tiles;                                // workgroups per slice
   const long long cap = max(1, num_cus * per_cu / sh.num_slices);
   if (groups > cap) groups = cap;
-  gemm_bf16_stream_kernel<TC, GATED, TR><<<(int)(groups * sh.num_slices), nwaves * 64, smem, stream>>>(
-      (const bf16_t*)X, (const bf16_t*)W, (TC*)Y, sh);
+  gemm_bf16_stream_kernel<TC, GATED, TR, NORM>
+      <<<(int)(groups * sh.num_slices), nwaves * 64, smem, stream>>>(
+          (const bf16_t*)X, (const bf16_t*)W, (TC*)Y, sh, nm);
   return 0;
 }
 
-template <typename TC, bool GATED>
+template <typename TC, bool GATED, bool NORM>
 static int launch_stream(const void* X, const void* W, void* Y, int T, int N, int K, long long ldx,
                          long long ldw, long long ldy, long long part_stride,
-                         hipStream_t stream) {
+                         const StreamNorm& nm, hipStream_t stream) {
   const int nitems = ceil_div(K, kStreamItem);
   const int slices = stream_slices(K);
   const int nwaves = max(4, ceil_div(nitems, slices));
@@ -820,8 +739,28 @@ static int launch_stream(const void* X, const void* W, void* Y, int T, int N, in
   // Tiles of 8 rows when 16-row tiles would leave compute units without work: a unit draws
   // only its share of the memory bandwidth, however much it has in flight.
   if ((long long)ceil_div(N, GATED ? 8 : 16) * slices < num_cus)
-    return launch_stream_tiles<TC, GATED, 8>(X, W, Y, sh, nwaves, num_cus, stream);
-  return launch_stream_tiles<TC, GATED, 16>(X, W, Y, sh, nwaves, num_cus, stream);
+    return launch_stream_tiles<TC, GATED, 8, NORM>(X, W, Y, sh, nm, nwaves, num_cus, stream);
+  return launch_stream_tiles<TC, GATED, 16, NORM>(X, W, Y, sh, nm, nwaves, num_cus, stream);
+}
+
+template <bool NORM>
+static int dispatch_stream(const char* name, const void* X, const void* W, void* Y, int y_dtype,
+                           int T, int N, int K, long long ldx, long long ldw, long long ldy,
+                           long long part_stride, int gated, const StreamNorm& nm,
+                           hipStream_t stream) {
+  RLIS_REQUIRE(!gated || y_dtype == RLIS_BF16, "%s: the gated form stores bfloat16", name);
+  int rc;
+  if (gated)
+    rc = launch_stream<bf16_t, true, NORM>(X, W, Y, T, N, K, ldx, ldw, ldy, part_stride, nm, stream);
+  else if (y_dtype == RLIS_F32)
+    rc = launch_stream<float, false, NORM>(X, W, Y, T, N, K, ldx, ldw, ldy, part_stride, nm, stream);
+  else if (y_dtype == RLIS_BF16)
+    rc = launch_stream<bf16_t, false, NORM>(X, W, Y, T, N, K, ldx, ldw, ldy, part_stride, nm, stream);
+  else
+    RLIS_REQUIRE(false, "%s: unknown output dtype %d", name, y_dtype);
+  if (rc) return rc;
+  RLIS_LAUNCH_CHECK(name);
+  return 0;
 }
 
 // Slices that rlis_gemm_bf16_stream cuts K into; with more than one, Y receives that many
@@ -839,18 +778,53 @@ RLIS_API int rlis_gemm_bf16_stream(const void* X, const void* W, void* Y, int y_
   RLIS_REQUIRE(slices == 1 || (!gated && y_dtype == RLIS_F32 && part_stride >= (long long)T * ldy),
                "gemm_bf16_stream: K=%d takes %d slices, which need float32 partial results and "
                "no gate", K, slices);
-  RLIS_REQUIRE(!gated || y_dtype == RLIS_BF16, "gemm_bf16_stream: the gated form stores bfloat16");
   if (T == 0) return 0;
-  int rc;
-  if (gated)
-    rc = launch_stream<bf16_t, true>(X, W, Y, T, N, K, ldx, ldw, ldy, part_stride, stream);
-  else if (y_dtype == RLIS_F32)
-    rc = launch_stream<float, false>(X, W, Y, T, N, K, ldx, ldw, ldy, part_stride, stream);
-  else if (y_dtype == RLIS_BF16)
-    rc = launch_stream<bf16_t, false>(X, W, Y, T, N, K, ldx, ldw, ldy, part_stride, stream);
-  else
-    RLIS_REQUIRE(false, "gemm_bf16_stream: unknown output dtype %d", y_dtype);
-  if (rc) return rc;
-  RLIS_LAUNCH_CHECK("gemm_bf16_stream");
-  return 0;
+  StreamNorm nm = {};
+  return dispatch_stream<false>("gemm_bf16_stream", X, W, Y, y_dtype, T, N, K, ldx, ldw, ldy,
+                                part_stride, gated, nm, stream);
+}
+
+// RMSNorm and projection in one pass, for T <= 16 tokens and K <= 4096:
+//   s = resid[row(t)] + sum of the `parts` deltas (delta may be null),
+//   y[t] = (s * rsqrt(mean(s^2) + eps) * norm_weight) W^T   (gated as above),
+// where row(t) = rows[t], or t when rows is null.  resid is (R, K) float32 contiguous; each
+// delta part is shaped like it (bfloat16, or float32 for partial sums), part_stride elements
+// apart.  When resid_out is given (only without rows, and never resid itself: other
+// workgroups still read that), it receives s.  The normalised row is rounded to bfloat16
+// before the scale by rsqrt is applied rather than after; the scale is exact in float32.
+RLIS_API int rlis_norm_linear_bf16(const float* resid, const void* delta, int delta_dtype,
+                                   int parts, long long part_stride, const void* norm_weight,
+                                   int norm_weight_dtype, float eps, const int* rows,
+                                   float* resid_out, const void* W, void* Y, int y_dtype, int T,
+                                   int N, int K, long long ldw, long long ldy, int gated,
+                                   hipStream_t stream) {
+  RLIS_REQUIRE(T >= 0 && T <= 16, "norm_linear: T=%d rows, at most 16", T);
+  RLIS_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && ldw % 8 == 0 && ldw >= K && ldy >= N,
+               "norm_linear: bad sizes N=%d K=%d ldw=%lld ldy=%lld", N, K, ldw, ldy);
+  RLIS_REQUIRE(stream_slices(K) == 1, "norm_linear: K=%d does not fit one k slice", K);
+  RLIS_REQUIRE(((uintptr_t)W % 16) == 0 && ((uintptr_t)resid % 16) == 0 &&
+                   ((uintptr_t)delta % 16) == 0 && ((uintptr_t)norm_weight % 16) == 0 &&
+                   ((uintptr_t)resid_out % 16) == 0,
+               "norm_linear: operands must be 16-byte aligned");
+  RLIS_REQUIRE(!delta || (parts >= 1 && (parts == 1 || delta_dtype == RLIS_F32)),
+               "norm_linear: %d delta parts of dtype %d", parts, delta_dtype);
+  RLIS_REQUIRE(!resid_out || (resid_out != resid && !rows),
+               "norm_linear: resid_out must be another buffer and excludes a row selection");
+  RLIS_REQUIRE((delta_dtype == RLIS_F32 || delta_dtype == RLIS_BF16) &&
+                   (norm_weight_dtype == RLIS_F32 || norm_weight_dtype == RLIS_BF16),
+               "norm_linear: unknown dtypes %d %d", delta_dtype, norm_weight_dtype);
+  if (T == 0) return 0;
+  StreamNorm nm;
+  nm.resid = resid;
+  nm.delta = delta;
+  nm.delta_f32 = delta_dtype == RLIS_F32;
+  nm.parts = delta ? parts : 0;
+  nm.part_stride = part_stride;
+  nm.weight = norm_weight;
+  nm.weight_f32 = norm_weight_dtype == RLIS_F32;
+  nm.eps = eps;
+  nm.rows = rows;
+  nm.resid_out = delta ? resid_out : nullptr;
+  return dispatch_stream<true>("norm_linear", nullptr, W, Y, y_dtype, T, N, K, K, ldw, ldy, 0,
+                               gated, nm, stream);
 }

@@ -14,7 +14,7 @@ from typing import Any, Dict, List, Optional, Sequence, Tuple
 import torch
 
 from ..parts.base import (Block, BuildContext, CacheBinding, CacheRequest, PartSpec,
-                          ResidualStream, TensorSpec, create, tensor_specs)
+                          ResidualStream, TensorSpec, create, normed, tensor_specs)
 
 
 @dataclass
@@ -154,5 +154,4 @@ class Model:
             self.layers[run.layer].forward(stream, step, pools.binding(self.bindings[i]))
         if step.num_logit_rows == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
-        h = self.final_norm.forward_rows(stream, step.logit_rows)
-        return self.head.forward(h)
+        return self.head.forward(normed(self.final_norm, stream, self.head, step.logit_rows))

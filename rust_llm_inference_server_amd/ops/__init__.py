@@ -18,13 +18,10 @@ _DT = {torch.float32: 0, torch.bfloat16: 1}
 
 # bf16 products with at most this many rows of x take the skinny kernel.
 SKINNY_MAX_ROWS = 64
-# ... with at most this many rows the streaming kernel (16 at most; 0 switches it off),
+# ... and with at most this many rows the streaming kernel (16 at most; 0 switches it off).
 STREAM_MAX_ROWS = 16
-# ... and with at most this many rows the row-streaming kernel.
-GEMV_MAX_ROWS = 2
-# ... or this many rows when the weight has at least GEMV_WIDE_N rows (the output head).
-GEMV_MAX_ROWS_WIDE = 4
-GEMV_WIDE_N = 32768
+# The norm in front of a projection goes into the streaming kernel where that applies.
+FUSE_NORM_LINEAR = True
 # "library": bf16 products with more rows and bf16 output go to torch.matmul (hipBLASLt);
 # "own": they take the hand-written matrix-core kernel.
 BF16_GEMM = "library"
@@ -190,11 +187,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     y = torch.empty((T, N), dtype=out_dtype, device=x.device)
     if T == 0:
         return y
-    if bf16 and aligned and (T <= GEMV_MAX_ROWS
-                             or (T <= GEMV_MAX_ROWS_WIDE and N >= GEMV_WIDE_N)):
-        lib.call("rlis_gemv_bf16_rows", x.data_ptr(), w.data_ptr(), y.data_ptr(), _DT[out_dtype],
-                 T, N, K, ldx, ldw, N, 0, stream)
-    elif bf16 and aligned:
+    if bf16 and aligned:
         name = "rlis_gemm_bf16_skinny" if T <= SKINNY_MAX_ROWS else "rlis_gemm_bf16_mfma"
         lib.call(name, x.data_ptr(), w.data_ptr(), y.data_ptr(), _DT[out_dtype], T, N, K, ldx,
                  ldw, N, stream)
@@ -202,6 +195,55 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         lib.call("rlis_gemm_plain", x.data_ptr(), _dt(x), w.data_ptr(), _dt(w), y.data_ptr(),
                  _DT[out_dtype], T, N, K, ldx, ldw, N, stream)
     return y
+
+
+def can_fuse_norm_linear(resid: torch.Tensor, w: torch.Tensor, rows: Optional[int] = None
+                         ) -> bool:
+    """Whether ``norm_linear`` applies: at most 16 rows, a bfloat16 weight over one k slice."""
+    T = resid.shape[0] if rows is None else rows
+    K = resid.shape[1]
+    return (0 < T <= STREAM_MAX_ROWS and FUSE_NORM_LINEAR and w.dtype == torch.bfloat16
+            and w.dim() == 2 and w.shape[1] == K and K % 8 == 0 and w.stride(1) == 1
+            and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0 and stream_slices(K) == 1)
+
+
+def norm_linear(resid: torch.Tensor, delta: Optional[torch.Tensor], norm_weight: torch.Tensor,
+                eps: float, w: torch.Tensor, out_dtype: torch.dtype, gated: bool = False,
+                rows: Optional[torch.Tensor] = None):
+    """RMSNorm of ``resid + delta`` and the product with ``w`` in one kernel (see
+    ``can_fuse_norm_linear``); ``gated`` as ``linear_swiglu``.  Returns ``(y, resid_sum)``:
+    without ``rows``, ``resid_sum`` is ``resid + delta`` in a new tensor (``resid`` itself when
+    there is no delta); with ``rows``, only those rows are produced and ``resid_sum`` is None."""
+    _check(resid, "residual", torch.float32, 2)
+    T, K = resid.shape
+    if not resid.is_contiguous():
+        raise KernelError("norm_linear: residual must be contiguous")
+    parts = 1 if delta is None else _delta_parts(resid, delta, "norm_linear")
+    _check(norm_weight, "norm weight", ndim=1)
+    if norm_weight.numel() != K or not norm_weight.is_contiguous():
+        raise KernelError(f"norm_linear: norm weight has {norm_weight.numel()} entries, rows {K}")
+    ldw = _rows_contig(w, "norm_linear weight")
+    if w.shape[1] != K or w.dtype != torch.bfloat16:
+        raise KernelError("norm_linear: the weight must be bfloat16 (N, K)")
+    N = w.shape[0]
+    if gated:
+        if N % 2:
+            raise KernelError("norm_linear: a gated weight needs an even number of rows")
+        N //= 2
+    if rows is not None:
+        R, rows_ptr, resid_sum = rows.numel(), _i32(rows, "rows"), None
+    else:
+        R, rows_ptr = T, None
+        resid_sum = resid if delta is None else torch.empty_like(resid)
+    y = torch.empty((R, N), dtype=out_dtype, device=resid.device)
+    if R:
+        lib.call("rlis_norm_linear_bf16", resid.data_ptr(),
+                 None if delta is None else delta.data_ptr(), 0 if delta is None else _dt(delta),
+                 parts, T * K, norm_weight.data_ptr(), _dt(norm_weight), float(eps), rows_ptr,
+                 None if (delta is None or rows is not None) else resid_sum.data_ptr(),
+                 w.data_ptr(), y.data_ptr(), _DT[out_dtype], R, N, K, ldw, N, int(bool(gated)),
+                 lib.stream_ptr())
+    return y, resid_sum
 
 
 def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
@@ -225,9 +267,6 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
     if T <= STREAM_MAX_ROWS and stream_slices(K) == 1:
         lib.call("rlis_gemm_bf16_stream", x.data_ptr(), w_gate_up.data_ptr(), y.data_ptr(), 1, T,
                  two_i // 2, K, ldx, ldw, two_i // 2, 0, 1, lib.stream_ptr())
-    elif T <= GEMV_MAX_ROWS:
-        lib.call("rlis_gemv_bf16_rows", x.data_ptr(), w_gate_up.data_ptr(), y.data_ptr(), 1, T,
-                 two_i // 2, K, ldx, ldw, two_i // 2, 1, lib.stream_ptr())
     else:
         lib.call("rlis_gemm_bf16_skinny_swiglu", x.data_ptr(), w_gate_up.data_ptr(), y.data_ptr(),
                  T, two_i // 2, K, ldx, ldw, two_i // 2, lib.stream_ptr())

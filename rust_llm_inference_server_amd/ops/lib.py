@@ -25,8 +25,8 @@ _SIGNATURES = {
     "rlis_gemm_bf16_mfma": [P, P, P, I, I, I, I, L, L, L, P],
     "rlis_gemm_bf16_skinny": [P, P, P, I, I, I, I, L, L, L, P],
     "rlis_gemm_bf16_skinny_swiglu": [P, P, P, I, I, I, L, L, L, P],
-    "rlis_gemv_bf16_rows": [P, P, P, I, I, I, I, L, L, L, I, P],
     "rlis_gemm_bf16_stream": [P, P, P, I, I, I, I, L, L, L, L, I, P],
+    "rlis_norm_linear_bf16": [P, P, I, I, L, P, I, F, P, P, P, P, I, I, I, I, L, L, I, P],
     "rlis_attn_generic": [P, I, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
     "rlis_attn_decode": [P, I, L, P, L, P, P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, P],
     "rlis_attn_decode_mfma": [P, L, P, L, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, P],

@@ -15,7 +15,7 @@ import torch
 
 from .. import ops
 from .base import (BuildContext, CacheBinding, CacheRequest, Mixer, PartSpec, TensorSpec, join,
-                   register)
+                   project, register)
 from .rope import shared_position
 
 
@@ -25,6 +25,7 @@ class PagedAttention(Mixer):
     ``window`` (None: all earlier positions), ``position`` (a PartSpec)."""
 
     graph_safe = True
+    takes_normed_input = True
 
     @classmethod
     def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
@@ -60,9 +61,9 @@ class PagedAttention(Mixer):
     def cache_request(self) -> CacheRequest:
         return CacheRequest(self.num_kv_heads, self.head_dim, self.window)
 
-    def forward(self, x: torch.Tensor, step: Any, binding: CacheBinding) -> torch.Tensor:
+    def forward(self, x: Any, step: Any, binding: CacheBinding) -> torch.Tensor:
         group = step.groups[binding.group]
-        qkv = ops.linear(x, self.w_qkv, self.act_dtype)
+        qkv = project(x, self.w_qkv, self.act_dtype)
         if step.max_context > self.position.max_positions:
             raise ValueError(f"sequence of {step.max_context} positions exceeds max_seq_len "
                              f"{self.position.max_positions}")

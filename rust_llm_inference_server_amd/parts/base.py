@@ -156,6 +156,55 @@ class Norm(Part):
     def forward_rows(self, stream: "ResidualStream", rows: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 
+    def fused_linear(self, stream: "ResidualStream", w: torch.Tensor, out_dtype: torch.dtype,
+                     gated: bool, rows: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+        """The norm and the projection behind it in one kernel: ``norm(stream) @ w.T`` (gated:
+        ``silu(. @ Wg.T) * (. @ Wu.T)`` for ``w = [Wg; Wu]``), with the effects of ``forward``
+        (or ``forward_rows``) on the stream.  None when this norm has no such kernel for these
+        operands; the caller then applies the norm and the projection one after the other."""
+        return None
+
+
+class NormedInput:
+    """A norm that has not been applied yet, handed to a part that sets ``takes_normed_input``
+    in place of the normalised activations, so that the part's first projection can take the
+    norm into its kernel.  ``tensor()`` applies the norm now; ``linear(w, ...)`` is the
+    projection of the normalised activations."""
+
+    __slots__ = ("norm", "stream", "rows")
+
+    def __init__(self, norm: Norm, stream: "ResidualStream", rows: Optional[torch.Tensor] = None):
+        self.norm, self.stream, self.rows = norm, stream, rows
+
+    def tensor(self) -> torch.Tensor:
+        if self.rows is None:
+            return self.norm.forward(self.stream)
+        return self.norm.forward_rows(self.stream, self.rows)
+
+    def linear(self, w: torch.Tensor, out_dtype: torch.dtype, gated: bool = False) -> torch.Tensor:
+        y = self.norm.fused_linear(self.stream, w, out_dtype, gated, self.rows)
+        if y is None:
+            from .. import ops
+            x = self.tensor()
+            y = ops.linear_swiglu(x, w) if gated else ops.linear(x, w, out_dtype)
+        return y
+
+
+def project(x: Any, w: torch.Tensor, out_dtype: torch.dtype, gated: bool = False) -> torch.Tensor:
+    """``x @ w.T`` (or the gated form) for activations ``x`` or a ``NormedInput``."""
+    if isinstance(x, NormedInput):
+        return x.linear(w, out_dtype, gated)
+    from .. import ops
+    return ops.linear_swiglu(x, w) if gated else ops.linear(x, w, out_dtype)
+
+
+def normed(norm: Norm, stream: "ResidualStream", consumer: Part,
+           rows: Optional[torch.Tensor] = None) -> Any:
+    """What ``consumer`` gets from ``norm``: the norm itself, unapplied, when it asks for that."""
+    if getattr(consumer, "takes_normed_input", False):
+        return NormedInput(norm, stream, rows)
+    return norm.forward(stream) if rows is None else norm.forward_rows(stream, rows)
+
 
 class PositionEncoding(Part):
     """Built once per distinct parameter set and shared by the mixers that name it."""
@@ -174,6 +223,8 @@ class Mixer(Part):
     # True when forward launches only device work that reads the step's device tensors, so
     # that a decode step may be captured into a HIP graph and replayed with new metadata.
     graph_safe = False
+    # True when forward takes ``x`` as a NormedInput (and projects it with ``project``).
+    takes_normed_input = False
 
     def cache_request(self) -> Optional[CacheRequest]:
         return None
@@ -188,6 +239,8 @@ class Mixer(Part):
 class FeedForward(Part):
     """``forward(x, step)`` maps activations ``(T, H)`` to ``(T, H)``, row by row (or to a
     stack of float32 partial sums of that, as a mixer may)."""
+
+    takes_normed_input = False       # as for a mixer
 
     def forward(self, x: torch.Tensor, step: Any) -> torch.Tensor:
         raise NotImplementedError
@@ -209,6 +262,8 @@ class Embedding(Part):
 
 
 class Head(Part):
+    takes_normed_input = False       # as for a mixer
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """Normalised rows ``(R, H)`` -> logits ``(R, V)`` float32."""
         raise NotImplementedError

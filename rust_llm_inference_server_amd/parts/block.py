@@ -6,7 +6,7 @@ from __future__ import annotations
 from typing import Any, Dict, List
 
 from .base import (Block, BuildContext, CacheBinding, PartSpec, ResidualStream, TensorSpec,
-                   create, join, register, tensor_specs)
+                   create, join, normed, register, tensor_specs)
 
 
 @register("block", "prenorm")
@@ -32,5 +32,6 @@ class PreNormBlock(Block):
         self.ffn_norm, self.feed_forward = built["ffn_norm"], built["feed_forward"]
 
     def forward(self, stream: ResidualStream, step: Any, binding: CacheBinding) -> None:
-        stream.add(self.mixer.forward(self.mixer_norm.forward(stream), step, binding))
-        stream.add(self.feed_forward.forward(self.ffn_norm.forward(stream), step))
+        stream.add(self.mixer.forward(normed(self.mixer_norm, stream, self.mixer), step, binding))
+        stream.add(self.feed_forward.forward(normed(self.ffn_norm, stream, self.feed_forward),
+                                             step))

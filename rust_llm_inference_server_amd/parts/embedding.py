@@ -11,7 +11,7 @@ from typing import Any, Dict, List
 import torch
 
 from .. import ops
-from .base import BuildContext, Embedding, Head, TensorSpec, join, register
+from .base import BuildContext, Embedding, Head, TensorSpec, join, project, register
 
 
 @register("embedding", "token")
@@ -36,6 +36,8 @@ class LinearHead(Head):
     """Parameters: ``vocab_size``, ``hidden_size``, ``tied_to`` (name of the tensor to share,
     or None for a weight of its own at ``prefix.weight``)."""
 
+    takes_normed_input = True
+
     @classmethod
     def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
         if params.get("tied_to"):
@@ -46,5 +48,5 @@ class LinearHead(Head):
         super().__init__(params, prefix, ctx)
         self.weight = ctx.take(params.get("tied_to") or join(prefix, "weight"))
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return ops.linear(x, self.weight, torch.float32)
+    def forward(self, x: Any) -> torch.Tensor:
+        return project(x, self.weight, torch.float32)

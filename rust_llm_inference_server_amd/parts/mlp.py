@@ -8,12 +8,14 @@ from typing import Any, Dict, List
 import torch
 
 from .. import ops
-from .base import BuildContext, FeedForward, TensorSpec, join, register
+from .base import BuildContext, FeedForward, TensorSpec, join, project, register
 
 
 @register("feed_forward", "swiglu")
 class SwiGLU(FeedForward):
     """Parameters: ``hidden_size``, ``intermediate_size``."""
+
+    takes_normed_input = True
 
     @classmethod
     def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
@@ -33,6 +35,6 @@ class SwiGLU(FeedForward):
         self.w_down = ctx.take(join(prefix, "down_proj.weight"))
         self.act_dtype = ctx.act_dtype
 
-    def forward(self, x: torch.Tensor, step: Any) -> torch.Tensor:
-        return ops.linear(ops.linear_swiglu(x, self.w_gate_up), self.w_down, self.act_dtype,
-                          partials=True)
+    def forward(self, x: Any, step: Any) -> torch.Tensor:
+        hidden = project(x, self.w_gate_up, self.act_dtype, gated=True)
+        return ops.linear(hidden, self.w_down, self.act_dtype, partials=True)

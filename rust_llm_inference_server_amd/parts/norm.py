@@ -3,7 +3,7 @@ directly, not as ``1 + w`` (crates/model/src/layers.rs:103-122, 141-146).  The i
 32-bit residual stream; statistics and both multiplies are 32-bit, one rounding at the store."""
 from __future__ import annotations
 
-from typing import Any, Dict, List
+from typing import Any, Dict, List, Optional
 
 import torch
 
@@ -32,3 +32,14 @@ class RMSNorm(Norm):
     def forward_rows(self, stream: ResidualStream, rows: torch.Tensor) -> torch.Tensor:
         return ops.add_rmsnorm(stream.x, stream.pending, self.weight, self.eps, self.out_dtype,
                                rows=rows)
+
+    def fused_linear(self, stream: ResidualStream, w: torch.Tensor, out_dtype: torch.dtype,
+                     gated: bool, rows: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+        count = stream.x.shape[0] if rows is None else rows.numel()
+        if self.out_dtype != torch.bfloat16 or not ops.can_fuse_norm_linear(stream.x, w, count):
+            return None
+        y, total = ops.norm_linear(stream.x, stream.pending, self.weight, self.eps, w, out_dtype,
+                                   gated=gated, rows=rows)
+        if rows is None:
+            stream.x, stream.pending = total, None
+        return y

@@ -46,6 +46,10 @@ def linear_swiglu(x, w_gate_up):
     return swiglu(linear(x, w_gate_up, x.dtype))
 
 
+def can_fuse_norm_linear(resid, w, rows=None):
+    return False
+
+
 def rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, cos, sin, positions, slots, k_pages,
                   v_pages, page_size, write_kv=True):
     T = qkv.shape[0]
@@ -133,7 +137,7 @@ def install(monkeypatch) -> None:
     import rust_llm_inference_server_amd.ops as ops
     import rust_llm_inference_server_amd.engine.runner as runner
     for name in ("embed", "add_residual", "add_rmsnorm", "swiglu", "linear", "linear_swiglu",
-                 "rope_kv_write",
+                 "can_fuse_norm_linear", "rope_kv_write",
                  "copy_pages", "decode_splits", "paged_attention", "sample_rows"):
         monkeypatch.setattr(ops, name, globals()[name])
     monkeypatch.setattr(runner, "default_device", lambda: torch.device("cpu"))

@@ -137,13 +137,13 @@ def test_linear_bfloat16(ops, out_dtype, T, N, K):
         torch.testing.assert_close(got, want, atol=2e-5 * max(1.0, scale) * math.sqrt(K / 64), rtol=1e-4)
     else:
         torch.testing.assert_close(got.float(), want, atol=scale / 128, rtol=1e-2)
-    old = ops.BF16_GEMM, ops.GEMV_MAX_ROWS
+    old = ops.BF16_GEMM, ops.STREAM_MAX_ROWS
     try:
         ops.BF16_GEMM = "own"
-        ops.GEMV_MAX_ROWS = 0 if T <= old[1] else 8       # the other kernel for this many rows
+        ops.STREAM_MAX_ROWS = 0                           # the other kernel for few rows
         got2 = ops.linear(x, w, out_dtype)
     finally:
-        ops.BF16_GEMM, ops.GEMV_MAX_ROWS = old
+        ops.BF16_GEMM, ops.STREAM_MAX_ROWS = old
     torch.testing.assert_close(got2.float(), got.float(), atol=scale / 128, rtol=1e-2)
 
 
@@ -183,6 +183,56 @@ def test_linear_streaming_kernel(ops, out_dtype, T, N, K):
                                    rtol=2e-2)
 
 
+@pytest.mark.parametrize("T,N,K,parts,rows", [(1, 2048, 2048, 0, False), (8, 3072, 2048, 1, False),
+                                              (16, 344, 104, 2, False), (5, 1001, 4096, 1, False),
+                                              (3, 128256, 256, 1, True), (7, 64, 776, 3, True),
+                                              (8, 16384, 2048, 1, False)])
+@pytest.mark.parametrize("norm_dtype", DTYPES, ids=["normw32", "normw16"])
+def test_norm_linear(ops, T, N, K, parts, rows, norm_dtype):
+    """RMSNorm fused into the streaming product, plain and gated, float32 and bfloat16 output:
+    no delta, a bfloat16 delta, float32 partial sums; a row selection; the summed residual that
+    comes back.  Against float64 formulas; the norm weight is far from one so that leaving it
+    out, or applying it after the product, would show."""
+    total = T + 5 if rows else T
+    resid = rnd(total, K, seed=1, scale=3.0)
+    if parts == 0:
+        delta = None
+    elif parts == 1:
+        delta = rnd(total, K, dtype=torch.bfloat16, seed=2)
+    else:
+        delta = rnd(parts, total, K, seed=2)
+    nw = (rnd(K, seed=3).abs() + 0.5).to(norm_dtype)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=4, scale=0.05)
+    sel = torch.tensor([(3 * i + 1) % total for i in range(T)], dtype=torch.int32, device=DEV) if rows else None
+    eps = 1e-5
+    s = resid.double()
+    if delta is not None:
+        s = s + (delta.double() if parts == 1 else delta.double().sum(0))
+    src = s if sel is None else s[sel.long()]
+    normed = src / torch.sqrt((src * src).mean(-1, keepdim=True) + eps) * nw.double()
+    want = normed @ w.double().t()
+    assert ops.can_fuse_norm_linear(resid, w, T)
+    resid_before = resid.clone()
+    for out_dtype in (torch.float32, torch.bfloat16):
+        got, total_out = ops.norm_linear(resid, delta, nw, eps, w, out_dtype, rows=sel)
+        assert got.dtype == out_dtype and got.shape == (T, N)
+        scale = max(1.0, want.abs().max().item())
+        torch.testing.assert_close(got.double(), want, atol=scale / 64, rtol=2e-2)
+        assert torch.equal(resid, resid_before)              # the input residual is left alone
+        if sel is not None:
+            assert total_out is None
+        elif delta is None:
+            assert total_out is resid
+        else:
+            torch.testing.assert_close(total_out.double(), s, atol=1e-5, rtol=1e-6)
+    if N % 2 == 0:
+        got, _ = ops.norm_linear(resid, delta, nw, eps, w, torch.bfloat16, gated=True, rows=sel)
+        g, u = want[:, :N // 2], want[:, N // 2:]
+        want_g = torch.nn.functional.silu(g) * u
+        torch.testing.assert_close(got.double(), want_g, atol=max(1.0, want_g.abs().max().item()) / 32,
+                                   rtol=3e-2)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,I,K", [(1, 8192, 2048), (8, 172, 104), (16, 320, 192), (33, 1000, 256),
                                    (8, 8192, 2048), (3, 1001, 4608), (8, 77, 14336),
@@ -197,12 +247,12 @@ def test_linear_swiglu(ops, dtype, T, I, K):
     want = (torch.nn.functional.silu(g) * u).float()
     got = ops.linear_swiglu(x, w)
     assert got.dtype == dtype and got.shape == (T, I)
-    old = ops.GEMV_MAX_ROWS
+    old = ops.STREAM_MAX_ROWS
     try:
-        ops.GEMV_MAX_ROWS = 0 if T <= old else 8              # the other kernel for this many rows
+        ops.STREAM_MAX_ROWS = 0                               # the other kernel for few rows
         other = ops.linear_swiglu(x, w)
     finally:
-        ops.GEMV_MAX_ROWS = old
+        ops.STREAM_MAX_ROWS = old
     torch.testing.assert_close(other.float(), got.float(), atol=0.05, rtol=2e-2)
     scale = max(1.0, want.abs().max().item())
     if dtype == torch.float32:
