@@ -439,8 +439,17 @@ def sample_rows(logits: torch.Tensor, keys: torch.Tensor, inv_temps: torch.Tenso
     R, V = logits.shape
     _check(inv_temps, "inv_temps", torch.float32)
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    # A large vocabulary is scanned in chunks by many workgroups and a second small kernel
+    # picks among the chunks' winners; the result is the same token.
+    chunks = min(64, max(1, V // 1024))
+    best = idx = None
+    if chunks > 1:
+        best = torch.empty((R, chunks), dtype=torch.float32, device=logits.device)
+        idx = torch.empty((R, chunks), dtype=torch.int32, device=logits.device)
     lib.call("rlis_sample_rows", logits.data_ptr(), stride, R, V, _i32(keys, "keys", R),
-             inv_temps.data_ptr(), out.data_ptr(), lib.stream_ptr())
+             inv_temps.data_ptr(), out.data_ptr(), chunks,
+             None if best is None else best.data_ptr(), None if idx is None else idx.data_ptr(),
+             lib.stream_ptr())
     return out
 
 

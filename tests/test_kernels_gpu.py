@@ -515,6 +515,13 @@ def test_sample_rows_greedy_and_ties(ops):
     big = rnd(5, 128256, seed=3)
     got = ops.sample_rows(big, torch.zeros(5, dtype=torch.int32, device=DEV), torch.zeros(5, device=DEV))
     assert got.tolist() == big.argmax(dim=-1).tolist()
+    # a vocabulary scanned in chunks: equal maxima in different chunks, and a row of -inf
+    wide = torch.full((3, 70001), -1.0, device=DEV)
+    wide[0, 69999] = wide[0, 1234] = wide[0, 40000] = 2.0
+    wide[1, 70000] = 0.5
+    wide[2] = float("-inf")
+    zi, zf = torch.zeros(3, dtype=torch.int32, device=DEV), torch.zeros(3, device=DEV)
+    assert ops.sample_rows(wide, zi, zf).tolist() == [1234, 70000, 0]
 
 
 def test_sample_rows_temperature_matches_host_reference(ops):
