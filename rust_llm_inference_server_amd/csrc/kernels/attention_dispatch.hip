@@ -17,7 +17,7 @@ DECL(32) DECL(64) DECL(96) DECL(128) DECL(160) DECL(192) DECL(224) DECL(256)
       const void* q, long long q_stride, void* out, long long out_stride, float* part_ml,      \
       float* part_acc, const void* k_pages, const void* v_pages, const int* block_tables,      \
       int max_pages, const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift,       \
-      int window, float scale, int splits, hipStream_t stream);
+      int window, float scale, int splits, const DecodeRope* rope, hipStream_t stream);
 DECL(32) DECL(64) DECL(96) DECL(128) DECL(160) DECL(192) DECL(224) DECL(256)
 #undef DECL
 
@@ -64,12 +64,36 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
 // One query token per sequence (bfloat16): q rows are the sequences themselves.  Needs at most
 // 16 query heads per KV head; part_ml (S, nh, splits, 2) and part_acc (S, nh, splits, d) float32
 // when splits > 1.
+//
+// positions == null: q is rotated and the pages hold the step's keys and values already.
+// Otherwise the kernel does that itself: q rows hold the k heads at column k_off and the v
+// heads at v_off; with cos/sin (float32 (max positions, rot / 2), rot = d = 64, 128 or 256) q
+// and the new k are rotated by positions[s], without them nothing is; with slots the new k and
+// v go to the pages at slots[s] (page * page_size + offset).
 RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
                                    long long out_stride, float* part_ml, float* part_acc,
-                                   const void* k_pages, const void* v_pages,
+                                   void* k_pages, void* v_pages,
                                    const int* block_tables, int max_pages, const int* ctx_lens,
                                    int S, int nh, int nkv, int d, int page_size, int window,
-                                   float scale, int splits, hipStream_t stream) {
+                                   float scale, int splits, const float* cos, const float* sin,
+                                   int rot, const int* positions, const int* slots,
+                                   long long k_off, long long v_off, hipStream_t stream) {
+  DecodeRope rope;
+  rope.cos = positions ? cos : nullptr;
+  rope.sin = positions ? sin : nullptr;
+  rope.positions = positions;
+  rope.slots = positions ? slots : nullptr;
+  rope.k_off = k_off;
+  rope.v_off = v_off;
+  rope.rot = rot;
+  RLIS_REQUIRE(!rope.cos || (sin && rot % 2 == 0 && ((uintptr_t)cos % 16) == 0 &&
+                             ((uintptr_t)sin % 16) == 0),
+               "attn_decode_mfma: rotation needs cos and sin tables, 16-byte aligned");
+  RLIS_REQUIRE(!rope.slots || (k_off >= (long long)nh * d && v_off >= 0 &&
+                               k_off + (long long)nkv * d <= q_stride &&
+                               v_off + (long long)nkv * d <= q_stride),
+               "attn_decode_mfma: k and v columns %lld, %lld do not fit rows of %lld", k_off,
+               v_off, q_stride);
   RLIS_REQUIRE(S >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0, "attn_decode_mfma: bad sizes");
   RLIS_REQUIRE(nh % nkv == 0 && nh / nkv <= 16,
                "attn_decode_mfma: %d query heads per KV head, at most 16", nkv ? nh / nkv : 0);
@@ -91,7 +115,7 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
 #define CALL(D)                                                                                 \
   rc = rlis_attn_decode_mfma_d##D(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,     \
                                   v_pages, block_tables, max_pages, ctx_lens, S, nh, nkv, d,    \
-                                  page_shift, window, scale, splits, stream)
+                                  page_shift, window, scale, splits, &rope, stream)
   if (d <= 32) CALL(32);
   else if (d <= 64) CALL(64);
   else if (d <= 96) CALL(96);

@@ -324,7 +324,20 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
 // lo32 = lo rounded down to 32, partition s covers [lo32 + s * part, lo32 + (s + 1) * part)
 // cut to [lo, ctx), part = ceil((ctx - lo32) / splits) rounded up to 256.  Page ids of a chunk
 // are fetched one chunk ahead of its keys and values, which are fetched one chunk ahead of use.
+//
+// With rope.positions the kernel also does what rope_kv_write does for the step's own tokens
+// (crates/model/src/llama.rs:205-222): every workgroup rotates its queries in registers
+// (rotate-half over the whole head, which must be as wide as this unit: the partner of a dim
+// is then in the same lane), and the workgroup whose partition holds the new key rotates it
+// and stores it and the new value to the pages before it reads them back.
 #define DECODE_KERNEL_NAME RLIS_CAT(rlis_attn_decode_mfma_kernel_d, RLIS_HEAD_DIM)
+
+namespace {
+__device__ __forceinline__ void load8f(const float* p, float (&v)[8]) {
+  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+}  // namespace
 
 constexpr int kDecodeWaves = 8;
 
@@ -333,7 +346,8 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
     long long out_stride, float* __restrict__ part_ml, float* __restrict__ part_acc,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ ctx_lens,
-    int nh, int nkv, int d, int page_shift, float scale, int window, int splits) {
+    int nh, int nkv, int d, int page_shift, float scale, int window, int splits,
+    const DecodeRope rope) {
   extern __shared__ float dsm[];           // ml: waves * g * 2 ; acc: waves * g * d
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int l16 = lane % 16, lq = lane / 16;
@@ -350,14 +364,60 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
   const int kbeg = lo32 + split * part;
   const int kend = min(ctx, kbeg + part);
 
+  const int pos = rope.positions ? rope.positions[seq] : 0;
+  if (rope.positions && rope.slots && kbeg < ctx && kend == ctx) {
+    // This workgroup's partition ends with the step's own key.
+    const int slot = rope.slots[seq];
+    if (slot >= 0) {
+      const long long page = slot >> page_shift;
+      const int off = slot & page_mask;
+      const bf16_t* krow = q + (long long)seq * q_stride + rope.k_off + kvh * d;
+      const bf16_t* vrow = q + (long long)seq * q_stride + rope.v_off + kvh * d;
+      bf16_t* kdst = const_cast<bf16_t*>(k_pages) + (((page * nkv + kvh) << page_shift) + off) * d;
+      bf16_t* vdst = const_cast<bf16_t*>(v_pages) + (((page * nkv + kvh) * d) << page_shift) + off;
+      const int half = rope.rot / 2;
+      for (int i = tid; i < d; i += 64 * kDecodeWaves) {
+        bf16_t kv = krow[i];
+        if (rope.cos && i < rope.rot) {
+          const int j = i < half ? i : i - half;
+          const float c = rope.cos[(long long)pos * half + j], s = rope.sin[(long long)pos * half + j];
+          const float x = bf16_to_f32(kv);
+          const float y = bf16_to_f32(i < half ? krow[i + half] : krow[i - half]);
+          kv = f32_to_bf16(i < half ? x * c - y * s : x * c + y * s);
+        }
+        kdst[i] = kv;
+        vdst[(long long)i << page_shift] = vrow[i];
+      }
+    }
+    __syncthreads();       // the stores are visible to the whole workgroup from here on
+  }
+
   Frag8 qf[D / 32];
 #pragma unroll
   for (int ks = 0; ks < D / 32; ++ks) {
     const int dim = ks * 32 + lq * 8;
-    if (l16 < g && dim < d)
-      qf[ks].u = *(const uint4*)(q + (long long)seq * q_stride + (kvh * g + l16) * d + dim);
-    else
-      qf[ks].u = make_uint4(0, 0, 0, 0);
+    const bool ok = l16 < g && dim < d;
+    const uint4 v = *(const uint4*)(q + (long long)seq * q_stride + (ok ? (kvh * g + l16) * d + dim : 0));
+    qf[ks].u = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+  }
+  if constexpr (D % 64 == 0) {
+    if (rope.positions && rope.cos) {         // the dispatcher has checked rot == d == D
+      constexpr int HS = D / 64;              // fragments between a dim and its partner
+      const float* cs = rope.cos + (long long)pos * (D / 2);
+      const float* sn = rope.sin + (long long)pos * (D / 2);
+#pragma unroll
+      for (int ks = 0; ks < HS; ++ks) {
+        float c[8], s[8];
+        load8f(cs + ks * 32 + lq * 8, c);
+        load8f(sn + ks * 32 + lq * 8, s);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float x1 = (float)qf[ks].v[e], x2 = (float)qf[ks + HS].v[e];
+          qf[ks].v[e] = (__bf16)(x1 * c[e] - x2 * s[e]);
+          qf[ks + HS].v[e] = (__bf16)(x2 * c[e] + x1 * s[e]);
+        }
+      }
+    }
   }
   float m_run = -INFINITY, l_run = 0.f;
   f32x4 o_acc[D / 16];
@@ -523,15 +583,18 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
     const void* q, long long q_stride, void* out, long long out_stride, float* part_ml,
     float* part_acc, const void* k_pages, const void* v_pages, const int* block_tables,
     int max_pages, const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift, int window,
-    float scale, int splits, hipStream_t stream) {
+    float scale, int splits, const DecodeRope* rope, hipStream_t stream) {
   if (S == 0) return 0;
+  RLIS_REQUIRE(!(rope->positions && rope->cos) || (D % 64 == 0 && rope->rot == D && d == D),
+               "attn_decode_mfma: rotation inside the kernel needs head_dim = rotated width = "
+               "64, 128 or 256 (got %d, %d)", d, rope->rot);
   const int g = nh / nkv;
   dim3 grid(nkv, S, splits);
   const size_t smem = (size_t)kDecodeWaves * g * (2 + d) * sizeof(float);
   DECODE_KERNEL_NAME<<<grid, 64 * kDecodeWaves, smem, stream>>>(
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, part_ml, part_acc,
       (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, max_pages, ctx_lens, nh, nkv, d,
-      page_shift, scale, window, splits);
+      page_shift, scale, window, splits, *rope);
   RLIS_LAUNCH_CHECK("attn_decode_mfma");
   return 0;
 }

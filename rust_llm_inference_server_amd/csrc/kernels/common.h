@@ -80,5 +80,17 @@ void rlis_set_error(const char* fmt, ...);
     }                                                                        \
   } while (0)
 
+// Rotation and cache write of a decode step's own tokens, when the decode attention kernel
+// does them itself: q rows are (q heads | ... k heads at k_off | ... v heads at v_off).
+struct DecodeRope {
+  const float* cos;       // (max positions, rot / 2) float32; null: nothing is rotated
+  const float* sin;
+  const int* positions;   // (S) position of each sequence's token; null: q comes rotated and
+                          // K, V are in the pages already
+  const int* slots;       // (S) page * page_size + offset of the new key; null: no cache write
+  long long k_off, v_off;
+  int rot;                // rotated width of a head
+};
+
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 static inline long long ceil_div_ll(long long a, long long b) { return (a + b - 1) / b; }

@@ -22,6 +22,8 @@ SKINNY_MAX_ROWS = 64
 STREAM_MAX_ROWS = 16
 # The norm in front of a projection goes into the streaming kernel where that applies.
 FUSE_NORM_LINEAR = True
+# The matrix-core decode attention rotates q and k and stores the new k, v itself where it can.
+FUSE_ROPE_DECODE = True
 # "library": bf16 products with more rows and bf16 output go to torch.matmul (hipBLASLt);
 # "own": they take the hand-written matrix-core kernel.
 BF16_GEMM = "library"
@@ -338,10 +340,63 @@ def decode_splits(num_seqs: int, num_kv_heads: int, group: int, max_context: int
     return max(1, min(math.ceil(512 / pairs), math.ceil(max_context / 256)))
 
 
+def _attention_kernel(qkv: torch.Tensor, nh: int, nkv: int, d: int, page_size: int, step,
+                      force: Optional[str]):
+    """(kind, matrix_decode): which attention kernel a batch takes."""
+    q_stride = qkv.stride(0)
+    kind = force or FORCE_ATTENTION
+    if kind is None:
+        if step.all_decode and d % 8 == 0 and d <= 256 and (nh // nkv) * d <= 2048:
+            kind = "decode"
+        elif (qkv.dtype == torch.bfloat16 and d % 16 == 0 and d <= 256 and page_size >= 8
+              and page_size & (page_size - 1) == 0 and q_stride % 8 == 0
+              and not step.all_decode):
+            kind = "prefill"
+        else:
+            kind = "generic"
+    g = nh // nkv
+    mfma = (kind == "decode" and qkv.dtype == torch.bfloat16 and d % 16 == 0 and g <= 16
+            and g * (d + 2) * 32 <= 65536
+            and page_size >= 8 and page_size & (page_size - 1) == 0 and q_stride % 8 == 0
+            and DECODE_ATTENTION != "vector")
+    return kind, mfma
+
+
+def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                   cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                   positions: torch.Tensor, slots: Optional[torch.Tensor],
+                   k_pages: torch.Tensor, v_pages: torch.Tensor, page_size: int,
+                   block_tables: torch.Tensor, step, scale: float,
+                   window: Optional[int] = None, write_kv: bool = True) -> torch.Tensor:
+    """``rope_kv_write`` followed by ``paged_attention``.  A decode batch that takes the
+    matrix-core decode kernel does both in that kernel when the whole head is rotated and is
+    64, 128 or 256 wide (or nothing is rotated); ``qkv`` is then left unrotated."""
+    nh, nkv, d = num_heads, num_kv_heads, head_dim
+    _rows_contig(qkv, "qkv")
+    kind, mfma = _attention_kernel(qkv, nh, nkv, d, page_size, step, None)
+    fusable = cos is None or (2 * cos.shape[1] == d and d in (64, 128, 256))
+    if mfma and fusable and FUSE_ROPE_DECODE and qkv.shape[1] == (nh + 2 * nkv) * d:
+        if cos is not None:
+            _check(cos, "cos", torch.float32, 2)
+            _check(sin, "sin", torch.float32, 2)
+            if cos.shape != sin.shape or not (cos.is_contiguous() and sin.is_contiguous()):
+                raise KernelError("rope_attention: cos and sin must match and be contiguous")
+        if write_kv and slots is None:
+            raise KernelError("rope_attention: a cache write needs slots")
+        return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
+                               scale, window,
+                               rope=(cos, sin, positions, slots if write_kv else None))
+    rope_kv_write(qkv, nh, nkv, d, cos, sin, positions, slots, k_pages, v_pages, page_size,
+                  write_kv=write_kv)
+    return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
+                           scale, window)
+
+
 def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                     k_pages: torch.Tensor, v_pages: torch.Tensor, page_size: int,
                     block_tables: torch.Tensor, step, scale: float,
-                    window: Optional[int] = None, force: Optional[str] = None) -> torch.Tensor:
+                    window: Optional[int] = None, force: Optional[str] = None,
+                    rope: Optional[tuple] = None) -> torch.Tensor:
     """Attention of the step's new tokens over the paged cache -> ``(T, nh * d)``.
 
     ``qkv`` holds the rotated queries in its first ``nh * d`` columns; K and V of the new
@@ -349,7 +404,9 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     metadata on the device).  The kernel is chosen from the shape of the batch: every
     sequence brings one token -> decode kernel; bfloat16 with multi-token sequences ->
     matrix-core prefill kernel; float32, or sizes those kernels refuse -> generic kernel.
-    ``force`` names one of 'generic', 'decode', 'prefill' for tests."""
+    ``force`` names one of 'generic', 'decode', 'prefill' for tests.  ``rope`` (from
+    ``rope_attention`` only): ``(cos, sin, positions, slots)`` for the matrix-core decode kernel
+    to rotate and store the step's tokens itself."""
     q_stride = _rows_contig(qkv, "qkv")
     T = qkv.shape[0]
     nh, nkv, d = num_heads, num_kv_heads, head_dim
@@ -374,16 +431,9 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     win = int(window) if window else 0
     out = torch.empty((T, nh * d), dtype=qkv.dtype, device=qkv.device)
     stream = lib.stream_ptr()
-    kind = force or FORCE_ATTENTION
-    if kind is None:
-        if step.all_decode and d % 8 == 0 and d <= 256 and (nh // nkv) * d <= 2048:
-            kind = "decode"
-        elif (qkv.dtype == torch.bfloat16 and d % 16 == 0 and d <= 256 and page_size >= 8
-              and page_size & (page_size - 1) == 0 and q_stride % 8 == 0
-              and not step.all_decode):
-            kind = "prefill"
-        else:
-            kind = "generic"
+    kind, mfma = _attention_kernel(qkv, nh, nkv, d, page_size, step, force)
+    if rope is not None and not mfma:
+        raise KernelError("attention: only the matrix-core decode kernel rotates and stores")
     if kind == "decode":
         if not step.all_decode:
             raise KernelError("attention: the decode kernel needs one token per sequence")
@@ -393,18 +443,22 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
         if splits > 1:
             part_ml = torch.empty((S, nh, splits, 2), dtype=torch.float32, device=qkv.device)
             part_acc = torch.empty((S, nh, splits, d), dtype=torch.float32, device=qkv.device)
-        g = nh // nkv
-        mfma = (qkv.dtype == torch.bfloat16 and d % 16 == 0 and g <= 16
-                and g * (d + 2) * 32 <= 65536
-                and page_size >= 8 and page_size & (page_size - 1) == 0 and q_stride % 8 == 0
-                and DECODE_ATTENTION != "vector")
         ml_ptr = None if part_ml is None else part_ml.data_ptr()
         acc_ptr = None if part_acc is None else part_acc.data_ptr()
         if mfma:
+            cos_p = sin_p = pos_p = slots_p = None
+            rot = 0
+            if rope is not None:
+                cos, sin, positions, slots = rope
+                pos_p = _i32(positions, "positions", S)
+                slots_p = None if slots is None else _i32(slots, "slots", S)
+                if cos is not None:
+                    cos_p, sin_p, rot = cos.data_ptr(), sin.data_ptr(), 2 * cos.shape[1]
             lib.call("rlis_attn_decode_mfma", qkv.data_ptr(), q_stride, out.data_ptr(), nh * d,
                      ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
                      block_tables.data_ptr(), max_pages, _i32(step.ctx_lens, "ctx_lens", S), S,
-                     nh, nkv, d, page_size, win, float(scale), splits, stream)
+                     nh, nkv, d, page_size, win, float(scale), splits, cos_p, sin_p, rot, pos_p,
+                     slots_p, nh * d, (nh + nkv) * d, stream)
         else:
             lib.call("rlis_attn_decode", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(),
                      nh * d, ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
@@ -454,4 +508,5 @@ def sample_rows(logits: torch.Tensor, keys: torch.Tensor, inv_temps: torch.Tenso
 
 
 __all__ = ["KernelError", "add_residual", "add_rmsnorm", "copy_pages", "decode_splits", "embed",
-           "linear", "linear_swiglu", "paged_attention", "rope_kv_write", "sample_rows", "swiglu"]
+           "linear", "linear_swiglu", "norm_linear", "paged_attention", "rope_attention",
+           "rope_kv_write", "sample_rows", "swiglu"]

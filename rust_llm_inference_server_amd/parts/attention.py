@@ -67,11 +67,9 @@ class PagedAttention(Mixer):
         if step.max_context > self.position.max_positions:
             raise ValueError(f"sequence of {step.max_context} positions exceeds max_seq_len "
                              f"{self.position.max_positions}")
-        ops.rope_kv_write(qkv, self.num_heads, self.num_kv_heads, self.head_dim,
-                          self.position.cos, self.position.sin, step.positions, group.slots,
-                          binding.k_pages, binding.v_pages, group.page_size,
-                          write_kv=binding.writes)
-        out = ops.paged_attention(qkv, self.num_heads, self.num_kv_heads, self.head_dim,
-                                  binding.k_pages, binding.v_pages, group.page_size,
-                                  group.block_tables, step, self.scale, self.window)
+        out = ops.rope_attention(qkv, self.num_heads, self.num_kv_heads, self.head_dim,
+                                 self.position.cos, self.position.sin, step.positions,
+                                 group.slots, binding.k_pages, binding.v_pages, group.page_size,
+                                 group.block_tables, step, self.scale, self.window,
+                                 write_kv=binding.writes)
         return ops.linear(out, self.w_o, self.act_dtype, partials=True)

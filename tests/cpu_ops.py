@@ -105,6 +105,14 @@ def paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, pa
     return out.to(qkv.dtype)
 
 
+def rope_attention(qkv, num_heads, num_kv_heads, head_dim, cos, sin, positions, slots, k_pages,
+                   v_pages, page_size, block_tables, step, scale, window=None, write_kv=True):
+    rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, cos, sin, positions, slots, k_pages,
+                  v_pages, page_size, write_kv=write_kv)
+    return paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, page_size,
+                           block_tables, step, scale, window)
+
+
 def _lowbias32(x):
     x ^= x >> 16
     x = (x * 0x7FEB352D) & 0xFFFFFFFF
@@ -137,7 +145,7 @@ def install(monkeypatch) -> None:
     import rust_llm_inference_server_amd.ops as ops
     import rust_llm_inference_server_amd.engine.runner as runner
     for name in ("embed", "add_residual", "add_rmsnorm", "swiglu", "linear", "linear_swiglu",
-                 "can_fuse_norm_linear", "rope_kv_write",
+                 "can_fuse_norm_linear", "rope_kv_write", "rope_attention",
                  "copy_pages", "decode_splits", "paged_attention", "sample_rows"):
         monkeypatch.setattr(ops, name, globals()[name])
     monkeypatch.setattr(runner, "default_device", lambda: torch.device("cpu"))

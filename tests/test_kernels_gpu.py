@@ -453,6 +453,50 @@ def test_attention_decode(ops, dtype, nh, nkv, d, ps, decode_kind):
     torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
 
 
+@pytest.mark.parametrize("nh,nkv,d,ps,rotate", [(32, 8, 64, 16, True), (24, 8, 128, 16, True),
+                                                (16, 2, 256, 16, True), (8, 8, 64, 32, False),
+                                                (5, 5, 48, 16, True), (9, 3, 112, 16, False)])
+@pytest.mark.parametrize("window", [None, 100])
+def test_rope_attention_decode_in_one_kernel(ops, nh, nkv, d, ps, rotate, window):
+    """The decode kernel that rotates q and k and stores the new k, v itself against
+    rope_kv_write followed by attention: same output, same pages; with and without a cache
+    write, unsplit and split (the new key then belongs to the last partition that has keys).
+    Head sizes 48 and 112 with rotation take the two-kernel path inside rope_attention."""
+    dtype = torch.bfloat16
+    lens = [1 + (i * 53) % 700 for i in range(19)] + [256, 257, 512, 513, 1]
+    cached, new = [l - 1 for l in lens], [1] * len(lens)
+    scale = 1.0 / math.sqrt(d)
+    qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=d + 1)
+    cos = sin = None
+    if rotate:
+        ang = rnd(max(lens) + 1, d // 2, seed=5, scale=3.0)
+        cos, sin = torch.cos(ang), torch.sin(ang)
+    tables = bt.cpu()
+    slots = torch.tensor([int(tables[s, (l - 1) // ps]) * ps + (l - 1) % ps for s, l in enumerate(lens)],
+                         dtype=torch.int32, device=DEV)
+    for write_kv in (True, False):
+        for splits in (None, 1, 3, 8):
+            step.decode_splits = splits
+            results = []
+            for fused in (False, True):
+                q2, k2, v2 = qkv.clone(), kp.clone(), vp.clone()
+                old = ops.FUSE_ROPE_DECODE
+                try:
+                    ops.FUSE_ROPE_DECODE = fused
+                    out = ops.rope_attention(q2, nh, nkv, d, cos, sin, step.positions, slots, k2, v2,
+                                             ps, bt, step, scale, window, write_kv=write_kv)
+                finally:
+                    ops.FUSE_ROPE_DECODE = old
+                results.append((out.float().cpu(), k2.float().cpu(), v2.cpu()))
+            (o0, k0, v0), (o1, k1, v1) = results
+            torch.testing.assert_close(o1, o0, atol=2e-2, rtol=2e-2)
+            torch.testing.assert_close(k1, k0, atol=2e-2, rtol=1e-2)      # one rounding apart at most
+            assert torch.equal(v1, v0)
+            if not write_kv:
+                assert torch.equal(k1, kp.float().cpu()) and torch.equal(v1, vp.cpu())
+    step.decode_splits = None
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_decode_long_split(ops, dtype, decode_kind):
     """Long contexts beside short ones with many partitions, some of them empty
