@@ -313,26 +313,63 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   }
 }
 
-// Grid (query head, sequence); merges the partitions of one head.
+// Grid (query head, sequence); merges the partitions of one head.  A thread owns output dims
+// j, j + blockDim, ...; the first kReduceAhead partitions' sums for its first dim are loaded
+// together with the maxima, before the weights exp(m_s - max m) are known, so that the whole
+// merge waits for memory once.  The weights go through LDS (`splits` floats); sums run over s
+// in order.
+constexpr int kReduceAhead = 16;
+
 template <typename TX>
 __global__ void attn_reduce_kernel(TX* __restrict__ out, long long out_stride,
                                    const float* __restrict__ part_ml,
                                    const float* __restrict__ part_acc,
                                    const int* __restrict__ token_rows, int nh, int d, int splits) {
+  extern __shared__ float reduce_w[];            // splits weights, then 8 floats of scratch
+  float* scratch = reduce_w + splits;
   const int h = blockIdx.x, seq = blockIdx.y;
   const int row = token_rows ? token_rows[seq] : seq;
   const long long base = ((long long)seq * nh + h) * splits;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, nwaves = blockDim.x / kWave;
+  const int j0 = threadIdx.x < d ? threadIdx.x : 0;
+  const float* acc0 = part_acc + base * d + j0;
+  float ahead[kReduceAhead];
+#pragma unroll
+  for (int s = 0; s < kReduceAhead; ++s) ahead[s] = acc0[(long long)min(s, splits - 1) * d];
   float big = -INFINITY;
-  for (int s = 0; s < splits; ++s)
+  for (int s = threadIdx.x; s < splits; s += blockDim.x)
     if (part_ml[(base + s) * 2 + 1] > 0.f) big = fmaxf(big, part_ml[(base + s) * 2]);
+  big = wave_max(big);
+  if (lane == 0) scratch[wave] = big;
+  __syncthreads();
+  for (int w = 0; w < nwaves; ++w) big = fmaxf(big, scratch[w]);
+  for (int s = threadIdx.x; s < splits; s += blockDim.x) {
+    const float ls = part_ml[(base + s) * 2 + 1];
+    reduce_w[s] = ls > 0.f ? expf(part_ml[(base + s) * 2] - big) : 0.f;
+  }
+  __syncthreads();
+  float lsum = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float e = reduce_w[s];
+    if (e > 0.f) lsum += part_ml[(base + s) * 2 + 1] * e;
+  }
   for (int j = threadIdx.x; j < d; j += blockDim.x) {
-    float lsum = 0.f, a = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float ls = part_ml[(base + s) * 2 + 1];
-      if (!(ls > 0.f)) continue;
-      const float e = expf(part_ml[(base + s) * 2] - big);
-      lsum += ls * e;
-      a += part_acc[(base + s) * d + j] * e;
+    float a = 0.f;
+    const float* acc = part_acc + base * d + j;
+    int s = 0;
+    if (j == j0) {
+#pragma unroll
+      for (; s < kReduceAhead; ++s) {
+        if (s >= splits) break;
+        const float e = reduce_w[s];
+        if (e > 0.f) a += ahead[s] * e;
+      }
+    }
+#pragma unroll 8
+    for (; s < splits; ++s) {
+      const float e = reduce_w[s];
+      const float v = acc[(long long)s * d];
+      if (e > 0.f) a += v * e;
     }
     st(out + (long long)row * out_stride + h * d + j, a / lsum);
   }
@@ -345,8 +382,8 @@ int rlis_launch_attn_reduce_bf16(void* out, long long out_stride, const float* p
                                  hipStream_t stream) {
   dim3 grid(nh, S);
   const int threads = d <= 64 ? 64 : (d <= 128 ? 128 : 256);
-  attn_reduce_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)out, out_stride, part_ml,
-                                                           part_acc, nullptr, nh, d, splits);
+  attn_reduce_kernel<bf16_t><<<grid, threads, (splits + 8) * sizeof(float), stream>>>(
+      (bf16_t*)out, out_stride, part_ml, part_acc, nullptr, nh, d, splits);
   RLIS_LAUNCH_CHECK("attn_reduce");
   return 0;
 }
@@ -390,7 +427,7 @@ RLIS_API int rlis_attn_decode(const void* q, int dtype, long long q_stride, void
                nh, nkv);
   RLIS_REQUIRE(d <= 256, "attn_decode: head_dim %d is above the limit of 256", d);
   RLIS_REQUIRE(d % 8 == 0, "attn_decode: head_dim %d must be a multiple of 8", d);
-  RLIS_REQUIRE(splits >= 1 && splits <= 65535 && S <= 65535, "attn_decode: bad grid");
+  RLIS_REQUIRE(splits >= 1 && splits <= 8192 && S <= 65535, "attn_decode: bad grid");
   RLIS_REQUIRE(splits == 1 || (part_ml && part_acc), "attn_decode: partitions need a workspace");
   if (S == 0) return 0;
   const int g = nh / nkv;
@@ -424,11 +461,11 @@ RLIS_API int rlis_attn_decode(const void* q, int dtype, long long q_stride, void
     dim3 grid(nh, S);
     const int threads = d <= 64 ? 64 : (d <= 128 ? 128 : 256);
     if (dtype == RLIS_F32)
-      attn_reduce_kernel<float><<<grid, threads, 0, stream>>>((float*)out, out_stride, part_ml,
-                                                              part_acc, token_rows, nh, d, splits);
+      attn_reduce_kernel<float><<<grid, threads, (splits + 8) * sizeof(float), stream>>>(
+          (float*)out, out_stride, part_ml, part_acc, token_rows, nh, d, splits);
     else
-      attn_reduce_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)out, out_stride, part_ml,
-                                                               part_acc, token_rows, nh, d, splits);
+      attn_reduce_kernel<bf16_t><<<grid, threads, (splits + 8) * sizeof(float), stream>>>(
+          (bf16_t*)out, out_stride, part_ml, part_acc, token_rows, nh, d, splits);
     RLIS_LAUNCH_CHECK("attn_reduce");
   }
   return 0;

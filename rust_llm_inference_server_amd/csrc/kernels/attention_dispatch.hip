@@ -107,7 +107,7 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
   RLIS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)k_pages % 16) == 0 &&
                    ((uintptr_t)v_pages % 16) == 0,
                "attn_decode_mfma: operands must be 16-byte aligned with row strides in steps of 8");
-  RLIS_REQUIRE(splits >= 1 && splits <= 65535 && S <= 65535, "attn_decode_mfma: bad grid");
+  RLIS_REQUIRE(splits >= 1 && splits <= 8192 && S <= 65535, "attn_decode_mfma: bad grid");
   RLIS_REQUIRE(splits == 1 || (part_ml && part_acc), "attn_decode_mfma: partitions need a workspace");
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;

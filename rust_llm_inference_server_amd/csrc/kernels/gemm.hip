@@ -500,47 +500,44 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
                                                                 const StreamShape sh,
                                                                 const StreamNorm nm) {
   extern __shared__ __attribute__((aligned(16))) unsigned char stream_smem[];
+  constexpr int kTileBytes = NORM ? kStreamTileBytes : TR * kStreamItem * 2;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, nwaves = blockDim.x / 64;
-  unsigned char* tile_s = stream_smem + wave * kStreamTileBytes;
-  float* red = (float*)(stream_smem + nwaves * kStreamTileBytes);      // [2][nwaves][256]
+  unsigned char* tile_s = stream_smem + wave * kTileBytes;
+  float* red = (float*)(stream_smem + nwaves * kTileBytes);            // [2][nwaves][256]
   const int half = lane / 32, l32 = lane % 32;          // loading: row parity, 16-byte chunk
   const int oi = lane % 16, og = lane / 16;             // operand: row (or token), k group
-  const uint4 zero = make_uint4(0, 0, 0, 0);
   const int T = sh.T, N = sh.N, K = sh.K;
   const int slice = blockIdx.x % sh.num_slices;
   const int tile_step = gridDim.x / sh.num_slices;
   const int nitems = (K + kStreamItem - 1) / kStreamItem;
-  const int item = slice * nwaves + wave;
+  const int item = slice * nwaves + wave;               // this wave's k item
   const bool has_item = item < nitems;
   const int kb = item * kStreamItem;
   const int ka = kb + l32 * 8;                          // this lane's k when loading weights
   const bool a_ok = has_item && ka < K;
+  // Loads are never predicated off (that would cost registers for the zeros): a row past the
+  // end reads row 0 instead and is not stored; a k past the end reads k = 0 and is zeroed.
+  const bf16_t* w_lane = W + (a_ok ? ka : 0);
 
   // Tile row r = 2 p + half of tile `tile` is weight row tile * rows + r; gated, the first
   // half of a tile's rows are the gate rows of consecutive columns and the second half their
   // up rows, N further down.  Everything but `half` and the lane's k is uniform over the wave.
   constexpr int cols_per_tile = GATED ? TR / 2 : TR;
-  // Loads are never predicated off (that would cost registers for the zeros): a row past the
-  // end reads row 0 instead and is not stored; a k past the end reads k = 0 and is zeroed.
-  const int ka_safe = a_ok ? ka : 0;
-  const bf16_t* w_lane = W + (long long)half * sh.ldw + ka_safe;
 #define RLIS_STREAM_LOAD_TILE(a, tile_)                                                         \
   {                                                                                             \
     const int tl_ = (tile_);                                                                    \
     if (tl_ < sh.num_tiles) {                                                                   \
-      const bf16_t* w_tile = w_lane + (long long)tl_ * cols_per_tile * sh.ldw;                  \
       const int col0 = tl_ * cols_per_tile + half;                                              \
+      const bf16_t* w_tile = w_lane + (long long)col0 * sh.ldw;                                 \
       _Pragma("unroll") for (int p = 0; p < TR / 2; ++p) {                                      \
-        {                                                                                       \
-          const int c = GATED ? (2 * p) % cols_per_tile : 2 * p; /* column within the tile */   \
-          const long long up = (GATED && 2 * p >= cols_per_tile) ? (long long)N * sh.ldw : 0;   \
-          const bf16_t* ptr = col0 + c < N ? w_tile + (long long)c * sh.ldw + up : W + ka_safe; \
-          const uint4 v_ = *(const uint4*)ptr;                                                  \
-          a[p].x = a_ok ? v_.x : 0u;                                                            \
-          a[p].y = a_ok ? v_.y : 0u;                                                            \
-          a[p].z = a_ok ? v_.z : 0u;                                                            \
-          a[p].w = a_ok ? v_.w : 0u;                                                            \
-        }                                                                                       \
+        const int c = GATED ? (2 * p) % cols_per_tile : 2 * p; /* column within the tile */     \
+        const long long up = (GATED && 2 * p >= cols_per_tile) ? (long long)N * sh.ldw : 0;     \
+        const bf16_t* ptr = col0 + c < N ? w_tile + (long long)c * sh.ldw + up : w_lane;        \
+        const uint4 v_ = *(const uint4*)ptr;                                                    \
+        a[p].x = a_ok ? v_.x : 0u;                                                              \
+        a[p].y = a_ok ? v_.y : 0u;                                                              \
+        a[p].z = a_ok ? v_.z : 0u;                                                              \
+        a[p].w = a_ok ? v_.w : 0u;                                                              \
       }                                                                                         \
     }                                                                                           \
   }
@@ -571,51 +568,81 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
     if (!has_item) {
       if (lane < 16) ss_s[wave * 16 + lane] = 0.f;
     } else {
-      for (int u = lane; u < T * 32; u += 64) {
-        const int t = u / 32, c = u % 32;
-        const int k = kb + c * 8;
-        const bool ok = k < K;
-        const long long src = nm.rows ? (long long)nm.rows[t] : (long long)t;
-        const long long at = src * K + (ok ? k : 0);
-        float v[8], d[8], w[8];
-        load8(nm.resid + at, v);
+      // A lane keeps its chunk of 8 k and walks over tokens lane / 32, + 2, + 4, ...; the
+      // loads of kU tokens are issued together.
+      constexpr int kU = 2;
+      const int c = l32, k = kb + c * 8;
+      const bool ok = k < K;
+      const int ks = ok ? k : 0;
+      float w[8];
+      if (nm.weight_f32)
+        load8((const float*)nm.weight + ks, w);
+      else
+        load8((const bf16_t*)nm.weight + ks, w);
+      for (int t0 = half; t0 < T; t0 += 2 * kU) {
+        float v[kU][8];
+        long long at[kU];
+#pragma unroll
+        for (int i = 0; i < kU; ++i) {
+          const int t = min(t0 + 2 * i, T - 1);               // repeats the last token: not used
+          at[i] = (nm.rows ? (long long)nm.rows[t] : (long long)t) * K + ks;
+          load8(nm.resid + at[i], v[i]);
+        }
         if (nm.delta) {
-          for (int s = 0; s < nm.parts; ++s) {
-            if (nm.delta_f32)
-              load8((const float*)nm.delta + s * nm.part_stride + at, d);
-            else
-              load8((const bf16_t*)nm.delta + s * nm.part_stride + at, d);
+          // two parts per round, so that their loads travel together with the residual's
+          for (int s = 0; s < nm.parts; s += 2) {
+            const bool two = s + 1 < nm.parts;
+            float d0[kU][8], d1[kU][8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] += d[e];
-          }
-          if (store_sum && ok) {
-            *(float4*)(nm.resid_out + at) = make_float4(v[0], v[1], v[2], v[3]);
-            *(float4*)(nm.resid_out + at + 4) = make_float4(v[4], v[5], v[6], v[7]);
+            for (int i = 0; i < kU; ++i) {
+              if (nm.delta_f32) {
+                const float* dp = (const float*)nm.delta + s * nm.part_stride + at[i];
+                load8(dp, d0[i]);
+                load8(two ? dp + nm.part_stride : dp, d1[i]);
+              } else {
+                const bf16_t* dp = (const bf16_t*)nm.delta + s * nm.part_stride + at[i];
+                load8(dp, d0[i]);
+                load8(two ? dp + nm.part_stride : dp, d1[i]);
+              }
+            }
+#pragma unroll
+            for (int i = 0; i < kU; ++i)
+#pragma unroll
+              for (int e = 0; e < 8; ++e) {
+                v[i][e] += d0[i][e];
+                if (two) v[i][e] += d1[i][e];
+              }
           }
         }
-        if (nm.weight_f32)
-          load8((const float*)nm.weight + (ok ? k : 0), w);
-        else
-          load8((const bf16_t*)nm.weight + (ok ? k : 0), w);
-        float ss = 0.f;
-        Frag8 xw;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float x = ok ? v[e] : 0.f;
-          ss += x * x;
-          xw.v[e] = (__bf16)(x * w[e]);
+        for (int i = 0; i < kU; ++i) {
+          const int t = t0 + 2 * i;
+          if (t < T) {
+            if (nm.delta && store_sum && ok) {
+              *(float4*)(nm.resid_out + at[i]) = make_float4(v[i][0], v[i][1], v[i][2], v[i][3]);
+              *(float4*)(nm.resid_out + at[i] + 4) = make_float4(v[i][4], v[i][5], v[i][6], v[i][7]);
+            }
+            float ss = 0.f;
+            Frag8 xw;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float x = ok ? v[i][e] : 0.f;
+              ss += x * x;
+              xw.v[e] = (__bf16)(x * w[e]);
+            }
+            *(uint4*)(tile_s + t * (kStreamItem * 2) + ((c ^ t) * 16)) = xw.u;
+#pragma unroll
+            for (int o = 16; o > 0; o >>= 1) ss += __shfl_xor(ss, o, kWave);
+            if (l32 == 0) ss_s[wave * 16 + t] = ss;
+          }
         }
-        *(uint4*)(tile_s + t * (kStreamItem * 2) + ((c ^ t) * 16)) = xw.u;
-#pragma unroll
-        for (int o = 16; o > 0; o >>= 1) ss += __shfl_xor(ss, o, kWave);
-        if (l32 == 0) ss_s[wave * 16 + t] = ss;
       }
       wave_lds_fence();
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const uint4 v = *(const uint4*)(tile_s + oi * (kStreamItem * 2) + (((4 * j + og) ^ oi) * 16));
-        const bool ok = oi < T;
-        b[j].u = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+        const bool tok = oi < T;
+        b[j].u = make_uint4(tok ? v.x : 0u, tok ? v.y : 0u, tok ? v.z : 0u, tok ? v.w : 0u);
       }
       wave_lds_fence();
     }
@@ -643,7 +670,8 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         Frag8 af;
-        af.u = *(const uint4*)(tile_s + oi * (kStreamItem * 2) + (((4 * j + og) ^ oi) * 16));
+        // tile rows beyond TR repeat the first ones: their products are not stored
+        af.u = *(const uint4*)(tile_s + (oi % TR) * (kStreamItem * 2) + (((4 * j + og) ^ (oi % TR)) * 16));
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af.v, b[j].v, acc, 0, 0, 0);
       }
       wave_lds_fence();
@@ -684,25 +712,27 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
 #undef RLIS_STREAM_LOAD_TILE
 }
 
-// Number of k slices a product over K is cut into (a function of K alone).
-static int stream_slices(int K) {
-  return ceil_div(ceil_div(K, kStreamItem), kStreamMaxWaves);
-}
+// A workgroup takes up to 16 k items, one per wave; longer rows are cut into slices.  Both
+// are functions of K alone.
+static int stream_slices(int K) { return ceil_div(ceil_div(K, kStreamItem), kStreamMaxWaves); }
+// The fused norm needs whole rows in one workgroup.
+constexpr int kStreamNormMaxK = kStreamMaxWaves * kStreamItem;
 
 template <typename TC, bool GATED, int TR, bool NORM>
 static int launch_stream_tiles(const void* X, const void* W, void* Y, StreamShape sh,
                                const StreamNorm& nm, int nwaves, int num_cus,
                                hipStream_t stream) {
+  constexpr int kTileBytes = NORM ? kStreamTileBytes : TR * kStreamItem * 2;
   static bool lds_raised = false;
   if (!lds_raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_stream_kernel<TC, GATED, TR, NORM>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       kStreamMaxWaves * (kStreamTileBytes + 2048));
+    hipError_t e = hipFuncSetAttribute(
+        (const void*)gemm_bf16_stream_kernel<TC, GATED, TR, NORM>,
+        hipFuncAttributeMaxDynamicSharedMemorySize, kStreamMaxWaves * (kTileBytes + 2048));
     RLIS_REQUIRE(e == hipSuccess, "gemm_bf16_stream: cannot raise the LDS limit: %s",
                  hipGetErrorString(e));
     lds_raised = true;
   }
-  const size_t smem = (size_t)nwaves * (kStreamTileBytes + 2048);
+  const size_t smem = (size_t)nwaves * (kTileBytes + 2048);
   const int per_cu = max(1, (int)((160 * 1024) / smem));
   const long long tiles = ceil_div_ll(sh.N, GATED ? TR / 2 : TR);
   RLIS_REQUIRE(tiles <= 0x3fffffffll, "gemm_bf16_stream: N=%d is too large", sh.N);
@@ -737,8 +767,10 @@ static int launch_stream(const void* X, const void* W, void* Y, int T, int N, in
   sh.num_slices = slices;
   sh.num_tiles = 0;
   // Tiles of 8 rows when 16-row tiles would leave compute units without work: a unit draws
-  // only its share of the memory bandwidth, however much it has in flight.
-  if ((long long)ceil_div(N, GATED ? 8 : 16) * slices < num_cus)
+  // only its share of the memory bandwidth, however much it has in flight.  With the fused
+  // norm every workgroup reads all of x, so fewer, larger tiles win earlier.
+  const long long tiles16 = (long long)ceil_div(N, GATED ? 8 : 16) * slices;
+  if (tiles16 < (NORM ? num_cus / 2 : num_cus))
     return launch_stream_tiles<TC, GATED, 8, NORM>(X, W, Y, sh, nm, nwaves, num_cus, stream);
   return launch_stream_tiles<TC, GATED, 16, NORM>(X, W, Y, sh, nm, nwaves, num_cus, stream);
 }
@@ -766,6 +798,9 @@ static int dispatch_stream(const char* name, const void* X, const void* W, void*
 // Slices that rlis_gemm_bf16_stream cuts K into; with more than one, Y receives that many
 // float32 partial results, part_stride elements apart, to be added in order.
 RLIS_API int rlis_gemm_bf16_stream_slices(int K) { return stream_slices(K); }
+
+// The longest row that rlis_norm_linear_bf16 takes.
+RLIS_API int rlis_norm_linear_max_k() { return kStreamNormMaxK; }
 
 // gated == 0: y (T, N) = x W^T.  gated != 0: W is (2N, K) = [Wg; Wu] and
 // y (T, N) = silu(x Wg^T) * (x Wu^T), K <= 4096.  T <= 16, bfloat16 operands, K a multiple of 8.
@@ -801,7 +836,7 @@ RLIS_API int rlis_norm_linear_bf16(const float* resid, const void* delta, int de
   RLIS_REQUIRE(T >= 0 && T <= 16, "norm_linear: T=%d rows, at most 16", T);
   RLIS_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && ldw % 8 == 0 && ldw >= K && ldy >= N,
                "norm_linear: bad sizes N=%d K=%d ldw=%lld ldy=%lld", N, K, ldw, ldy);
-  RLIS_REQUIRE(stream_slices(K) == 1, "norm_linear: K=%d does not fit one k slice", K);
+  RLIS_REQUIRE(K <= kStreamNormMaxK, "norm_linear: K=%d, at most %d", K, kStreamNormMaxK);
   RLIS_REQUIRE(((uintptr_t)W % 16) == 0 && ((uintptr_t)resid % 16) == 0 &&
                    ((uintptr_t)delta % 16) == 0 && ((uintptr_t)norm_weight % 16) == 0 &&
                    ((uintptr_t)resid_out % 16) == 0,

@@ -206,7 +206,8 @@ def can_fuse_norm_linear(resid: torch.Tensor, w: torch.Tensor, rows: Optional[in
     K = resid.shape[1]
     return (0 < T <= STREAM_MAX_ROWS and FUSE_NORM_LINEAR and w.dtype == torch.bfloat16
             and w.dim() == 2 and w.shape[1] == K and K % 8 == 0 and w.stride(1) == 1
-            and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0 and stream_slices(K) == 1)
+            and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0
+            and K <= lib.load().rlis_norm_linear_max_k())
 
 
 def norm_linear(resid: torch.Tensor, delta: Optional[torch.Tensor], norm_weight: torch.Tensor,

@@ -62,6 +62,8 @@ def load() -> ctypes.CDLL:
         fn.argtypes = argtypes
     lib.rlis_gemm_bf16_stream_slices.restype = c_int
     lib.rlis_gemm_bf16_stream_slices.argtypes = [I]
+    lib.rlis_norm_linear_max_k.restype = c_int
+    lib.rlis_norm_linear_max_k.argtypes = []
     _LIB = lib
     return lib
 
