@@ -16,7 +16,8 @@ from .lib import KernelError
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 
-# bf16 products with at most this many rows of x take the skinny kernel.
+# bf16 products with at most this many rows of x take the skinny kernel (where the library's
+# GEMM is not used, see BF16_GEMM).
 SKINNY_MAX_ROWS = 64
 # ... and with at most this many rows the streaming kernel (16 at most; 0 switches it off).
 STREAM_MAX_ROWS = 16
@@ -24,8 +25,8 @@ STREAM_MAX_ROWS = 16
 FUSE_NORM_LINEAR = True
 # The matrix-core decode attention rotates q and k and stores the new k, v itself where it can.
 FUSE_ROPE_DECODE = True
-# "library": bf16 products with more rows and bf16 output go to torch.matmul (hipBLASLt);
-# "own": they take the hand-written matrix-core kernel.
+# "library": bf16 products with more rows than the streaming kernel takes go to torch
+# (hipBLASLt); "own": they take the hand-written skinny and matrix-core kernels.
 BF16_GEMM = "library"
 # None: attention kernels are chosen from the batch; "generic": the generic kernel always
 # (what the command line's --attention v1 asks for).
@@ -156,8 +157,9 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     """``x @ w.T`` for ``x (T, K)`` and ``w (N, K)``, float32 accumulation.
 
     A float32 weight (or float32 ``x``) takes the plain FMA kernel, the true 32-bit product.
-    bfloat16 operands take the streaming kernel up to 16 rows, the skinny kernel up to 64, else
-    the matrix-core GEMM (ours for float32 output, the library's or ours for bfloat16 output).
+    bfloat16 operands take the streaming kernel up to 16 rows; more rows go to the library's
+    GEMM (hipBLASLt through torch), or with ``BF16_GEMM = "own"`` to the skinny kernel up to 64
+    rows and the hand-written matrix-core GEMM beyond.
 
     ``partials``: the caller hands the result to the residual stream and takes it as a stack
     ``(S, T, N)`` of float32 partial sums too (one per k slice of the streaming kernel, added in
@@ -173,9 +175,10 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     bf16 = x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
     aligned = (K % 8 == 0 and ldx % 8 == 0 and ldw % 8 == 0
                and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
-    if bf16 and aligned and T > SKINNY_MAX_ROWS and out_dtype == torch.bfloat16 \
-            and BF16_GEMM == "library":
-        return torch.matmul(x, w.t())
+    if bf16 and aligned and T > STREAM_MAX_ROWS and BF16_GEMM == "library":
+        if out_dtype == torch.bfloat16:
+            return torch.matmul(x, w.t())
+        return torch.mm(x, w.t(), out_dtype=torch.float32)    # float32 accumulation and result
     if bf16 and aligned and 0 < T <= STREAM_MAX_ROWS:
         slices = stream_slices(K)
         if slices == 1 or partials:
@@ -252,22 +255,26 @@ def norm_linear(resid: torch.Tensor, delta: Optional[torch.Tensor], norm_weight:
 def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
     """``silu(x @ Wg.T) * (x @ Wu.T)`` for ``w_gate_up = [Wg; Wu]`` of shape ``(2 I, K)``.
 
-    Up to 64 rows of bfloat16 take one kernel that never stores the ``(T, 2 I)`` intermediate;
-    everything else is the product followed by the SwiGLU kernel."""
+    Up to 16 rows of bfloat16 (64 with ``BF16_GEMM = "own"``) take one kernel that never stores
+    the ``(T, 2 I)`` intermediate; everything else is the product followed by the SwiGLU
+    kernel."""
     T, K = x.shape
     two_i = w_gate_up.shape[0]
     if two_i % 2:
         raise KernelError("linear_swiglu: the fused weight needs an even number of rows")
     ldx = _rows_contig(x, "linear_swiglu x")
     ldw = _rows_contig(w_gate_up, "linear_swiglu weight")
-    fused = (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
-             and 0 < T <= SKINNY_MAX_ROWS and K == w_gate_up.shape[1] and K % 8 == 0
-             and ldx % 8 == 0 and ldw % 8 == 0 and x.data_ptr() % 16 == 0
-             and w_gate_up.data_ptr() % 16 == 0)
-    if not fused:
+    fusable = (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
+               and 0 < T and K == w_gate_up.shape[1] and K % 8 == 0
+               and ldx % 8 == 0 and ldw % 8 == 0 and x.data_ptr() % 16 == 0
+               and w_gate_up.data_ptr() % 16 == 0)
+    streamed = fusable and T <= STREAM_MAX_ROWS and stream_slices(K) == 1
+    skinny = fusable and not streamed and T <= SKINNY_MAX_ROWS and \
+        (BF16_GEMM == "own" or T <= STREAM_MAX_ROWS)
+    if not (streamed or skinny):
         return swiglu(linear(x, w_gate_up, x.dtype))
     y = torch.empty((T, two_i // 2), dtype=torch.bfloat16, device=x.device)
-    if T <= STREAM_MAX_ROWS and stream_slices(K) == 1:
+    if streamed:
         lib.call("rlis_gemm_bf16_stream", x.data_ptr(), w_gate_up.data_ptr(), y.data_ptr(), 1, T,
                  two_i // 2, K, ldx, ldw, two_i // 2, 0, 1, lib.stream_ptr())
     else:

@@ -247,12 +247,12 @@ def test_linear_swiglu(ops, dtype, T, I, K):
     want = (torch.nn.functional.silu(g) * u).float()
     got = ops.linear_swiglu(x, w)
     assert got.dtype == dtype and got.shape == (T, I)
-    old = ops.STREAM_MAX_ROWS
+    old = ops.STREAM_MAX_ROWS, ops.BF16_GEMM
     try:
-        ops.STREAM_MAX_ROWS = 0                               # the other kernel for few rows
+        ops.STREAM_MAX_ROWS, ops.BF16_GEMM = 0, "own"         # the skinny kernel up to 64 rows
         other = ops.linear_swiglu(x, w)
     finally:
-        ops.STREAM_MAX_ROWS = old
+        ops.STREAM_MAX_ROWS, ops.BF16_GEMM = old
     torch.testing.assert_close(other.float(), got.float(), atol=0.05, rtol=2e-2)
     scale = max(1.0, want.abs().max().item())
     if dtype == torch.float32:
