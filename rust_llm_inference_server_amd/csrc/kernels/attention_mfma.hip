@@ -55,7 +55,8 @@ constexpr int BM = 64;
 
 }  // namespace
 
-__global__ __launch_bounds__(256) void KERNEL_NAME(
+// Up to three waves per SIMD: the staging registers must not be traded for a fourth.
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) void KERNEL_NAME(
     const bf16_t* __restrict__ q, long long q_stride, bf16_t* __restrict__ out,
     long long out_stride, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_seqlens,
@@ -112,71 +113,84 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
   const int kt0 = (klo / BN) * BN;
   const int wave_q_last = min(n_new - 1, wave_q_first + 15);
 
-  // Staging registers for the next tile.
+  // Staging for the tiles to come.  A tile's page ids are fetched four tiles ahead of its use,
+  // its keys and values two tiles ahead (two register sets taking turns), so that neither the
+  // table lookup nor the loads themselves are waited for.  The loads are unconditional, so
+  // that the compiler can count them: a key past the end of the tile's range reads the last
+  // key in range instead (its score is masked), a dim past d reads dim d - 8 (it meets a zero
+  // of q, or a row of O^T that is not stored).  Values past the end of the range inside a
+  // group of 8 keys are whatever the page holds: the pages start as zeros and only ever hold
+  // values that a model wrote, and their probabilities are exactly zero.
   constexpr int K_CHUNKS = BN * (D / 8);
   constexpr int KCH = (K_CHUNKS + 255) / 256;
   constexpr int VCH = (D * (BN / 8) + 255) / 256;
-  uint4 kreg[KCH], vreg[VCH];
   const int v_chunks = d * (BN / 8);
-  auto load_tile = [&](int k0) {
+  int k_key[KCH], k_dim[KCH], v_key[VCH], v_dim[VCH];   // this thread's chunks within a tile
 #pragma unroll
-    for (int i = 0; i < KCH; ++i) {
-      const int c = tid + i * 256;
-      const int key = c / (D / 8), dc = c % (D / 8);
-      const int kpos = k0 + key;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (c < K_CHUNKS && kpos < khi && dc * 8 < d) {
-        const long long page = table[kpos >> page_shift];
-        const int off = kpos & page_mask;
-        v = *(const uint4*)(k_pages + (((page * nkv + kvh) << page_shift) + off) * d + dc * 8);
-      }
-      kreg[i] = v;
-    }
+  for (int i = 0; i < KCH; ++i) {
+    const int c = min(tid + i * 256, K_CHUNKS - 1);
+    k_key[i] = c / (D / 8);
+    k_dim[i] = min((c % (D / 8)) * 8, d - 8);
+  }
 #pragma unroll
-    for (int i = 0; i < VCH; ++i) {
-      const int c = tid + i * 256;
-      Frag8 v;
-      v.u = make_uint4(0, 0, 0, 0);
-      if (c < v_chunks) {
-        const int dim = c / (BN / 8), kg = c % (BN / 8);
-        const int kpos = k0 + kg * 8;
-        if (kpos < khi) {
-          const long long page = table[kpos >> page_shift];
-          const int off = kpos & page_mask;
-          v.u = *(const uint4*)(v_pages +
-                                (((page * nkv + kvh) * (long long)d + dim) << page_shift) + off);
-          if (kpos + 8 > khi) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-              if (kpos + e >= khi) v.e[e] = 0;
-          }
-        }
-      }
-      vreg[i] = v.u;
-    }
-  };
-  auto store_tile = [&]() {
-#pragma unroll
-    for (int i = 0; i < KCH; ++i) {
-      const int c = tid + i * 256;
-      if (c < K_CHUNKS) *(uint4*)(Ks + (c / (D / 8)) * KS + (c % (D / 8)) * 8) = kreg[i];
-    }
-#pragma unroll
-    for (int i = 0; i < VCH; ++i) {
-      const int c = tid + i * 256;
-      if (c < v_chunks) *(uint4*)(Vs + (c / (BN / 8)) * VS + (c % (BN / 8)) * 8) = vreg[i];
-    }
-  };
+  for (int i = 0; i < VCH; ++i) {
+    const int c = min(tid + i * 256, v_chunks - 1);
+    v_dim[i] = c / (BN / 8);
+    v_key[i] = (c % (BN / 8)) * 8;
+  }
+  const int last_key = khi - 1, last_group = (khi - 1) & ~7;
+  // Two sets of staging registers (A, B) and of page ids; plain arrays and macros, so that they
+  // stay in registers.
+  uint4 tile_ka[KCH], tile_va[VCH], tile_kb[KCH], tile_vb[VCH];
+  int page_ka[KCH], page_va[VCH], page_kb[KCH], page_vb[VCH];
+#define RLIS_LOAD_PAGES(k0_, PK, PV)                                                           \
+  {                                                                                            \
+    _Pragma("unroll") for (int i = 0; i < KCH; ++i)                                            \
+        PK[i] = table[max(0, min((k0_) + k_key[i], last_key)) >> page_shift];                  \
+    _Pragma("unroll") for (int i = 0; i < VCH; ++i)                                            \
+        PV[i] = table[max(0, min((k0_) + v_key[i], last_group)) >> page_shift];                \
+  }
+#define RLIS_LOAD_TILE(k0_, PK, PV, TK, TV)                                                    \
+  {                                                                                            \
+    _Pragma("unroll") for (int i = 0; i < KCH; ++i) {                                          \
+      const int off_ = max(0, min((k0_) + k_key[i], last_key)) & page_mask;                    \
+      TK[i] = *(const uint4*)(k_pages +                                                        \
+                              ((((long long)PK[i] * nkv + kvh) << page_shift) + off_) * d +    \
+                              k_dim[i]);                                                       \
+    }                                                                                          \
+    _Pragma("unroll") for (int i = 0; i < VCH; ++i) {                                          \
+      const int off_ = max(0, min((k0_) + v_key[i], last_group)) & page_mask;                  \
+      TV[i] = *(const uint4*)(v_pages +                                                        \
+                              ((((long long)PV[i] * nkv + kvh) * d + v_dim[i]) << page_shift) + \
+                              off_);                                                           \
+    }                                                                                          \
+  }
+#define RLIS_STORE_TILE(TK, TV)                                                                \
+  {                                                                                            \
+    _Pragma("unroll") for (int i = 0; i < KCH; ++i) {                                          \
+      const int c_ = tid + i * 256;                                                            \
+      if (c_ < K_CHUNKS) *(uint4*)(Ks + (c_ / (D / 8)) * KS + (c_ % (D / 8)) * 8) = TK[i];     \
+    }                                                                                          \
+    _Pragma("unroll") for (int i = 0; i < VCH; ++i) {                                          \
+      const int c_ = tid + i * 256;                                                            \
+      if (c_ < v_chunks) *(uint4*)(Vs + (c_ / (BN / 8)) * VS + (c_ % (BN / 8)) * 8) = TV[i];   \
+    }                                                                                          \
+  }
 
   const float scale2 = scale * 1.4426950408889634f;      // scores in the base-2 domain
-  if (kt0 < khi) {
-    load_tile(kt0);
-    store_tile();
-  }
+  if (kt0 < khi) {           // else this tile has no keys at all (it cannot happen: khi > P + qb)
+  RLIS_LOAD_PAGES(kt0, page_ka, page_va);
+  RLIS_LOAD_PAGES(kt0 + BN, page_kb, page_vb);
+  RLIS_LOAD_TILE(kt0, page_ka, page_va, tile_ka, tile_va);
+  RLIS_LOAD_TILE(kt0 + BN, page_kb, page_vb, tile_kb, tile_vb);
+  RLIS_LOAD_PAGES(kt0 + 2 * BN, page_ka, page_va);
+  RLIS_LOAD_PAGES(kt0 + 3 * BN, page_kb, page_vb);
+  RLIS_STORE_TILE(tile_ka, tile_va);
+  RLIS_LOAD_TILE(kt0 + 2 * BN, page_ka, page_va, tile_ka, tile_va);
+  RLIS_LOAD_PAGES(kt0 + 4 * BN, page_ka, page_va);
   __syncthreads();
-  for (int k0 = kt0; k0 < khi; k0 += BN) {
-    const bool more = k0 + BN < khi;
-    if (more) load_tile(k0 + BN);
+  // The arithmetic of one tile, which LDS holds.
+  auto compute = [&](int k0) __attribute__((always_inline)) {
 
     // Tiles wholly after this wave's last query contribute nothing to it.
     const bool wave_active = (wave_q_first < n_new) && (k0 <= P + wave_q_last);
@@ -263,11 +277,30 @@ __global__ __launch_bounds__(256) void KERNEL_NAME(
         }
       }
     }
-    __syncthreads();
-    if (more) {
-      store_tile();
-      __syncthreads();
-    }
+  };
+  // On entry of the step for tile k0: LDS holds tile k0; the `next` registers hold tile k0 + BN
+  // and the other set tile k0 + 2 BN (in flight); the `next` page ids are those of tile
+  // k0 + 3 BN, the other set's those of tile k0 + 4 BN.  After the arithmetic the next tile goes
+  // to LDS and its registers take tile k0 + 3 BN, whose page ids arrived long since.
+#define RLIS_STEP(k0_, PK, PV, TK, TV)                \
+  {                                                   \
+    compute(k0_);                                     \
+    __syncthreads();                                  \
+    if ((k0_) + BN < khi) {                           \
+      RLIS_STORE_TILE(TK, TV);                        \
+      __syncthreads();                                \
+    }                                                 \
+    RLIS_LOAD_TILE((k0_) + 3 * BN, PK, PV, TK, TV);   \
+    RLIS_LOAD_PAGES((k0_) + 5 * BN, PK, PV);          \
+  }
+  for (int k0 = kt0; k0 < khi; k0 += 2 * BN) {
+    RLIS_STEP(k0, page_kb, page_vb, tile_kb, tile_vb);
+    if (k0 + BN < khi) RLIS_STEP(k0 + BN, page_ka, page_va, tile_ka, tile_va);
+  }
+#undef RLIS_STEP
+#undef RLIS_STORE_TILE
+#undef RLIS_LOAD_TILE
+#undef RLIS_LOAD_PAGES
   }
 
   // ---- normalise and store: this lane holds dims db * 16 + lq * 4 + [0, 4) of its query ----
