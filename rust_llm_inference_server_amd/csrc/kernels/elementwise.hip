@@ -156,6 +156,83 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_small_kernel(
   }
 }
 
+// The all-bfloat16 case with rows of a multiple of 8 and at most 256 * 8 * CH elements: eight
+// elements per thread and chunk, 16- and 32-byte accesses.
+template <int CH>
+__global__ __launch_bounds__(256) void add_rmsnorm_bf16x8_kernel(
+    float* __restrict__ resid, const bf16_t* __restrict__ delta, const bf16_t* __restrict__ weight,
+    bf16_t* __restrict__ out, const int* __restrict__ rows, int H, float eps, int write_resid) {
+  __shared__ float red[256 / kWave];
+  const int r = blockIdx.x;
+  const long long src = rows ? (long long)rows[r] : (long long)r;
+  float* x = resid + src * H;
+  const bf16_t* d = delta ? delta + src * H : nullptr;
+  float v[CH][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int ch = 0; ch < CH; ++ch) {
+    const int j = (threadIdx.x + ch * 256) * 8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[ch][e] = 0.f;
+    if (j < H) {
+      const float4 a = *(const float4*)(x + j), b = *(const float4*)(x + j + 4);
+      v[ch][0] = a.x; v[ch][1] = a.y; v[ch][2] = a.z; v[ch][3] = a.w;
+      v[ch][4] = b.x; v[ch][5] = b.y; v[ch][6] = b.z; v[ch][7] = b.w;
+      if (d) {
+        const uint4 dv = *(const uint4*)(d + j);
+        const uint32_t dw[4] = {dv.x, dv.y, dv.z, dv.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[ch][2 * e] += __uint_as_float(dw[e] << 16);
+          v[ch][2 * e + 1] += __uint_as_float(dw[e] & 0xffff0000u);
+        }
+        if (write_resid) {
+          *(float4*)(x + j) = make_float4(v[ch][0], v[ch][1], v[ch][2], v[ch][3]);
+          *(float4*)(x + j + 4) = make_float4(v[ch][4], v[ch][5], v[ch][6], v[ch][7]);
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += v[ch][e] * v[ch][e];
+    }
+  }
+  ss = block_sum<256>(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+  bf16_t* o = out + (long long)r * H;
+#pragma unroll
+  for (int ch = 0; ch < CH; ++ch) {
+    const int j = (threadIdx.x + ch * 256) * 8;
+    if (j < H) {
+      const uint4 wv = *(const uint4*)(weight + j);
+      const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+      uint32_t ow[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float r0 = v[ch][2 * e] * inv * __uint_as_float(ww[e] << 16);
+        const float r1 = v[ch][2 * e + 1] * inv * __uint_as_float(ww[e] & 0xffff0000u);
+        ow[e] = (uint32_t)f32_to_bf16(r0) | ((uint32_t)f32_to_bf16(r1) << 16);
+      }
+      *(uint4*)(o + j) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+    }
+  }
+}
+
+// True when the vectorised kernel took the call.
+static bool launch_add_rmsnorm_bf16x8(float* resid, const void* delta, const void* weight, void* out,
+                                      const int* rows, int R, int H, float eps, int write_resid,
+                                      int parts, hipStream_t stream) {
+  if (H % 8 != 0 || H > 256 * 8 * 4 || parts != 1) return false;
+  if (((uintptr_t)resid | (uintptr_t)delta | (uintptr_t)weight | (uintptr_t)out) % 16) return false;
+#define LAUNCH(CH)                                                                               \
+  add_rmsnorm_bf16x8_kernel<CH><<<R, 256, 0, stream>>>(resid, (const bf16_t*)delta,              \
+                                                       (const bf16_t*)weight, (bf16_t*)out, rows, \
+                                                       H, eps, write_resid)
+  if (H <= 256 * 8) LAUNCH(1);
+  else if (H <= 256 * 16) LAUNCH(2);
+  else LAUNCH(4);
+#undef LAUNCH
+  return true;
+}
+
 template <typename TD, typename TW, typename TO>
 static void launch_add_rmsnorm(float* resid, const void* delta, const void* weight, void* out,
                                const int* rows, int R, int H, float eps, int write_resid,
@@ -183,6 +260,12 @@ RLIS_API int rlis_add_rmsnorm(float* resid, const void* delta, int delta_dtype,
   RLIS_REQUIRE(!(rows && write_resid && delta),
                "add_rmsnorm: writing the residual back needs all rows, not a selection");
   if (R == 0) return 0;
+  if ((!delta || delta_dtype == RLIS_BF16) && weight_dtype == RLIS_BF16 && out_dtype == RLIS_BF16 &&
+      launch_add_rmsnorm_bf16x8(resid, delta, weight, out, rows, R, H, eps, write_resid, parts,
+                                stream)) {
+    RLIS_LAUNCH_CHECK("add_rmsnorm");
+    return 0;
+  }
   const int key = (delta ? delta_dtype : out_dtype) * 4 + weight_dtype * 2 + out_dtype;
 #define CASE(k, TD, TW, TO)                                                                  \
   case k:                                                                                    \
@@ -224,10 +307,40 @@ __global__ void swiglu_kernel(TX* __restrict__ out, const TX* __restrict__ gu, i
   }
 }
 
+// bfloat16 rows whose width is a multiple of 8: eight columns per thread, 16-byte accesses.
+__global__ void swiglu_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ gu,
+                                     int I8 /* I / 8 */, long long total8) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (; i < total8; i += stride) {
+    const long long t = i / I8;
+    const int c = (int)(i - t * I8);
+    const uint4 gv = *(const uint4*)(gu + (t * 2 * I8 + c) * 8);
+    const uint4 uv = *(const uint4*)(gu + (t * 2 * I8 + I8 + c) * 8);
+    const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
+      const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
+      const float r0 = g0 / (1.0f + expf(-g0)) * u0, r1 = g1 / (1.0f + expf(-g1)) * u1;
+      ow[j] = (uint32_t)f32_to_bf16(r0) | ((uint32_t)f32_to_bf16(r1) << 16);
+    }
+    *(uint4*)(out + i * 8) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+  }
+}
+
 RLIS_API int rlis_swiglu(void* out, const void* gu, int dtype, int T, int I, hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && I > 0, "swiglu: bad sizes T=%d I=%d", T, I);
   const long long total = (long long)T * I;
   if (total == 0) return 0;
+  if (dtype == RLIS_BF16 && I % 8 == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)gu % 16) == 0) {
+    const long long total8 = total / 8;
+    const int blocks8 = (int)(ceil_div_ll(total8, 256) < 16384 ? ceil_div_ll(total8, 256) : 16384);
+    swiglu_bf16x8_kernel<<<blocks8, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, I / 8, total8);
+    RLIS_LAUNCH_CHECK("swiglu");
+    return 0;
+  }
   const int blocks = (int)(ceil_div_ll(total, 256) < 8192 ? ceil_div_ll(total, 256) : 8192);
   if (dtype == RLIS_F32)
     swiglu_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gu, I, total);

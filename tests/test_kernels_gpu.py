@@ -55,7 +55,8 @@ def test_embed(ops, dtype, V, H, T):
 
 @pytest.mark.parametrize("out_dtype", DTYPES)
 @pytest.mark.parametrize("w_dtype", DTYPES)
-@pytest.mark.parametrize("T,H,eps", [(5, 100, 1e-5), (3, 2048, 1e-6), (2, 8192, 1e-5), (1, 7, 0.1)])
+@pytest.mark.parametrize("T,H,eps", [(5, 100, 1e-5), (3, 2048, 1e-6), (2, 8192, 1e-5), (1, 7, 0.1),
+                                     (4, 3072, 1e-5), (3, 4104, 1e-6), (2, 1000, 1e-5), (2, 8200, 1e-5)])
 def test_add_rmsnorm(ops, out_dtype, w_dtype, T, H, eps):
     resid = rnd(T, H, seed=1) * 3
     delta = rnd(T, H, dtype=out_dtype, seed=2)
@@ -100,7 +101,7 @@ def test_add_residual(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("T,I", [(3, 172), (17, 8192), (1, 5)])
+@pytest.mark.parametrize("T,I", [(3, 172), (17, 8192), (1, 5), (5, 1000), (300, 520)])
 def test_swiglu(ops, dtype, T, I):
     gu = rnd(T, 2 * I, dtype=dtype, scale=2.0)
     want = torch.nn.functional.silu(gu[:, :I].float()) * gu[:, I:].float()
