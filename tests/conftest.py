@@ -49,7 +49,17 @@ TINY_C = {
     "vocab_size": 331, "rms_norm_eps": 1e-5, "rope_theta": 10000.0, "rope_scaling": None,
     "max_position_embeddings": 512, "tie_word_embeddings": False,
 }
-TINY = {"a": TINY_A, "b": TINY_B, "c": TINY_C}
+# Head size 64 (the smallest for which the decode kernel rotates and stores by itself), a width
+# that is neither a power of two nor heads * head size, a prime vocabulary, frequency scaling.
+TINY_D = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 136, "intermediate_size": 200,
+    "num_hidden_layers": 2, "num_attention_heads": 6, "num_key_value_heads": 2, "head_dim": 64,
+    "vocab_size": 523, "rms_norm_eps": 1e-5, "rope_theta": 100000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 4.0, "low_freq_factor": 1.0,
+                     "high_freq_factor": 4.0, "original_max_position_embeddings": 32},
+    "max_position_embeddings": 256, "tie_word_embeddings": True,
+}
+TINY = {"a": TINY_A, "b": TINY_B, "c": TINY_C, "d": TINY_D}
 
 
 def make_model_folder(path, config, seed, dtype=torch.float32):
