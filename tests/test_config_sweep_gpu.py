@@ -1,0 +1,58 @@
+"""Configurations drawn at random within what config.json allows (head sizes in steps of 16, any
+number of heads and groups, widths and vocabularies that are no power of two or multiple of
+8), each replayed as a mixed trace with page reuse, in float32 and bfloat16, against the plain
+implementation.  The point is sizes that no hand-picked configuration happens to have."""
+import random
+
+import pytest
+import torch
+
+import plain_llama as plain
+import traces
+from conftest import make_model_folder
+from test_replay_gpu import TOL, check, make_runner
+
+pytestmark = pytest.mark.gpu
+
+
+def draw_config(seed: int) -> dict:
+    rng = random.Random(seed)
+    head_dim = rng.choice([16, 32, 48, 64, 80, 96, 112, 128])
+    kv = rng.choice([1, 2, 3, 4])
+    heads = kv * rng.choice([1, 2, 3, 4, 7])
+    scaling = None
+    if rng.random() < 0.5:
+        scaling = {"rope_type": "llama3", "factor": rng.choice([2.0, 8.0, 32.0]),
+                   "low_freq_factor": 1.0, "high_freq_factor": rng.choice([2.0, 4.0]),
+                   "original_max_position_embeddings": rng.choice([16, 64])}
+    return {
+        "architectures": ["LlamaForCausalLM"],
+        "hidden_size": rng.choice([36, 72, 100, 136, 200, 264, 328]) + rng.choice([0, 2, 4]),
+        "intermediate_size": rng.randrange(24, 400),
+        "num_hidden_layers": rng.choice([1, 2, 3]),
+        "num_attention_heads": heads, "num_key_value_heads": kv, "head_dim": head_dim,
+        "vocab_size": rng.randrange(50, 700),
+        "rms_norm_eps": rng.choice([1e-5, 1e-6, 1e-3]),
+        "rope_theta": rng.choice([10000.0, 500000.0, 1e6]),
+        "rope_scaling": scaling,
+        "max_position_embeddings": 160,
+        "tie_word_embeddings": rng.random() < 0.5,
+    }
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_configuration_mixed_trace(seed, tmp_path):
+    cfg = draw_config(seed)
+    lengths = [3, 40, 17, 70, 1, 130, 9]
+    for dtype, tdt in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
+        folder = make_model_folder(tmp_path / dtype, cfg, seed=seed, dtype=tdt)
+        w, c = plain.read_weights(folder), plain.read_config(folder)
+        reqs = traces.random_requests(cfg["vocab_size"], lengths, seed=seed + 1)
+        ref = {k: plain.forward(w, c, t) for k, t in reqs.items()}
+        steps, max_tokens = traces.trace_mixed(reqs, seed=seed)
+        runner = make_runner(folder, dtype, max_tokens, page_size=16)
+        outputs = traces.replay_in_process(runner, steps)
+        worst = check(steps, outputs, reqs, ref, cfg["vocab_size"], TOL[dtype])
+        print(f"seed {seed} {dtype}: {cfg['hidden_size']}x{cfg['num_attention_heads']}/"
+              f"{cfg['num_key_value_heads']}x{cfg['head_dim']} worst |diff| {worst:.3e}")
+        assert runner.cache.num_free_pages(0) == runner.cache.num_pages(0)
