@@ -458,72 +458,53 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
   for (int db = 0; db < D / 16; ++db) o_acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
   const float scale2 = scale * 1.4426950408889634f;
 
-  struct Chunk {
-    Frag8 k[2][D / 32];
-    Frag8 v[D / 16];
-  };
-  struct Pages {            // page of this lane's K row (two row blocks) and V keys (two halves)
-    int k[2], v[2];
-  };
-  auto load_pages = [&](int c0, Pages& pg) {
+  // A wave takes its chunks two at a time: the page ids of both, then all their keys and
+  // values, are on their way before the first product, and the page ids of the next two follow
+  // at once.  The loads are unconditional, so that the compiler can count them: a key past the
+  // end of the partition reads the last key in it instead (its score is masked, its
+  // probability exactly zero; values past the end inside a group of 4 keys are whatever the
+  // page holds, and the pages only ever hold zeros or values that a model wrote); a dim past d
+  // reads one below d (it meets a zero of q, or a row of O^T that is not stored).
+  const int last_key = kend - 1, last_quad = (kend - 1) & ~3;
+  int k_dim[D / 32], v_dim[D / 16];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int key = c0 + i * 16 + l16, key4 = c0 + i * 16 + lq * 4;
-      pg.k[i] = key < kend ? table[key >> page_shift] : 0;
-      pg.v[i] = key4 < kend ? table[key4 >> page_shift] : 0;
-    }
-  };
-  auto load_chunk = [&](int c0, const Pages& pg, Chunk& ch) {
+  for (int ks = 0; ks < D / 32; ++ks) k_dim[ks] = min(ks * 32 + lq * 8, d - 8);
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
-      const int key = c0 + nb * 16 + l16;
-      const bool ok = key < kend;
-      const bf16_t* kp =
-          k_pages + ((((long long)pg.k[nb] * nkv + kvh) << page_shift) + (key & page_mask)) * d;
-#pragma unroll
-      for (int ks = 0; ks < D / 32; ++ks) {
-        const int dim = ks * 32 + lq * 8;
-        ch.k[nb][ks].u = (ok && dim < d) ? *(const uint4*)(kp + dim) : make_uint4(0, 0, 0, 0);
-      }
-    }
-#pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      const int key4 = c0 + half * 16 + lq * 4;        // four keys, inside one page
-      const bool ok = key4 < kend;
-      const int off = key4 & page_mask;
-#pragma unroll
-      for (int db = 0; db < D / 16; ++db) {
-        const int dim = db * 16 + l16;
-        ch.v[db].h[half] = (ok && dim < d)
-            ? *(const uint2*)(v_pages + ((((long long)pg.v[half] * nkv + kvh) * d + dim) << page_shift) + off)
-            : make_uint2(0, 0);
-      }
-    }
-  };
-
-  int c0 = kbeg + wave * 32;
-  Chunk cur;
-  Pages pg_next;
-  if (c0 < kend) {
-    Pages pg;
-    load_pages(c0, pg);
-    load_chunk(c0, pg, cur);
-    load_pages(c0 + kStride, pg_next);
+  for (int db = 0; db < D / 16; ++db) v_dim[db] = min(db * 16 + l16, d - 1);
+  Frag8 k_a[2][D / 32], v_a[D / 16], k_b[2][D / 32], v_b[D / 16];
+  int pk_a[2], pv_a[2], pk_b[2], pv_b[2];
+#define RLIS_DEC_PAGES(c0_, PK, PV)                                                             \
+  {                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < 2; ++i) {                                             \
+      PK[i] = table[max(0, min((c0_) + i * 16 + l16, last_key)) >> page_shift];                 \
+      PV[i] = table[max(0, min((c0_) + i * 16 + lq * 4, last_quad)) >> page_shift];             \
+    }                                                                                           \
   }
-  for (; c0 < kend; c0 += kStride) {
-    Chunk nxt;
-    const bool more = c0 + kStride < kend;
-    if (more) {
-      load_chunk(c0 + kStride, pg_next, nxt);
-      load_pages(c0 + 2 * kStride, pg_next);
-    }
+#define RLIS_DEC_CHUNK(c0_, PK, PV, KF, VF)                                                     \
+  {                                                                                             \
+    _Pragma("unroll") for (int nb = 0; nb < 2; ++nb) {                                          \
+      const int key_ = max(0, min((c0_) + nb * 16 + l16, last_key));                            \
+      const bf16_t* kp_ =                                                                       \
+          k_pages + ((((long long)PK[nb] * nkv + kvh) << page_shift) + (key_ & page_mask)) * d; \
+      _Pragma("unroll") for (int ks = 0; ks < D / 32; ++ks)                                     \
+          KF[nb][ks].u = *(const uint4*)(kp_ + k_dim[ks]);                                      \
+    }                                                                                           \
+    _Pragma("unroll") for (int hf = 0; hf < 2; ++hf) {                                          \
+      const int off_ = max(0, min((c0_) + hf * 16 + lq * 4, last_quad)) & page_mask;            \
+      const bf16_t* vp_ = v_pages + ((((long long)PV[hf] * nkv + kvh) * d) << page_shift) + off_; \
+      _Pragma("unroll") for (int db = 0; db < D / 16; ++db)                                     \
+          VF[db].h[hf] = *(const uint2*)(vp_ + ((long long)v_dim[db] << page_shift));           \
+    }                                                                                           \
+  }
+  auto compute = [&](int c0, const Frag8 (&kf)[2][D / 32], const Frag8 (&vf)[D / 16])
+                     __attribute__((always_inline)) {
     f32x4 s[2];
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
       s[nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < D / 32; ++ks)
-        s[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[nb][ks].v, qf[ks].v, s[nb], 0, 0, 0);
+        s[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[nb][ks].v, qf[ks].v, s[nb], 0, 0, 0);
     }
     float mx = -INFINITY;
 #pragma unroll
@@ -559,12 +540,35 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
       if (db * 16 < d) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) o_acc[db][r] *= corr;
-        // keys whose values were never loaded (beyond kend) have p = 0 and zero fragments
-        o_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.v[db].v, pf, o_acc[db], 0, 0, 0);
+        o_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db].v, pf, o_acc[db], 0, 0, 0);
       }
     }
-    if (more) cur = nxt;
+  };
+
+  int c0 = kbeg + wave * 32;
+  if (part <= kStride) {
+    // At most one chunk for every wave of the workgroup.
+    if (c0 < kend) {
+      RLIS_DEC_PAGES(c0, pk_a, pv_a);
+      RLIS_DEC_CHUNK(c0, pk_a, pv_a, k_a, v_a);
+      compute(c0, k_a, v_a);
+    }
+  } else {
+    if (c0 < kend) {
+      RLIS_DEC_PAGES(c0, pk_a, pv_a);
+      RLIS_DEC_PAGES(c0 + kStride, pk_b, pv_b);
+    }
+    for (; c0 < kend; c0 += 2 * kStride) {
+      RLIS_DEC_CHUNK(c0, pk_a, pv_a, k_a, v_a);
+      RLIS_DEC_CHUNK(c0 + kStride, pk_b, pv_b, k_b, v_b);
+      RLIS_DEC_PAGES(c0 + 2 * kStride, pk_a, pv_a);
+      RLIS_DEC_PAGES(c0 + 3 * kStride, pk_b, pv_b);
+      compute(c0, k_a, v_a);
+      if (c0 + kStride < kend) compute(c0 + kStride, k_b, v_b);
+    }
   }
+#undef RLIS_DEC_CHUNK
+#undef RLIS_DEC_PAGES
 
   // ---- merge the waves (in wave order), then store the partition ------------------
   float* ml_s = dsm;                       // [wave][head][2]
