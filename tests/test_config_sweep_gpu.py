@@ -56,3 +56,44 @@ def test_random_configuration_mixed_trace(seed, tmp_path):
         print(f"seed {seed} {dtype}: {cfg['hidden_size']}x{cfg['num_attention_heads']}/"
               f"{cfg['num_key_value_heads']}x{cfg['head_dim']} worst |diff| {worst:.3e}")
         assert runner.cache.num_free_pages(0) == runner.cache.num_pages(0)
+
+
+# Layer sizes of the larger shapes the engine is meant for (Llama-3.2-3B and Llama-3.1-8B), with
+# one layer and a small vocabulary so that the plain implementation stays quick: widths of 12
+# and 16 k items, a feed-forward width that takes two k slices, head size 128.
+LARGE_LAYERS = {
+    "3b-layer": dict(hidden_size=3072, intermediate_size=8192, num_attention_heads=24,
+                     num_key_value_heads=8, head_dim=128, factor=32.0, tie=True),
+    "8b-layer": dict(hidden_size=4096, intermediate_size=14336, num_attention_heads=32,
+                     num_key_value_heads=8, head_dim=128, factor=8.0, tie=False),
+}
+
+
+@pytest.mark.parametrize("name", sorted(LARGE_LAYERS))
+def test_layer_sizes_of_larger_models(name, tmp_path):
+    p = LARGE_LAYERS[name]
+    cfg = {
+        "architectures": ["LlamaForCausalLM"], "hidden_size": p["hidden_size"],
+        "intermediate_size": p["intermediate_size"], "num_hidden_layers": 1,
+        "num_attention_heads": p["num_attention_heads"],
+        "num_key_value_heads": p["num_key_value_heads"], "head_dim": p["head_dim"],
+        "vocab_size": 1000, "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
+        "rope_scaling": {"rope_type": "llama3", "factor": p["factor"], "low_freq_factor": 1.0,
+                         "high_freq_factor": 4.0, "original_max_position_embeddings": 8192},
+        "max_position_embeddings": 128, "tie_word_embeddings": p["tie"],
+    }
+    folder = make_model_folder(tmp_path / "m", cfg, seed=11, dtype=torch.bfloat16)
+    w, c = plain.read_weights(folder), plain.read_config(folder)
+    reqs = traces.random_requests(cfg["vocab_size"], [70, 9, 40], seed=5)
+    ref = {k: plain.forward(w, c, t) for k, t in reqs.items()}
+    spread = max(r.abs().max().item() for r in ref.values())
+    for dtype in ("float32", "bfloat16"):
+        # The gates of the tiny models are absolute, for logits of about +-1; these logits are
+        # larger, so the gates go with their size.
+        tol = TOL[dtype] * max(1.0, spread)
+        for build in (traces.trace_tail, traces.trace_mixed):
+            steps, max_tokens = build(reqs)
+            runner = make_runner(folder, dtype, max_tokens, page_size=16)
+            outputs = traces.replay_in_process(runner, steps)
+            worst = check(steps, outputs, reqs, ref, cfg["vocab_size"], tol)
+            print(f"{name} {dtype} {build.__name__}: worst |diff| {worst:.3e}, largest |logit| {spread:.2f}")
