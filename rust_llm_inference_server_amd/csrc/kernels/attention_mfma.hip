@@ -33,6 +33,7 @@
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // 16 bytes in flight, a plain vector
 
 union Frag8 {
   uint4 u;
@@ -141,7 +142,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) voi
   const int last_key = khi - 1, last_group = (khi - 1) & ~7;
   // Two sets of staging registers (A, B) and of page ids; plain arrays and macros, so that they
   // stay in registers.
-  uint4 tile_ka[KCH], tile_va[VCH], tile_kb[KCH], tile_vb[VCH];
+  u32x4 tile_ka[KCH], tile_va[VCH], tile_kb[KCH], tile_vb[VCH];
   int page_ka[KCH], page_va[VCH], page_kb[KCH], page_vb[VCH];
 #define RLIS_LOAD_PAGES(k0_, PK, PV)                                                           \
   {                                                                                            \
@@ -154,13 +155,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) voi
   {                                                                                            \
     _Pragma("unroll") for (int i = 0; i < KCH; ++i) {                                          \
       const int off_ = max(0, min((k0_) + k_key[i], last_key)) & page_mask;                    \
-      TK[i] = *(const uint4*)(k_pages +                                                        \
+      TK[i] = *(const u32x4*)(k_pages +                                                        \
                               ((((long long)PK[i] * nkv + kvh) << page_shift) + off_) * d +    \
                               k_dim[i]);                                                       \
     }                                                                                          \
     _Pragma("unroll") for (int i = 0; i < VCH; ++i) {                                          \
       const int off_ = max(0, min((k0_) + v_key[i], last_group)) & page_mask;                  \
-      TV[i] = *(const uint4*)(v_pages +                                                        \
+      TV[i] = *(const u32x4*)(v_pages +                                                        \
                               ((((long long)PV[i] * nkv + kvh) * d + v_dim[i]) << page_shift) + \
                               off_);                                                           \
     }                                                                                          \
@@ -169,11 +170,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) voi
   {                                                                                            \
     _Pragma("unroll") for (int i = 0; i < KCH; ++i) {                                          \
       const int c_ = tid + i * 256;                                                            \
-      if (c_ < K_CHUNKS) *(uint4*)(Ks + (c_ / (D / 8)) * KS + (c_ % (D / 8)) * 8) = TK[i];     \
+      if (c_ < K_CHUNKS) *(u32x4*)(Ks + (c_ / (D / 8)) * KS + (c_ % (D / 8)) * 8) = TK[i];     \
     }                                                                                          \
     _Pragma("unroll") for (int i = 0; i < VCH; ++i) {                                          \
       const int c_ = tid + i * 256;                                                            \
-      if (c_ < v_chunks) *(uint4*)(Vs + (c_ / (BN / 8)) * VS + (c_ % (BN / 8)) * 8) = TV[i];   \
+      if (c_ < v_chunks) *(u32x4*)(Vs + (c_ / (BN / 8)) * VS + (c_ % (BN / 8)) * 8) = TV[i];   \
     }                                                                                          \
   }
 
