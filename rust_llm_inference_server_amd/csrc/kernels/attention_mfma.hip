@@ -547,14 +547,15 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
   };
 
   int c0 = kbeg + wave * 32;
-  if (part <= kStride) {
-    // At most one chunk for every wave of the workgroup.
-    if (c0 < kend) {
+  constexpr bool kPairs = D <= 128;      // wider heads have no registers for two chunks
+  if (part <= kStride || !kPairs) {
+    // One chunk at a time: at most one for every wave of the workgroup, or a wide head.
+    for (; c0 < kend; c0 += kStride) {
       RLIS_DEC_PAGES(c0, pk_a, pv_a);
       RLIS_DEC_CHUNK(c0, pk_a, pv_a, k_a, v_a);
       compute(c0, k_a, v_a);
     }
-  } else {
+  } else if constexpr (kPairs) {
     if (c0 < kend) {
       RLIS_DEC_PAGES(c0, pk_a, pv_a);
       RLIS_DEC_PAGES(c0 + kStride, pk_b, pv_b);
