@@ -30,6 +30,9 @@ HIP_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-fPIC", "-std=c++17", "-fvisibility=hidden",
     # Packed float32 forms are kept out of the generated code.
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # Matrix-core results go to ordinary vector registers: the softmax and the epilogues read
+    # them with vector instructions, and copies out of the accumulator file cost as much.
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wno-unused-command-line-argument",
 ]
 CXX_FLAGS = ["-O2", "-fPIC", "-std=c++17", "-fvisibility=hidden", "-Wall"]

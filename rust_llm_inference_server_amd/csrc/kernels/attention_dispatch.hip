@@ -35,6 +35,7 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
   (void)reserved;
   RLIS_REQUIRE(num_tiles >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0,
                "attn_prefill_mfma: bad sizes");
+  RLIS_REQUIRE(scale > 0.f, "attn_prefill_mfma: the score scale must be positive, got %g", scale);
   RLIS_REQUIRE(nh % nkv == 0, "attn_prefill_mfma: %d query heads are not a multiple of %d KV heads",
                nh, nkv);
   RLIS_REQUIRE(d % 16 == 0 && d <= 256,
@@ -95,6 +96,7 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
                "attn_decode_mfma: k and v columns %lld, %lld do not fit rows of %lld", k_off,
                v_off, q_stride);
   RLIS_REQUIRE(S >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0, "attn_decode_mfma: bad sizes");
+  RLIS_REQUIRE(scale > 0.f, "attn_decode_mfma: the score scale must be positive, got %g", scale);
   RLIS_REQUIRE(nh % nkv == 0 && nh / nkv <= 16,
                "attn_decode_mfma: %d query heads per KV head, at most 16", nkv ? nh / nkv : 0);
   RLIS_REQUIRE(d % 16 == 0 && d <= 256,

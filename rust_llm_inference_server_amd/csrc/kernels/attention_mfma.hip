@@ -211,15 +211,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) voi
       // ---- scale, mask (only where a tile meets the diagonal, the window or the end) -----
       const bool plain_tile = (k0 + BN - 1 <= P + wave_q_first) &&
                               (window <= 0 || k0 > P + wave_q_first + 15 - window);
+      // The scale (positive) is applied inside the exponent, with one fused multiply-add per
+      // score; the maximum is taken over the raw scores and scaled once.
       float mx = -INFINITY;
       if (plain_tile) {
 #pragma unroll
         for (int nb = 0; nb < BN / 16; ++nb)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            s[nb][r] *= scale2;
-            mx = fmaxf(mx, s[nb][r]);
-          }
+          for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[nb][r]);
       } else {
 #pragma unroll
         for (int nb = 0; nb < BN / 16; ++nb)
@@ -227,14 +226,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) voi
           for (int r = 0; r < 4; ++r) {
             const int kpos = k0 + nb * 16 + lq * 4 + r;
             const bool ok = (kpos <= my_qpos) && (window <= 0 || kpos > my_qpos - window);
-            const float sv = ok ? s[nb][r] * scale2 : -INFINITY;
+            const float sv = ok ? s[nb][r] : -INFINITY;
             s[nb][r] = sv;
             mx = fmaxf(mx, sv);
           }
       }
       mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
       mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-      const float m_new = fmaxf(m_run, mx);
+      const float m_new = fmaxf(m_run, mx * scale2);             // -inf stays -inf
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;   // a query with no key yet
       const float corr = __builtin_amdgcn_exp2f(m_run - m_safe);  // 0 when m_run is -inf
       float sum = 0.f;
@@ -242,7 +241,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) voi
       for (int nb = 0; nb < BN / 16; ++nb)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const float p = __builtin_amdgcn_exp2f(s[nb][r] - m_safe);   // exp2(-inf) = 0
+          const float p = __builtin_amdgcn_exp2f(fmaf(s[nb][r], scale2, -m_safe));  // exp2(-inf) = 0
           s[nb][r] = p;
           sum += p;
         }
@@ -513,13 +512,13 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int key = c0 + nb * 16 + lq * 4 + r;
-        const float sv = (key >= lo && key < kend) ? s[nb][r] * scale2 : -INFINITY;
+        const float sv = (key >= lo && key < kend) ? s[nb][r] : -INFINITY;
         s[nb][r] = sv;
         mx = fmaxf(mx, sv);
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
     mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-    const float m_new = fmaxf(m_run, mx);
+    const float m_new = fmaxf(m_run, mx * scale2);    // scale2 > 0; -inf stays -inf
     const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
     const float corr = __builtin_amdgcn_exp2f(m_run - m_safe);
     float sum = 0.f;
@@ -528,7 +527,7 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
     for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float p = __builtin_amdgcn_exp2f(s[nb][r] - m_safe);
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[nb][r], scale2, -m_safe));
         sum += p;
         pf[nb * 4 + r] = (__bf16)p;
       }
