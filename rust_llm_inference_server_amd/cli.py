@@ -17,14 +17,24 @@ import sys
 import tempfile
 from typing import List, Optional
 
-_DTYPES = {"f32": "float32", "float32": "float32", "bf16": "bfloat16", "bfloat16": "bfloat16"}
+_DTYPES = {"f32": "float32", "fp32": "float32", "float32": "float32",
+           "bf16": "bfloat16", "bfloat16": "bfloat16"}
+
+
+def _dtype(name: str) -> str:
+    if name in ("f16", "fp16", "float16", "half"):
+        raise argparse.ArgumentTypeError(
+            "f16 (the reference's default) is not built here: use bf16 or f32")
+    if name not in _DTYPES:
+        raise argparse.ArgumentTypeError(f"unknown dtype '{name}': one of {', '.join(sorted(_DTYPES))}")
+    return name
 
 
 def _add_model_args(p: argparse.ArgumentParser) -> None:
     p.add_argument("--model", help="a folder with config.json and *.safetensors")
     p.add_argument("--tokenizer", help="folder with tokenizer.json (needed for text prompts)")
-    p.add_argument("--dtype", default="bf16", choices=sorted(_DTYPES),
-                   help="weight and activation dtype (default bf16)")
+    p.add_argument("--dtype", default="bf16", type=_dtype,
+                   help="weight and activation dtype: bf16 (default) or f32 / fp32")
     p.add_argument("--device", default="hip", help="'hip' (the GPU); there is no CPU path")
     p.add_argument("--max-seq-len", type=int, default=2048,
                    help="longest prompt plus completion, in tokens")
@@ -37,7 +47,8 @@ def _add_model_args(p: argparse.ArgumentParser) -> None:
 def _add_engine_args(p: argparse.ArgumentParser) -> None:
     p.add_argument("--kv-cache-gb", type=float, default=1.0, help="size of the page pool")
     p.add_argument("--num-pages", type=int, default=None, help="pool size in pages, overrides --kv-cache-gb")
-    p.add_argument("--block-size", type=int, default=16, help="tokens per page")
+    p.add_argument("--block-size", "--page-size", dest="block_size", type=int, default=16,
+                   help="tokens per page")
     p.add_argument("--max-num-seqs", type=int, default=64, help="most sequences in one step")
     p.add_argument("--max-batched-tokens", type=int, default=2048,
                    help="most tokens in one step; longer prompts are prefilled in portions")
@@ -175,7 +186,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     p.add_argument("--bos", type=int, default=None, help="BOS id put at the start of each window")
     p.add_argument("--ctx", type=int, default=512, help="window length; the second half is scored")
     p.add_argument("--max-windows", type=int, default=0, help="score only the first N windows (0 = all)")
-    p.add_argument("--block-size", type=int, default=16)
+    p.add_argument("--block-size", "--page-size", dest="block_size", type=int, default=16)
     args = ap.parse_args(argv)
     return run_generate(args) if args.command == "generate" else run_perplexity(args)
 

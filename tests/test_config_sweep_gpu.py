@@ -97,3 +97,26 @@ def test_layer_sizes_of_larger_models(name, tmp_path):
             outputs = traces.replay_in_process(runner, steps)
             worst = check(steps, outputs, reqs, ref, cfg["vocab_size"], tol)
             print(f"{name} {dtype} {build.__name__}: worst |diff| {worst:.3e}, largest |logit| {spread:.2f}")
+
+
+def test_whole_llama_1b_shape(tmp_path):
+    """All 16 layers of the Llama-3.2-1B shape with random weights: the 32-bit path within the
+    reference's gate for its own parity run (1e-4), bfloat16 within the gate scaled by the size of
+    these logits, for the tail-decoded and the mixed trace."""
+    from rust_llm_inference_server_amd.config import preset_dict
+    cfg = preset_dict("llama-3.2-1b")
+    cfg["max_position_embeddings"] = 256
+    folder = make_model_folder(tmp_path / "m", cfg, seed=0, dtype=torch.bfloat16)
+    w, c = plain.read_weights(folder), plain.read_config(folder)
+    reqs = traces.random_requests(cfg["vocab_size"], [48, 9, 33], seed=5)
+    ref = {k: plain.forward(w, c, t) for k, t in reqs.items()}
+    spread = max(r.abs().max().item() for r in ref.values())
+    for dtype, tol in (("float32", TOL["float32"]), ("bfloat16", TOL["bfloat16"] * max(1.0, spread))):
+        for build in (traces.trace_tail, traces.trace_mixed):
+            steps, max_tokens = build(reqs)
+            runner = make_runner(folder, dtype, max_tokens, page_size=16)
+            outputs = traces.replay_in_process(runner, steps)
+            worst = check(steps, outputs, reqs, ref, cfg["vocab_size"], tol)
+            print(f"1b {dtype} {build.__name__}: worst |diff| {worst:.3e}, largest |logit| {spread:.2f}")
+            del runner
+            torch.cuda.empty_cache()
