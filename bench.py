@@ -11,6 +11,7 @@ fraction of the bf16 matrix peak, the decode step's achieved fraction of the HBM
 throughput at batch 1 and 64 after 512-token prompts.  Weights are random (N(0, 0.02)),
 prompts are uniform random token ids."""
 import argparse
+import copy
 import json
 import os
 import sys
@@ -76,27 +77,38 @@ def main() -> int:
         return [torch.randint(0, V, (length,), generator=g).tolist() for _ in range(n)]
 
     def decode_run(batch, context, steps, warmup):
-        """tokens/s and ms/step of `steps` decode steps whose last one reaches `context`."""
-        prompt_len = context - (steps + warmup)
+        """tokens/s and ms/step of `steps` decode steps of `batch` requests, none of which goes
+        beyond `context`.  Prompts are prefilled in portions under the engine's token budget
+        while earlier requests already decode, so every request is given room for the steps
+        that the prefill of the others takes; the timed steps are pure decode steps."""
+        budget = max(args.max_batched_tokens, batch)
+        prefill_steps = -(-batch * context // budget) + 1
+        new_tokens = steps + warmup + prefill_steps + 1
+        prompt_len = max(1, context - new_tokens)
         pages = batch * (-(-context // page) + 1) + 8
-        engine = Engine(model, EngineConfig(max_num_seqs=max(batch, 1),
-                                            max_batched_tokens=max(args.max_batched_tokens, batch),
+        engine = Engine(model, EngineConfig(max_num_seqs=max(batch, 1), max_batched_tokens=budget,
                                             num_pages=pages, block_size=page,
                                             max_seq_len=context + 8, watermark_pages=0))
-        sp = SamplingParams(max_tokens=steps + warmup + 1, ignore_eos=True)
+        sp = SamplingParams(max_tokens=new_tokens, ignore_eos=True)
         for p in prompts(batch, prompt_len):
             engine.add_request(p, sp)
-        while engine.stats().generated_tokens < batch:       # prefill, in portions
-            engine.step()
-        for _ in range(warmup - 1):
+        while engine.stats().prefill_tokens < batch * prompt_len or engine.stats().waiting:
+            engine.step()                                     # prefill, in portions
+        for _ in range(warmup):
             engine.step()
         torch.cuda.synchronize()
+        before = copy.copy(engine.stats())
         t0 = time.perf_counter()
         for _ in range(steps):
             engine.step()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        mean_ctx = context - steps / 2
+        after = copy.copy(engine.stats())
+        if (after.generated_tokens - before.generated_tokens != batch * steps
+                or after.prefill_tokens != before.prefill_tokens
+                or after.preemptions != before.preemptions):
+            raise RuntimeError("the timed steps were not pure decode steps of the whole batch")
+        mean_ctx = prompt_len + (before.generated_tokens + after.generated_tokens) / 2 / batch
         return batch * steps / dt, dt / steps * 1e3, mean_ctx
 
     # ---- prefill: one prompt of T tokens in one step, last-row logits ------------------
@@ -141,7 +153,7 @@ def main() -> int:
             print(f"[bench] decode b{b}: {v:.0f} tok/s, {ms:.3f} ms/step", file=sys.stderr, flush=True)
 
     print(json.dumps({
-        "metric": "decode tok/s at batch 8 (Llama-3.2-1B shape)", "value": round(value, 1),
+        "metric": f"decode tok/s at batch {args.batch} ({args.model} shape)", "value": round(value, 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",

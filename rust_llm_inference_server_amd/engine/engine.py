@@ -178,10 +178,11 @@ class Engine:
         row = 0
         for (seq_id, start, end), last in zip(sched.seqs, final):
             self.scheduler.advance(seq_id, end)
-            if not last:
-                self.stats_.prefill_tokens += end - start
-                continue
             seq = self._seqs[seq_id]
+            # prompt tokens of this portion (recomputed ones after a preemption count again)
+            self.stats_.prefill_tokens += max(0, min(end, seq.prompt_len) - start)
+            if not last:
+                continue
             mode = seq.sampler.device_mode(len(seq.tokens))
             if mode is not None:
                 device_rows.append((row, seq_id))
