@@ -609,6 +609,65 @@ def test_copy_pages(ops, dtype):
     torch.testing.assert_close(pages, want, atol=0, rtol=0)
 
 
+# ------------------------------------------------------------------ large pools
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_pages_past_two_to_the_31_elements(ops, dtype):
+    """A pool whose last pages start beyond element 2^31 of the K and V arrays (a few GB per
+    layer, small on a 288 GB card): cache write, the three attention kernels and the page copy
+    give bit for bit what they give for the same pages at the start of a small pool."""
+    nh, nkv, d, ps = 8, 8, 64, 16
+    cached, new = [0, 40, 130, 17, 300], [33, 2, 70, 1, 1]
+    scale = 1.0 / math.sqrt(d)
+    qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=2)
+    small = kp.shape[0]
+    big = (1 << 31) // (nkv * ps * d) + small + 5
+    shift = big - small
+    kb = torch.empty(big, nkv, ps, d, dtype=dtype, device=DEV)
+    vb = torch.empty(big, nkv, d, ps, dtype=dtype, device=DEV)
+    assert kb[shift:].storage_offset() > (1 << 31)
+    kb[shift:], vb[shift:] = kp, vp
+    bt_big = bt + shift
+    inv = plain.inv_freqs(d, 10000.0, None)
+    cos, sin = (t.to(DEV) for t in plain.rope_tables(inv, range(512)))
+    tables = bt.cpu()
+    pos = step.positions.cpu().tolist()
+    seq = step.seq_of_token.cpu().tolist()
+    slots = torch.tensor([int(tables[s, p // ps]) * ps + p % ps for s, p in zip(seq, pos)],
+                         dtype=torch.int32, device=DEV)
+    q_small, q_big = qkv.clone(), qkv.clone()
+    ops.rope_kv_write(q_small, nh, nkv, d, cos, sin, step.positions, slots, kp, vp, ps)
+    ops.rope_kv_write(q_big, nh, nkv, d, cos, sin, step.positions, slots + shift * ps, kb, vb, ps)
+    assert torch.equal(q_small, q_big)
+    assert torch.equal(kb[shift:], kp) and torch.equal(vb[shift:], vp)
+    kinds = ["generic"] + (["prefill"] if dtype == torch.bfloat16 else [])
+    for kind in kinds:
+        a = ops.paged_attention(q_small, nh, nkv, d, kp, vp, ps, bt, step, scale, None, force=kind)
+        b = ops.paged_attention(q_big, nh, nkv, d, kb, vb, ps, bt_big, step, scale, None, force=kind)
+        assert torch.equal(a, b), kind
+    # single tokens: the decode kernels, with and without the rotation and cache write inside
+    lens = [c + n for c, n in zip(cached, new)]
+    dq, _, _, _, dstep, *_ = paged_case([l - 1 for l in lens], [1] * len(lens), nh, nkv, d, ps, dtype, seed=3)
+    dstep.decode_splits = 3
+    a = ops.paged_attention(dq, nh, nkv, d, kp, vp, ps, bt, dstep, scale, None, force="decode")
+    b = ops.paged_attention(dq, nh, nkv, d, kb, vb, ps, bt_big, dstep, scale, None, force="decode")
+    assert torch.equal(a, b)
+    dslots = torch.tensor([int(tables[s, (l - 1) // ps]) * ps + (l - 1) % ps for s, l in enumerate(lens)],
+                          dtype=torch.int32, device=DEV)
+    a = ops.rope_attention(dq.clone(), nh, nkv, d, cos, sin, dstep.positions, dslots, kp, vp, ps, bt,
+                           dstep, scale, None)
+    b = ops.rope_attention(dq.clone(), nh, nkv, d, cos, sin, dstep.positions, dslots + shift * ps, kb, vb,
+                           ps, bt_big, dstep, scale, None)
+    assert torch.equal(a, b)
+    assert torch.equal(kb[shift:], kp) and torch.equal(vb[shift:], vp)
+    # page copy to and from the far end
+    pool = kb.reshape(1, big, -1)
+    src = torch.tensor([shift + 1, 0], dtype=torch.int32, device=DEV)
+    dst = torch.tensor([2, big - 1], dtype=torch.int32, device=DEV)
+    first, far = pool[0, 0].clone(), pool[0, shift + 1].clone()
+    ops.copy_pages(pool, src, dst)
+    assert torch.equal(pool[0, 2], far) and torch.equal(pool[0, big - 1], first)
+
+
 # ----------------------------------------------------------------- refusals
 def test_kernels_refuse_what_they_cannot_do(ops):
     with pytest.raises(ops.KernelError):
