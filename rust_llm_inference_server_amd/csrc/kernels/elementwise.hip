@@ -410,6 +410,118 @@ __global__ void rope_kv_write_kernel(TX* __restrict__ qkv, long long row_stride,
   }
 }
 
+// bfloat16 with every head segment a multiple of 8 wide: 16-byte accesses.  The first
+// `qk_blocks` workgroups rotate q in place and k into its page, kRopeTokQK tokens each; the
+// others take kRopeTokV tokens each and turn their v rows through LDS, so that lanes which are
+// neighbours in a page's (d, offset) layout store neighbouring offsets (tokens with adjacent
+// slots fill whole 32-byte runs, whatever their alignment).
+constexpr int kRopeTokQK = 2;
+constexpr int kRopeTokV = 16;
+constexpr int kRopeVCols = 1024;               // v columns staged per pass
+constexpr int kRopeVRow = kRopeVCols + 8;      // padded: rows stay 16-byte aligned, banks spread
+
+__device__ __forceinline__ void unpack8(const uint4 u, float (&v)[8]) {
+  const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = __uint_as_float(w[i] << 16);
+    v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+__device__ __forceinline__ uint4 pack8(const float (&v)[8]) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    w[i] = (uint32_t)f32_to_bf16(v[2 * i]) | ((uint32_t)f32_to_bf16(v[2 * i + 1]) << 16);
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+__global__ __launch_bounds__(256) void rope_kv_write_bf16x8_kernel(
+    bf16_t* __restrict__ qkv, long long row_stride, int k_off, int v_off, int T, int nh, int nkv,
+    int d, int rot_dim, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int* __restrict__ positions, const int* __restrict__ slots,
+    bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages, int page_size, int write_kv,
+    int qk_blocks) {
+  const int tid = threadIdx.x;
+  const int half = rot_dim / 2;
+  if ((int)blockIdx.x < qk_blocks) {
+    const int t0 = blockIdx.x * kRopeTokQK;
+    const int hc = half / 8;                             // chunks of 8 pairs per head
+    const int heads = nh + (write_kv ? nkv : 0);
+    const int per_tok = heads * hc;
+    for (int i = tid; i < kRopeTokQK * per_tok; i += blockDim.x) {
+      const int tt = i / per_tok, r = i - tt * per_tok, t = t0 + tt;
+      if (t >= T) break;
+      const int h = r / hc, j = (r - h * hc) * 8;
+      const bool is_k = h >= nh;
+      const int slot = is_k ? slots[t] : 0;
+      if (slot < 0) continue;
+      bf16_t* src = qkv + (long long)t * row_stride + (is_k ? k_off + (h - nh) * d : h * d);
+      bf16_t* dst = src;
+      if (is_k) {
+        const long long page = slot / page_size;
+        const int off = slot - (int)page * page_size;
+        dst = k_pages + ((page * nkv + (h - nh)) * page_size + off) * d;
+      }
+      const long long cs = (long long)positions[t] * half + j;
+      float x1[8], x2[8], c[8], s[8], o1[8], o2[8];
+      unpack8(*(const uint4*)(src + j), x1);
+      unpack8(*(const uint4*)(src + j + half), x2);
+      *(float4*)&c[0] = *(const float4*)(cos_t + cs);
+      *(float4*)&c[4] = *(const float4*)(cos_t + cs + 4);
+      *(float4*)&s[0] = *(const float4*)(sin_t + cs);
+      *(float4*)&s[4] = *(const float4*)(sin_t + cs + 4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        o1[e] = x1[e] * c[e] - x2[e] * s[e];
+        o2[e] = x2[e] * c[e] + x1[e] * s[e];
+      }
+      *(uint4*)(dst + j) = pack8(o1);
+      *(uint4*)(dst + j + half) = pack8(o2);
+    }
+    if (write_kv && d > rot_dim) {                       // the dims of k that are not rotated
+      const int tc = (d - rot_dim) / 8, per = nkv * tc;
+      for (int i = tid; i < kRopeTokQK * per; i += blockDim.x) {
+        const int tt = i / per, r = i - tt * per, t = t0 + tt;
+        if (t >= T) break;
+        const int h = r / tc, j = rot_dim + (r - h * tc) * 8;
+        const int slot = slots[t];
+        if (slot < 0) continue;
+        const long long page = slot / page_size;
+        const int off = slot - (int)page * page_size;
+        *(uint4*)(k_pages + ((page * nkv + h) * page_size + off) * d + j) =
+            *(const uint4*)(qkv + (long long)t * row_stride + k_off + h * d + j);
+      }
+    }
+    return;
+  }
+  __shared__ __attribute__((aligned(16))) bf16_t v_s[kRopeTokV * kRopeVRow];
+  __shared__ int slot_s[kRopeTokV];
+  const int t0 = ((int)blockIdx.x - qk_blocks) * kRopeTokV;
+  if (tid < kRopeTokV) slot_s[tid] = t0 + tid < T ? slots[t0 + tid] : -1;
+  const int cols = nkv * d;
+  for (int c0 = 0; c0 < cols; c0 += kRopeVCols) {
+    const int nc = min(kRopeVCols, cols - c0), nc8 = nc / 8;
+    __syncthreads();                                     // slots are there; the tile is free
+    for (int i = tid; i < kRopeTokV * nc8; i += blockDim.x) {
+      const int tt = i / nc8, c = (i - tt * nc8) * 8;
+      if (t0 + tt < T)
+        *(uint4*)(v_s + tt * kRopeVRow + c) =
+            *(const uint4*)(qkv + (long long)(t0 + tt) * row_stride + v_off + c0 + c);
+    }
+    __syncthreads();
+    for (int i = tid; i < kRopeTokV * nc; i += blockDim.x) {
+      const int tt = i % kRopeTokV, c = i / kRopeTokV;
+      const int slot = slot_s[tt];
+      if (slot < 0) continue;
+      const int col = c0 + c, h = col / d, j = col - h * d;
+      const long long page = slot / page_size;
+      const int off = slot - (int)page * page_size;
+      v_pages[((page * nkv + h) * d + j) * page_size + off] = v_s[tt * kRopeVRow + c];
+    }
+  }
+}
+
 RLIS_API int rlis_rope_kv_write(void* qkv, int dtype, long long row_stride, int k_off, int v_off,
                                 int T, int nh, int nkv, int d, int rot_dim, const float* cos_t,
                                 const float* sin_t, const int* positions, const int* slots,
@@ -421,6 +533,19 @@ RLIS_API int rlis_rope_kv_write(void* qkv, int dtype, long long row_stride, int 
   RLIS_REQUIRE(!write_kv || (page_size > 0 && k_pages && v_pages && slots),
                "rope_kv_write: cache write asked for without pages");
   if (T == 0) return 0;
+  const bool by8 = dtype == RLIS_BF16 && d % 8 == 0 && rot_dim % 16 == 0 && row_stride % 8 == 0 &&
+                   k_off % 8 == 0 && v_off % 8 == 0 && ((uintptr_t)qkv % 16) == 0 &&
+                   ((uintptr_t)cos_t % 16) == 0 && ((uintptr_t)sin_t % 16) == 0 &&
+                   (!write_kv || (((uintptr_t)k_pages % 16) == 0 && T <= (1 << 30)));
+  if (by8) {
+    const int qk_blocks = ceil_div(T, kRopeTokQK);
+    const int v_blocks = write_kv ? ceil_div(T, kRopeTokV) : 0;
+    rope_kv_write_bf16x8_kernel<<<qk_blocks + v_blocks, 256, 0, stream>>>(
+        (bf16_t*)qkv, row_stride, k_off, v_off, T, nh, nkv, d, rot_dim, cos_t, sin_t, positions,
+        slots, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, write_kv, qk_blocks);
+    RLIS_LAUNCH_CHECK("rope_kv_write");
+    return 0;
+  }
   if (dtype == RLIS_F32)
     rope_kv_write_kernel<float><<<T, 256, 0, stream>>>(
         (float*)qkv, row_stride, k_off, v_off, nh, nkv, d, rot_dim, cos_t, sin_t, positions,

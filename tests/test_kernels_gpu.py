@@ -281,27 +281,44 @@ def test_linear_rows_do_not_depend_on_the_batch(ops):
 
 # ---------------------------------------------------------- rotation + cache write
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T", [11, 77])
 @pytest.mark.parametrize("nh,nkv,d,rot,ps", [(4, 1, 16, 16, 16), (6, 2, 32, 32, 8), (5, 5, 48, 48, 16),
-                                              (3, 1, 80, 40, 32), (32, 8, 64, 64, 16)])
-def test_rope_kv_write(ops, dtype, nh, nkv, d, rot, ps):
-    T, pages = 11, 9
-    inv = plain.inv_freqs(rot, 10000.0, None)
-    positions = torch.tensor([0, 1, 2, 40, 41, 7, 100, 3, 4, 5, 6], dtype=torch.int32)
-    cos_all, sin_all = plain.rope_tables(inv, range(128))
+                                              (3, 1, 80, 40, 32), (32, 8, 64, 64, 16), (2, 2, 80, 48, 16),
+                                              (16, 8, 256, 256, 16), (3, 3, 24, 0, 8)])
+def test_rope_kv_write(ops, dtype, T, nh, nkv, d, rot, ps):
+    """Scattered slots (T = 11) and runs of adjacent slots that start in the middle of a page,
+    with tokens that are not stored (slot -1) among them (T = 77)."""
+    g = torch.Generator().manual_seed(T)
+    positions = torch.randint(0, 128, (T,), generator=g, dtype=torch.int32)
+    positions[:3] = torch.tensor([0, 1, 127])
+    if rot:
+        inv = plain.inv_freqs(rot, 10000.0, None)
+        cos_all, sin_all = plain.rope_tables(inv, range(128))
+    else:
+        cos_all = sin_all = None
     qkv = rnd(T, (nh + 2 * nkv) * d, dtype=dtype, seed=4)
-    slots = torch.randperm(pages * ps, generator=torch.Generator().manual_seed(1))[:T].to(torch.int32)
+    if T == 11:
+        pages = 9
+        slots = torch.randperm(pages * ps, generator=g)[:T].to(torch.int32)
+    else:
+        pages = (3 * ps + 64 + 37) // ps + 2
+        slots = torch.cat([torch.arange(5, 5 + 40), torch.arange(3 * ps + 64, 3 * ps + 64 + 37)]).to(torch.int32)
+        slots[[7, 50, 76]] = -1
     k_pages = torch.zeros(pages, nkv, ps, d, dtype=dtype, device=DEV)
     v_pages = torch.zeros(pages, nkv, d, ps, dtype=dtype, device=DEV)
     src = qkv.clone()
-    ops.rope_kv_write(qkv, nh, nkv, d, cos_all.to(DEV), sin_all.to(DEV), positions.to(DEV),
+    ops.rope_kv_write(qkv, nh, nkv, d, None if cos_all is None else cos_all.to(DEV),
+                      None if sin_all is None else sin_all.to(DEV), positions.to(DEV),
                       slots.to(DEV), k_pages, v_pages, ps)
     x = src.float().cpu()
     q = x[:, :nh * d].reshape(T, nh, d)
     k = x[:, nh * d:(nh + nkv) * d].reshape(T, nkv, d)
     v = x[:, (nh + nkv) * d:].reshape(T, nkv, d)
-    cos, sin = cos_all[positions.long()], sin_all[positions.long()]
 
     def rotate(t):          # (T, heads, d): rotate the first `rot` dims, pass the rest
+        if not rot:
+            return t
+        cos, sin = cos_all[positions.long()], sin_all[positions.long()]
         r = plain.rope_apply(t[..., :rot].transpose(0, 1), cos, sin).transpose(0, 1)
         return torch.cat([r, t[..., rot:]], dim=-1)
 
@@ -309,14 +326,19 @@ def test_rope_kv_write(ops, dtype, nh, nkv, d, rot, ps):
     torch.testing.assert_close(qkv[:, :nh * d].float().cpu().reshape(T, nh, d), rotate(q), **t)
     torch.testing.assert_close(qkv[:, nh * d:].cpu(), src[:, nh * d:].cpu(), atol=0, rtol=0)
     kr = rotate(k)
+    kp, vp = k_pages.float().cpu(), v_pages.float().cpu()
     for i in range(T):
+        if int(slots[i]) < 0:
+            continue
         page, off = int(slots[i]) // ps, int(slots[i]) % ps
-        torch.testing.assert_close(k_pages[page, :, off, :].float().cpu(), kr[i], **t)
-        torch.testing.assert_close(v_pages[page, :, :, off].float().cpu(), v[i], atol=0, rtol=0)
+        torch.testing.assert_close(kp[page, :, off, :], kr[i], **t)
+        torch.testing.assert_close(vp[page, :, :, off], v[i], atol=0, rtol=0)
     # rows that were not written stay zero
     written = torch.zeros(pages * ps, dtype=torch.bool)
-    written[slots.long()] = True
-    assert k_pages.float().abs().sum(dim=(1, 3)).reshape(-1)[~written].max().item() == 0.0
+    written[slots[slots >= 0].long()] = True
+    k_rows = kp.abs().sum(dim=3).transpose(1, 2).reshape(pages * ps, nkv)
+    v_rows = vp.abs().sum(dim=2).transpose(1, 2).reshape(pages * ps, nkv)
+    assert k_rows[~written].max().item() == 0.0 and v_rows[~written].max().item() == 0.0
 
 
 def test_rope_position_zero_is_identity_and_norm_is_kept(ops):
