@@ -412,12 +412,12 @@ __global__ void rope_kv_write_kernel(TX* __restrict__ qkv, long long row_stride,
 
 // bfloat16 with every head segment a multiple of 8 wide: 16-byte accesses.  The first
 // `qk_blocks` workgroups rotate q in place and k into its page, kRopeTokQK tokens each; the
-// others take kRopeTokV tokens each and turn their v rows through LDS, so that lanes which are
-// neighbours in a page's (d, offset) layout store neighbouring offsets (tokens with adjacent
-// slots fill whole 32-byte runs, whatever their alignment).
+// others take kRopeTokV tokens times kRopeVCols value columns each and turn them through LDS, so
+// that lanes which are neighbours in a page's (d, offset) layout store neighbouring offsets
+// (tokens with adjacent slots fill whole 32-byte runs, whatever their alignment).
 constexpr int kRopeTokQK = 2;
 constexpr int kRopeTokV = 16;
-constexpr int kRopeVCols = 1024;               // v columns staged per pass
+constexpr int kRopeVCols = 256;                // v columns per workgroup
 constexpr int kRopeVRow = kRopeVCols + 8;      // padded: rows stay 16-byte aligned, banks spread
 
 __device__ __forceinline__ void unpack8(const uint4 u, float (&v)[8]) {
@@ -495,30 +495,34 @@ __global__ __launch_bounds__(256) void rope_kv_write_bf16x8_kernel(
     }
     return;
   }
+  // Values: a tile of kRopeTokV tokens times kRopeVCols columns per workgroup.
   __shared__ __attribute__((aligned(16))) bf16_t v_s[kRopeTokV * kRopeVRow];
-  __shared__ int slot_s[kRopeTokV];
-  const int t0 = ((int)blockIdx.x - qk_blocks) * kRopeTokV;
-  if (tid < kRopeTokV) slot_s[tid] = t0 + tid < T ? slots[t0 + tid] : -1;
+  __shared__ long long page_s[kRopeTokV];                // -1: the token is not stored
+  __shared__ int off_s[kRopeTokV];
   const int cols = nkv * d;
-  for (int c0 = 0; c0 < cols; c0 += kRopeVCols) {
-    const int nc = min(kRopeVCols, cols - c0), nc8 = nc / 8;
-    __syncthreads();                                     // slots are there; the tile is free
-    for (int i = tid; i < kRopeTokV * nc8; i += blockDim.x) {
-      const int tt = i / nc8, c = (i - tt * nc8) * 8;
-      if (t0 + tt < T)
-        *(uint4*)(v_s + tt * kRopeVRow + c) =
-            *(const uint4*)(qkv + (long long)(t0 + tt) * row_stride + v_off + c0 + c);
-    }
-    __syncthreads();
-    for (int i = tid; i < kRopeTokV * nc; i += blockDim.x) {
-      const int tt = i % kRopeTokV, c = i / kRopeTokV;
-      const int slot = slot_s[tt];
-      if (slot < 0) continue;
-      const int col = c0 + c, h = col / d, j = col - h * d;
-      const long long page = slot / page_size;
-      const int off = slot - (int)page * page_size;
-      v_pages[((page * nkv + h) * d + j) * page_size + off] = v_s[tt * kRopeVRow + c];
-    }
+  const int chunks = (cols + kRopeVCols - 1) / kRopeVCols;
+  const int vb = (int)blockIdx.x - qk_blocks;
+  const int t0 = (vb / chunks) * kRopeTokV, c0 = (vb % chunks) * kRopeVCols;
+  if (tid < kRopeTokV) {
+    const int slot = t0 + tid < T ? slots[t0 + tid] : -1;
+    const int page = slot < 0 ? -1 : slot / page_size;
+    page_s[tid] = page;
+    off_s[tid] = slot < 0 ? 0 : slot - page * page_size;
+  }
+  const int nc = min(kRopeVCols, cols - c0), nc8 = nc / 8;
+  for (int i = tid; i < kRopeTokV * nc8; i += blockDim.x) {
+    const int tt = i / nc8, c = (i - tt * nc8) * 8;
+    if (t0 + tt < T)
+      *(uint4*)(v_s + tt * kRopeVRow + c) =
+          *(const uint4*)(qkv + (long long)(t0 + tt) * row_stride + v_off + c0 + c);
+  }
+  __syncthreads();
+  for (int i = tid; i < kRopeTokV * nc; i += blockDim.x) {
+    const int tt = i % kRopeTokV, c = i / kRopeTokV;
+    const long long page = page_s[tt];
+    if (page < 0) continue;
+    const int col = c0 + c, h = col / d, j = col - h * d;
+    v_pages[((page * nkv + h) * d + j) * page_size + off_s[tt]] = v_s[tt * kRopeVRow + c];
   }
 }
 
@@ -539,7 +543,7 @@ RLIS_API int rlis_rope_kv_write(void* qkv, int dtype, long long row_stride, int 
                    (!write_kv || (((uintptr_t)k_pages % 16) == 0 && T <= (1 << 30)));
   if (by8) {
     const int qk_blocks = ceil_div(T, kRopeTokQK);
-    const int v_blocks = write_kv ? ceil_div(T, kRopeTokV) : 0;
+    const int v_blocks = write_kv ? ceil_div(T, kRopeTokV) * ceil_div(nkv * d, kRopeVCols) : 0;
     rope_kv_write_bf16x8_kernel<<<qk_blocks + v_blocks, 256, 0, stream>>>(
         (bf16_t*)qkv, row_stride, k_off, v_off, T, nh, nkv, d, rot_dim, cos_t, sin_t, positions,
         slots, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, write_kv, qk_blocks);

@@ -16,7 +16,7 @@ def test_presets_parse_and_cover_the_benchmark_shapes():
     assert (c.hidden_size, c.num_hidden_layers, c.num_attention_heads, c.num_key_value_heads,
             c.head_dim, c.intermediate_size, c.vocab_size) == (2048, 16, 32, 8, 64, 8192, 128256)
     assert c.tie_word_embeddings and c.rope_scaling.factor == 32.0
-    # 32 KiB of K and V per token in bf16 (crates/model/src/config.rs:49-52; DESIGN.md:66-69)
+    # 32 KiB of K and V per token in bf16 (crates/model/src/config.rs:49-52)
     assert c.kv_bytes_per_token(2) == 32 * 1024
     c8 = LlamaConfig.from_dict(preset_dict("llama-3.1-8b"))
     assert not c8.tie_word_embeddings and c8.kv_bytes_per_token(2) == 128 * 1024
