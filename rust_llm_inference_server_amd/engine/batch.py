@@ -53,17 +53,28 @@ class StepContext:
     max_new: int
     all_decode: bool
     decode_splits: Optional[int] = None
+    # Sequences that bring a single token come first in the step: sequences (and token rows)
+    # [0, num_single) are theirs, so that a decode kernel can take them beside the portions.
+    num_single: int = 0
+    max_single_context: int = 0
+    multi_tile_map: Optional[torch.Tensor] = None     # tile_map without the single tokens' tiles
+    num_multi_tiles: int = 0
     # Host copies, for parts that plan on the host.
     host_start_pos: List[int] = field(default_factory=list)
     host_new: List[int] = field(default_factory=list)
     host_state_slots: List[int] = field(default_factory=list)
+    host_order: List[int] = field(default_factory=list)   # entry index of every sequence
 
 
 def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
                vocab_size: int) -> StepContext:
-    """Lay out a step.  Every entry's request must hold reserved positions for its tokens."""
+    """Lay out a step.  Every entry's request must hold reserved positions for its tokens.
+
+    Inside the step the sequences are ordered single tokens first (``host_order`` maps them back
+    to the entries); ``logit_rows`` keeps the order of the entries and of their ``want``."""
     if not entries:
         raise ValueError("a step needs at least one request")
+    order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens) != 1)
     ps = cache.page_size
     ids: List[int] = []
     positions: List[int] = []
@@ -78,7 +89,9 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
     tables: List[List[List[int]]] = [[] for _ in range(ng)]
     slots: List[List[int]] = [[] for _ in range(ng)]
     seen = set()
-    for s, e in enumerate(entries):
+    base_of = [0] * len(entries)
+    for s, i in enumerate(order):
+        e = entries[i]
         n = len(e.tokens)
         if n == 0:
             raise ValueError("empty sequence in batch")          # llama.rs:231-233
@@ -95,7 +108,7 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
             if not 0 <= int(t) < vocab_size:
                 raise ValueError(f"request {e.seq_id}: token id {t} is outside the vocabulary "
                                  f"of {vocab_size}")
-        base = len(ids)
+        base = base_of[i] = len(ids)
         ids.extend(int(t) for t in e.tokens)
         positions.extend(range(computed, computed + n))
         seq_of_token.extend([s] * n)
@@ -106,7 +119,6 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
         for w in e.want:
             if not 0 <= int(w) < n:
                 raise ValueError(f"request {e.seq_id}: wanted index {w} is outside its {n} tokens")
-            logit_rows.append(base + int(w))
         tiles.extend((computed + min(n, qb + PREFILL_TILE), s, qb)
                      for qb in range(0, n, PREFILL_TILE))
         for g in range(ng):
@@ -117,7 +129,11 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
                 if page < 0:
                     raise ValueError(f"request {e.seq_id}: position {p} has no page reserved")
                 slots[g].append(page * ps + p % ps)
+    for i, e in enumerate(entries):
+        logit_rows.extend(base_of[i] + int(w) for w in e.want)
     T, S = len(ids), len(entries)
+    new = [len(entries[i].tokens) for i in order]
+    num_single = sum(1 for n in new if n == 1)
     widths = [max(8, -(-max(len(t) for t in tables[g]) // 8) * 8) for g in range(ng)]
     flat: List[int] = []
     offsets = {}
@@ -138,6 +154,8 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
     # Longest tiles first: the prefill attention kernel hands them out in this order.
     tiles.sort(key=lambda t: -t[0])
     put("tiles", [x for _, s_, qb in tiles for x in (s_, qb)])
+    multi = [t for t in tiles if t[1] >= num_single]
+    put("tiles_multi", [x for _, s_, qb in multi for x in (s_, qb)])
     for g in range(ng):
         put(f"slots{g}", slots[g])
         rows: List[int] = []
@@ -162,7 +180,8 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
         seq_of_token=view("seq_of_token"), cu_seqlens=view("cu"), start_pos=view("start_pos"),
         ctx_lens=view("ctx_lens"), logit_rows=view("logit_rows"), num_logit_rows=len(logit_rows),
         state_slots=view("state_slots"), tile_map=view("tiles"), num_tiles=len(tiles),
-        groups=groups, max_context=max(ctx_lens), max_new=max(len(e.tokens) for e in entries),
-        all_decode=all(len(e.tokens) == 1 for e in entries),
-        host_start_pos=start_pos, host_new=[len(e.tokens) for e in entries],
-        host_state_slots=state_slots)
+        groups=groups, max_context=max(ctx_lens), max_new=max(new),
+        all_decode=num_single == S, num_single=num_single,
+        max_single_context=max(ctx_lens[:num_single], default=0),
+        multi_tile_map=view("tiles_multi"), num_multi_tiles=len(multi),
+        host_start_pos=start_pos, host_new=new, host_state_slots=state_slots, host_order=order)

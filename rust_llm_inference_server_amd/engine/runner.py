@@ -148,8 +148,8 @@ class ModelRunner:
                 if start == 0:
                     self.pools.zero_state(slot)      # a fresh (or recomputed) request
         logits = self.model.forward(step, self.pools)
-        for e, start in zip(entries, step.host_start_pos):
-            self.cache.advance(e.seq_id, start + len(e.tokens))
+        for i, start in zip(step.host_order, step.host_start_pos):
+            self.cache.advance(entries[i].seq_id, start + len(entries[i].tokens))
         return logits
 
     def _decode_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:

@@ -21,6 +21,8 @@ _DT = {torch.float32: 0, torch.bfloat16: 1}
 SKINNY_MAX_ROWS = 64
 # ... and with at most this many rows the streaming kernel (16 at most; 0 switches it off).
 STREAM_MAX_ROWS = 16
+# Single tokens in a batch that also holds portions of prompts take the decode attention kernel.
+SPLIT_MIXED_ATTENTION = True
 # The norm in front of a projection goes into the streaming kernel where that applies.
 FUSE_NORM_LINEAR = True
 # The matrix-core decode attention rotates q and k and stores the new k, v itself where it can.
@@ -348,6 +350,15 @@ def decode_splits(num_seqs: int, num_kv_heads: int, group: int, max_context: int
     return max(1, min(math.ceil(512 / pairs), math.ceil(max_context / 256)))
 
 
+def _decode_mfma_ok(qkv: torch.Tensor, nh: int, nkv: int, d: int, page_size: int) -> bool:
+    """Whether single tokens of this layout can take the matrix-core decode kernel."""
+    g = nh // nkv
+    return (qkv.dtype == torch.bfloat16 and d % 16 == 0 and d <= 256 and g <= 16
+            and g * (d + 2) * 32 <= 65536
+            and page_size >= 8 and page_size & (page_size - 1) == 0 and qkv.stride(0) % 8 == 0
+            and DECODE_ATTENTION != "vector")
+
+
 def _attention_kernel(qkv: torch.Tensor, nh: int, nkv: int, d: int, page_size: int, step,
                       force: Optional[str]):
     """(kind, matrix_decode): which attention kernel a batch takes."""
@@ -362,11 +373,7 @@ def _attention_kernel(qkv: torch.Tensor, nh: int, nkv: int, d: int, page_size: i
             kind = "prefill"
         else:
             kind = "generic"
-    g = nh // nkv
-    mfma = (kind == "decode" and qkv.dtype == torch.bfloat16 and d % 16 == 0 and g <= 16
-            and g * (d + 2) * 32 <= 65536
-            and page_size >= 8 and page_size & (page_size - 1) == 0 and q_stride % 8 == 0
-            and DECODE_ATTENTION != "vector")
+    mfma = kind == "decode" and _decode_mfma_ok(qkv, nh, nkv, d, page_size)
     return kind, mfma
 
 
@@ -442,18 +449,16 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     kind, mfma = _attention_kernel(qkv, nh, nkv, d, page_size, step, force)
     if rope is not None and not mfma:
         raise KernelError("attention: only the matrix-core decode kernel rotates and stores")
-    if kind == "decode":
-        if not step.all_decode:
-            raise KernelError("attention: the decode kernel needs one token per sequence")
-        S = step.num_seqs
-        splits = step.decode_splits or decode_splits(S, nkv, nh // nkv, step.max_context)
+    def decode(S: int, max_context: int, matrix: bool, splits: Optional[int]) -> None:
+        """The first S sequences, one token each (their token rows are the first S too)."""
+        splits = splits or decode_splits(S, nkv, nh // nkv, max_context)
         part_ml = part_acc = None
         if splits > 1:
             part_ml = torch.empty((S, nh, splits, 2), dtype=torch.float32, device=qkv.device)
             part_acc = torch.empty((S, nh, splits, d), dtype=torch.float32, device=qkv.device)
         ml_ptr = None if part_ml is None else part_ml.data_ptr()
         acc_ptr = None if part_acc is None else part_acc.data_ptr()
-        if mfma:
+        if matrix:
             cos_p = sin_p = pos_p = slots_p = None
             rot = 0
             if rope is not None:
@@ -472,15 +477,29 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                      nh * d, ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
                      block_tables.data_ptr(), max_pages, _i32(step.ctx_lens, "ctx_lens", S), None,
                      S, nh, nkv, d, page_size, float(scale), win, splits, stream)
+
+    if kind == "decode":
+        if not step.all_decode:
+            raise KernelError("attention: the decode kernel needs one token per sequence")
+        decode(step.num_seqs, step.max_context, mfma, step.decode_splits)
     elif kind == "prefill":
         if qkv.dtype != torch.bfloat16:
             raise KernelError("attention: the matrix-core prefill kernel is bfloat16 only")
-        lib.call("rlis_attn_prefill_mfma", qkv.data_ptr(), q_stride, out.data_ptr(), nh * d,
-                 k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,
-                 _i32(step.cu_seqlens, "cu_seqlens", step.num_seqs + 1),
-                 _i32(step.start_pos, "start_pos", step.num_seqs),
-                 _i32(step.tile_map, "tile_map", 2 * step.num_tiles), step.num_tiles, nh, nkv, d,
-                 page_size, win, float(scale), 0, stream)
+        tile_map, num_tiles = step.tile_map, step.num_tiles
+        # Single tokens beside portions of prompts: the step lists them first, and the decode
+        # kernel reads their keys and values once for the whole group of heads, where a
+        # 64-query tile of the prefill kernel would walk the context for one query per head.
+        singles = getattr(step, "num_single", 0) if force is None and SPLIT_MIXED_ATTENTION else 0
+        if singles and _decode_mfma_ok(qkv, nh, nkv, d, page_size):
+            decode(singles, step.max_single_context, True, None)
+            tile_map, num_tiles = step.multi_tile_map, step.num_multi_tiles
+        if num_tiles:
+            lib.call("rlis_attn_prefill_mfma", qkv.data_ptr(), q_stride, out.data_ptr(), nh * d,
+                     k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,
+                     _i32(step.cu_seqlens, "cu_seqlens", step.num_seqs + 1),
+                     _i32(step.start_pos, "start_pos", step.num_seqs),
+                     _i32(tile_map, "tile_map", 2 * num_tiles), num_tiles, nh, nkv, d,
+                     page_size, win, float(scale), 0, stream)
     elif kind == "generic":
         lib.call("rlis_attn_generic", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(), nh * d,
                  k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,

@@ -406,6 +406,12 @@ def paged_case(lens_cached, lens_new, nh, nkv, d, ps, dtype, seed=0, q_scale=1.0
     step.max_context, step.max_new = max(totals), max(lens_new)
     step.all_decode = all(n == 1 for n in lens_new)
     step.decode_splits = None
+    # single tokens that lead the batch, as the engine's steps order them
+    lead = next((i for i, n in enumerate(lens_new) if n != 1), S)
+    if all(n > 1 for n in lens_new[lead:]):
+        multi = [x for s, n in enumerate(lens_new) if s >= lead for qb in range(0, n, 64) for x in (s, qb)]
+        step.num_single, step.max_single_context = lead, max(totals[:lead], default=0)
+        step.multi_tile_map, step.num_multi_tiles = i32(multi), len(multi) // 2
     return (qkv.to(DEV), k_pages.to(DEV), v_pages.to(DEV), bt.to(DEV), step, ks, vs, cu)
 
 
@@ -440,6 +446,33 @@ def test_attention_mixed_batch(ops, dtype, nh, nkv, d, ps, kind):
     got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, None, force=kind)
     want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, None)
     torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
+
+
+@pytest.mark.parametrize("nh,nkv,d,ps", [(32, 8, 64, 16), (24, 8, 128, 16), (6, 2, 32, 8), (5, 5, 48, 16),
+                                         (34, 2, 16, 16)])
+@pytest.mark.parametrize("window", [None, 70])
+def test_attention_single_tokens_beside_portions(ops, nh, nkv, d, ps, window):
+    """Single tokens that lead a batch of portions take the decode kernel, the portions the
+    prefill kernel: same result as the plain implementation, and as the prefill kernel alone.
+    17 query heads per KV head are more than the decode kernel takes: then nothing is split."""
+    dtype = torch.bfloat16
+    cached = [5, 63, 300, 1000, 0, 40, 0, 130, 17]
+    new = [1, 1, 1, 1, 33, 70, 2, 129, 64]
+    scale = 1.0 / math.sqrt(d)
+    qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=nh + 1)
+    assert step.num_single == 4 and step.num_multi_tiles == 8
+    want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, window)
+    got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window)
+    torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
+    whole = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window, force="prefill")
+    torch.testing.assert_close(got.float(), whole.float(), atol=2e-2, rtol=2e-2)
+    assert torch.equal(got[4:], whole[4:])                 # the portions' rows: same kernel, same tiles
+    old = ops.SPLIT_MIXED_ATTENTION
+    try:
+        ops.SPLIT_MIXED_ATTENTION = False
+        assert torch.equal(ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window), whole)
+    finally:
+        ops.SPLIT_MIXED_ATTENTION = old
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -62,3 +62,38 @@ def test_step_errors(cpu_ops, tiny_folders):
     out = runner.step([StepEntry(1, [1, 2], [1]), StepEntry(2, [3], [])])
     assert out.shape == (1, 256)
     assert runner.num_computed(1) == 2 and runner.num_computed(2) == 1
+
+
+def test_step_layout_puts_single_tokens_first(cpu_ops, tiny_folders):
+    """Inside a step the requests that bring one token come first (their rows are the first
+    rows, so that a decode kernel can take them beside the portions); the logits come back in
+    the order of the entries and of their `want` all the same."""
+    from rust_llm_inference_server_amd.engine import ModelRunner, StepEntry, build_step, load_model
+    model = load_model(tiny_folders["a"], "float32", max_positions=128, device=torch.device("cpu"))
+    runner = ModelRunner(model, num_pages=16, page_size=16, max_num_seqs=8)
+    for seq, n in ((1, 40), (2, 9), (3, 70), (4, 5)):
+        runner.reserve(seq, n)
+    runner.step([StepEntry(2, list(range(8)), []), StepEntry(4, [7, 8, 9, 10], [])])
+    entries = [StepEntry(1, list(range(10, 43 - 3)), [0, 29]), StepEntry(2, [5], [0]),
+               StepEntry(3, list(range(70)), [69]), StepEntry(4, [6], [])]
+    step = build_step(entries, runner.cache, torch.device("cpu"), 256)
+    assert step.host_order == [1, 3, 0, 2] and step.num_single == 2 and not step.all_decode
+    assert step.host_new == [1, 1, 30, 70] and step.host_start_pos == [8, 4, 0, 0]
+    assert step.max_single_context == 9 and step.max_context == 70
+    assert step.ids.tolist()[:2] == [5, 6] and step.positions.tolist()[:3] == [8, 4, 0]
+    assert step.cu_seqlens.tolist() == [0, 1, 2, 32, 102]
+    assert step.logit_rows.tolist() == [2, 31, 0, 101]            # entry order, then want order
+    tiles = step.tile_map.reshape(-1, 2).tolist()
+    multi = step.multi_tile_map.reshape(-1, 2).tolist()
+    assert sorted(tiles) == [[0, 0], [1, 0], [2, 0], [3, 0], [3, 64]]
+    assert multi == [[3, 64], [3, 0], [2, 0]] and step.num_multi_tiles == 3
+    # and the runner's answer does not depend on the order the entries come in
+    want = runner.step(entries)
+    assert [runner.num_computed(s) for s in (1, 2, 3, 4)] == [30, 9, 70, 5]
+    for seq in (1, 2, 3, 4):
+        runner.free(seq)
+    for seq, n in ((1, 40), (2, 9), (3, 70), (4, 5)):
+        runner.reserve(seq, n)
+    runner.step([StepEntry(4, [7, 8, 9, 10], []), StepEntry(2, list(range(8)), [])])
+    again = runner.step([entries[2], entries[3], entries[1], entries[0]])
+    assert (again[[2, 3, 1, 0]] - want).abs().max().item() < 1e-5
