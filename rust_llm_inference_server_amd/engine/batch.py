@@ -11,6 +11,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 PREFILL_TILE = 64     # new tokens per workgroup of the matrix-core prefill attention
@@ -76,20 +77,20 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
         raise ValueError("a step needs at least one request")
     order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens) != 1)
     ps = cache.page_size
-    ids: List[int] = []
-    positions: List[int] = []
-    seq_of_token: List[int] = []
+    S = len(entries)
+    ids: List[np.ndarray] = []
+    positions: List[np.ndarray] = []
     cu = [0]
     start_pos: List[int] = []
     ctx_lens: List[int] = []
-    logit_rows: List[int] = []
     state_slots: List[int] = []
+    new: List[int] = []
     tiles: List[Tuple[int, int, int]] = []      # (keys the tile walks, sequence, first index)
     ng = cache.num_groups
     tables: List[List[List[int]]] = [[] for _ in range(ng)]
-    slots: List[List[int]] = [[] for _ in range(ng)]
+    slots: List[List[np.ndarray]] = [[] for _ in range(ng)]
     seen = set()
-    base_of = [0] * len(entries)
+    base_of = [0] * S
     for s, i in enumerate(order):
         e = entries[i]
         n = len(e.tokens)
@@ -104,15 +105,19 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
         if computed + n > reserved:
             # paged.rs:258-263 "position {pos} has no block reserved"
             raise ValueError(f"request {e.seq_id}: position {reserved} has no page reserved")
-        for t in e.tokens:
-            if not 0 <= int(t) < vocab_size:
-                raise ValueError(f"request {e.seq_id}: token id {t} is outside the vocabulary "
-                                 f"of {vocab_size}")
-        base = base_of[i] = len(ids)
-        ids.extend(int(t) for t in e.tokens)
-        positions.extend(range(computed, computed + n))
-        seq_of_token.extend([s] * n)
-        cu.append(base + n)
+        toks = np.asarray(e.tokens, dtype=np.int64)
+        if toks.ndim != 1:
+            raise ValueError(f"request {e.seq_id}: its tokens must be a flat list")
+        if int(toks.min()) < 0 or int(toks.max()) >= vocab_size:
+            bad = int(toks[(toks < 0) | (toks >= vocab_size)][0])
+            raise ValueError(f"request {e.seq_id}: token id {bad} is outside the vocabulary "
+                             f"of {vocab_size}")
+        base_of[i] = cu[-1]
+        ids.append(toks)
+        pos = np.arange(computed, computed + n, dtype=np.int64)
+        positions.append(pos)
+        cu.append(cu[-1] + n)
+        new.append(n)
         start_pos.append(computed)
         ctx_lens.append(computed + n)
         state_slots.append(max(slot, 0))
@@ -124,28 +129,32 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
         for g in range(ng):
             table = cache.table(e.seq_id, g)
             tables[g].append(table)
-            for p in range(computed, computed + n):
-                page = table[p // ps]
-                if page < 0:
-                    raise ValueError(f"request {e.seq_id}: position {p} has no page reserved")
-                slots[g].append(page * ps + p % ps)
-    for i, e in enumerate(entries):
-        logit_rows.extend(base_of[i] + int(w) for w in e.want)
-    T, S = len(ids), len(entries)
-    new = [len(entries[i].tokens) for i in order]
+            pages = np.asarray(table, dtype=np.int64)[pos // ps]
+            if int(pages.min()) < 0:
+                p = int(pos[pages < 0][0])
+                raise ValueError(f"request {e.seq_id}: position {p} has no page reserved")
+            slots[g].append(pages * ps + pos % ps)
+    logit_rows = [base_of[i] + int(w) for i, e in enumerate(entries) for w in e.want]
+    T = cu[-1]
     num_single = sum(1 for n in new if n == 1)
     widths = [max(8, -(-max(len(t) for t in tables[g]) // 8) * 8) for g in range(ng)]
-    flat: List[int] = []
+    chunks: List[np.ndarray] = []
     offsets = {}
+    filled = 0
 
     def put(name, values):
-        offsets[name] = (len(flat), len(values))
-        flat.extend(values)
-        flat.extend([0] * (-len(flat) % 4))     # keep every array 16-byte aligned
+        nonlocal filled
+        arr = np.asarray(values, dtype=np.int32).reshape(-1)
+        offsets[name] = (filled, arr.size)
+        pad = -arr.size % 4                     # keep every array 16-byte aligned
+        chunks.append(arr)
+        if pad:
+            chunks.append(np.zeros(pad, dtype=np.int32))
+        filled += arr.size + pad
 
-    put("ids", ids)
-    put("positions", positions)
-    put("seq_of_token", seq_of_token)
+    put("ids", np.concatenate(ids))
+    put("positions", np.concatenate(positions))
+    put("seq_of_token", np.repeat(np.arange(S, dtype=np.int32), new))
     put("cu", cu)
     put("start_pos", start_pos)
     put("ctx_lens", ctx_lens)
@@ -157,13 +166,13 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
     multi = [t for t in tiles if t[1] >= num_single]
     put("tiles_multi", [x for _, s_, qb in multi for x in (s_, qb)])
     for g in range(ng):
-        put(f"slots{g}", slots[g])
-        rows: List[int] = []
-        for t in tables[g]:
-            rows.extend(max(p, 0) for p in t)
-            rows.extend([0] * (widths[g] - len(t)))
+        put(f"slots{g}", np.concatenate(slots[g]))
+        rows = np.zeros((S, widths[g]), dtype=np.int32)
+        for r, t in enumerate(tables[g]):
+            rows[r, :len(t)] = np.maximum(np.asarray(t, dtype=np.int32), 0)
         put(f"tables{g}", rows)
-    host = torch.tensor(flat, dtype=torch.int32)
+    host = torch.from_numpy(np.concatenate(chunks))
+
     if device.type == "cuda":
         host = host.pin_memory()
     dev = host.to(device, non_blocking=True)

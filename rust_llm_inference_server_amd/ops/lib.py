@@ -79,5 +79,11 @@ def call(name: str, *args) -> None:
         raise KernelError(lib.rlis_last_error().decode("utf-8", "replace"))
 
 
+_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr() -> int:
+    """torch's current HIP stream of the current device, as the kernels' launch argument."""
+    if _RAW_STREAM is not None:
+        return _RAW_STREAM(torch.cuda.current_device())    # the same stream, looked up faster
     return torch.cuda.current_stream().cuda_stream
