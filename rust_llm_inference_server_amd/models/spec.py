@@ -111,7 +111,8 @@ class Model:
         self.final_norm = create("norm", spec.final_norm, spec.final_norm_prefix, ctx)
         self.head = create("head", spec.head, spec.head_prefix, ctx)
         self.runs = spec.runs()
-        self.graph_safe = all(getattr(l.mixer, "graph_safe", False) for l in self.layers)
+        self.graph_safe = all(getattr(p, "graph_safe", False)
+                              for p in (self.embedding, *self.layers, self.final_norm, self.head))
         self._plan_cache()
 
     # ---------------------------------------------------------------- cache plan

@@ -133,6 +133,11 @@ def join(prefix: str, name: str) -> str:
 class Part:
     category = ""
     kind = ""
+    # True when the part's forward launches only device work that reads the step's device
+    # tensors (no host decision on device data, no synchronisation), so that a decode step may
+    # be captured into a HIP graph and replayed with new metadata.  A model's decode steps are
+    # captured only when every part of it says so; a new part starts out on the safe side.
+    graph_safe = False
 
     @classmethod
     def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
@@ -220,9 +225,6 @@ class Mixer(Part):
     mixer with state must leave, after a step, the state as it is after the last token the
     step brought for that request."""
 
-    # True when forward launches only device work that reads the step's device tensors, so
-    # that a decode step may be captured into a HIP graph and replayed with new metadata.
-    graph_safe = False
     # True when forward takes ``x`` as a NormedInput (and projects it with ``project``).
     takes_normed_input = False
 

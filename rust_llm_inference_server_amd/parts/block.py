@@ -31,6 +31,11 @@ class PreNormBlock(Block):
         self.mixer_norm, self.mixer = built["mixer_norm"], built["mixer"]
         self.ffn_norm, self.feed_forward = built["ffn_norm"], built["feed_forward"]
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(p.graph_safe for p in (self.mixer_norm, self.mixer, self.ffn_norm,
+                                          self.feed_forward))
+
     def forward(self, stream: ResidualStream, step: Any, binding: CacheBinding) -> None:
         stream.add(self.mixer.forward(normed(self.mixer_norm, stream, self.mixer), step, binding))
         stream.add(self.feed_forward.forward(normed(self.ffn_norm, stream, self.feed_forward),

@@ -18,6 +18,8 @@ from .base import BuildContext, Embedding, Head, TensorSpec, join, project, regi
 class TokenEmbedding(Embedding):
     """Parameters: ``vocab_size``, ``hidden_size``."""
 
+    graph_safe = True
+
     @classmethod
     def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
         return [TensorSpec(join(prefix, "weight"), (params["vocab_size"], params["hidden_size"]))]
@@ -35,6 +37,8 @@ class TokenEmbedding(Embedding):
 class LinearHead(Head):
     """Parameters: ``vocab_size``, ``hidden_size``, ``tied_to`` (name of the tensor to share,
     or None for a weight of its own at ``prefix.weight``)."""
+
+    graph_safe = True
 
     takes_normed_input = True
 

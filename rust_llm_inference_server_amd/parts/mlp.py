@@ -15,6 +15,8 @@ from .base import BuildContext, FeedForward, TensorSpec, join, project, register
 class SwiGLU(FeedForward):
     """Parameters: ``hidden_size``, ``intermediate_size``."""
 
+    graph_safe = True
+
     takes_normed_input = True
 
     @classmethod

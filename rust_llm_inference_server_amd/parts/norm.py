@@ -15,6 +15,8 @@ from .base import BuildContext, Norm, ResidualStream, TensorSpec, join, register
 class RMSNorm(Norm):
     """Parameters: ``size`` (hidden width), ``eps``."""
 
+    graph_safe = True
+
     @classmethod
     def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
         return [TensorSpec(join(prefix, "weight"), (params["size"],), init="ones_normal")]
