@@ -231,8 +231,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) voi
             mx = fmaxf(mx, sv);
           }
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      mx = xor32_max(xor16_max(mx));
       const float m_new = fmaxf(m_run, mx * scale2);             // -inf stays -inf
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;   // a query with no key yet
       const float corr = __builtin_amdgcn_exp2f(m_run - m_safe);  // 0 when m_run is -inf
@@ -245,8 +244,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) voi
           s[nb][r] = p;
           sum += p;
         }
-      sum += __shfl_xor(sum, 16, kWave);
-      sum += __shfl_xor(sum, 32, kWave);
+      sum = xor32_sum(xor16_sum(sum));
       l_run = l_run * corr + sum;
       m_run = m_new;
       // The accumulator needs rescaling only when some query's maximum moved.
@@ -516,8 +514,7 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
         s[nb][r] = sv;
         mx = fmaxf(mx, sv);
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    mx = xor32_max(xor16_max(mx));
     const float m_new = fmaxf(m_run, mx * scale2);    // scale2 > 0; -inf stays -inf
     const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
     const float corr = __builtin_amdgcn_exp2f(m_run - m_safe);
@@ -531,8 +528,7 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
         sum += p;
         pf[nb * 4 + r] = (__bf16)p;
       }
-    sum += __shfl_xor(sum, 16, kWave);
-    sum += __shfl_xor(sum, 32, kWave);
+    sum = xor32_sum(xor16_sum(sum));
     l_run = l_run * corr + sum;
     m_run = m_new;
 #pragma unroll

@@ -33,15 +33,42 @@ __device__ __forceinline__ float ld(const bf16_t* p) { return bf16_to_f32(*p); }
 __device__ __forceinline__ void st(float* p, float v) { *p = v; }
 __device__ __forceinline__ void st(bf16_t* p, float v) { *p = f32_to_bf16(v); }
 
+// Sum and maximum of a value with its partner 16 or 32 lanes away (lane ^ 16, lane ^ 32): every
+// lane gets the result.  gfx950 swaps 16- and 32-lane halves of two registers in the vector
+// unit (v_permlane16_swap: odd rows of the first with even rows of the second;
+// v_permlane32_swap: upper half of the first with lower half of the second), which spares the
+// trip through LDS that a general shuffle takes.  Swapping a value with itself leaves one
+// register holding rows [0, 0, 2, 2] (halves [lo, lo]) and the other [1, 1, 3, 3] ([hi, hi]).
+__device__ __forceinline__ float xor16_sum(float v) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float xor32_sum(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float xor16_max(float v) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float xor32_max(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
+  v = xor32_sum(v);
+  v = xor16_sum(v);
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
   return v;
 }
 
 __device__ __forceinline__ float wave_max(float v) {
+  v = xor32_max(v);
+  v = xor16_max(v);
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  for (int o = 8; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
   return v;
 }
 
