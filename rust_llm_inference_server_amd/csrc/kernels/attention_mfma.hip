@@ -42,6 +42,10 @@ union Frag8 {
   bf16_t e[8];
 };
 
+#ifndef RLIS_PREFILL_BUFS
+#define RLIS_PREFILL_BUFS (RLIS_HEAD_DIM <= 64 ? 2 : 1)
+#endif
+
 #define RLIS_CAT2(a, b) a##b
 #define RLIS_CAT(a, b) RLIS_CAT2(a, b)
 #define KERNEL_NAME RLIS_CAT(rlis_attn_prefill_mfma_kernel_d, RLIS_HEAD_DIM)
@@ -53,6 +57,9 @@ constexpr int BN = D <= 128 ? 64 : 32;
 constexpr int KS = D + 8;     // K tile row stride (bf16 elements)
 constexpr int VS = BN + 8;    // V tile row stride
 constexpr int BM = 64;
+// Two LDS tiles taking turns (one barrier per tile instead of two) where that does not cost a
+// resident workgroup.
+constexpr int kTileBufs = RLIS_PREFILL_BUFS;
 
 }  // namespace
 
@@ -63,8 +70,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) voi
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_seqlens,
     const int* __restrict__ start_pos, const int* __restrict__ tile_map, int nh, int nkv, int d,
     int page_shift, float scale, int window, int num_tiles, int tiles_per_round) {
-  __shared__ __attribute__((aligned(16))) bf16_t Ks[BN * KS];
-  __shared__ __attribute__((aligned(16))) bf16_t Vs[D * VS];
+  __shared__ __attribute__((aligned(16))) bf16_t Ks_all[kTileBufs * BN * KS];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs_all[kTileBufs * D * VS];
 
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int l16 = lane % 16, lq = lane / 16;
@@ -166,8 +173,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) voi
                               off_);                                                           \
     }                                                                                          \
   }
-#define RLIS_STORE_TILE(TK, TV)                                                                \
+#define RLIS_STORE_TILE(TK, TV, buf_)                                                          \
   {                                                                                            \
+    bf16_t* Ks = Ks_all + (buf_) * (BN * KS);                                                  \
+    bf16_t* Vs = Vs_all + (buf_) * (D * VS);                                                   \
     _Pragma("unroll") for (int i = 0; i < KCH; ++i) {                                          \
       const int c_ = tid + i * 256;                                                            \
       if (c_ < K_CHUNKS) *(u32x4*)(Ks + (c_ / (D / 8)) * KS + (c_ % (D / 8)) * 8) = TK[i];     \
@@ -186,12 +195,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) voi
   RLIS_LOAD_TILE(kt0 + BN, page_kb, page_vb, tile_kb, tile_vb);
   RLIS_LOAD_PAGES(kt0 + 2 * BN, page_ka, page_va);
   RLIS_LOAD_PAGES(kt0 + 3 * BN, page_kb, page_vb);
-  RLIS_STORE_TILE(tile_ka, tile_va);
+  RLIS_STORE_TILE(tile_ka, tile_va, 0);
   RLIS_LOAD_TILE(kt0 + 2 * BN, page_ka, page_va, tile_ka, tile_va);
   RLIS_LOAD_PAGES(kt0 + 4 * BN, page_ka, page_va);
   __syncthreads();
   // The arithmetic of one tile, which LDS holds.
-  auto compute = [&](int k0) __attribute__((always_inline)) {
+  auto compute = [&](int k0, int buf) __attribute__((always_inline)) {
+    const bf16_t* Ks = Ks_all + buf * (BN * KS);
+    const bf16_t* Vs = Vs_all + buf * (D * VS);
 
     // Tiles wholly after this wave's last query contribute nothing to it.
     const bool wave_active = (wave_q_first < n_new) && (k0 <= P + wave_q_last);
@@ -278,22 +289,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) voi
   };
   // On entry of the step for tile k0: LDS holds tile k0; the `next` registers hold tile k0 + BN
   // and the other set tile k0 + 2 BN (in flight); the `next` page ids are those of tile
-  // k0 + 3 BN, the other set's those of tile k0 + 4 BN.  After the arithmetic the next tile goes
-  // to LDS and its registers take tile k0 + 3 BN, whose page ids arrived long since.
-#define RLIS_STEP(k0_, PK, PV, TK, TV)                \
+  // k0 + 3 BN, the other set's those of tile k0 + 4 BN.  The next tile goes to LDS (after the
+  // arithmetic and a barrier with one LDS tile; before the arithmetic, into the other tile,
+  // with two) and its registers take tile k0 + 3 BN, whose page ids arrived long since.
+#define RLIS_STEP(k0_, PK, PV, TK, TV, cur_)          \
   {                                                   \
-    compute(k0_);                                     \
-    __syncthreads();                                  \
-    if ((k0_) + BN < khi) {                           \
-      RLIS_STORE_TILE(TK, TV);                        \
+    if (kTileBufs == 2) {                             \
+      if ((k0_) + BN < khi) RLIS_STORE_TILE(TK, TV, 1 - (cur_)); \
+      RLIS_LOAD_TILE((k0_) + 3 * BN, PK, PV, TK, TV); \
+      RLIS_LOAD_PAGES((k0_) + 5 * BN, PK, PV);        \
+      compute(k0_, cur_);                             \
       __syncthreads();                                \
+    } else {                                          \
+      compute(k0_, 0);                                \
+      __syncthreads();                                \
+      if ((k0_) + BN < khi) {                         \
+        RLIS_STORE_TILE(TK, TV, 0);                   \
+        __syncthreads();                              \
+      }                                               \
+      RLIS_LOAD_TILE((k0_) + 3 * BN, PK, PV, TK, TV); \
+      RLIS_LOAD_PAGES((k0_) + 5 * BN, PK, PV);        \
     }                                                 \
-    RLIS_LOAD_TILE((k0_) + 3 * BN, PK, PV, TK, TV);   \
-    RLIS_LOAD_PAGES((k0_) + 5 * BN, PK, PV);          \
   }
   for (int k0 = kt0; k0 < khi; k0 += 2 * BN) {
-    RLIS_STEP(k0, page_kb, page_vb, tile_kb, tile_vb);
-    if (k0 + BN < khi) RLIS_STEP(k0 + BN, page_ka, page_va, tile_ka, tile_va);
+    RLIS_STEP(k0, page_kb, page_vb, tile_kb, tile_vb, 0);
+    if (k0 + BN < khi) RLIS_STEP(k0 + BN, page_ka, page_va, tile_ka, tile_va, 1);
   }
 #undef RLIS_STEP
 #undef RLIS_STORE_TILE
