@@ -130,7 +130,13 @@ class Sampler:
 def sample_on_device(logits: torch.Tensor, modes: Sequence[Tuple[int, float]]) -> List[int]:
     """One token per row of ``logits`` with the device kernel; ``modes`` as ``device_mode``."""
     from .. import ops
-    keys = torch.tensor([k - (1 << 32) if k >= (1 << 31) else k for k, _ in modes],
-                        dtype=torch.int32, device=logits.device)
-    inv_t = torch.tensor([t for _, t in modes], dtype=torch.float32, device=logits.device)
+    # keys (32-bit patterns) and inverse temperatures travel in one buffer, one copy
+    both = np.empty((2, len(modes)), dtype=np.uint32)
+    both[0] = [k for k, _ in modes]
+    both[1] = np.asarray([t for _, t in modes], dtype=np.float32).view(np.uint32)
+    host = torch.from_numpy(both.view(np.int32))
+    if logits.is_cuda:
+        host = host.pin_memory()
+    dev = host.to(logits.device, non_blocking=True)
+    keys, inv_t = dev[0], dev[1].view(torch.float32)
     return ops.sample_rows(logits, keys, inv_t).tolist()
