@@ -97,6 +97,34 @@ def test_captured_decode_steps_match_eager_ones(case, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_of_a_sequence(case, dtype):
+    """Sequences fed one token at a time from position 0 (no prompt step before them), two of
+    them side by side and a third that joins later, through captured and through eager decode
+    steps: the first positions of a sequence meet an empty cache, a page with one key, and
+    partitions without keys."""
+    name, cfg, per_dtype = case
+    folder, reqs, ref = per_dtype[dtype]
+    keys = [k for k, t in reqs.items() if len(t) >= 17][:3]
+    small = {k: reqs[k][:17] for k in keys}
+    steps = []
+    for p in range(17 + 5):
+        entries = []
+        for i, k in enumerate(keys):
+            q = p - (5 if i == 2 else 0)                # the third joins five steps later
+            if 0 <= q < 17:
+                entries.append({"id": k, "tokens": [small[k][q]], "want": [0]})
+        end = [e["id"] for e in entries if (p - (5 if e["id"] == keys[2] else 0)) == 16]
+        steps.append({"step": p, "entries": entries, "end": end})
+    for use_graphs in (True, False):
+        runner = make_runner(folder, dtype, 3 * 64, page_size=8 if name == "b" else 16,
+                             use_graphs=use_graphs)
+        outputs = traces.replay_in_process(runner, steps)
+        small_ref = {k: ref[k][:17] for k in keys}
+        check(steps, outputs, small, small_ref, cfg["vocab_size"], TOL[dtype])
+        assert runner.cache.num_free_pages(0) == runner.cache.num_pages(0)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(case, dtype, tmp_path):
     """The program itself, as a child process fed step by step, on the mixed trace."""
     name, cfg, per_dtype = case
