@@ -8,7 +8,7 @@
       const void* q, long long q_stride, void* out, long long out_stride, const void* k_pages, \
       const void* v_pages, const int* block_tables, int max_pages, const int* cu_seqlens,     \
       const int* start_pos, const int* tile_map, int num_tiles, int nh, int nkv, int d,       \
-      int page_shift, int window, float scale, hipStream_t stream);
+      int page_shift, int window, float scale, int tile_queries, hipStream_t stream);
 DECL(32) DECL(64) DECL(96) DECL(128) DECL(160) DECL(192) DECL(224) DECL(256)
 #undef DECL
 
@@ -30,9 +30,12 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
                                     const void* v_pages, const int* block_tables, int max_pages,
                                     const int* cu_seqlens, const int* start_pos,
                                     const int* tile_map, int num_tiles, int nh, int nkv, int d,
-                                    int page_size, int window, float scale, int reserved,
+                                    int page_size, int window, float scale, int tile_queries,
                                     hipStream_t stream) {
-  (void)reserved;
+  // tile_map lists tiles of tile_queries new tokens: 64 (0 means that too) or 128.
+  if (tile_queries == 0) tile_queries = 64;
+  RLIS_REQUIRE(tile_queries == 64 || tile_queries == 128,
+               "attn_prefill_mfma: tiles of %d queries, 64 or 128 only", tile_queries);
   RLIS_REQUIRE(num_tiles >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0,
                "attn_prefill_mfma: bad sizes");
   RLIS_REQUIRE(scale > 0.f, "attn_prefill_mfma: the score scale must be positive, got %g", scale);
@@ -50,7 +53,8 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
 #define CALL(D)                                                                                 \
   return rlis_attn_prefill_mfma_d##D(q, q_stride, out, out_stride, k_pages, v_pages,            \
                                      block_tables, max_pages, cu_seqlens, start_pos, tile_map,  \
-                                     num_tiles, nh, nkv, d, page_shift, window, scale, stream)
+                                     num_tiles, nh, nkv, d, page_shift, window, scale,         \
+                                     tile_queries, stream)
   if (d <= 32) CALL(32);
   if (d <= 64) CALL(64);
   if (d <= 96) CALL(96);

@@ -1,8 +1,11 @@
 // Prefill attention over the paged cache on the matrix cores (bfloat16 operands, float32
 // accumulation and softmax), one compile unit per padded head size RLIS_HEAD_DIM.
 //
-// A workgroup of four waves serves 64 consecutive new tokens of one sequence for one query
-// head; each wave owns 16 of them.  Keys are walked in tiles of BN positions aligned to BN,
+// A workgroup of four waves serves 64 (or, QB = 2, 128) consecutive new tokens of one sequence
+// for one query head; each wave owns 16 (32, as two blocks of 16) of them.  With two query blocks
+// every K and V fragment that a wave reads from LDS serves two products, which halves the LDS
+// traffic per flop: long prompts, whose tiles are plenty, take that form.  Keys are walked in
+// tiles of BN positions aligned to BN,
 // read through the block table: the K tile [key][dim] and the V tile [dim][key] (the cache
 // keeps V transposed inside a page, so both are copied as they lie) go to LDS once per
 // workgroup, the next tile travelling global -> registers while the current one is computed.
@@ -53,23 +56,31 @@ union Frag8 {
 namespace {
 
 constexpr int D = RLIS_HEAD_DIM;
-constexpr int BN = D <= 128 ? 64 : 32;
+// Keys per tile: 64 up to head size 128, 32 beyond; with two query blocks per wave the
+// accumulators take twice the registers, and 32 keys per tile from head size 96 on keep the
+// staging and score registers within what two waves per SIMD can have.
+__host__ __device__ constexpr int tile_keys(int QB) {
+  return (D > 128 || (QB == 2 && D > 64)) ? 32 : 64;
+}
 constexpr int KS = D + 8;     // K tile row stride (bf16 elements)
-constexpr int VS = BN + 8;    // V tile row stride
-constexpr int BM = 64;
+constexpr int BM = 64;       // queries per workgroup and query block
 // Two LDS tiles taking turns (one barrier per tile instead of two) where that does not cost a
 // resident workgroup.
 constexpr int kTileBufs = RLIS_PREFILL_BUFS;
 
 }  // namespace
 
-// Up to three waves per SIMD: the staging registers must not be traded for a fourth.
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) void KERNEL_NAME(
+// Up to three waves per SIMD (two with two query blocks): the staging registers must not be
+// traded for another.
+template <int QB>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, QB == 1 ? 3 : 2))) void KERNEL_NAME(
     const bf16_t* __restrict__ q, long long q_stride, bf16_t* __restrict__ out,
     long long out_stride, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_seqlens,
     const int* __restrict__ start_pos, const int* __restrict__ tile_map, int nh, int nkv, int d,
     int page_shift, float scale, int window, int num_tiles, int tiles_per_round) {
+  constexpr int BN = tile_keys(QB);
+  constexpr int VS = BN + 8;    // V tile row stride
   __shared__ __attribute__((aligned(16))) bf16_t Ks_all[kTileBufs * BN * KS];
   __shared__ __attribute__((aligned(16))) bf16_t Vs_all[kTileBufs * D * VS];
 
@@ -94,32 +105,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) voi
   const int* table = block_tables + (long long)seq * max_pages;
   const int page_mask = (1 << page_shift) - 1;
 
-  // This lane's query: new-token index qb + wave * 16 + l16.  Its fragments serve as the
-  // B operand (column l16) of S^T = K Q^T.
-  const int wave_q_first = qb + wave * 16;
-  const int my_qi = wave_q_first + l16;
-  const int my_qpos = P + my_qi;
-  Frag8 qf[D / 32];
+  // This lane's queries: new-token indices qb + wave * 16 QB + b * 16 + l16, one per block b.
+  // Their fragments serve as the B operand (column l16) of S^T = K Q^T.
+  const int wave_q_first = qb + wave * 16 * QB;
+  int my_qi[QB], my_qpos[QB];
+  Frag8 qf[QB][D / 32];
 #pragma unroll
-  for (int ks = 0; ks < D / 32; ++ks) {
-    const int dim = ks * 32 + lq * 8;
-    if (my_qi < n_new && dim < d)
-      qf[ks].u = *(const uint4*)(q + (long long)(tok_begin + my_qi) * q_stride + h * d + dim);
-    else
-      qf[ks].u = make_uint4(0, 0, 0, 0);
+  for (int b = 0; b < QB; ++b) {
+    my_qi[b] = wave_q_first + b * 16 + l16;
+    my_qpos[b] = P + my_qi[b];
+#pragma unroll
+    for (int ks = 0; ks < D / 32; ++ks) {
+      const int dim = ks * 32 + lq * 8;
+      if (my_qi[b] < n_new && dim < d)
+        qf[b][ks].u = *(const uint4*)(q + (long long)(tok_begin + my_qi[b]) * q_stride + h * d + dim);
+      else
+        qf[b][ks].u = make_uint4(0, 0, 0, 0);
+    }
   }
 
-  float m_run = -INFINITY, l_run = 0.f;
-  f32x4 o_acc[D / 16];      // O^T: rows are dims db * 16 + lq * 4 + r, the column is this query
+  float m_run[QB], l_run[QB];
+  f32x4 o_acc[QB][D / 16];  // O^T: rows are dims db * 16 + lq * 4 + r, the column is this query
 #pragma unroll
-  for (int db = 0; db < D / 16; ++db) o_acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int b = 0; b < QB; ++b) {
+    m_run[b] = -INFINITY;
+    l_run[b] = 0.f;
+#pragma unroll
+    for (int db = 0; db < D / 16; ++db) o_acc[b][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
 
-  const int q_last = min(n_new, qb + BM) - 1;           // last new-token index of the tile
+  const int q_last = min(n_new, qb + BM * QB) - 1;      // last new-token index of the tile
   const int khi = P + q_last + 1;                        // keys [klo, khi) matter to the tile
   int klo = 0;
   if (window > 0) klo = max(0, P + qb - window + 1);
   const int kt0 = (klo / BN) * BN;
-  const int wave_q_last = min(n_new - 1, wave_q_first + 15);
+  const int wave_q_last = min(n_new - 1, wave_q_first + 16 * QB - 1);
 
   // Staging for the tiles to come.  A tile's page ids are fetched four tiles ahead of its use,
   // its keys and values two tiles ahead (two register sets taking turns), so that neither the
@@ -208,72 +228,85 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) voi
     const bool wave_active = (wave_q_first < n_new) && (k0 <= P + wave_q_last);
     if (wave_active) {
       // ---- S^T = K Q^T: block nb holds keys k0 + nb * 16 + lq * 4 + r for query l16 --------
-      f32x4 s[BN / 16];
+      f32x4 s[QB][BN / 16];
 #pragma unroll
       for (int nb = 0; nb < BN / 16; ++nb) {
-        s[nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int b = 0; b < QB; ++b) s[b][nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < D / 32; ++ks) {
           Frag8 kf;
           kf.u = *(const uint4*)(Ks + (nb * 16 + l16) * KS + ks * 32 + lq * 8);
-          s[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[ks].v, s[nb], 0, 0, 0);
+#pragma unroll
+          for (int b = 0; b < QB; ++b)
+            s[b][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[b][ks].v, s[b][nb], 0, 0, 0);
         }
       }
       // ---- scale, mask (only where a tile meets the diagonal, the window or the end) -----
       const bool plain_tile = (k0 + BN - 1 <= P + wave_q_first) &&
-                              (window <= 0 || k0 > P + wave_q_first + 15 - window);
+                              (window <= 0 || k0 > P + wave_q_first + 16 * QB - 1 - window);
       // The scale (positive) is applied inside the exponent, with one fused multiply-add per
       // score; the maximum is taken over the raw scores and scaled once.
-      float mx = -INFINITY;
-      if (plain_tile) {
+      bool moved = false;
+      float corr[QB];
 #pragma unroll
-        for (int nb = 0; nb < BN / 16; ++nb)
+      for (int b = 0; b < QB; ++b) {
+        float mx = -INFINITY;
+        if (plain_tile) {
 #pragma unroll
-          for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[nb][r]);
-      } else {
+          for (int nb = 0; nb < BN / 16; ++nb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[b][nb][r]);
+        } else {
+#pragma unroll
+          for (int nb = 0; nb < BN / 16; ++nb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int kpos = k0 + nb * 16 + lq * 4 + r;
+              const bool ok = (kpos <= my_qpos[b]) && (window <= 0 || kpos > my_qpos[b] - window);
+              const float sv = ok ? s[b][nb][r] : -INFINITY;
+              s[b][nb][r] = sv;
+              mx = fmaxf(mx, sv);
+            }
+        }
+        mx = xor32_max(xor16_max(mx));
+        const float m_new = fmaxf(m_run[b], mx * scale2);          // -inf stays -inf
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;   // a query with no key yet
+        corr[b] = __builtin_amdgcn_exp2f(m_run[b] - m_safe);       // 0 when m_run is -inf
+        float sum = 0.f;
 #pragma unroll
         for (int nb = 0; nb < BN / 16; ++nb)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const int kpos = k0 + nb * 16 + lq * 4 + r;
-            const bool ok = (kpos <= my_qpos) && (window <= 0 || kpos > my_qpos - window);
-            const float sv = ok ? s[nb][r] : -INFINITY;
-            s[nb][r] = sv;
-            mx = fmaxf(mx, sv);
+            const float p = __builtin_amdgcn_exp2f(fmaf(s[b][nb][r], scale2, -m_safe));  // exp2(-inf) = 0
+            s[b][nb][r] = p;
+            sum += p;
           }
+        sum = xor32_sum(xor16_sum(sum));
+        l_run[b] = l_run[b] * corr[b] + sum;
+        m_run[b] = m_new;
+        moved = moved || corr[b] != 1.0f;
       }
-      mx = xor32_max(xor16_max(mx));
-      const float m_new = fmaxf(m_run, mx * scale2);             // -inf stays -inf
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;   // a query with no key yet
-      const float corr = __builtin_amdgcn_exp2f(m_run - m_safe);  // 0 when m_run is -inf
-      float sum = 0.f;
+      // The accumulators need rescaling only when some query's maximum moved.
+      if (__any(moved)) {
 #pragma unroll
-      for (int nb = 0; nb < BN / 16; ++nb)
+        for (int b = 0; b < QB; ++b)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float p = __builtin_amdgcn_exp2f(fmaf(s[nb][r], scale2, -m_safe));  // exp2(-inf) = 0
-          s[nb][r] = p;
-          sum += p;
-        }
-      sum = xor32_sum(xor16_sum(sum));
-      l_run = l_run * corr + sum;
-      m_run = m_new;
-      // The accumulator needs rescaling only when some query's maximum moved.
-      if (__any(corr != 1.0f)) {
+          for (int db = 0; db < D / 16; ++db)
 #pragma unroll
-        for (int db = 0; db < D / 16; ++db)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) o_acc[db][r] *= corr;
+            for (int r = 0; r < 4; ++r) o_acc[b][db][r] *= corr[b];
       }
       // ---- O^T += V^T P^T: P^T fragments come straight from the registers ----------------
 #pragma unroll
       for (int st = 0; st < BN / 32; ++st) {
-        bf16x8 pf;
+        bf16x8 pf[QB];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          pf[j] = (__bf16)s[2 * st][j];
-          pf[4 + j] = (__bf16)s[2 * st + 1][j];
-        }
+        for (int b = 0; b < QB; ++b)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            pf[b][j] = (__bf16)s[b][2 * st][j];
+            pf[b][4 + j] = (__bf16)s[b][2 * st + 1][j];
+          }
 #pragma unroll
         for (int db = 0; db < D / 16; ++db) {
           if (db * 16 < d) {
@@ -281,7 +314,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) voi
             const bf16_t* vrow = Vs + (db * 16 + l16) * VS + st * 32 + lq * 4;
             vf.h[0] = *(const uint2*)(vrow);
             vf.h[1] = *(const uint2*)(vrow + 16);
-            o_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf, o_acc[db], 0, 0, 0);
+#pragma unroll
+            for (int b = 0; b < QB; ++b)
+              o_acc[b][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[b], o_acc[b][db], 0, 0, 0);
           }
         }
       }
@@ -321,30 +356,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) voi
 #undef RLIS_LOAD_PAGES
   }
 
-  // ---- normalise and store: this lane holds dims db * 16 + lq * 4 + [0, 4) of its query ----
-  if (my_qi < n_new) {
-    const float inv_l = 1.0f / l_run;
-    bf16_t* orow = out + (long long)(tok_begin + my_qi) * out_stride + h * d;
+  // ---- normalise and store: this lane holds dims db * 16 + lq * 4 + [0, 4) of its queries --
 #pragma unroll
-    for (int db = 0; db < D / 16; ++db) {
-      const int dim = db * 16 + lq * 4;
-      if (dim < d) {
-        union { uint2 u; bf16_t e[4]; } o;
+  for (int b = 0; b < QB; ++b) {
+    if (my_qi[b] < n_new) {
+      const float inv_l = 1.0f / l_run[b];
+      bf16_t* orow = out + (long long)(tok_begin + my_qi[b]) * out_stride + h * d;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) o.e[r] = f32_to_bf16(o_acc[db][r] * inv_l);
-        *(uint2*)(orow + dim) = o.u;
+      for (int db = 0; db < D / 16; ++db) {
+        const int dim = db * 16 + lq * 4;
+        if (dim < d) {
+          union { uint2 u; bf16_t e[4]; } o;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o.e[r] = f32_to_bf16(o_acc[b][db][r] * inv_l);
+          *(uint2*)(orow + dim) = o.u;
+        }
       }
     }
   }
 }
 
-// tile_map holds num_tiles pairs (sequence, first new-token index of a 64-token tile), sorted
-// by falling number of keys the tile walks.
+// tile_map holds num_tiles pairs (sequence, first new-token index of a tile of tile_queries =
+// 64 or 128 tokens), sorted by falling number of keys the tile walks.
 RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
     const void* q, long long q_stride, void* out, long long out_stride, const void* k_pages,
     const void* v_pages, const int* block_tables, int max_pages, const int* cu_seqlens,
     const int* start_pos, const int* tile_map, int num_tiles, int nh, int nkv, int d,
-    int page_shift, int window, float scale, hipStream_t stream) {
+    int page_shift, int window, float scale, int tile_queries, hipStream_t stream) {
   if (num_tiles == 0) return 0;
   const long long blocks = (long long)num_tiles * nh;
   if (blocks >= (1ll << 31)) {
@@ -353,10 +391,16 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
   }
   // 256 compute units: a round is the tiles whose blocks fill them once.
   const int tiles_per_round = (nh <= 256 && 256 % nh == 0) ? 256 / nh : 0;
-  KERNEL_NAME<<<(int)blocks, 256, 0, stream>>>(
-      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,
-      (const bf16_t*)v_pages, block_tables, max_pages, cu_seqlens, start_pos, tile_map, nh, nkv, d,
-      page_shift, scale, window, num_tiles, tiles_per_round);
+  if (tile_queries == 2 * BM)
+    KERNEL_NAME<2><<<(int)blocks, 256, 0, stream>>>(
+        (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,
+        (const bf16_t*)v_pages, block_tables, max_pages, cu_seqlens, start_pos, tile_map, nh, nkv,
+        d, page_shift, scale, window, num_tiles, tiles_per_round);
+  else
+    KERNEL_NAME<1><<<(int)blocks, 256, 0, stream>>>(
+        (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,
+        (const bf16_t*)v_pages, block_tables, max_pages, cu_seqlens, start_pos, tile_map, nh, nkv,
+        d, page_shift, scale, window, num_tiles, tiles_per_round);
   RLIS_LAUNCH_CHECK("attn_prefill_mfma");
   return 0;
 }

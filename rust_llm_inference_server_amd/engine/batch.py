@@ -15,6 +15,7 @@ import numpy as np
 import torch
 
 PREFILL_TILE = 64     # new tokens per workgroup of the matrix-core prefill attention
+WIDE_TILE = 128       # ... of its form with two query blocks per wave
 
 
 @dataclass
@@ -60,6 +61,8 @@ class StepContext:
     max_single_context: int = 0
     multi_tile_map: Optional[torch.Tensor] = None     # tile_map without the single tokens' tiles
     num_multi_tiles: int = 0
+    wide_tile_map: Optional[torch.Tensor] = None      # the same two lists in tiles of 128 tokens
+    wide_multi_tile_map: Optional[torch.Tensor] = None
     # Host copies, for parts that plan on the host.
     host_start_pos: List[int] = field(default_factory=list)
     host_new: List[int] = field(default_factory=list)
@@ -86,6 +89,7 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
     state_slots: List[int] = []
     new: List[int] = []
     tiles: List[Tuple[int, int, int]] = []      # (keys the tile walks, sequence, first index)
+    wide: List[Tuple[int, int, int]] = []       # the same in tiles of WIDE_TILE tokens
     ng = cache.num_groups
     tables: List[List[List[int]]] = [[] for _ in range(ng)]
     slots: List[List[np.ndarray]] = [[] for _ in range(ng)]
@@ -126,6 +130,7 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
                 raise ValueError(f"request {e.seq_id}: wanted index {w} is outside its {n} tokens")
         tiles.extend((computed + min(n, qb + PREFILL_TILE), s, qb)
                      for qb in range(0, n, PREFILL_TILE))
+        wide.extend((computed + min(n, qb + WIDE_TILE), s, qb) for qb in range(0, n, WIDE_TILE))
         for g in range(ng):
             table = cache.table(e.seq_id, g)
             tables[g].append(table)
@@ -165,6 +170,9 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
     put("tiles", [x for _, s_, qb in tiles for x in (s_, qb)])
     multi = [t for t in tiles if t[1] >= num_single]
     put("tiles_multi", [x for _, s_, qb in multi for x in (s_, qb)])
+    wide.sort(key=lambda t: -t[0])
+    put("wide", [x for _, s_, qb in wide for x in (s_, qb)])
+    put("wide_multi", [x for _, s_, qb in wide if s_ >= num_single for x in (s_, qb)])
     for g in range(ng):
         put(f"slots{g}", np.concatenate(slots[g]))
         rows = np.zeros((S, widths[g]), dtype=np.int32)
@@ -193,4 +201,5 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
         all_decode=num_single == S, num_single=num_single,
         max_single_context=max(ctx_lens[:num_single], default=0),
         multi_tile_map=view("tiles_multi"), num_multi_tiles=len(multi),
+        wide_tile_map=view("wide"), wide_multi_tile_map=view("wide_multi"),
         host_start_pos=start_pos, host_new=new, host_state_slots=state_slots, host_order=order)

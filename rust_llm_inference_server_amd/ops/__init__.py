@@ -23,6 +23,9 @@ SKINNY_MAX_ROWS = 64
 STREAM_MAX_ROWS = 16
 # Single tokens in a batch that also holds portions of prompts take the decode attention kernel.
 SPLIT_MIXED_ATTENTION = True
+# The prefill attention takes tiles of 128 queries when that still makes this many workgroups
+# (half as many when the longest context has 4096 positions or more).
+PREFILL_WIDE_MIN_GROUPS = 768
 # The norm in front of a projection goes into the streaming kernel where that applies.
 FUSE_NORM_LINEAR = True
 # The matrix-core decode attention rotates q and k and stores the new k, v itself where it can.
@@ -493,13 +496,24 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
         if singles and _decode_mfma_ok(qkv, nh, nkv, d, page_size):
             decode(singles, step.max_single_context, True, None)
             tile_map, num_tiles = step.multi_tile_map, step.num_multi_tiles
+        # Tiles of 128 queries (two query blocks per wave, half the LDS traffic per flop) where
+        # they still fill the chip: plenty of them, or fewer with long walks over cached keys.
+        # The step brings them for the same set of sequences.
+        tile_queries = 64
+        wide = getattr(step, "wide_multi_tile_map" if tile_map is not step.tile_map
+                       else "wide_tile_map", None)
+        if wide is not None and d <= 128:
+            groups = wide.numel() // 2 * nh
+            if groups >= PREFILL_WIDE_MIN_GROUPS or (2 * groups >= PREFILL_WIDE_MIN_GROUPS
+                                                     and step.max_context >= 4096):
+                tile_map, num_tiles, tile_queries = wide, wide.numel() // 2, 128
         if num_tiles:
             lib.call("rlis_attn_prefill_mfma", qkv.data_ptr(), q_stride, out.data_ptr(), nh * d,
                      k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,
                      _i32(step.cu_seqlens, "cu_seqlens", step.num_seqs + 1),
                      _i32(step.start_pos, "start_pos", step.num_seqs),
                      _i32(tile_map, "tile_map", 2 * num_tiles), num_tiles, nh, nkv, d,
-                     page_size, win, float(scale), 0, stream)
+                     page_size, win, float(scale), tile_queries, stream)
     elif kind == "generic":
         lib.call("rlis_attn_generic", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(), nh * d,
                  k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,

@@ -406,12 +406,16 @@ def paged_case(lens_cached, lens_new, nh, nkv, d, ps, dtype, seed=0, q_scale=1.0
     step.max_context, step.max_new = max(totals), max(lens_new)
     step.all_decode = all(n == 1 for n in lens_new)
     step.decode_splits = None
+    wide = [x for s, n in enumerate(lens_new) for qb in range(0, n, 128) for x in (s, qb)]
+    step.wide_tile_map = i32(wide)
     # single tokens that lead the batch, as the engine's steps order them
     lead = next((i for i, n in enumerate(lens_new) if n != 1), S)
     if all(n > 1 for n in lens_new[lead:]):
         multi = [x for s, n in enumerate(lens_new) if s >= lead for qb in range(0, n, 64) for x in (s, qb)]
         step.num_single, step.max_single_context = lead, max(totals[:lead], default=0)
         step.multi_tile_map, step.num_multi_tiles = i32(multi), len(multi) // 2
+        step.wide_multi_tile_map = i32([x for s, n in enumerate(lens_new) if s >= lead
+                                        for qb in range(0, n, 128) for x in (s, qb)])
     return (qkv.to(DEV), k_pages.to(DEV), v_pages.to(DEV), bt.to(DEV), step, ks, vs, cu)
 
 
@@ -473,6 +477,33 @@ def test_attention_single_tokens_beside_portions(ops, nh, nkv, d, ps, window):
         assert torch.equal(ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window), whole)
     finally:
         ops.SPLIT_MIXED_ATTENTION = old
+
+
+@pytest.mark.parametrize("nh,nkv,d,ps", [(32, 8, 64, 16), (24, 8, 128, 16), (6, 2, 32, 8), (5, 5, 48, 16),
+                                         (3, 1, 96, 32), (9, 3, 112, 16), (4, 2, 256, 16)])
+@pytest.mark.parametrize("window", [None, 70, 200])
+def test_attention_prefill_tiles_of_128_queries(ops, nh, nkv, d, ps, window):
+    """The prefill kernel with two query blocks per wave (tiles of 128 new tokens, which long
+    prompts take) against the plain implementation and against its 64-token form: portions that
+    end inside a tile, inside a query block, with and without cached positions, single tokens
+    among them.  Head sizes beyond 128 keep the 64-token form."""
+    dtype = torch.bfloat16
+    cached = [0, 5, 40, 0, 63, 130, 17, 300]
+    new = [33, 1, 70, 2, 129, 257, 128, 200]
+    scale = 1.0 / math.sqrt(d)
+    qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=nh + 2)
+    want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, window)
+    narrow = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window)
+    old = ops.PREFILL_WIDE_MIN_GROUPS
+    try:
+        ops.PREFILL_WIDE_MIN_GROUPS = 0
+        got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window)
+    finally:
+        ops.PREFILL_WIDE_MIN_GROUPS = old
+    torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
+    torch.testing.assert_close(got.float(), narrow.float(), atol=2e-2, rtol=2e-2)
+    if d <= 64:
+        assert torch.equal(got, narrow)            # the same tiles of keys, the same sums
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
