@@ -9,7 +9,13 @@ back), bracketed by device synchronisation.  On the same line: a 2,048-token pre
 fraction of the bf16 matrix peak, the decode step's achieved fraction of the HBM roofline
 (bytes that must be read: every weight once plus the live requests' cache), and decode
 throughput at batch 1 and 64 after 512-token prompts.  Weights are random (N(0, 0.02)),
-prompts are uniform random token ids."""
+prompts are uniform random token ids.
+
+    python bench.py --serve --model llama-3.2-3b --max-batched-tokens 512
+
+measures another workload instead (its own JSON line): R requests with prompts of uniform
+random length under continuous batching with chunked prefill, N new tokens each with seeded
+temperature sampling, timed from the first request's arrival to the last one's end."""
 import argparse
 import copy
 import json
@@ -40,6 +46,12 @@ def main() -> int:
     ap.add_argument("--skip-prefill", action="store_true")
     ap.add_argument("--max-batched-tokens", type=int, default=8192,
                     help="token budget of the engine steps that prefill the decode runs")
+    ap.add_argument("--serve", action="store_true",
+                    help="time a batch of requests through Engine.generate instead")
+    ap.add_argument("--requests", type=int, default=64)
+    ap.add_argument("--min-prompt", type=int, default=128)
+    ap.add_argument("--max-prompt", type=int, default=2048)
+    ap.add_argument("--new-tokens", type=int, default=256)
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (single-GPU engine)")
@@ -110,6 +122,44 @@ def main() -> int:
             raise RuntimeError("the timed steps were not pure decode steps of the whole batch")
         mean_ctx = prompt_len + (before.generated_tokens + after.generated_tokens) / 2 / batch
         return batch * steps / dt, dt / steps * 1e3, mean_ctx
+
+    if args.serve:
+        # ---- continuous batching: R requests, chunked prefill under the token budget ---------
+        lens = torch.randint(args.min_prompt, args.max_prompt + 1, (args.requests,), generator=g).tolist()
+        reqs = [torch.randint(0, V, (n,), generator=g).tolist() for n in lens]
+        pages = sum(-(-(n + args.new_tokens) // page) + 1 for n in lens) + 64
+        sp = SamplingParams(max_tokens=args.new_tokens, ignore_eos=True, temperature=0.8, seed=1)
+        best = None
+        for trial in range(2):                       # the first run also captures the graphs
+            engine = Engine(model, EngineConfig(
+                max_num_seqs=args.requests, max_batched_tokens=max(args.max_batched_tokens, args.requests),
+                num_pages=pages, block_size=page, max_seq_len=args.max_prompt + args.new_tokens + 8))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            outs = engine.generate(reqs, sp)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+            stats = engine.stats()
+            print(f"[bench] serve run {trial}: {dt:.3f}s, {stats.steps} steps, "
+                  f"{stats.preemptions} preemptions", file=sys.stderr, flush=True)
+        generated = sum(len(o.token_ids) for o in outs)
+        print(json.dumps({
+            "metric": f"served tok/s, {args.requests} requests ({args.model} shape)",
+            "value": round(generated / best, 1), "unit": "generated tokens/s", "n_gpus": 1,
+            "seconds": round(best, 4), "higher_is_better": True,
+            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
+            "config": {"model": args.model, "layers": L, "layers_full": full_layers,
+                       "requests": args.requests, "min_prompt": args.min_prompt,
+                       "max_prompt": args.max_prompt, "new_tokens": args.new_tokens,
+                       "max_batched_tokens": args.max_batched_tokens, "page_size": page,
+                       "prompt_tokens": sum(lens), "generated_tokens": generated,
+                       "steps": stats.steps, "mean_ttft_ms": round(
+                           sum(o.ttft for o in outs) / len(outs) * 1e3, 1)},
+            "total_tokens_per_s": round((generated + sum(lens)) / best, 1),
+        }))
+        return 0
 
     # ---- prefill: one prompt of T tokens in one step, last-row logits ------------------
     T = args.prefill_tokens
