@@ -57,10 +57,10 @@ namespace {
 
 constexpr int D = RLIS_HEAD_DIM;
 // Keys per tile: 64 up to head size 128, 32 beyond; with two query blocks per wave the
-// accumulators take twice the registers, and 32 keys per tile from head size 96 on keep the
-// staging and score registers within what two waves per SIMD can have.
+// accumulators take twice the registers, and 32 keys per tile keep the staging and score
+// registers within what three (head size up to 64) or two waves per SIMD can have.
 __host__ __device__ constexpr int tile_keys(int QB) {
-  return (D > 128 || (QB == 2 && D > 64)) ? 32 : 64;
+  return (D > 128 || QB == 2) ? 32 : 64;
 }
 constexpr int KS = D + 8;     // K tile row stride (bf16 elements)
 constexpr int BM = 64;       // queries per workgroup and query block
@@ -73,7 +73,7 @@ constexpr int kTileBufs = RLIS_PREFILL_BUFS;
 // Up to three waves per SIMD (two with two query blocks): the staging registers must not be
 // traded for another.
 template <int QB>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, QB == 1 ? 3 : 2))) void KERNEL_NAME(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, QB == 1 ? (D <= 64 ? 4 : 3) : (D <= 64 ? 3 : 2)))) void KERNEL_NAME(
     const bf16_t* __restrict__ q, long long q_stride, bf16_t* __restrict__ out,
     long long out_stride, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_seqlens,

@@ -502,8 +502,6 @@ def test_attention_prefill_tiles_of_128_queries(ops, nh, nkv, d, ps, window):
         ops.PREFILL_WIDE_MIN_GROUPS = old
     torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
     torch.testing.assert_close(got.float(), narrow.float(), atol=2e-2, rtol=2e-2)
-    if d <= 64:
-        assert torch.equal(got, narrow)            # the same tiles of keys, the same sums
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
