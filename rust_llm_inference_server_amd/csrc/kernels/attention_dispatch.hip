@@ -8,7 +8,8 @@
       const void* q, long long q_stride, void* out, long long out_stride, const void* k_pages, \
       const void* v_pages, const int* block_tables, int max_pages, const int* cu_seqlens,     \
       const int* start_pos, const int* tile_map, int num_tiles, int nh, int nkv, int d,       \
-      int page_shift, int window, float scale, int tile_queries, hipStream_t stream);
+      int page_shift, int window, float scale, int tile_queries, int splits, int row0,        \
+      float* part_ml, float* part_acc, hipStream_t stream);
 DECL(32) DECL(64) DECL(96) DECL(128) DECL(160) DECL(192) DECL(224) DECL(256)
 #undef DECL
 
@@ -25,19 +26,27 @@ int rlis_launch_attn_reduce_bf16(void* out, long long out_stride, const float* p
                                  const float* part_acc, int S, int nh, int d, int splits,
                                  hipStream_t stream);
 
+// splits > 1: the keys of every tile are cut into that many runs, one workgroup each, whose
+// partial results go to part_ml (rows, nh, splits, 2) and part_acc (rows, nh, splits, d)
+// float32 and are merged afterwards; `rows` output rows from row0 on are those that the tiles
+// cover (all of them: a row that no tile covers would be merged from nothing).
 RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out,
                                     long long out_stride, const void* k_pages,
                                     const void* v_pages, const int* block_tables, int max_pages,
                                     const int* cu_seqlens, const int* start_pos,
                                     const int* tile_map, int num_tiles, int nh, int nkv, int d,
                                     int page_size, int window, float scale, int tile_queries,
-                                    hipStream_t stream) {
+                                    int splits, int row0, int rows, float* part_ml,
+                                    float* part_acc, hipStream_t stream) {
   // tile_map lists tiles of tile_queries new tokens: 64 (0 means that too) or 128.
   if (tile_queries == 0) tile_queries = 64;
   RLIS_REQUIRE(tile_queries == 64 || tile_queries == 128,
                "attn_prefill_mfma: tiles of %d queries, 64 or 128 only", tile_queries);
   RLIS_REQUIRE(num_tiles >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0,
                "attn_prefill_mfma: bad sizes");
+  RLIS_REQUIRE(splits >= 1 && splits <= 64, "attn_prefill_mfma: %d key runs, 1 to 64", splits);
+  RLIS_REQUIRE(splits == 1 || (part_ml && part_acc && row0 >= 0 && rows > 0 && d % 4 == 0),
+               "attn_prefill_mfma: key runs need a workspace and the range of rows they cover");
   RLIS_REQUIRE(scale > 0.f, "attn_prefill_mfma: the score scale must be positive, got %g", scale);
   RLIS_REQUIRE(nh % nkv == 0, "attn_prefill_mfma: %d query heads are not a multiple of %d KV heads",
                nh, nkv);
@@ -50,20 +59,26 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
   RLIS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)k_pages % 16) == 0 &&
                    ((uintptr_t)v_pages % 16) == 0,
                "attn_prefill_mfma: operands must be 16-byte aligned with row strides in steps of 8");
+  int rc;
 #define CALL(D)                                                                                 \
-  return rlis_attn_prefill_mfma_d##D(q, q_stride, out, out_stride, k_pages, v_pages,            \
-                                     block_tables, max_pages, cu_seqlens, start_pos, tile_map,  \
-                                     num_tiles, nh, nkv, d, page_shift, window, scale,         \
-                                     tile_queries, stream)
+  rc = rlis_attn_prefill_mfma_d##D(q, q_stride, out, out_stride, k_pages, v_pages,              \
+                                   block_tables, max_pages, cu_seqlens, start_pos, tile_map,    \
+                                   num_tiles, nh, nkv, d, page_shift, window, scale,            \
+                                   tile_queries, splits, row0, part_ml, part_acc, stream)
   if (d <= 32) CALL(32);
-  if (d <= 64) CALL(64);
-  if (d <= 96) CALL(96);
-  if (d <= 128) CALL(128);
-  if (d <= 160) CALL(160);
-  if (d <= 192) CALL(192);
-  if (d <= 224) CALL(224);
-  CALL(256);
+  else if (d <= 64) CALL(64);
+  else if (d <= 96) CALL(96);
+  else if (d <= 128) CALL(128);
+  else if (d <= 160) CALL(160);
+  else if (d <= 192) CALL(192);
+  else if (d <= 224) CALL(224);
+  else CALL(256);
 #undef CALL
+  if (rc) return rc;
+  if (splits > 1 && num_tiles > 0)
+    return rlis_launch_attn_reduce_bf16((bf16_t*)out + (long long)row0 * out_stride, out_stride,
+                                        part_ml, part_acc, rows, nh, d, splits, stream);
+  return 0;
 }
 
 // One query token per sequence (bfloat16): q rows are the sequences themselves.  Needs at most

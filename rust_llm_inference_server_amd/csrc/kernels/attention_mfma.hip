@@ -73,12 +73,13 @@ constexpr int kTileBufs = RLIS_PREFILL_BUFS;
 // Up to three waves per SIMD (two with two query blocks): the staging registers must not be
 // traded for another.
 template <int QB>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, QB == 1 ? (D <= 64 ? 4 : 3) : (D <= 64 ? 3 : 2)))) void KERNEL_NAME(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 && D <= 64) ? 4 : 1, QB == 1 ? (D <= 64 ? 4 : 3) : (D <= 64 ? 3 : 2)))) void KERNEL_NAME(
     const bf16_t* __restrict__ q, long long q_stride, bf16_t* __restrict__ out,
     long long out_stride, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_seqlens,
     const int* __restrict__ start_pos, const int* __restrict__ tile_map, int nh, int nkv, int d,
-    int page_shift, float scale, int window, int num_tiles, int tiles_per_round) {
+    int page_shift, float scale, int window, int num_tiles, int tiles_per_round, int splits,
+    int row0, float* __restrict__ part_ml, float* __restrict__ part_acc) {
   constexpr int BN = tile_keys(QB);
   constexpr int VS = BN + 8;    // V tile row stride
   __shared__ __attribute__((aligned(16))) bf16_t Ks_all[kTileBufs * BN * KS];
@@ -90,8 +91,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, QB == 1 
   // One round of blocks (tiles_per_round tiles x all heads) fills the compute units once; every
   // other round walks its tiles backwards, so that a unit that drew a long tile in one round
   // draws a short one in the next.
+  // With `splits` > 1 the keys of a tile are cut into that many runs of whole key tiles, one
+  // workgroup each (splits fastest after the heads): few tiles with long walks over cached
+  // keys then still fill the chip.  Such workgroups store unnormalised sums with their maximum
+  // and denominator, which attn_reduce (attention.hip) merges.
   const int h = blockIdx.x % nh;
-  int tile = blockIdx.x / nh;
+  const int split = (blockIdx.x / nh) % splits;
+  int tile = blockIdx.x / nh / splits;
   if (tiles_per_round > 0) {
     const int round = tile / tiles_per_round, within = tile % tiles_per_round;
     const bool whole = (round + 1) * tiles_per_round <= num_tiles;
@@ -135,10 +141,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, QB == 1 
   }
 
   const int q_last = min(n_new, qb + BM * QB) - 1;      // last new-token index of the tile
-  const int khi = P + q_last + 1;                        // keys [klo, khi) matter to the tile
+  const int khi_all = P + q_last + 1;                    // keys [klo, khi_all) matter to the tile
   int klo = 0;
   if (window > 0) klo = max(0, P + qb - window + 1);
-  const int kt0 = (klo / BN) * BN;
+  const int kt0_all = (klo / BN) * BN;
+  int kt0 = kt0_all, khi = khi_all;                      // this workgroup's run of them
+  if (splits > 1) {
+    const int per = ((khi_all - kt0_all + BN - 1) / BN + splits - 1) / splits;
+    kt0 = kt0_all + split * per * BN;
+    khi = min(khi_all, kt0 + per * BN);
+  }
   const int wave_q_last = min(n_new - 1, wave_q_first + 16 * QB - 1);
 
   // Staging for the tiles to come.  A tile's page ids are fetched four tiles ahead of its use,
@@ -208,7 +220,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, QB == 1 
   }
 
   const float scale2 = scale * 1.4426950408889634f;      // scores in the base-2 domain
-  if (kt0 < khi) {           // else this tile has no keys at all (it cannot happen: khi > P + qb)
+  if (kt0 < khi) {           // else this run has no keys (only with splits)
   RLIS_LOAD_PAGES(kt0, page_ka, page_va);
   RLIS_LOAD_PAGES(kt0 + BN, page_kb, page_vb);
   RLIS_LOAD_TILE(kt0, page_ka, page_va, tile_ka, tile_va);
@@ -360,16 +372,35 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, QB == 1 
 #pragma unroll
   for (int b = 0; b < QB; ++b) {
     if (my_qi[b] < n_new) {
-      const float inv_l = 1.0f / l_run[b];
-      bf16_t* orow = out + (long long)(tok_begin + my_qi[b]) * out_stride + h * d;
+      const long long row = tok_begin + my_qi[b];
+      if (splits == 1) {
+        const float inv_l = 1.0f / l_run[b];
+        bf16_t* orow = out + row * out_stride + h * d;
 #pragma unroll
-      for (int db = 0; db < D / 16; ++db) {
-        const int dim = db * 16 + lq * 4;
-        if (dim < d) {
-          union { uint2 u; bf16_t e[4]; } o;
+        for (int db = 0; db < D / 16; ++db) {
+          const int dim = db * 16 + lq * 4;
+          if (dim < d) {
+            union { uint2 u; bf16_t e[4]; } o;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) o.e[r] = f32_to_bf16(o_acc[b][db][r] * inv_l);
-          *(uint2*)(orow + dim) = o.u;
+            for (int r = 0; r < 4; ++r) o.e[r] = f32_to_bf16(o_acc[b][db][r] * inv_l);
+            *(uint2*)(orow + dim) = o.u;
+          }
+        }
+      } else {
+        const long long idx = ((row - row0) * nh + h) * splits + split;
+        float* arow = part_acc + idx * d;
+#pragma unroll
+        for (int db = 0; db < D / 16; ++db) {
+          const int dim = db * 16 + lq * 4;
+          if (dim < d)
+            *(float4*)(arow + dim) = make_float4(o_acc[b][db][0], o_acc[b][db][1],
+                                                 o_acc[b][db][2], o_acc[b][db][3]);
+        }
+        if (lq == 0) {
+          // attn_reduce works with natural-log maxima: m * ln 2 (-inf, with a denominator of
+          // zero, where the query sees no key of this run)
+          part_ml[idx * 2] = m_run[b] * 0.6931471805599453f;
+          part_ml[idx * 2 + 1] = l_run[b];
         }
       }
     }
@@ -382,25 +413,26 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
     const void* q, long long q_stride, void* out, long long out_stride, const void* k_pages,
     const void* v_pages, const int* block_tables, int max_pages, const int* cu_seqlens,
     const int* start_pos, const int* tile_map, int num_tiles, int nh, int nkv, int d,
-    int page_shift, int window, float scale, int tile_queries, hipStream_t stream) {
+    int page_shift, int window, float scale, int tile_queries, int splits, int row0,
+    float* part_ml, float* part_acc, hipStream_t stream) {
   if (num_tiles == 0) return 0;
-  const long long blocks = (long long)num_tiles * nh;
+  const long long blocks = (long long)num_tiles * nh * splits;
   if (blocks >= (1ll << 31)) {
     rlis_set_error("attn_prefill_mfma: too many tiles");
     return 1;
   }
   // 256 compute units: a round is the tiles whose blocks fill them once.
-  const int tiles_per_round = (nh <= 256 && 256 % nh == 0) ? 256 / nh : 0;
+  const int tiles_per_round = (splits == 1 && nh <= 256 && 256 % nh == 0) ? 256 / nh : 0;
   if (tile_queries == 2 * BM)
     KERNEL_NAME<2><<<(int)blocks, 256, 0, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,
         (const bf16_t*)v_pages, block_tables, max_pages, cu_seqlens, start_pos, tile_map, nh, nkv,
-        d, page_shift, scale, window, num_tiles, tiles_per_round);
+        d, page_shift, scale, window, num_tiles, tiles_per_round, splits, row0, part_ml, part_acc);
   else
     KERNEL_NAME<1><<<(int)blocks, 256, 0, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,
         (const bf16_t*)v_pages, block_tables, max_pages, cu_seqlens, start_pos, tile_map, nh, nkv,
-        d, page_shift, scale, window, num_tiles, tiles_per_round);
+        d, page_shift, scale, window, num_tiles, tiles_per_round, splits, row0, part_ml, part_acc);
   RLIS_LAUNCH_CHECK("attn_prefill_mfma");
   return 0;
 }

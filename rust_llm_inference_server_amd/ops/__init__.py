@@ -26,6 +26,11 @@ SPLIT_MIXED_ATTENTION = True
 # The prefill attention takes tiles of 128 queries when that still makes this many workgroups
 # (half as many when the longest context has 4096 positions or more).
 PREFILL_WIDE_MIN_GROUPS = 768
+# The prefill attention cuts the keys of its tiles into runs (one workgroup each, merged
+# afterwards) while that still fits the chip's compute units at once, with at least this many
+# keys a run (0 units: never).
+PREFILL_SPLIT_UNITS = 256
+PREFILL_SPLIT_MIN_KEYS = 512
 # The norm in front of a projection goes into the streaming kernel where that applies.
 FUSE_NORM_LINEAR = True
 # The matrix-core decode attention rotates q and k and stores the new k, v itself where it can.
@@ -493,9 +498,10 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
         # kernel reads their keys and values once for the whole group of heads, where a
         # 64-query tile of the prefill kernel would walk the context for one query per head.
         singles = getattr(step, "num_single", 0) if force is None and SPLIT_MIXED_ATTENTION else 0
+        row0 = 0                      # the first row that the prefill kernel's tiles cover
         if singles and _decode_mfma_ok(qkv, nh, nkv, d, page_size):
             decode(singles, step.max_single_context, True, None)
-            tile_map, num_tiles = step.multi_tile_map, step.num_multi_tiles
+            tile_map, num_tiles, row0 = step.multi_tile_map, step.num_multi_tiles, singles
         # Tiles of 128 queries (two query blocks per wave, half the LDS traffic per flop) where
         # they still fill the chip: plenty of them, or fewer with long walks over cached keys.
         # The step brings them for the same set of sequences.
@@ -508,12 +514,27 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                                                      and step.max_context >= 4096):
                 tile_map, num_tiles, tile_queries = wide, wide.numel() // 2, 128
         if num_tiles:
+            # Few tiles with long walks over cached keys (a portion of a long prompt): the keys
+            # of every tile are cut into runs, one workgroup each, and merged afterwards.
+            splits = getattr(step, "prefill_splits", None)
+            if splits is None:
+                # as many runs as keep every compute unit's resident workgroups in one round
+                # (4 of them up to head size 64, 3 with 128-query tiles, 2 beyond)
+                resident = 2 if d > 64 else (3 if tile_queries == 128 else 4)
+                splits = max(1, min(PREFILL_SPLIT_UNITS * resident // (num_tiles * nh),
+                                    step.max_context // PREFILL_SPLIT_MIN_KEYS, 16))
+            part_ml = part_acc = None
+            if splits > 1:
+                part_ml = torch.empty((T - row0, nh, splits, 2), dtype=torch.float32, device=qkv.device)
+                part_acc = torch.empty((T - row0, nh, splits, d), dtype=torch.float32, device=qkv.device)
             lib.call("rlis_attn_prefill_mfma", qkv.data_ptr(), q_stride, out.data_ptr(), nh * d,
                      k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,
                      _i32(step.cu_seqlens, "cu_seqlens", step.num_seqs + 1),
                      _i32(step.start_pos, "start_pos", step.num_seqs),
                      _i32(tile_map, "tile_map", 2 * num_tiles), num_tiles, nh, nkv, d,
-                     page_size, win, float(scale), tile_queries, stream)
+                     page_size, win, float(scale), tile_queries, splits, row0, T - row0,
+                     None if part_ml is None else part_ml.data_ptr(),
+                     None if part_acc is None else part_acc.data_ptr(), stream)
     elif kind == "generic":
         lib.call("rlis_attn_generic", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(), nh * d,
                  k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,

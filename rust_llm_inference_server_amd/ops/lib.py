@@ -31,7 +31,8 @@ _SIGNATURES = {
     "rlis_attn_decode": [P, I, L, P, L, P, P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, P],
     "rlis_attn_decode_mfma": [P, L, P, L, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, P, P, I, P, P, L, L,
                               P],
-    "rlis_attn_prefill_mfma": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P],
+    "rlis_attn_prefill_mfma": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, I, I, P, P,
+                               P],
     "rlis_sample_rows": [P, L, I, I, P, P, P, I, P, P, P],
 }
 

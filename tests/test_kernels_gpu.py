@@ -504,6 +504,34 @@ def test_attention_prefill_tiles_of_128_queries(ops, nh, nkv, d, ps, window):
     torch.testing.assert_close(got.float(), narrow.float(), atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("nh,nkv,d,ps", [(32, 8, 64, 16), (24, 8, 128, 16), (6, 2, 32, 8), (3, 1, 96, 32),
+                                         (4, 2, 256, 16)])
+@pytest.mark.parametrize("window", [None, 70])
+@pytest.mark.parametrize("splits", [2, 3, 7])
+def test_attention_prefill_with_keys_cut_into_runs(ops, nh, nkv, d, ps, window, splits):
+    """The prefill kernel with every tile's keys cut into runs that separate workgroups take and
+    a merge afterwards (what a portion of a long prompt gets): against the plain
+    implementation, with both tile sizes; runs without keys, queries that see no key of a run,
+    single tokens handled by the decode kernel beside them."""
+    dtype = torch.bfloat16
+    cached = [5, 300, 0, 40, 0, 130, 700]
+    new = [1, 1, 33, 70, 2, 129, 200]
+    scale = 1.0 / math.sqrt(d)
+    qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=nh + 3)
+    want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, window)
+    step.prefill_splits = splits
+    old = ops.PREFILL_WIDE_MIN_GROUPS
+    try:
+        for wide in (False, True):
+            ops.PREFILL_WIDE_MIN_GROUPS = 0 if wide else 1 << 30
+            got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window)
+            torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
+            whole = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window, force="prefill")
+            torch.testing.assert_close(whole.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
+    finally:
+        ops.PREFILL_WIDE_MIN_GROUPS = old
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("kind", ["generic", "prefill", "decode"])
 @pytest.mark.parametrize("window", [1, 7, 64, 100])
