@@ -69,8 +69,10 @@ def main() -> int:
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
-    cfg["max_position_embeddings"] = min(cfg["max_position_embeddings"],
-                                         max(args.context, args.prefill_tokens, 4096) + 64)
+    longest = max(args.context, args.prefill_tokens, 4096)
+    if args.serve:
+        longest = max(longest, args.max_prompt + args.new_tokens)
+    cfg["max_position_embeddings"] = min(cfg["max_position_embeddings"], longest + 64)
     page = 16
     K, W = args.steps, args.warmup
     elem = 2 if args.dtype == "bfloat16" else 4
