@@ -27,8 +27,8 @@ SPLIT_MIXED_ATTENTION = True
 # (half as many when the longest context has 4096 positions or more).
 PREFILL_WIDE_MIN_GROUPS = 768
 # The prefill attention cuts the keys of its tiles into runs (one workgroup each, merged
-# afterwards) while that still fits the chip's compute units at once, with at least this many
-# keys a run (0 units: never).
+# afterwards) when its tiles leave compute units without work: as many runs as the units hold
+# at once, with at least this many keys a run (0 units: never).
 PREFILL_SPLIT_UNITS = 256
 PREFILL_SPLIT_MIN_KEYS = 512
 # The norm in front of a projection goes into the streaming kernel where that applies.
@@ -520,9 +520,11 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
             if splits is None:
                 # as many runs as keep every compute unit's resident workgroups in one round
                 # (4 of them up to head size 64, 3 with 128-query tiles, 2 beyond)
-                resident = 2 if d > 64 else (3 if tile_queries == 128 else 4)
-                splits = max(1, min(PREFILL_SPLIT_UNITS * resident // (num_tiles * nh),
-                                    step.max_context // PREFILL_SPLIT_MIN_KEYS, 16))
+                splits, groups = 1, num_tiles * nh
+                if groups <= PREFILL_SPLIT_UNITS:
+                    resident = 2 if d > 64 else (3 if tile_queries == 128 else 4)
+                    splits = max(1, min(PREFILL_SPLIT_UNITS * resident // groups,
+                                        step.max_context // PREFILL_SPLIT_MIN_KEYS, 16))
             part_ml = part_acc = None
             if splits > 1:
                 part_ml = torch.empty((T - row0, nh, splits, 2), dtype=torch.float32, device=qkv.device)
