@@ -124,6 +124,77 @@ def test_first_tokens_of_a_sequence(case, dtype):
         assert runner.cache.num_free_pages(0) == runner.cache.num_pages(0)
 
 
+LONG = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 128, "intermediate_size": 176,
+    "num_hidden_layers": 2, "num_attention_heads": 8, "num_key_value_heads": 2, "head_dim": 64,
+    "vocab_size": 301, "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                     "high_freq_factor": 4.0, "original_max_position_embeddings": 1024},
+    "max_position_embeddings": 4096, "tie_word_embeddings": True,
+}
+
+
+@pytest.mark.parametrize("wide", [False, True], ids=["tiles64", "tiles128"])
+def test_long_prompt_whole_and_in_portions(tmp_path, wide):
+    """A prompt of 2,600 tokens in one step and in portions of 512 and 200 beside a decoding
+    request, bfloat16: the long walks over cached keys take the prefill attention's forms for
+    them (keys cut into runs and merged; tiles of 128 queries), which tiny prompts never reach.
+    One key far back is made to stand out for the last token, so that a lost run would show."""
+    from rust_llm_inference_server_amd import ops
+    folder = make_model_folder(tmp_path / "long", LONG, seed=5, dtype=torch.bfloat16)
+    w, c = plain.read_weights(folder), plain.read_config(folder)
+    reqs = traces.random_requests(LONG["vocab_size"], [2600, 40], seed=4)
+    reqs["r0"][-1] = reqs["r0"][700]                      # the last token meets itself far back
+    ref = {k: plain.forward(w, c, t) for k, t in reqs.items()}
+    long_t, short_t = reqs["r0"], reqs["r1"]
+    steps = [{"step": 0, "entries": [{"id": "whole", "tokens": long_t, "want": [0, 1299, 2599]}],
+              "end": ["whole"]},
+             {"step": 1, "entries": [{"id": "r1", "tokens": short_t[:30], "want": []}], "end": []}]
+    pos, dec = 0, 30
+    for n in [512, 200] * 4:
+        n = min(n, len(long_t) - pos)
+        if n == 0:
+            break
+        entries = [{"id": "r0", "tokens": long_t[pos:pos + n], "want": [0, n - 1]}]
+        if dec < len(short_t):
+            entries.append({"id": "r1", "tokens": [short_t[dec]], "want": [0]})
+            dec += 1
+        steps.append({"step": len(steps), "entries": entries, "end": []})
+        pos += n
+    assert pos == len(long_t)
+    steps[-1]["end"] = ["r0", "r1"]
+    old, call = ops.PREFILL_WIDE_MIN_GROUPS, ops.lib.call
+    seen = []                                   # (tile_queries, splits) of every prefill launch
+
+    def spy(name, *args):
+        if name == "rlis_attn_prefill_mfma":
+            seen.append((args[18], args[19]))
+        return call(name, *args)
+
+    try:
+        ops.PREFILL_WIDE_MIN_GROUPS = 0 if wide else 1 << 30
+        ops.lib.call = spy
+        runner = make_runner(folder, "bfloat16", 2 * 2624 + 64, page_size=16)
+        outputs = traces.replay_in_process(runner, steps)
+    finally:
+        ops.PREFILL_WIDE_MIN_GROUPS, ops.lib.call = old, call
+    assert any(runs > 1 for _, runs in seen) and any(runs == 1 for _, runs in seen)
+    assert {tq for tq, _ in seen} == ({128} if wide else {64})
+    whole = outputs[0]
+    want = ref["r0"]
+    assert (whole - want[[0, 1299, 2599]]).abs().max().item() < TOL["bfloat16"]
+    pos, dec = 0, 30
+    for st in steps[2:]:
+        n = len(st["entries"][0]["tokens"])
+        got = outputs[st["step"]]
+        assert (got[:2] - want[[pos, pos + n - 1]]).abs().max().item() < TOL["bfloat16"], f"portion at {pos}"
+        if len(st["entries"]) > 1:
+            assert (got[2] - ref["r1"][dec]).abs().max().item() < TOL["bfloat16"], f"decoded token {dec}"
+            dec += 1
+        pos += n
+    assert runner.cache.num_free_pages(0) == runner.cache.num_pages(0)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(case, dtype, tmp_path):
     """The program itself, as a child process fed step by step, on the mixed trace."""
