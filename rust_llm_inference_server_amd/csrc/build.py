@@ -1,9 +1,12 @@
 """Compiles the native code in-tree: the gfx950 kernels (hipcc) and the host runtime (g++).
 
-Two libraries are built into ``rust_llm_inference_server_amd/_lib``:
+These libraries are built into ``rust_llm_inference_server_amd/_lib``:
 
-* ``librlis_kernels.so``  - every ``kernels/*.hip`` (and the per-head-size attention units);
-* ``librlis_runtime.so``  - ``runtime/*.cpp``: page manager and scheduler, no GPU needed.
+* ``librlis_kernels.so``   - ``kernels/*.hip`` but the matrix-core attention;
+* ``librlis_attn_dN.so``   - the matrix-core attention (``kernels/attention_mfma.hip``) for head
+  sizes up to N = 32, 64, ... 256, one library each: a model needs one of them, and only that
+  one is built and loaded for it;
+* ``librlis_runtime.so``   - ``runtime/*.cpp``: page manager and scheduler, no GPU needed.
 
 ``ensure(name)`` returns the path of a library, building it first when it is absent or older
 than its sources; a line is printed before each compile step so that a first call in a fresh
@@ -67,34 +70,49 @@ def _lib_dir() -> str:
         return d
 
 
+ATTENTION_UNIT_SOURCE = "attention_mfma.hip"
+
+
+def attention_unit(head_dim: int) -> str:
+    """The library kind that serves ``head_dim`` on the matrix cores."""
+    padded = -(-head_dim // 32) * 32
+    if padded not in MFMA_ATTENTION_HEAD_DIMS:
+        raise ValueError(f"no matrix-core attention unit for head size {head_dim}")
+    return f"attn_d{padded}"
+
+
+def all_kinds() -> List[str]:
+    return ["runtime", "kernels"] + [f"attn_d{d}" for d in MFMA_ATTENTION_HEAD_DIMS]
+
+
+def _is_hip(kind: str) -> bool:
+    return kind != "runtime"
+
+
 def _sources(kind: str) -> List[str]:
-    sub = "kernels" if kind == "kernels" else "runtime"
-    ext = (".hip",) if kind == "kernels" else (".cpp",)
-    d = os.path.join(HERE, sub)
-    return sorted(os.path.join(d, f) for f in os.listdir(d) if f.endswith(ext))
+    d = os.path.join(HERE, "kernels" if _is_hip(kind) else "runtime")
+    if kind.startswith("attn_d"):
+        return [os.path.join(d, ATTENTION_UNIT_SOURCE)]
+    ext = (".hip",) if _is_hip(kind) else (".cpp",)
+    return sorted(os.path.join(d, f) for f in os.listdir(d)
+                  if f.endswith(ext) and f != ATTENTION_UNIT_SOURCE)
 
 
 def _headers(kind: str) -> List[str]:
-    sub = "kernels" if kind == "kernels" else "runtime"
-    d = os.path.join(HERE, sub)
+    d = os.path.join(HERE, "kernels" if _is_hip(kind) else "runtime")
     return sorted(os.path.join(d, f) for f in os.listdir(d) if f.endswith((".h", ".hpp")))
 
 
 def _units(kind: str) -> List[Tuple[str, str, List[str]]]:
     """(object name, source, extra defines) for every compile step."""
-    units = []
-    for src in _sources(kind):
-        base = os.path.splitext(os.path.basename(src))[0]
-        if kind == "kernels" and base == "attention_mfma":
-            for d in MFMA_ATTENTION_HEAD_DIMS:
-                units.append((f"{base}_d{d}", src, [f"-DRLIS_HEAD_DIM={d}"]))
-        else:
-            units.append((base, src, []))
-    return units
+    if kind.startswith("attn_d"):
+        src, = _sources(kind)
+        return [(f"attention_mfma_{kind[5:]}", src, [f"-DRLIS_HEAD_DIM={kind[6:]}"])]
+    return [(os.path.splitext(os.path.basename(src))[0], src, []) for src in _sources(kind)]
 
 
 def source_hash(kind: str) -> str:
-    h = hashlib.sha256()
+    h = hashlib.sha256(kind.encode())
     for path in _sources(kind) + _headers(kind) + [os.path.abspath(__file__)]:
         h.update(os.path.basename(path).encode())
         with open(path, "rb") as f:
@@ -123,40 +141,48 @@ def _run(cmd: Sequence[str], what: str) -> None:
     _say(f"{what} done in {time.time() - t0:.1f}s")
 
 
-def build(kind: str, jobs: Optional[int] = None) -> str:
-    """Compile library ``kind`` ('kernels' or 'runtime') from scratch and return its path."""
-    out = lib_path(kind)
-    obj_dir = os.path.join(os.path.dirname(out), f"_build_{kind}")
+def build_many(kinds: Sequence[str], jobs: Optional[int] = None) -> List[str]:
+    """Compile the libraries ``kinds`` from scratch (all their units through one pool) and
+    return their paths."""
+    lib_dir = _lib_dir()
+    obj_dir = os.path.join(lib_dir, f"_build_{os.getpid()}")
     os.makedirs(obj_dir, exist_ok=True)
-    units = _units(kind)
-    if kind == "kernels":
-        cc, flags = _hipcc(), HIP_FLAGS
-    else:
-        cc, flags = shutil.which("g++") or "g++", CXX_FLAGS
-    jobs = jobs or min(8, os.cpu_count() or 1, len(units))
-    _say(f"compiling {len(units)} {kind} units with {os.path.basename(cc)} ({jobs} at a time)")
-    objs: Dict[str, str] = {}
+    work: List[Tuple[str, Tuple[str, str, List[str]]]] = [(k, u) for k in kinds for u in _units(k)]
+    jobs = jobs or min(8, os.cpu_count() or 1, len(work))
+    _say(f"compiling {len(work)} units of {', '.join(kinds)} ({jobs} at a time)")
 
-    def compile_one(unit: Tuple[str, str, List[str]]) -> str:
-        name, src, defs = unit
-        obj = os.path.join(obj_dir, name + ".o")
+    def compile_one(item: Tuple[str, Tuple[str, str, List[str]]]) -> str:
+        kind, (name, src, defs) = item
+        cc, flags = (_hipcc(), HIP_FLAGS) if _is_hip(kind) else (shutil.which("g++") or "g++", CXX_FLAGS)
+        obj = os.path.join(obj_dir, f"{kind}.{name}.o")
         _say(f"  {name} ...")
         _run([cc, *flags, *defs, "-c", src, "-o", obj], f"  {name}")
         return obj
 
+    objs: Dict[str, List[str]] = {k: [] for k in kinds}
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
-        for unit, obj in zip(units, pool.map(compile_one, units)):
-            objs[unit[0]] = obj
-    tmp = out + f".tmp{os.getpid()}"
-    link = [cc, "-shared", "-o", tmp, *objs.values()]
-    if kind == "kernels":
-        link[1:1] = [f"--offload-arch={ARCH}", "-fPIC"]
-    _run(link, f"linking {os.path.basename(out)}")
-    os.replace(tmp, out)
-    with open(out + ".hash", "w") as f:
-        f.write(source_hash(kind))
+        for (kind, _), obj in zip(work, pool.map(compile_one, work)):
+            objs[kind].append(obj)
+    outs = []
+    for kind in kinds:
+        out = lib_path(kind)
+        tmp = out + f".tmp{os.getpid()}"
+        if _is_hip(kind):
+            link = [_hipcc(), f"--offload-arch={ARCH}", "-fPIC", "-shared", "-o", tmp, *objs[kind]]
+        else:
+            link = [shutil.which("g++") or "g++", "-shared", "-o", tmp, *objs[kind]]
+        _run(link, f"linking {os.path.basename(out)}")
+        os.replace(tmp, out)
+        with open(out + ".hash", "w") as f:
+            f.write(source_hash(kind))
+        outs.append(out)
     shutil.rmtree(obj_dir, ignore_errors=True)
-    return out
+    return outs
+
+
+def build(kind: str, jobs: Optional[int] = None) -> str:
+    """Compile library ``kind`` ('kernels', 'runtime' or an attention unit) from scratch."""
+    return build_many([kind], jobs)[0]
 
 
 def ensure(kind: str) -> str:
@@ -168,8 +194,7 @@ def ensure(kind: str) -> str:
 
 
 def build_all() -> None:
-    build("runtime")
-    build("kernels")
+    build_many(all_kinds())
 
 
 if __name__ == "__main__":

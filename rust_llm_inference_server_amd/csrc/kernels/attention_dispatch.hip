@@ -1,26 +1,50 @@
-// Picks the matrix-core prefill attention unit built for the head size at hand.  Each unit
-// (attention_mfma.hip compiled with RLIS_HEAD_DIM = 32, 64, ... 256) serves head sizes up to
-// its own, padding the rest with zeros.
+// Checks the arguments of the matrix-core attention kernels and hands them to the unit built
+// for the head size at hand.  Each unit (attention_mfma.hip compiled with RLIS_HEAD_DIM = 32,
+// 64, ... 256) serves head sizes up to its own, padding the rest with zeros.
 #include "common.h"
 
-#define DECL(D)                                                                               \
-  extern "C" int rlis_attn_prefill_mfma_d##D(                                                 \
-      const void* q, long long q_stride, void* out, long long out_stride, const void* k_pages, \
-      const void* v_pages, const int* block_tables, int max_pages, const int* cu_seqlens,     \
-      const int* start_pos, const int* tile_map, int num_tiles, int nh, int nkv, int d,       \
-      int page_shift, int window, float scale, int tile_queries, int splits, int row0,        \
-      float* part_ml, float* part_acc, hipStream_t stream);
-DECL(32) DECL(64) DECL(96) DECL(128) DECL(160) DECL(192) DECL(224) DECL(256)
-#undef DECL
+typedef int (*PrefillUnit)(const void* q, long long q_stride, void* out, long long out_stride,
+                           const void* k_pages, const void* v_pages, const int* block_tables,
+                           int max_pages, const int* cu_seqlens, const int* start_pos,
+                           const int* tile_map, int num_tiles, int nh, int nkv, int d,
+                           int page_shift, int window, float scale, int tile_queries, int splits,
+                           int row0, float* part_ml, float* part_acc, hipStream_t stream);
+typedef int (*DecodeUnit)(const void* q, long long q_stride, void* out, long long out_stride,
+                          float* part_ml, float* part_acc, const void* k_pages,
+                          const void* v_pages, const int* block_tables, int max_pages,
+                          const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift,
+                          int window, float scale, int splits, const DecodeRope* rope,
+                          hipStream_t stream);
 
-#define DECL(D)                                                                                \
-  extern "C" int rlis_attn_decode_mfma_d##D(                                                   \
-      const void* q, long long q_stride, void* out, long long out_stride, float* part_ml,      \
-      float* part_acc, const void* k_pages, const void* v_pages, const int* block_tables,      \
-      int max_pages, const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift,       \
-      int window, float scale, int splits, const DecodeRope* rope, hipStream_t stream);
-DECL(32) DECL(64) DECL(96) DECL(128) DECL(160) DECL(192) DECL(224) DECL(256)
-#undef DECL
+// The units (attention_mfma.hip compiled for a padded head size of 32, 64, ... 256) are
+// libraries of their own, built and loaded when a model needs them and registered here.
+constexpr int kUnits = 8;
+static PrefillUnit prefill_units[kUnits];
+static DecodeUnit decode_units[kUnits];
+
+static int unit_index(int d) { return (d + 31) / 32 - 1; }
+
+RLIS_API int rlis_attn_register_unit(int padded_head_dim, void* prefill, void* decode) {
+  RLIS_REQUIRE(padded_head_dim % 32 == 0 && padded_head_dim >= 32 && padded_head_dim <= 32 * kUnits &&
+                   prefill && decode,
+               "attn_register_unit: bad unit for head size %d", padded_head_dim);
+  prefill_units[unit_index(padded_head_dim)] = (PrefillUnit)prefill;
+  decode_units[unit_index(padded_head_dim)] = (DecodeUnit)decode;
+  return 0;
+}
+
+// What a unit's return code says.
+static int unit_result(const char* name, int rc, int d) {
+  if (rc == 0) return 0;
+  if (rc == 1) rlis_set_error("%s: too many tiles", name);
+  else if (rc == 2)
+    rlis_set_error("%s: rotation inside the kernel needs head_dim = rotated width = 64, 128 or "
+                   "256 (got %d)", name, d);
+  else if (rc >= 1000)
+    rlis_set_error("%s: launch failed: %s", name, hipGetErrorString((hipError_t)(rc - 1000)));
+  else rlis_set_error("%s: unit error %d", name, rc);
+  return 1;
+}
 
 int rlis_launch_attn_reduce_bf16(void* out, long long out_stride, const float* part_ml,
                                  const float* part_acc, int S, int nh, int d, int splits,
@@ -59,21 +83,14 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
   RLIS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)k_pages % 16) == 0 &&
                    ((uintptr_t)v_pages % 16) == 0,
                "attn_prefill_mfma: operands must be 16-byte aligned with row strides in steps of 8");
-  int rc;
-#define CALL(D)                                                                                 \
-  rc = rlis_attn_prefill_mfma_d##D(q, q_stride, out, out_stride, k_pages, v_pages,              \
-                                   block_tables, max_pages, cu_seqlens, start_pos, tile_map,    \
-                                   num_tiles, nh, nkv, d, page_shift, window, scale,            \
-                                   tile_queries, splits, row0, part_ml, part_acc, stream)
-  if (d <= 32) CALL(32);
-  else if (d <= 64) CALL(64);
-  else if (d <= 96) CALL(96);
-  else if (d <= 128) CALL(128);
-  else if (d <= 160) CALL(160);
-  else if (d <= 192) CALL(192);
-  else if (d <= 224) CALL(224);
-  else CALL(256);
-#undef CALL
+  const PrefillUnit unit = prefill_units[unit_index(d)];
+  RLIS_REQUIRE(unit != nullptr, "attn_prefill_mfma: the unit for head size %d is not loaded", d);
+  const int rc = unit_result(
+      "attn_prefill_mfma",
+      unit(q, q_stride, out, out_stride, k_pages, v_pages, block_tables, max_pages, cu_seqlens,
+           start_pos, tile_map, num_tiles, nh, nkv, d, page_shift, window, scale, tile_queries,
+           splits, row0, part_ml, part_acc, stream),
+      d);
   if (rc) return rc;
   if (splits > 1 && num_tiles > 0)
     return rlis_launch_attn_reduce_bf16((bf16_t*)out + (long long)row0 * out_stride, out_stride,
@@ -132,20 +149,13 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
   RLIS_REQUIRE(splits == 1 || (part_ml && part_acc), "attn_decode_mfma: partitions need a workspace");
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;
-  int rc;
-#define CALL(D)                                                                                 \
-  rc = rlis_attn_decode_mfma_d##D(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,     \
-                                  v_pages, block_tables, max_pages, ctx_lens, S, nh, nkv, d,    \
-                                  page_shift, window, scale, splits, &rope, stream)
-  if (d <= 32) CALL(32);
-  else if (d <= 64) CALL(64);
-  else if (d <= 96) CALL(96);
-  else if (d <= 128) CALL(128);
-  else if (d <= 160) CALL(160);
-  else if (d <= 192) CALL(192);
-  else if (d <= 224) CALL(224);
-  else CALL(256);
-#undef CALL
+  const DecodeUnit unit = decode_units[unit_index(d)];
+  RLIS_REQUIRE(unit != nullptr, "attn_decode_mfma: the unit for head size %d is not loaded", d);
+  const int rc = unit_result(
+      "attn_decode_mfma",
+      unit(q, q_stride, out, out_stride, part_ml, part_acc, k_pages, v_pages, block_tables,
+           max_pages, ctx_lens, S, nh, nkv, d, page_shift, window, scale, splits, &rope, stream),
+      d);
   if (rc) return rc;
   if (splits > 1 && S > 0)
     return rlis_launch_attn_reduce_bf16(out, out_stride, part_ml, part_acc, S, nh, d, splits, stream);

@@ -49,6 +49,17 @@ union Frag8 {
 #define RLIS_PREFILL_BUFS (RLIS_HEAD_DIM <= 64 ? 2 : 1)
 #endif
 
+// A unit is a library of its own, loaded when a model needs its head size: it reports through
+// return codes (kUnit...), which the dispatcher turns into messages.
+constexpr int kUnitTooManyTiles = 1;
+constexpr int kUnitBadRotation = 2;
+constexpr int kUnitLaunchFailed = 1000;       // + the hipError_t
+#define RLIS_UNIT_LAUNCH_CHECK()                                 \
+  do {                                                           \
+    hipError_t e_ = hipGetLastError();                           \
+    if (e_ != hipSuccess) return kUnitLaunchFailed + (int)e_;    \
+  } while (0)
+
 #define RLIS_CAT2(a, b) a##b
 #define RLIS_CAT(a, b) RLIS_CAT2(a, b)
 #define KERNEL_NAME RLIS_CAT(rlis_attn_prefill_mfma_kernel_d, RLIS_HEAD_DIM)
@@ -417,10 +428,7 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
     float* part_ml, float* part_acc, hipStream_t stream) {
   if (num_tiles == 0) return 0;
   const long long blocks = (long long)num_tiles * nh * splits;
-  if (blocks >= (1ll << 31)) {
-    rlis_set_error("attn_prefill_mfma: too many tiles");
-    return 1;
-  }
+  if (blocks >= (1ll << 31)) return kUnitTooManyTiles;
   // 256 compute units: a round is the tiles whose blocks fill them once.
   const int tiles_per_round = (splits == 1 && nh <= 256 && 256 % nh == 0) ? 256 / nh : 0;
   if (tile_queries == 2 * BM)
@@ -433,7 +441,7 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,
         (const bf16_t*)v_pages, block_tables, max_pages, cu_seqlens, start_pos, tile_map, nh, nkv,
         d, page_shift, scale, window, num_tiles, tiles_per_round, splits, row0, part_ml, part_acc);
-  RLIS_LAUNCH_CHECK("attn_prefill_mfma");
+  RLIS_UNIT_LAUNCH_CHECK();
   return 0;
 }
 
@@ -715,9 +723,9 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
     int max_pages, const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift, int window,
     float scale, int splits, const DecodeRope* rope, hipStream_t stream) {
   if (S == 0) return 0;
-  RLIS_REQUIRE(!(rope->positions && rope->cos) || (D % 64 == 0 && rope->rot == D && d == D),
-               "attn_decode_mfma: rotation inside the kernel needs head_dim = rotated width = "
-               "64, 128 or 256 (got %d, %d)", d, rope->rot);
+  // rotation inside the kernel needs head_dim = rotated width = 64, 128 or 256
+  if (rope->positions && rope->cos && !(D % 64 == 0 && rope->rot == D && d == D))
+    return kUnitBadRotation;
   const int g = nh / nkv;
   dim3 grid(nkv, S, splits);
   const size_t smem = (size_t)kDecodeWaves * g * (2 + d) * sizeof(float);
@@ -725,6 +733,6 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, part_ml, part_acc,
       (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, max_pages, ctx_lens, nh, nkv, d,
       page_shift, scale, window, splits, *rope);
-  RLIS_LAUNCH_CHECK("attn_decode_mfma");
+  RLIS_UNIT_LAUNCH_CHECK();
   return 0;
 }

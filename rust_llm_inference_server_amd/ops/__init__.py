@@ -467,6 +467,7 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
         ml_ptr = None if part_ml is None else part_ml.data_ptr()
         acc_ptr = None if part_acc is None else part_acc.data_ptr()
         if matrix:
+            lib.ensure_attention_unit(d)
             cos_p = sin_p = pos_p = slots_p = None
             rot = 0
             if rope is not None:
@@ -514,6 +515,7 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                                                      and step.max_context >= 4096):
                 tile_map, num_tiles, tile_queries = wide, wide.numel() // 2, 128
         if num_tiles:
+            lib.ensure_attention_unit(d)
             # Few tiles with long walks over cached keys (a portion of a long prompt): the keys
             # of every tile are cut into runs, one workgroup each, and merged afterwards.
             splits = getattr(step, "prefill_splits", None)

@@ -63,10 +63,39 @@ def load() -> ctypes.CDLL:
         fn.argtypes = argtypes
     lib.rlis_gemm_bf16_stream_slices.restype = c_int
     lib.rlis_gemm_bf16_stream_slices.argtypes = [I]
+    lib.rlis_attn_register_unit.restype = c_int
+    lib.rlis_attn_register_unit.argtypes = [I, P, P]
     lib.rlis_norm_linear_max_k.restype = c_int
     lib.rlis_norm_linear_max_k.argtypes = []
     _LIB = lib
     return lib
+
+
+_UNITS: dict = {}      # padded head size -> the loaded unit library
+
+
+def ensure_attention_unit(head_dim: int) -> None:
+    """Build (when absent), load and register the matrix-core attention unit that serves
+    ``head_dim``: a model needs one, and only that one is compiled for it."""
+    padded = -(-head_dim // 32) * 32
+    if padded in _UNITS:
+        return
+    main = load()
+    from ..csrc import build
+    try:
+        kind = build.attention_unit(head_dim)
+    except ValueError as e:
+        raise KernelError(str(e)) from None
+    unit = ctypes.CDLL(build.ensure(kind))
+    fns = []
+    for name in (f"rlis_attn_prefill_mfma_d{padded}", f"rlis_attn_decode_mfma_d{padded}"):
+        fn = getattr(unit, name, None)
+        if fn is None:
+            raise RuntimeError(f"{unit._name} does not export {name}; rebuild the kernels")
+        fns.append(ctypes.cast(fn, c_void_p))
+    if main.rlis_attn_register_unit(padded, *fns) != 0:
+        raise KernelError(main.rlis_last_error().decode("utf-8", "replace"))
+    _UNITS[padded] = unit
 
 
 def loaded_path() -> Optional[str]:
