@@ -14,7 +14,6 @@ import argparse
 import json
 import os
 import sys
-import tempfile
 from typing import List, Optional
 
 _DTYPES = {"f32": "float32", "fp32": "float32", "float32": "float32",

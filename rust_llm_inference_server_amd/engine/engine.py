@@ -14,7 +14,7 @@ its sampling being keyed by position, continues with the same tokens (engine.rs 
 from __future__ import annotations
 
 import time
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, Iterable, List, Optional, Sequence, Tuple, Union
 
 import torch

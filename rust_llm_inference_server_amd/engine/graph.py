@@ -15,12 +15,11 @@ replay with eager work in between."""
 from __future__ import annotations
 
 import ctypes
-from typing import Dict, List, Optional, Sequence
+from typing import Optional, Sequence
 
 import numpy as np
 import torch
 
-from .. import ops
 from .batch import GroupStep, StepContext
 
 

@@ -9,18 +9,17 @@ program, the perplexity tool and the benchmark all call it.  Its contract is the
 crates/model/src/paged.rs:154-161, 255-296)."""
 from __future__ import annotations
 
-import os
 from typing import Dict, List, Optional, Sequence, Union
 
 import torch
 
 from ..cache.manager import CacheManager, GroupSpec
 from ..cache.pools import CachePools
-from ..models.spec import Model, ModelSpec
+from ..models.spec import Model
 from ..registry import architecture_of, read_config_dict
 from ..weights.loader import load_weights
 from ..weights.random_init import random_weights
-from .batch import StepContext, StepEntry, build_step
+from .batch import StepEntry, build_step
 
 DTYPES = {"float32": torch.float32, "fp32": torch.float32, "f32": torch.float32,
           "bfloat16": torch.bfloat16, "bf16": torch.bfloat16}

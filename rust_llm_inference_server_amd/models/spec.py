@@ -9,11 +9,11 @@ step: embedding, the run order, final norm on the wanted rows, head."""
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional, Sequence, Tuple
+from typing import Any, Dict, List, Optional, Tuple
 
 import torch
 
-from ..parts.base import (Block, BuildContext, CacheBinding, CacheRequest, PartSpec,
+from ..parts.base import (Block, BuildContext, CacheRequest, PartSpec,
                           ResidualStream, TensorSpec, create, normed, tensor_specs)
 
 

@@ -5,7 +5,7 @@ from __future__ import annotations
 
 from typing import Any, Dict, List
 
-from .base import (Block, BuildContext, CacheBinding, PartSpec, ResidualStream, TensorSpec,
+from .base import (Block, BuildContext, CacheBinding, ResidualStream, TensorSpec,
                    create, join, normed, register, tensor_specs)
 
 

@@ -9,12 +9,12 @@ dtype only (crates/model/src/llama.rs:33-64); so does this loader, tensor by ten
 from __future__ import annotations
 
 import fnmatch
-from typing import Dict, Iterable, List, Optional, Sequence
+from typing import Dict, Iterable, List, Sequence
 
 import torch
 
 from ..parts.base import TensorSpec
-from .safetensors_io import SafetensorsError, open_folder
+from .safetensors_io import open_folder
 
 # Buffers some exporters write beside the weights; they carry nothing the model reads.
 IGNORED_PATTERNS = ("*.rotary_emb.inv_freq", "*.attn.bias", "*.attn.masked_bias")

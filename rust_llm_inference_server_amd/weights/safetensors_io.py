@@ -9,7 +9,7 @@ import json
 import mmap
 import os
 import struct
-from typing import Dict, Iterable, List, Optional, Tuple
+from typing import Dict, List, Optional, Tuple
 
 import torch
 

@@ -8,8 +8,6 @@ their code.
 """
 from __future__ import annotations
 
-import math
-from typing import Optional
 
 import torch
 

@@ -5,7 +5,6 @@ import pytest
 import torch
 
 import plain_llama as plain
-from conftest import TINY
 from rust_llm_inference_server_amd.config import EngineConfig
 from rust_llm_inference_server_amd.sampling import SamplingParams
 

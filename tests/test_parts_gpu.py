@@ -2,9 +2,7 @@
 a layer with a window beside layers without, a layer named twice in the run order, a layer
 that reads another layer's cache, and a toy mixer with state of its own that the test defines
 and registers without touching the package.  Everything runs on the GPU against plain code."""
-import json
 import math
-import os
 
 import pytest
 import torch

@@ -4,7 +4,6 @@ under every way of cutting the work: whole prompts; most of a prompt in one step
 requests mixed, portions of some beside single tokens of others, with so few pages that they
 are used again.  In float32 (the true 32-bit path) and in bfloat16, for three tiny
 configurations that differ in every size and option."""
-import os
 
 import pytest
 import torch
