@@ -331,7 +331,7 @@ __global__ void attn_reduce_kernel(TX* __restrict__ out, long long out_stride,
   const int row = token_rows ? token_rows[seq] : seq;
   const long long base = ((long long)seq * nh + h) * splits;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, nwaves = blockDim.x / kWave;
-  const int j0 = threadIdx.x < d ? threadIdx.x : 0;
+  const int j0 = (int)threadIdx.x < d ? (int)threadIdx.x : 0;
   const float* acc0 = part_acc + base * d + j0;
   float ahead[kReduceAhead];
 #pragma unroll
