@@ -23,8 +23,8 @@ SKINNY_MAX_ROWS = 64
 STREAM_MAX_ROWS = 16
 # Single tokens in a batch that also holds portions of prompts take the decode attention kernel.
 SPLIT_MIXED_ATTENTION = True
-# The prefill attention takes tiles of 128 queries when that still makes this many workgroups
-# (half as many when the longest context has 4096 positions or more).
+# The prefill attention takes tiles of 128 queries when that makes this many workgroups, or when
+# contexts are long (4096 positions, or 2048 cached ones); 1 << 30: never.
 PREFILL_WIDE_MIN_GROUPS = 768
 # The prefill attention cuts the keys of its tiles into runs (one workgroup each, merged
 # afterwards) when its tiles leave compute units without work: as many runs as the units hold
@@ -504,15 +504,16 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
             decode(singles, step.max_single_context, True, None)
             tile_map, num_tiles, row0 = step.multi_tile_map, step.num_multi_tiles, singles
         # Tiles of 128 queries (two query blocks per wave, half the LDS traffic per flop) where
-        # they still fill the chip: plenty of them, or fewer with long walks over cached keys.
-        # The step brings them for the same set of sequences.
+        # they are plenty, or where the walks over keys are long (few such tiles still fill the
+        # chip then, their keys cut into runs).  The step brings them for the same sequences.
         tile_queries = 64
         wide = getattr(step, "wide_multi_tile_map" if tile_map is not step.tile_map
                        else "wide_tile_map", None)
         if wide is not None and d <= 128:
             groups = wide.numel() // 2 * nh
-            if groups >= PREFILL_WIDE_MIN_GROUPS or (2 * groups >= PREFILL_WIDE_MIN_GROUPS
-                                                     and step.max_context >= 4096):
+            cached = step.max_context - getattr(step, "max_new", 0)
+            if groups >= PREFILL_WIDE_MIN_GROUPS or (PREFILL_WIDE_MIN_GROUPS < (1 << 30) and (
+                    step.max_context >= 4096 or cached >= 2048)):
                 tile_map, num_tiles, tile_queries = wide, wide.numel() // 2, 128
         if num_tiles:
             lib.ensure_attention_unit(d)
