@@ -39,7 +39,7 @@ def prompts_for(vocab, lengths, seed=0):
 
 
 def test_greedy_generation_matches_the_plain_implementation(backend, tiny_folders):
-    """BASELINE workload 0/1 in small: prompts 5/17/33 (and 1/9/40), 8 greedy tokens each."""
+    """Prompts of 5, 17 and 33 tokens (and 1, 9 and 40), 8 greedy tokens each."""
     for name, lengths in (("a", [5, 17, 33]), ("b", [1, 9, 40])):
         folder = tiny_folders[name]
         w, c = plain.read_weights(folder), plain.read_config(folder)
