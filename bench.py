@@ -69,7 +69,8 @@ def main() -> int:
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
-    longest = max(args.context, args.prefill_tokens, 4096)
+    # room for the timed steps themselves when they are more than the context holds
+    longest = max(args.context, args.prefill_tokens, 4096, args.steps + args.warmup + 128)
     if args.serve:
         longest = max(longest, args.max_prompt + args.new_tokens)
     cfg["max_position_embeddings"] = min(cfg["max_position_embeddings"], longest + 64)
@@ -99,7 +100,8 @@ def main() -> int:
         budget = max(args.max_batched_tokens, batch)
         prefill_steps = -(-batch * context // budget) + 1
         new_tokens = steps + warmup + prefill_steps + 1
-        prompt_len = max(1, context - new_tokens)
+        context = max(context, new_tokens + 16)           # more steps than the context holds
+        prompt_len = context - new_tokens
         pages = batch * (-(-context // page) + 1) + 8
         engine = Engine(model, EngineConfig(max_num_seqs=max(batch, 1), max_batched_tokens=budget,
                                             num_pages=pages, block_size=page,
