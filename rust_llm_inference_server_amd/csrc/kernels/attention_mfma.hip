@@ -45,9 +45,6 @@ union Frag8 {
   bf16_t e[8];
 };
 
-#ifndef RLIS_PREFILL_BUFS
-#define RLIS_PREFILL_BUFS (RLIS_HEAD_DIM <= 64 ? 2 : 1)
-#endif
 
 // A unit is a library of its own, loaded when a model needs its head size: it reports through
 // return codes (kUnit...), which the dispatcher turns into messages.
@@ -77,7 +74,9 @@ constexpr int KS = D + 8;     // K tile row stride (bf16 elements)
 constexpr int BM = 64;       // queries per workgroup and query block
 // Two LDS tiles taking turns (one barrier per tile instead of two) where that does not cost a
 // resident workgroup.
-constexpr int kTileBufs = RLIS_PREFILL_BUFS;
+__host__ __device__ constexpr int tile_bufs(int QB) {
+  return (D <= 64 || (QB == 2 && D <= 128)) ? 2 : 1;
+}
 
 }  // namespace
 
@@ -93,6 +92,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
     int row0, float* __restrict__ part_ml, float* __restrict__ part_acc) {
   constexpr int BN = tile_keys(QB);
   constexpr int VS = BN + 8;    // V tile row stride
+  constexpr int kTileBufs = tile_bufs(QB);
   __shared__ __attribute__((aligned(16))) bf16_t Ks_all[kTileBufs * BN * KS];
   __shared__ __attribute__((aligned(16))) bf16_t Vs_all[kTileBufs * D * VS];
 
