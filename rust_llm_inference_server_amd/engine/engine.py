@@ -33,10 +33,11 @@ class Completion:
     """What a finished request returns (engine.rs:139-158 ``Finish``)."""
     request_id: int
     token_ids: List[int]
-    finish_reason: str                 # "stop" or "length"
+    finish_reason: str                 # "stop", "length" or "error"
     prompt_tokens: int
     ttft: float                        # seconds from arrival to the first token
     decode_time: float                 # seconds from the first token to the last
+    error: Optional[str] = None        # with "error": what the failed step said
 
     @property
     def completion_tokens(self) -> int:
@@ -153,7 +154,9 @@ class Engine:
     # --------------------------------------------------------------------- step
     def step(self) -> List[Tuple[int, Optional[int], bool]]:
         """One scheduled batch.  Returns ``(request id, token or None, finished)`` for every
-        request that produced a token (``None`` with ``finished``: it stopped at an EOS)."""
+        request that produced a token (``None`` with ``finished``: it stopped at an EOS).
+        If the model step raises, the requests of that batch finish with reason ``error``
+        and the exception goes on to the caller; requests outside the batch are untouched."""
         sched = self.scheduler.schedule()
         self.stats_.preemptions = self.scheduler.num_preemptions
         if not sched.seqs:
@@ -163,7 +166,6 @@ class Engine:
                     self.cancel(seq_id)
                 raise RuntimeError("scheduler made no progress")
             return []
-        self.runner.apply_copies(sched.copies)
         entries, final = [], []
         for seq_id, start, end in sched.seqs:
             seq = self._seqs[seq_id]
@@ -171,7 +173,15 @@ class Engine:
             entries.append(StepEntry(seq_id, seq.tokens[start:end],
                                      [end - start - 1] if last else []))
             final.append(last)
-        logits = self.runner.step(entries)
+        try:
+            self.runner.apply_copies(sched.copies)
+            logits = self.runner.step(entries)
+        except Exception as exc:
+            # engine.rs:523-528: a failed step fails its own requests and no others; their
+            # pages are free again and the engine goes on with the rest.
+            for seq_id, _, _ in sched.seqs:
+                self._finish(self._seqs[seq_id], "error", error=f"{type(exc).__name__}: {exc}")
+            raise
         self.stats_.steps += 1
         # Rows that yield a token, split between the device kernel and the host sampler.
         device_rows, device_modes, host_rows = [], [], []
@@ -230,14 +240,14 @@ class Engine:
         self.scheduler.append_token(seq.id)
         return (seq.id, token, False)
 
-    def _finish(self, seq: _Sequence, reason: str) -> None:
+    def _finish(self, seq: _Sequence, reason: str, error: Optional[str] = None) -> None:
         seq.finish_reason = reason
         self.scheduler.remove(seq.id)
         del self._seqs[seq.id]
         self._finished[seq.id] = Completion(
             request_id=seq.id, token_ids=seq.tokens[seq.prompt_len:], finish_reason=reason,
             prompt_tokens=seq.prompt_len, ttft=(seq.first_token_at or seq.arrived) - seq.arrived,
-            decode_time=(seq.last_token_at or 0.0) - (seq.first_token_at or 0.0))
+            decode_time=(seq.last_token_at or 0.0) - (seq.first_token_at or 0.0), error=error)
 
     # ----------------------------------------------------------------- generate
     def generate(self, prompts: Sequence[Sequence[int]],

@@ -140,3 +140,32 @@ def test_cancel_returns_the_pages(backend, tiny_folders):
         engine.step()
     assert engine.pop_finished(b).finish_reason == "length" and engine.pop_finished(a) is None
     assert engine.runner.cache.num_free_pages() == 16
+
+
+def test_a_failed_step_fails_only_its_own_requests(backend, tiny_folders):
+    """crates/engine/src/engine.rs:523-528.  The first step holds a portion of the long request
+    alone (it uses the whole budget); the model step is made to raise once."""
+    model = load(tiny_folders["a"], backend, max_positions=128)
+    engine = engine_for(model, num_pages=16, max_batched_tokens=16)
+    a = engine.add_request(prompts_for(256, [20])[0], SamplingParams.greedy(4))
+    b = engine.add_request(prompts_for(256, [5], seed=1)[0], SamplingParams.greedy(4))
+    real, calls = engine.runner.step, []
+
+    def failing(entries):
+        calls.append([e.seq_id for e in entries])
+        if len(calls) == 1:
+            raise RuntimeError("the device said no")
+        return real(entries)
+
+    engine.runner.step = failing
+    with pytest.raises(RuntimeError, match="the device said no"):
+        engine.step()
+    assert calls == [[a]]
+    failed = engine.pop_finished(a)
+    assert failed.finish_reason == "error" and "the device said no" in failed.error
+    assert engine.runner.cache.num_free_pages() == 16
+    while engine.has_work():
+        engine.step()
+    done = engine.pop_finished(b)
+    assert done.finish_reason == "length" and len(done.token_ids) == 4 and done.error is None
+    assert engine.runner.cache.num_free_pages() == 16
