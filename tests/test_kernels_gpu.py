@@ -435,14 +435,18 @@ LAYOUTS = [(4, 1, 16, 16), (6, 2, 32, 8), (5, 5, 48, 16), (32, 8, 64, 16), (24, 
            (8, 8, 64, 32), (12, 2, 128, 64), (3, 1, 80, 8), (16, 2, 256, 16), (9, 3, 112, 16)]
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
+def kinds_and_dtypes(*kinds):
+    """Every kernel family with the dtypes it takes: the matrix-core prefill kernel is
+    bfloat16 only."""
+    return [pytest.param(k, dt, id=f"{k}-{str(dt).split('.')[-1]}") for k in kinds for dt in DTYPES
+            if k != "prefill" or dt == torch.bfloat16]
+
+
 @pytest.mark.parametrize("nh,nkv,d,ps", LAYOUTS)
-@pytest.mark.parametrize("kind", ["generic", "prefill"])
+@pytest.mark.parametrize("kind,dtype", kinds_and_dtypes("generic", "prefill"))
 def test_attention_mixed_batch(ops, dtype, nh, nkv, d, ps, kind):
     """Portions of prompts (with and without cached positions, across page and tile edges)
     beside single tokens, in one batch, through scattered block tables."""
-    if kind == "prefill" and dtype != torch.bfloat16:
-        pytest.skip("the matrix-core prefill kernel is bfloat16 only")
     cached = [0, 5, 40, 0, 63, 130, 17]
     new = [33, 1, 70, 2, 1, 129, 64]
     scale = 1.0 / math.sqrt(d)
@@ -532,12 +536,9 @@ def test_attention_prefill_with_keys_cut_into_runs(ops, nh, nkv, d, ps, window, 
         ops.PREFILL_WIDE_MIN_GROUPS = old
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("kind", ["generic", "prefill", "decode"])
+@pytest.mark.parametrize("kind,dtype", kinds_and_dtypes("generic", "prefill", "decode"))
 @pytest.mark.parametrize("window", [1, 7, 64, 100])
 def test_attention_window(ops, dtype, kind, window, decode_kind):
-    if kind == "prefill" and dtype != torch.bfloat16:
-        pytest.skip("the matrix-core prefill kernel is bfloat16 only")
     nh, nkv, d, ps = 6, 2, 32, 8
     cached, new = ([0, 30, 200, 99], [50, 90, 3, 1]) if kind != "decode" else ([0, 30, 200, 99, 6], [1] * 5)
     scale = 0.2
@@ -626,13 +627,10 @@ def test_attention_decode_long_split(ops, dtype, decode_kind):
         torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("kind", ["generic", "prefill", "decode"])
+@pytest.mark.parametrize("kind,dtype", kinds_and_dtypes("generic", "prefill", "decode"))
 def test_attention_finds_a_far_key(ops, dtype, kind, decode_kind):
     """One key among hundreds is made to stand out (its key vector equals the scaled query
     direction); the output must be that key's value, wherever its page lies."""
-    if kind == "prefill" and dtype != torch.bfloat16:
-        pytest.skip("the matrix-core prefill kernel is bfloat16 only")
     nh, nkv, d, ps = 4, 2, 64, 16
     total = 777
     cached, new = ([total - 1], [1]) if kind == "decode" else ([total - 3], [3])

@@ -198,8 +198,6 @@ def test_long_prompt_whole_and_in_portions(tmp_path, wide):
 def test_trace_run_program(case, dtype, tmp_path):
     """The program itself, as a child process fed step by step, on the mixed trace."""
     name, cfg, per_dtype = case
-    if name == "c":
-        pytest.skip("one configuration less through the child process keeps the suite short")
     folder, reqs, ref = per_dtype[dtype]
     steps, max_tokens = traces.trace_mixed(reqs, seed=1)
     outputs = traces.replay_program(folder, dtype, steps, max_tokens, str(tmp_path / "out"),
