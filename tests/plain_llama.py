@@ -198,6 +198,30 @@ def greedy_generate(w: Dict[str, torch.Tensor], cfg: dict, prompt: Sequence[int]
 
 
 # ----------------------------------------------------------------------- sampling
+def perplexity(w: Dict[str, torch.Tensor], cfg: dict, tokens: Sequence[int], bos: int, ctx: int,
+               max_windows: int = 0) -> dict:
+    """crates/engine/src/perplexity.rs:26-80: windows of ``ctx`` tokens, the first token of
+    each replaced by BOS, rows ctx/2 .. ctx-2 scored against the tokens that follow them;
+    ppl = exp(mean NLL), one standard error = ppl * sqrt(var / n)."""
+    windows = len(tokens) // ctx
+    if max_windows > 0:
+        windows = min(windows, max_windows)
+    first = ctx // 2
+    nll: List[float] = []
+    for wi in range(windows):
+        chunk = [int(t) for t in tokens[wi * ctx:(wi + 1) * ctx]]
+        chunk[0] = bos
+        logits = forward(w, cfg, chunk).double()
+        for row in range(first, ctx - 1):
+            r = logits[row]
+            nll.append(float(torch.logsumexp(r, 0) - r[chunk[row + 1]]))
+    n = len(nll)
+    mean = sum(nll) / n
+    var = max(sum(x * x for x in nll) / n - mean * mean, 0.0)
+    return {"ppl": math.exp(mean), "ppl_stderr": math.exp(mean) * math.sqrt(var / n),
+            "mean_nll": mean, "tokens_scored": n, "windows": windows}
+
+
 def lowbias32(x: int) -> int:
     """crates/model/src/sampling.rs:11-18."""
     x &= 0xFFFFFFFF

@@ -169,3 +169,28 @@ def test_a_failed_step_fails_only_its_own_requests(backend, tiny_folders):
     done = engine.pop_finished(b)
     assert done.finish_reason == "length" and len(done.token_ids) == 4 and done.error is None
     assert engine.runner.cache.num_free_pages() == 16
+
+
+def test_perplexity_matches_the_plain_implementation(backend, tiny_folders):
+    """crates/engine/src/perplexity.rs:26-80, windows of 16 and of 13 tokens over 70."""
+    from rust_llm_inference_server_amd.engine import ModelRunner
+    from rust_llm_inference_server_amd.engine.perplexity import perplexity
+    folder = tiny_folders["b"]
+    w, c = plain.read_weights(folder), plain.read_config(folder)
+    tokens = prompts_for(c["vocab_size"], [70], seed=9)[0]
+    runner = ModelRunner(load(folder, backend), num_pages=4, page_size=8, max_num_seqs=2)
+    for ctx, max_windows in ((16, 0), (13, 3)):
+        seen = []
+        got = perplexity(runner, tokens, bos=1, ctx=ctx, max_windows=max_windows,
+                         progress=lambda done, total, ppl: seen.append((done, total)))
+        want = plain.perplexity(w, c, tokens, bos=1, ctx=ctx, max_windows=max_windows)
+        assert (got.windows, got.tokens_scored) == (want["windows"], want["tokens_scored"])
+        assert seen == [(i + 1, got.windows) for i in range(got.windows)]
+        assert abs(got.mean_nll - want["mean_nll"]) < 1e-5
+        assert abs(got.ppl - want["ppl"]) < 1e-4 * want["ppl"]
+        assert abs(got.ppl_stderr - want["ppl_stderr"]) < 1e-3 * want["ppl"]
+    assert runner.cache.num_free_pages() == 4
+    with pytest.raises(ValueError, match="ctx must be at least 4"):
+        perplexity(runner, tokens, bos=1, ctx=3)
+    with pytest.raises(ValueError, match="shorter than one window"):
+        perplexity(runner, tokens[:10], bos=1, ctx=16)

@@ -235,3 +235,24 @@ def test_gumbel_max_frequencies_follow_softmax():
     for i in range(n):
         counts[plain.sample_row(l, plain.row_key(42, i), 1 / 0.7)] += 1
     assert (counts / n - torch.softmax(l / 0.7, 0)).abs().max().item() < 0.03
+
+
+def test_perplexity_of_uniform_logits_is_the_vocabulary_size():
+    """With an output head of zeros every logit is 0, every token costs ln(V): the perplexity
+    is V and its standard error 0, whatever the tokens; and the count of scored tokens is
+    windows * (ctx - 1 - ctx // 2)  (crates/engine/src/perplexity.rs:44-59)."""
+    cfg = dict(TINY_B)
+    g = torch.Generator().manual_seed(0)
+    w = {}
+    from rust_llm_inference_server_amd.registry import architecture_of
+    arch = architecture_of(cfg)
+    for spec in arch.build_spec(arch.parse_config(cfg)).tensor_specs():
+        w[spec.name] = torch.randn(spec.shape, generator=g) * 0.05
+    w["lm_head.weight"].zero_()
+    c = dict(cfg)
+    tokens = torch.randint(0, cfg["vocab_size"], (70,), generator=g).tolist()
+    out = plain.perplexity(w, c, tokens, bos=1, ctx=16)
+    assert out["windows"] == 4 and out["tokens_scored"] == 4 * 7
+    assert abs(out["ppl"] - cfg["vocab_size"]) < 1e-6 * cfg["vocab_size"]
+    assert out["ppl_stderr"] < 1e-4
+    assert plain.perplexity(w, c, tokens, bos=1, ctx=16, max_windows=2)["windows"] == 2
