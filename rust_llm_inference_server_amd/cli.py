@@ -164,7 +164,7 @@ def run_perplexity(args) -> int:
     return 0
 
 
-def main(argv: Optional[List[str]] = None) -> int:
+def build_parser() -> argparse.ArgumentParser:
     ap = argparse.ArgumentParser(prog="rlis", description="Llama inference engine for MI355X")
     sub = ap.add_subparsers(dest="command", required=True)
     g = sub.add_parser("generate", help="generate a completion for one prompt")
@@ -186,7 +186,11 @@ def main(argv: Optional[List[str]] = None) -> int:
     p.add_argument("--ctx", type=int, default=512, help="window length; the second half is scored")
     p.add_argument("--max-windows", type=int, default=0, help="score only the first N windows (0 = all)")
     p.add_argument("--block-size", "--page-size", dest="block_size", type=int, default=16)
-    args = ap.parse_args(argv)
+    return ap
+
+
+def main(argv: Optional[List[str]] = None) -> int:
+    args = build_parser().parse_args(argv)
     return run_generate(args) if args.command == "generate" else run_perplexity(args)
 
 

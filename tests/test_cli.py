@@ -1,0 +1,88 @@
+"""The command line: option names and defaults are the reference's
+(crates/server/src/main.rs:31-127), and both subcommands run a tiny random model on the GPU."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+import plain_llama as plain
+from rust_llm_inference_server_amd import cli
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_option_names_and_defaults_are_the_references():
+    ap = cli.build_parser()
+    g = ap.parse_args(["generate", "--model", "m", "--prompt-ids", "1 2"])
+    # main.rs:46-61 (model), 63-86 (generate), 106-127 (engine)
+    assert (g.max_seq_len, g.max_tokens, g.temperature, g.top_p, g.top_k, g.repetition_penalty,
+            g.seed) == (2048, 128, 0.0, 1.0, 0, 1.0, None)
+    assert (g.kv_cache_gb, g.block_size, g.max_num_seqs, g.max_batched_tokens, g.scheduler,
+            g.attention, g.no_prefix_caching) == (1.0, 16, 64, 2048, "continuous", "v2", False)
+    p = ap.parse_args(["perplexity", "--model", "m", "--ids-file", "f"])
+    assert (p.ctx, p.max_windows) == (512, 0)             # main.rs:31-43
+    assert ap.parse_args(["generate", "--page-size", "8", "--scheduler", "static"]).block_size == 8
+
+
+@pytest.mark.parametrize("argv,message", [
+    (["generate", "--dtype", "f16"], "f16"),
+    (["generate", "--scheduler", "fair"], "invalid choice"),
+    (["serve"], "invalid choice"),
+])
+def test_refused_options(argv, message, capsys):
+    with pytest.raises(SystemExit):
+        cli.build_parser().parse_args(argv)
+    assert message in capsys.readouterr().err
+
+
+def test_refused_runs():
+    with pytest.raises(SystemExit, match="GPU only"):
+        cli.main(["generate", "--device", "cpu", "--model", "m", "--prompt-ids", "1"])
+    with pytest.raises(SystemExit, match="--random-weights needs --config"):
+        cli.main(["generate", "--random-weights", "--prompt-ids", "1"])
+    with pytest.raises(SystemExit, match="--model is required"):
+        cli.main(["generate", "--prompt-ids", "1"])
+
+
+@pytest.mark.gpu
+def test_generate_prints_the_greedy_tokens(tiny_folders, capsys):
+    folder = tiny_folders["b"]
+    w, c = plain.read_weights(folder), plain.read_config(folder)
+    prompt = [5, 17, 3, 99, 250, 7, 7, 12, 300]
+    rc = cli.main(["generate", "--model", folder, "--dtype", "f32", "--max-seq-len", "128",
+                   "--num-pages", "32", "--block-size", "8", "--max-tokens", "6",
+                   "--prompt-ids", ",".join(map(str, prompt))])
+    out = capsys.readouterr()
+    assert rc == 0
+    assert [int(t) for t in out.out.split()] == plain.greedy_generate(w, c, prompt, 6)
+    assert "prompt 9 tok | output 6 tok (length) | ttft" in out.err and "tok/s" in out.err
+
+
+@pytest.mark.gpu
+def test_the_program_generates_and_scores(tiny_folders, tmp_path):
+    """``bin/rlis`` as a child process: generation with a seeded temperature twice (the same
+    tokens), and the perplexity report as JSON on standard output."""
+    folder = tiny_folders["a"]
+    w, c = plain.read_weights(folder), plain.read_config(folder)
+    base = [sys.executable, os.path.join(ROOT, "bin", "rlis")]
+    common = ["--model", folder, "--dtype", "f32", "--max-seq-len", "128"]
+    runs = [subprocess.run(base + ["generate"] + common + [
+        "--num-pages", "16", "--prompt-ids", "3 1 4 1 5", "--max-tokens", "5",
+        "--temperature", "0.8", "--seed", "11"], capture_output=True, text=True, timeout=300)
+        for _ in range(2)]
+    assert all(r.returncode == 0 for r in runs), runs[0].stderr
+    assert runs[0].stdout.split() == runs[1].stdout.split() and len(runs[0].stdout.split()) == 5
+    tokens = [(7 * i + 3) % c["vocab_size"] for i in range(50)]
+    ids = tmp_path / "ids.txt"
+    ids.write_text(" ".join(map(str, tokens)))
+    r = subprocess.run(base + ["perplexity"] + common + ["--ids-file", str(ids), "--ctx", "16",
+                                                          "--bos", "1"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    report = json.loads(r.stdout.strip().splitlines()[-1])
+    want = plain.perplexity(w, c, tokens, bos=1, ctx=16)
+    assert report["windows"] == 3 and report["tokens_scored"] == want["tokens_scored"]
+    assert abs(report["ppl"] - want["ppl"]) < 1e-4 * want["ppl"]
+    assert "PPL = " in r.stderr
