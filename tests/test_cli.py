@@ -86,3 +86,37 @@ def test_the_program_generates_and_scores(tiny_folders, tmp_path):
     assert report["windows"] == 3 and report["tokens_scored"] == want["tokens_scored"]
     assert abs(report["ppl"] - want["ppl"]) < 1e-4 * want["ppl"]
     assert "PPL = " in r.stderr
+
+
+def test_bench_measures_one_gpu_only():
+    """For more than one GPU bench.py prints one line that says so and exits with 2."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2
+    assert len(r.stdout.strip().splitlines()) == 1 and "one GPU" in r.stdout
+
+
+@pytest.mark.gpu
+def test_bench_line_has_the_agreed_fields():
+    """A short run at a reduced number of layers: one JSON line with the fields of the
+    contract, a flat configuration of at most 20 keys that names both layer counts."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--layers", "2",
+                        "--steps", "4", "--warmup", "2", "--context", "256"],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if l.startswith("{")]
+    assert len(lines) == 1
+    rec = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
+                "higher_is_better", "scaling", "vs_baseline", "dtype", "data", "config",
+                "prefill", "roofline", "points"):
+        assert key in rec, key
+    assert rec["n_gpus"] == 1 and rec["steps"] == 4 and rec["warmup"] == 2
+    cfg = rec["config"]
+    assert len(cfg) <= 20 and all(not isinstance(v, (dict, list)) for v in cfg.values())
+    assert cfg["layers"] == 2 and cfg["layers_full"] == 16
+    assert set(rec["prefill"]) == {"value", "tokens", "ms", "frac"} and rec["prefill"]["tokens"] == 2048
+    assert rec["roofline"]["bound"] == "hbm" and rec["roofline"]["peak"] == 8000.0
+    assert abs(rec["roofline"]["frac"] - rec["roofline"]["achieved"] / 8000.0) < 1e-3
+    assert set(rec["points"]) == {"decode_b1", "decode_b64"}
+    assert abs(rec["value"] - 8 / rec["ms_per_step"] * 1e3) < 0.01 * rec["value"]
