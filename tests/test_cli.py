@@ -120,3 +120,10 @@ def test_bench_line_has_the_agreed_fields():
     assert abs(rec["roofline"]["frac"] - rec["roofline"]["achieved"] / 8000.0) < 1e-3
     assert set(rec["points"]) == {"decode_b1", "decode_b64"}
     assert abs(rec["value"] - 8 / rec["ms_per_step"] * 1e3) < 0.01 * rec["value"]
+
+
+@pytest.mark.gpu
+def test_smoke_entry_point(capsys):
+    import __graft_entry__ as entry
+    entry.smoke()
+    assert "smoke ok" in capsys.readouterr().out
