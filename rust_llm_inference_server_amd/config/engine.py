@@ -27,8 +27,10 @@ class EngineConfig:
             raise ValueError("max_num_seqs must be positive")
         if self.block_size <= 0:
             raise ValueError("block_size must be positive")
-        if self.max_batched_tokens < self.max_num_seqs:
-            # scheduler.rs:113-117: the budget must cover one decode token per sequence.
-            raise ValueError("max_batched_tokens must be at least max_num_seqs")
+        if self.max_batched_tokens <= 0:
+            raise ValueError("max_batched_tokens must be positive")
+        # A budget below max_num_seqs is raised to it by the engine, as the reference does
+        # (engine.rs:263-271): the scheduler needs one decode token per sequence
+        # (scheduler.rs:113-117).
         if self.scheduler not in ("continuous", "static"):
             raise ValueError(f"scheduler must be 'continuous' or 'static', got {self.scheduler!r}")

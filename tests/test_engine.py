@@ -194,3 +194,31 @@ def test_perplexity_matches_the_plain_implementation(backend, tiny_folders):
         perplexity(runner, tokens, bos=1, ctx=3)
     with pytest.raises(ValueError, match="shorter than one window"):
         perplexity(runner, tokens[:10], bos=1, ctx=16)
+
+
+def test_pool_size_watermark_and_budget_follow_the_references_rules(backend, tiny_folders):
+    """crates/engine/src/engine.rs:252-280: pages = pool bytes / (bytes of K and V per token *
+    block size); watermark = max(1, pages / 100); the budget is at least max_num_seqs; the
+    longest request is bounded by the rope table and by the pool."""
+    from rust_llm_inference_server_amd.engine import Engine
+    model = load(tiny_folders["a"], backend, max_positions=128)        # float32
+    per_token = 2 * 2 * 1 * 16 * 4                                     # K and V, layers, kv heads, d
+    cfg = EngineConfig(kv_cache_gb=0.001, block_size=16, max_num_seqs=8, max_batched_tokens=4,
+                       max_seq_len=128)
+    engine = Engine(model, cfg)
+    pages = int(0.001 * (1 << 30)) // (per_token * 16)
+    assert engine.runner.cache.num_pages(0) == pages == 262
+    assert engine.scheduler.max_batched_tokens == 8
+    assert engine.scheduler.max_seq_tokens == (pages - max(1, pages // 100)) * 16
+    assert engine.max_seq_len == 128
+    small = Engine(model, EngineConfig(num_pages=5, block_size=8, max_num_seqs=2, max_seq_len=128))
+    assert small.max_seq_len == (5 - 1) * 8
+    with pytest.raises(ValueError, match="at least 2"):
+        Engine(model, EngineConfig(num_pages=1, block_size=8, max_num_seqs=2))
+    defaults = EngineConfig()                                          # engine.rs:31-63
+    assert (defaults.max_num_seqs, defaults.max_batched_tokens, defaults.kv_cache_gb,
+            defaults.block_size, defaults.scheduler) == (64, 2048, 1.0, 16, "continuous")
+    for bad in (dict(max_num_seqs=0), dict(block_size=0), dict(scheduler="fair"),
+                dict(max_batched_tokens=0)):
+        with pytest.raises(ValueError):
+            EngineConfig(**bad).validate()
