@@ -14,7 +14,9 @@ kernels clear nothing) and are checked against the eager step in the tests, repl
 replay with eager work in between."""
 from __future__ import annotations
 
+import contextlib
 import ctypes
+import gc
 from typing import Optional, Sequence
 
 import numpy as np
@@ -29,6 +31,23 @@ def bucket_for(n: int, limit: int) -> int:
     while b < n:
         b *= 2
     return min(b, max(limit, n))
+
+
+@contextlib.contextmanager
+def no_collection():
+    """Keeps Python's cyclic collector from running inside the block.  Under stream capture it
+    must not: what it finds (an earlier engine's graphs, pinned buffers, events: they sit in
+    reference cycles) is destroyed through HIP calls that a capturing stream refuses, and an
+    error inside a destructor ends the process.  Garbage is collected before the block and
+    waits until after it."""
+    gc.collect()
+    enabled = gc.isenabled()
+    gc.disable()
+    try:
+        yield
+    finally:
+        if enabled:
+            gc.enable()
 
 
 class DecodeGraph:
@@ -137,7 +156,7 @@ class DecodeGraph:
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        with no_collection(), torch.cuda.graph(graph):
             self.logits = runner.model.forward(self.step, runner.pools)
         self.graph = graph
         graph.replay()

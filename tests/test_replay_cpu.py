@@ -97,3 +97,35 @@ def test_step_layout_puts_single_tokens_first(cpu_ops, tiny_folders):
     runner.step([StepEntry(4, [7, 8, 9, 10], []), StepEntry(2, list(range(8)), [])])
     again = runner.step([entries[2], entries[3], entries[1], entries[0]])
     assert (again[[2, 3, 1, 0]] - want).abs().max().item() < 1e-5
+
+
+def test_no_collection_holds_the_cyclic_collector_off():
+    """What graph capture runs under: garbage is collected before the block, none inside it
+    (not even at the lowest thresholds), and the collector is back afterwards."""
+    import gc
+    import weakref
+    from rust_llm_inference_server_amd.engine.graph import no_collection
+
+    class Node:
+        pass
+
+    def cycle():
+        a, b = Node(), Node()
+        a.other, b.other = b, a
+        return weakref.ref(a)
+
+    before = cycle()
+    thresholds = gc.get_threshold()
+    gc.set_threshold(1, 1, 1)
+    try:
+        with no_collection():
+            assert before() is None and not gc.isenabled()
+            inside = cycle()
+            junk = [[i] for i in range(2000)]            # allocations that would trigger a pass
+            assert inside() is not None
+            del junk
+        assert gc.isenabled()
+        gc.collect()
+        assert inside() is None
+    finally:
+        gc.set_threshold(*thresholds)

@@ -95,6 +95,30 @@ def test_captured_decode_steps_match_eager_ones(case, dtype):
             torch.testing.assert_close(out_g[k], out_e[k], atol=TOL[dtype] / 4, rtol=0)
 
 
+def test_capture_beside_the_garbage_of_an_earlier_runner(case):
+    """A runner that has captured graphs is dropped without a collection (runner and graphs
+    refer to each other, so only the cyclic collector frees them); the next runner captures
+    its graphs while the collector would run at every allocation.  Capture holds it off:
+    destroying graphs, pinned buffers and events under a capturing stream is refused by HIP."""
+    import gc
+    name, cfg, per_dtype = case
+    folder, reqs, ref = per_dtype["float32"]
+    steps, max_tokens = traces.trace_tail(reqs)
+    first = make_runner(folder, "float32", max_tokens, 16, use_graphs=True)
+    traces.replay_in_process(first, steps)
+    assert first._graphs
+    del first
+    thresholds = gc.get_threshold()
+    gc.set_threshold(1, 1, 1)
+    try:
+        second = make_runner(folder, "float32", max_tokens, 16, use_graphs=True)
+        outputs = traces.replay_in_process(second, steps)
+    finally:
+        gc.set_threshold(*thresholds)
+    assert second._graphs
+    check(steps, outputs, reqs, ref, cfg["vocab_size"], TOL["float32"])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_first_tokens_of_a_sequence(case, dtype):
     """Sequences fed one token at a time from position 0 (no prompt step before them), two of
