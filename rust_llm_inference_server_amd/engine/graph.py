@@ -17,6 +17,7 @@ from __future__ import annotations
 import contextlib
 import ctypes
 import gc
+import weakref
 from typing import Optional, Sequence
 
 import numpy as np
@@ -54,7 +55,7 @@ class DecodeGraph:
     """The captured decode step of one batch-size bucket."""
 
     def __init__(self, runner, bucket: int):
-        self.runner = runner
+        self.runner = weakref.proxy(runner)     # the runner owns its graphs: no cycle
         self.bucket = B = bucket
         model, cache = runner.model, runner.cache
         dev = runner.device
