@@ -222,3 +222,48 @@ def test_pool_size_watermark_and_budget_follow_the_references_rules(backend, tin
                 dict(max_batched_tokens=0)):
         with pytest.raises(ValueError):
             EngineConfig(**bad).validate()
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_workloads_give_what_each_request_gives_alone(backend, tiny_folders, seed):
+    """Requests of random lengths and sampling parameters, arriving while others run, under a
+    random budget, page size and a pool small enough to preempt now and then: every request
+    ends with the tokens it produces alone in a roomy engine, and every page comes back."""
+    import random
+    rng = random.Random(seed)
+    name = rng.choice(["a", "b"])
+    model = load(tiny_folders[name], backend, max_positions=128)
+    vocab = plain.read_config(tiny_folders[name])["vocab_size"]
+    n = rng.randrange(4, 9)
+    prompts = prompts_for(vocab, [rng.choice([1, 2, 7, 16, 17, 33, 60]) for _ in range(n)], seed)
+    params = []
+    for i in range(n):
+        mt = rng.randrange(1, 20)
+        kind = rng.choice(["greedy", "temperature", "host"])
+        if kind == "greedy":
+            params.append(SamplingParams.greedy(mt))
+        elif kind == "temperature":
+            params.append(SamplingParams(temperature=rng.choice([0.5, 1.0]), seed=100 + i, max_tokens=mt))
+        else:
+            params.append(SamplingParams(temperature=0.9, top_k=rng.choice([0, 5]), top_p=rng.choice([1.0, 0.8]),
+                                         repetition_penalty=rng.choice([1.0, 1.2]), seed=200 + i, max_tokens=mt))
+    alone = [engine_for(model).generate([p], sp)[0].token_ids for p, sp in zip(prompts, params)]
+    block = rng.choice([8, 16])
+    longest = max(len(p) + sp.max_tokens for p, sp in zip(prompts, params))
+    pages = -(-longest // block) + rng.randrange(1, 6)
+    engine = engine_for(model, num_pages=pages, block_size=block, watermark_pages=rng.choice([0, 1]),
+                        max_num_seqs=rng.choice([2, 4, 8]), max_batched_tokens=rng.choice([8, 24, 64]))
+    ids, pending, steps = {}, list(range(n)), 0
+    while pending or engine.has_work():
+        for _ in range(rng.randrange(0, 3)):                  # arrivals between steps
+            if pending:
+                i = pending.pop(0)
+                ids[engine.add_request(prompts[i], params[i])] = i
+        if engine.has_work():
+            engine.step()
+        steps += 1
+        assert steps < 5000
+    got = {ids[k]: engine.pop_finished(k) for k in ids}
+    assert [got[i].token_ids for i in range(n)] == alone
+    assert engine.runner.cache.num_free_pages() == pages
+    engine.runner.cache.check_invariants()
