@@ -647,6 +647,39 @@ def test_attention_finds_a_far_key(ops, dtype, kind, decode_kind):
     torch.testing.assert_close(got[-1, :d].float().cpu(), vs[0][far, 0, :], **tol(dtype, 1e-4, 2e-2))
 
 
+@pytest.mark.parametrize("kind,dtype", kinds_and_dtypes("generic", "prefill", "decode"))
+@pytest.mark.parametrize("window", [5, 64, 100, 300])
+def test_attention_window_edge(ops, dtype, kind, window, decode_kind):
+    """The last query sees keys p - window + 1 .. p.  The key just outside the window is made
+    to stand out: it must not be seen.  Then the first key inside is made to stand out twice as
+    much: the output must be its value.  An edge that is off by one fails one of the two."""
+    nh, nkv, d, ps = 4, 2, 64, 16
+    total = 555
+    cached, new = ([total - 1], [1]) if kind == "decode" else ([total - 3], [3])
+    qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=window)
+    table = bt[0].tolist()
+    qdir = qkv[-1, :d].float()                  # last token, head 0 (KV head 0)
+    qdir = qdir / qdir.norm()
+    p = total - 1
+
+    def stand_out(pos, by):
+        kp[table[pos // ps], 0, pos % ps, :] = (qdir * by).to(dtype)
+        ks[0][pos, 0, :] = kp[table[pos // ps], 0, pos % ps, :].float().cpu()
+
+    def run():
+        got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, 1.0, window, force=kind)
+        want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, 1.0, window)
+        torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
+        return got[-1, :d].float().cpu()
+
+    stand_out(p - window, 50.0)
+    unseen = run()
+    assert (unseen - vs[0][p - window, 0, :]).abs().max() > 0.1
+    stand_out(p - window + 1, 100.0)
+    seen = run()
+    torch.testing.assert_close(seen, vs[0][p - window + 1, 0, :], **tol(dtype, 1e-4, 2e-2))
+
+
 def test_attention_one_key_returns_its_value(ops):
     nh, nkv, d, ps = 4, 2, 32, 8
     for kind in ("generic", "decode"):
