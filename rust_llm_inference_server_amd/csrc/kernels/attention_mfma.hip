@@ -70,6 +70,12 @@ constexpr int D = RLIS_HEAD_DIM;
 __host__ __device__ constexpr int tile_keys(int QB) {
   return (D > 128 || QB == 2) ? 32 : 64;
 }
+// LDS row strides.  A 16-byte read of a wave is served in four cycles, sixteen lanes each
+// (lanes 0-3, 12-15, 20-27 in the first, 4-11, 16-19, 28-31 in the second, and the same
+// plus 32), and a cycle is free of bank conflicts when its sixteen 16-byte pieces fall on
+// sixteen different quarters of the 64 banks.  For 16 rows read at every second row (the K
+// tile, see below) that holds with a row stride of 16 bytes mod 32; for 16 consecutive rows
+// (the V^T tile) with a stride of 32 bytes mod 64.
 constexpr int KS = D + 8;     // K tile row stride (bf16 elements)
 constexpr int BM = 64;       // queries per workgroup and query block
 // Two LDS tiles taking turns (one barrier per tile instead of two) where that does not cost a
@@ -91,7 +97,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
     int page_shift, float scale, int window, int num_tiles, int tiles_per_round, int splits,
     int row0, float* __restrict__ part_ml, float* __restrict__ part_acc) {
   constexpr int BN = tile_keys(QB);
-  constexpr int VS = BN + 8;    // V tile row stride
+  constexpr int VS = BN + 16;   // V tile row stride
   constexpr int kTileBufs = tile_bufs(QB);
   __shared__ __attribute__((aligned(16))) bf16_t Ks_all[kTileBufs * BN * KS];
   __shared__ __attribute__((aligned(16))) bf16_t Vs_all[kTileBufs * D * VS];
@@ -250,7 +256,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
     // Tiles wholly after this wave's last query contribute nothing to it.
     const bool wave_active = (wave_q_first < n_new) && (k0 <= P + wave_q_last);
     if (wave_active) {
-      // ---- S^T = K Q^T: block nb holds keys k0 + nb * 16 + lq * 4 + r for query l16 --------
+      // ---- S^T = K Q^T for query l16.  Blocks 2 st and 2 st + 1 share the 32 keys from
+      // k0 + 32 st on: row i of the even block is key 2 i of them, row i of the odd block
+      // key 2 i + 1, so that the eight scores a lane holds of the pair (rows lq * 4 + r) are
+      // the eight consecutive keys lq * 8 ... + 7, which is what one 16-byte read of a V^T
+      // row delivers for the second product.
       f32x4 s[QB][BN / 16];
 #pragma unroll
       for (int nb = 0; nb < BN / 16; ++nb) {
@@ -259,7 +269,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
 #pragma unroll
         for (int ks = 0; ks < D / 32; ++ks) {
           Frag8 kf;
-          kf.u = *(const uint4*)(Ks + (nb * 16 + l16) * KS + ks * 32 + lq * 8);
+          kf.u = *(const uint4*)(Ks + ((nb / 2) * 32 + 2 * l16 + (nb % 2)) * KS + ks * 32 + lq * 8);
 #pragma unroll
           for (int b = 0; b < QB; ++b)
             s[b][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[b][ks].v, s[b][nb], 0, 0, 0);
@@ -285,7 +295,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
           for (int nb = 0; nb < BN / 16; ++nb)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              const int kpos = k0 + nb * 16 + lq * 4 + r;
+              const int kpos = k0 + (nb / 2) * 32 + lq * 8 + 2 * r + (nb % 2);
               const bool ok = (kpos <= my_qpos[b]) && (window <= 0 || kpos > my_qpos[b] - window);
               const float sv = ok ? s[b][nb][r] : -INFINITY;
               s[b][nb][r] = sv;
@@ -327,16 +337,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
         for (int b = 0; b < QB; ++b)
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            pf[b][j] = (__bf16)s[b][2 * st][j];
-            pf[b][4 + j] = (__bf16)s[b][2 * st + 1][j];
+            pf[b][2 * j] = (__bf16)s[b][2 * st][j];
+            pf[b][2 * j + 1] = (__bf16)s[b][2 * st + 1][j];
           }
 #pragma unroll
         for (int db = 0; db < D / 16; ++db) {
           if (db * 16 < d) {
             Frag8 vf;
-            const bf16_t* vrow = Vs + (db * 16 + l16) * VS + st * 32 + lq * 4;
-            vf.h[0] = *(const uint2*)(vrow);
-            vf.h[1] = *(const uint2*)(vrow + 16);
+            vf.u = *(const uint4*)(Vs + (db * 16 + l16) * VS + st * 32 + lq * 8);
 #pragma unroll
             for (int b = 0; b < QB; ++b)
               o_acc[b][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[b], o_acc[b][db], 0, 0, 0);
