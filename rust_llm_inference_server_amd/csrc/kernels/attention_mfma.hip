@@ -342,13 +342,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
           }
 #pragma unroll
         for (int db = 0; db < D / 16; ++db) {
-          if (db * 16 < d) {
-            Frag8 vf;
-            vf.u = *(const uint4*)(Vs + (db * 16 + l16) * VS + st * 32 + lq * 8);
+          // Unconditional, so that reads and products of all blocks can overlap: rows of V^T
+          // past d hold whatever LDS held and feed rows of O^T that are never stored.
+          Frag8 vf;
+          vf.u = *(const uint4*)(Vs + (db * 16 + l16) * VS + st * 32 + lq * 8);
 #pragma unroll
-            for (int b = 0; b < QB; ++b)
-              o_acc[b][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[b], o_acc[b][db], 0, 0, 0);
-          }
+          for (int b = 0; b < QB; ++b)
+            o_acc[b][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[b], o_acc[b][db], 0, 0, 0);
         }
       }
     }
@@ -644,12 +644,10 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
     l_run = l_run * corr + sum;
     m_run = m_new;
 #pragma unroll
-    for (int db = 0; db < D / 16; ++db) {
-      if (db * 16 < d) {
+    for (int db = 0; db < D / 16; ++db) {   // blocks past d: rows of O^T that are never stored
 #pragma unroll
-        for (int r = 0; r < 4; ++r) o_acc[db][r] *= corr;
-        o_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db].v, pf, o_acc[db], 0, 0, 0);
-      }
+      for (int r = 0; r < 4; ++r) o_acc[db][r] *= corr;
+      o_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db].v, pf, o_acc[db], 0, 0, 0);
     }
   };
 
