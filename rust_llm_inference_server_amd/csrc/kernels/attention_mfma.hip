@@ -200,26 +200,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
   // stay in registers.
   u32x4 tile_ka[KCH], tile_va[VCH], tile_kb[KCH], tile_vb[VCH];
   int page_ka[KCH], page_va[VCH], page_kb[KCH], page_vb[VCH];
+  // Addresses: 64 bits only for page id times the elements of a page; what lies inside a page
+  // (head, offset, dim) fits 32 bits and costs one multiply-add.  Keys are never negative, so
+  // the clamp is a minimum alone.
+  const unsigned page_elems = ((unsigned)nkv << page_shift) * (unsigned)d;
+  unsigned k_in[KCH], v_in[VCH];                        // inside a page, without the key's offset
+#pragma unroll
+  for (int i = 0; i < KCH; ++i) k_in[i] = ((unsigned)kvh << page_shift) * (unsigned)d + k_dim[i];
+#pragma unroll
+  for (int i = 0; i < VCH; ++i) v_in[i] = ((unsigned)(kvh * d + v_dim[i])) << page_shift;
 #define RLIS_LOAD_PAGES(k0_, PK, PV)                                                           \
   {                                                                                            \
     _Pragma("unroll") for (int i = 0; i < KCH; ++i)                                            \
-        PK[i] = table[max(0, min((k0_) + k_key[i], last_key)) >> page_shift];                  \
+        PK[i] = table[min((k0_) + k_key[i], last_key) >> page_shift];                          \
     _Pragma("unroll") for (int i = 0; i < VCH; ++i)                                            \
-        PV[i] = table[max(0, min((k0_) + v_key[i], last_group)) >> page_shift];                \
+        PV[i] = table[min((k0_) + v_key[i], last_group) >> page_shift];                        \
   }
 #define RLIS_LOAD_TILE(k0_, PK, PV, TK, TV)                                                    \
   {                                                                                            \
     _Pragma("unroll") for (int i = 0; i < KCH; ++i) {                                          \
-      const int off_ = max(0, min((k0_) + k_key[i], last_key)) & page_mask;                    \
-      TK[i] = *(const u32x4*)(k_pages +                                                        \
-                              ((((long long)PK[i] * nkv + kvh) << page_shift) + off_) * d +    \
-                              k_dim[i]);                                                       \
+      const unsigned off_ = (unsigned)(min((k0_) + k_key[i], last_key) & page_mask);           \
+      TK[i] = *(const u32x4*)(k_pages + ((unsigned long long)(unsigned)PK[i] * page_elems +    \
+                                         (off_ * (unsigned)d + k_in[i])));                     \
     }                                                                                          \
     _Pragma("unroll") for (int i = 0; i < VCH; ++i) {                                          \
-      const int off_ = max(0, min((k0_) + v_key[i], last_group)) & page_mask;                  \
-      TV[i] = *(const u32x4*)(v_pages +                                                        \
-                              ((((long long)PV[i] * nkv + kvh) * d + v_dim[i]) << page_shift) + \
-                              off_);                                                           \
+      const unsigned off_ = (unsigned)(min((k0_) + v_key[i], last_group) & page_mask);         \
+      TV[i] = *(const u32x4*)(v_pages + ((unsigned long long)(unsigned)PV[i] * page_elems +    \
+                                         (v_in[i] + off_)));                                   \
     }                                                                                          \
   }
 #define RLIS_STORE_TILE(TK, TV, buf_)                                                          \
