@@ -590,27 +590,33 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
   for (int db = 0; db < D / 16; ++db) v_dim[db] = min(db * 16 + l16, d - 1);
   Frag8 k_a[2][D / 32], v_a[D / 16], k_b[2][D / 32], v_b[D / 16];
   int pk_a[2], pv_a[2], pk_b[2], pv_b[2];
+  // Addresses: 64 bits only for page id times the elements of a page (keys are never negative,
+  // so the clamp is a minimum alone).
+  const unsigned page_elems = ((unsigned)nkv << page_shift) * (unsigned)d;
+  const unsigned k_head = ((unsigned)kvh << page_shift) * (unsigned)d;
+  const unsigned v_head = ((unsigned)(kvh * d)) << page_shift;
 #define RLIS_DEC_PAGES(c0_, PK, PV)                                                             \
   {                                                                                             \
     _Pragma("unroll") for (int i = 0; i < 2; ++i) {                                             \
-      PK[i] = table[max(0, min((c0_) + i * 16 + l16, last_key)) >> page_shift];                 \
-      PV[i] = table[max(0, min((c0_) + i * 16 + lq * 4, last_quad)) >> page_shift];             \
+      PK[i] = table[min((c0_) + i * 16 + l16, last_key) >> page_shift];                         \
+      PV[i] = table[min((c0_) + i * 16 + lq * 4, last_quad) >> page_shift];                     \
     }                                                                                           \
   }
 #define RLIS_DEC_CHUNK(c0_, PK, PV, KF, VF)                                                     \
   {                                                                                             \
     _Pragma("unroll") for (int nb = 0; nb < 2; ++nb) {                                          \
-      const int key_ = max(0, min((c0_) + nb * 16 + l16, last_key));                            \
-      const bf16_t* kp_ =                                                                       \
-          k_pages + ((((long long)PK[nb] * nkv + kvh) << page_shift) + (key_ & page_mask)) * d; \
+      const unsigned off_ = (unsigned)(min((c0_) + nb * 16 + l16, last_key) & page_mask);       \
+      const bf16_t* kp_ = k_pages + ((unsigned long long)(unsigned)PK[nb] * page_elems +        \
+                                     (k_head + off_ * (unsigned)d));                            \
       _Pragma("unroll") for (int ks = 0; ks < D / 32; ++ks)                                     \
           KF[nb][ks].u = *(const uint4*)(kp_ + k_dim[ks]);                                      \
     }                                                                                           \
     _Pragma("unroll") for (int hf = 0; hf < 2; ++hf) {                                          \
-      const int off_ = max(0, min((c0_) + hf * 16 + lq * 4, last_quad)) & page_mask;            \
-      const bf16_t* vp_ = v_pages + ((((long long)PV[hf] * nkv + kvh) * d) << page_shift) + off_; \
+      const unsigned off_ = (unsigned)(min((c0_) + hf * 16 + lq * 4, last_quad) & page_mask);   \
+      const bf16_t* vp_ = v_pages + ((unsigned long long)(unsigned)PV[hf] * page_elems +        \
+                                     (v_head + off_));                                          \
       _Pragma("unroll") for (int db = 0; db < D / 16; ++db)                                     \
-          VF[db].h[hf] = *(const uint2*)(vp_ + ((long long)v_dim[db] << page_shift));           \
+          VF[db].h[hf] = *(const uint2*)(vp_ + ((unsigned)v_dim[db] << page_shift));            \
     }                                                                                           \
   }
   auto compute = [&](int c0, const Frag8 (&kf)[2][D / 32], const Frag8 (&vf)[D / 16])
