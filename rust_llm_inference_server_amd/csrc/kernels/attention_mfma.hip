@@ -173,11 +173,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
   // Staging for the tiles to come.  A tile's page ids are fetched four tiles ahead of its use,
   // its keys and values two tiles ahead (two register sets taking turns), so that neither the
   // table lookup nor the loads themselves are waited for.  The loads are unconditional, so
-  // that the compiler can count them: a key past the end of the tile's range reads the last
-  // key in range instead (its score is masked), a dim past d reads dim d - 8 (it meets a zero
-  // of q, or a row of O^T that is not stored).  Values past the end of the range inside a
-  // group of 8 keys are whatever the page holds: the pages start as zeros and only ever hold
-  // values that a model wrote, and their probabilities are exactly zero.
+  // that the compiler can count them: a key past the end of the range reads its place in the
+  // last page of the range (its score is masked), a dim past d reads dim d - 8 (it meets a
+  // zero of q, or a row of O^T that is not stored).  Keys and values past the end are whatever
+  // the page holds: the pages start as zeros and only ever hold what a model wrote, and their
+  // probabilities are exactly zero.
   constexpr int K_CHUNKS = BN * (D / 8);
   constexpr int KCH = (K_CHUNKS + 255) / 256;
   constexpr int VCH = (D * (BN / 8) + 255) / 256;
@@ -195,39 +195,46 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
     v_dim[i] = c / (BN / 8);
     v_key[i] = (c % (BN / 8)) * 8;
   }
-  const int last_key = khi - 1, last_group = (khi - 1) & ~7;
+  // Addresses.  Tiles start at multiples of their size and pages are powers of two, so the
+  // page of a chunk is (k0 >> page_shift) + a constant of the thread, and its place inside the
+  // page is a constant of the thread plus (k0 & page_mask), which is zero unless pages are
+  // larger than tiles: what changes from tile to tile is uniform over the workgroup.  The page
+  // index is clamped to the last page of the range; 64 bits are needed only for page id times
+  // the elements of a page.
+  const int last_page = (khi - 1) >> page_shift;
+  const unsigned page_elems = ((unsigned)nkv << page_shift) * (unsigned)d;
+  int k_pg[KCH], v_pg[VCH];
+  unsigned k_in[KCH], v_in[VCH];
+#pragma unroll
+  for (int i = 0; i < KCH; ++i) {
+    k_pg[i] = k_key[i] >> page_shift;
+    k_in[i] = (((unsigned)kvh << page_shift) + (unsigned)(k_key[i] & page_mask)) * (unsigned)d + k_dim[i];
+  }
+#pragma unroll
+  for (int i = 0; i < VCH; ++i) {
+    v_pg[i] = v_key[i] >> page_shift;
+    v_in[i] = (((unsigned)(kvh * d + v_dim[i])) << page_shift) + (unsigned)(v_key[i] & page_mask);
+  }
   // Two sets of staging registers (A, B) and of page ids; plain arrays and macros, so that they
   // stay in registers.
   u32x4 tile_ka[KCH], tile_va[VCH], tile_kb[KCH], tile_vb[VCH];
   int page_ka[KCH], page_va[VCH], page_kb[KCH], page_vb[VCH];
-  // Addresses: 64 bits only for page id times the elements of a page; what lies inside a page
-  // (head, offset, dim) fits 32 bits and costs one multiply-add.  Keys are never negative, so
-  // the clamp is a minimum alone.
-  const unsigned page_elems = ((unsigned)nkv << page_shift) * (unsigned)d;
-  unsigned k_in[KCH], v_in[VCH];                        // inside a page, without the key's offset
-#pragma unroll
-  for (int i = 0; i < KCH; ++i) k_in[i] = ((unsigned)kvh << page_shift) * (unsigned)d + k_dim[i];
-#pragma unroll
-  for (int i = 0; i < VCH; ++i) v_in[i] = ((unsigned)(kvh * d + v_dim[i])) << page_shift;
 #define RLIS_LOAD_PAGES(k0_, PK, PV)                                                           \
   {                                                                                            \
-    _Pragma("unroll") for (int i = 0; i < KCH; ++i)                                            \
-        PK[i] = table[min((k0_) + k_key[i], last_key) >> page_shift];                          \
-    _Pragma("unroll") for (int i = 0; i < VCH; ++i)                                            \
-        PV[i] = table[min((k0_) + v_key[i], last_group) >> page_shift];                        \
+    const int pg0_ = (k0_) >> page_shift;                                                      \
+    _Pragma("unroll") for (int i = 0; i < KCH; ++i) PK[i] = table[min(pg0_ + k_pg[i], last_page)]; \
+    _Pragma("unroll") for (int i = 0; i < VCH; ++i) PV[i] = table[min(pg0_ + v_pg[i], last_page)]; \
   }
 #define RLIS_LOAD_TILE(k0_, PK, PV, TK, TV)                                                    \
   {                                                                                            \
-    _Pragma("unroll") for (int i = 0; i < KCH; ++i) {                                          \
-      const unsigned off_ = (unsigned)(min((k0_) + k_key[i], last_key) & page_mask);           \
-      TK[i] = *(const u32x4*)(k_pages + ((unsigned long long)(unsigned)PK[i] * page_elems +    \
-                                         (off_ * (unsigned)d + k_in[i])));                     \
-    }                                                                                          \
-    _Pragma("unroll") for (int i = 0; i < VCH; ++i) {                                          \
-      const unsigned off_ = (unsigned)(min((k0_) + v_key[i], last_group) & page_mask);         \
-      TV[i] = *(const u32x4*)(v_pages + ((unsigned long long)(unsigned)PV[i] * page_elems +    \
-                                         (v_in[i] + off_)));                                   \
-    }                                                                                          \
+    const unsigned off0_ = (unsigned)((k0_) & page_mask);                                      \
+    const unsigned koff0_ = off0_ * (unsigned)d;                                               \
+    _Pragma("unroll") for (int i = 0; i < KCH; ++i)                                            \
+        TK[i] = *(const u32x4*)(k_pages + ((unsigned long long)(unsigned)PK[i] * page_elems +  \
+                                           (k_in[i] + koff0_)));                               \
+    _Pragma("unroll") for (int i = 0; i < VCH; ++i)                                            \
+        TV[i] = *(const u32x4*)(v_pages + ((unsigned long long)(unsigned)PV[i] * page_elems +  \
+                                           (v_in[i] + off0_)));                                \
   }
 #define RLIS_STORE_TILE(TK, TV, buf_)                                                          \
   {                                                                                            \
