@@ -180,7 +180,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
   // probabilities are exactly zero.
   constexpr int K_CHUNKS = BN * (D / 8);
   constexpr int KCH = (K_CHUNKS + 255) / 256;
-  constexpr int VCH = (D * (BN / 8) + 255) / 256;
+  constexpr int V_CHUNKS = D * (BN / 8);     // rows past d receive copies of the last chunk
+  constexpr int VCH = (V_CHUNKS + 255) / 256;
   const int v_chunks = d * (BN / 8);
   int k_key[KCH], k_dim[KCH], v_key[VCH], v_dim[VCH];   // this thread's chunks within a tile
 #pragma unroll
@@ -222,8 +223,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
 #define RLIS_LOAD_PAGES(k0_, PK, PV)                                                           \
   {                                                                                            \
     const int pg0_ = (k0_) >> page_shift;                                                      \
-    _Pragma("unroll") for (int i = 0; i < KCH; ++i) PK[i] = table[min(pg0_ + k_pg[i], last_page)]; \
-    _Pragma("unroll") for (int i = 0; i < VCH; ++i) PV[i] = table[min(pg0_ + v_pg[i], last_page)]; \
+    _Pragma("unroll") for (int i = 0; i < KCH; ++i) PK[i] = table[(unsigned)min(pg0_ + k_pg[i], last_page)]; \
+    _Pragma("unroll") for (int i = 0; i < VCH; ++i) PV[i] = table[(unsigned)min(pg0_ + v_pg[i], last_page)]; \
   }
 #define RLIS_LOAD_TILE(k0_, PK, PV, TK, TV)                                                    \
   {                                                                                            \
@@ -242,11 +243,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
     bf16_t* Vs = Vs_all + (buf_) * (D * VS);                                                   \
     _Pragma("unroll") for (int i = 0; i < KCH; ++i) {                                          \
       const int c_ = tid + i * 256;                                                            \
-      if (c_ < K_CHUNKS) *(u32x4*)(Ks + (c_ / (D / 8)) * KS + (c_ % (D / 8)) * 8) = TK[i];     \
+      if (K_CHUNKS % 256 == 0 || c_ < K_CHUNKS)                                                \
+        *(u32x4*)(Ks + (c_ / (D / 8)) * KS + (c_ % (D / 8)) * 8) = TK[i];                      \
     }                                                                                          \
     _Pragma("unroll") for (int i = 0; i < VCH; ++i) {                                          \
       const int c_ = tid + i * 256;                                                            \
-      if (c_ < v_chunks) *(u32x4*)(Vs + (c_ / (BN / 8)) * VS + (c_ % (BN / 8)) * 8) = TV[i];   \
+      if (V_CHUNKS % 256 == 0 || c_ < V_CHUNKS)                                                \
+        *(u32x4*)(Vs + (c_ / (BN / 8)) * VS + (c_ % (BN / 8)) * 8) = TV[i];                    \
     }                                                                                          \
   }
 
