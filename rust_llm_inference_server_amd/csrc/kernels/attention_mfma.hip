@@ -332,7 +332,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
             s[b][nb][r] = p;
             sum += p;
           }
-        sum = xor32_sum(xor16_sum(sum));
+        // The denominator stays a partial sum per lane (the four lanes of a query share its
+        // maximum, hence corr); the lanes are added once, after the last tile.
         l_run[b] = l_run[b] * corr[b] + sum;
         m_run[b] = m_new;
         moved = moved || corr[b] != 1.0f;
@@ -405,6 +406,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
   }
 
   // ---- normalise and store: this lane holds dims db * 16 + lq * 4 + [0, 4) of its queries --
+#pragma unroll
+  for (int b = 0; b < QB; ++b) l_run[b] = xor32_sum(xor16_sum(l_run[b]));
 #pragma unroll
   for (int b = 0; b < QB; ++b) {
     if (my_qi[b] < n_new) {
@@ -663,8 +666,7 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
         sum += p;
         pf[nb * 4 + r] = (__bf16)p;
       }
-    sum = xor32_sum(xor16_sum(sum));
-    l_run = l_run * corr + sum;
+    l_run = l_run * corr + sum;        // per lane; the four lanes of a head are added at the end
     m_run = m_new;
 #pragma unroll
     for (int db = 0; db < D / 16; ++db) {   // blocks past d: rows of O^T that are never stored
@@ -701,6 +703,7 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
 #undef RLIS_DEC_PAGES
 
   // ---- merge the waves (in wave order), then store the partition ------------------
+  l_run = xor32_sum(xor16_sum(l_run));
   float* ml_s = dsm;                       // [wave][head][2]
   float* acc_s = dsm + kDecodeWaves * g * 2;   // [wave][head][d]
   if (l16 < g) {
