@@ -516,7 +516,8 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
   const int ka = kb + l32 * 8;                          // this lane's k when loading weights
   const bool a_ok = has_item && ka < K;
   // Loads are never predicated off (that would cost registers for the zeros): a row past the
-  // end reads row 0 instead and is not stored; a k past the end reads k = 0 and is zeroed.
+  // end reads row 0 instead and is not stored; a k past the end reads k = 0 instead and meets
+  // a zero in the rows of x (weights are finite).
   const bf16_t* w_lane = W + (a_ok ? ka : 0);
 
   // Tile row r = 2 p + half of tile `tile` is weight row tile * rows + r; gated, the first
@@ -533,11 +534,11 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
         const int c = GATED ? (2 * p) % cols_per_tile : 2 * p; /* column within the tile */     \
         const long long up = (GATED && 2 * p >= cols_per_tile) ? (long long)N * sh.ldw : 0;     \
         const bf16_t* ptr = col0 + c < N ? w_tile + (long long)c * sh.ldw + up : w_lane;        \
-        const uint4 v_ = *(const uint4*)ptr;                                                    \
-        a[p].x = a_ok ? v_.x : 0u;                                                              \
-        a[p].y = a_ok ? v_.y : 0u;                                                              \
-        a[p].z = a_ok ? v_.z : 0u;                                                              \
-        a[p].w = a_ok ? v_.w : 0u;                                                              \
+        const uint4 v_ = *(const uint4*)ptr;   /* a k past the end meets a zero of x */         \
+        a[p].x = v_.x;          /* member by member: a struct copy would go through scratch */  \
+        a[p].y = v_.y;                                                                          \
+        a[p].z = v_.z;                                                                          \
+        a[p].w = v_.w;                                                                          \
       }                                                                                         \
     }                                                                                           \
   }
