@@ -722,17 +722,23 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
   __syncthreads();
   for (int i = tid; i < g * d; i += 64 * kDecodeWaves) {
     const int hh = i / d, j = i % d;
+    // Without branches, so that all the reads are issued together: a wave that saw no key has
+    // maximum -inf, weight 0 (selected, since -inf - -inf is no number) and sums of zeros.
+    float mw[kDecodeWaves], lw[kDecodeWaves], aw[kDecodeWaves];
     float big = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < kDecodeWaves; ++w) big = fmaxf(big, ml_s[(w * g + hh) * 2]);
+    for (int w = 0; w < kDecodeWaves; ++w) {
+      mw[w] = ml_s[(w * g + hh) * 2];
+      lw[w] = ml_s[(w * g + hh) * 2 + 1];
+      aw[w] = acc_s[(w * g + hh) * d + j];
+      big = fmaxf(big, mw[w]);
+    }
     float lsum = 0.f, a = 0.f;
 #pragma unroll
     for (int w = 0; w < kDecodeWaves; ++w) {
-      const float mw = ml_s[(w * g + hh) * 2];
-      if (mw == -INFINITY) continue;
-      const float e = __builtin_amdgcn_exp2f(mw - big);
-      lsum += ml_s[(w * g + hh) * 2 + 1] * e;
-      a += acc_s[(w * g + hh) * d + j] * e;
+      const float e = (mw[w] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw[w] - big);
+      lsum += lw[w] * e;
+      a += aw[w] * e;
     }
     const int h = kvh * g + hh;
     if (splits == 1) {
