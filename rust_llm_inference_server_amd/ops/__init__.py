@@ -351,11 +351,13 @@ def copy_pages(pages: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> Non
 
 # ----------------------------------------------------------------------- attention
 def decode_splits(num_seqs: int, num_kv_heads: int, group: int, max_context: int) -> int:
-    """Partitions per context for the decode kernel: enough workgroups to fill 256 compute
-    units twice, at least 256 positions each (the rule of crates/model/src/
-    paged_attention.rs:21-36, with the target sized for this chip)."""
+    """Partitions per context for the decode kernel (the rule of crates/model/src/
+    paged_attention.rs:21-36 with targets measured on this chip): as many as bring the launch
+    to one workgroup per compute unit, never more than 16 (beyond that the merge costs more
+    than the partitions gain) and at least 256 positions each.  From 32 requests of 8 KV heads
+    on that is one partition, and no merge kernel."""
     pairs = max(1, num_seqs * num_kv_heads * math.ceil(group / 8))
-    return max(1, min(math.ceil(512 / pairs), math.ceil(max_context / 256)))
+    return max(1, min(256 // pairs, 16, math.ceil(max_context / 256)))
 
 
 def _decode_mfma_ok(qkv: torch.Tensor, nh: int, nkv: int, d: int, page_size: int) -> bool:
