@@ -30,7 +30,7 @@ PREFILL_WIDE_MIN_GROUPS = 768
 # afterwards) when its tiles leave compute units without work: as many runs as the units hold
 # at once, with at least this many keys a run (0 units: never).
 PREFILL_SPLIT_UNITS = 256
-PREFILL_SPLIT_MIN_KEYS = 512
+PREFILL_SPLIT_MIN_KEYS = 1024
 # The norm in front of a projection goes into the streaming kernel where that applies.
 FUSE_NORM_LINEAR = True
 # The matrix-core decode attention rotates q and k and stores the new k, v itself where it can.
