@@ -23,8 +23,9 @@ SKINNY_MAX_ROWS = 64
 STREAM_MAX_ROWS = 16
 # Single tokens in a batch that also holds portions of prompts take the decode attention kernel.
 SPLIT_MIXED_ATTENTION = True
-# The prefill attention takes tiles of 128 queries when that makes this many workgroups, or when
-# contexts are long (4096 positions, or 2048 cached ones); 1 << 30: never.
+# The prefill attention takes tiles of 128 queries when that makes this many workgroups (5/3 as
+# many up to head size 64), or when contexts are long (4096 positions, or 2048 cached ones);
+# 1 << 30: never.
 PREFILL_WIDE_MIN_GROUPS = 768
 # The prefill attention cuts the keys of its tiles into runs (one workgroup each, merged
 # afterwards) when its tiles leave compute units without work: as many runs as the units hold
@@ -514,7 +515,9 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
         if wide is not None and d <= 128:
             groups = wide.numel() // 2 * nh
             cached = step.max_context - getattr(step, "max_new", 0)
-            if groups >= PREFILL_WIDE_MIN_GROUPS or (PREFILL_WIDE_MIN_GROUPS < (1 << 30) and (
+            # (measured: up to head size 64 the smaller tiles hold out to 5/3 as many groups)
+            enough = PREFILL_WIDE_MIN_GROUPS if d > 64 else PREFILL_WIDE_MIN_GROUPS * 5 // 3
+            if groups >= enough or (PREFILL_WIDE_MIN_GROUPS < (1 << 30) and (
                     step.max_context >= 4096 or cached >= 2048)):
                 tile_map, num_tiles, tile_queries = wide, wide.numel() // 2, 128
         if num_tiles:
