@@ -97,7 +97,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
     int page_shift, float scale, int window, int num_tiles, int tiles_per_round, int splits,
     int row0, float* __restrict__ part_ml, float* __restrict__ part_acc) {
   constexpr int BN = tile_keys(QB);
-  constexpr int VS = BN + 16;   // V tile row stride
+  // V^T tile rows: 64 keys padded to a stride of 32 bytes mod 64; 32 keys unpadded, with the
+  // 16-byte piece index XORed with (-(row / 4)) & 3, which frees reads and stores of conflicts.
+  constexpr int VS = BN == 32 ? 32 : BN + 16;
   constexpr int kTileBufs = tile_bufs(QB);
   __shared__ __attribute__((aligned(16))) bf16_t Ks_all[kTileBufs * BN * KS];
   __shared__ __attribute__((aligned(16))) bf16_t Vs_all[kTileBufs * D * VS];
@@ -249,7 +251,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
     _Pragma("unroll") for (int i = 0; i < VCH; ++i) {                                          \
       const int c_ = tid + i * 256;                                                            \
       if (V_CHUNKS % 256 == 0 || c_ < V_CHUNKS)                                                \
-        *(u32x4*)(Vs + (c_ / (BN / 8)) * VS + (c_ % (BN / 8)) * 8) = TV[i];                    \
+        *(u32x4*)(Vs + (c_ / (BN / 8)) * VS +                                                  \
+                  ((c_ % (BN / 8)) ^ (BN == 32 ? ((0 - ((c_ / (BN / 8)) >> 2)) & 3) : 0)) * 8) = TV[i]; \
     }                                                                                          \
   }
 
@@ -363,7 +366,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
           // Unconditional, so that reads and products of all blocks can overlap: rows of V^T
           // past d hold whatever LDS held and feed rows of O^T that are never stored.
           Frag8 vf;
-          vf.u = *(const uint4*)(Vs + (db * 16 + l16) * VS + st * 32 + lq * 8);
+          vf.u = *(const uint4*)(Vs + (db * 16 + l16) * VS + st * 32 +
+                                 (lq ^ (BN == 32 ? ((0 - (l16 >> 2)) & 3) : 0)) * 8);
 #pragma unroll
           for (int b = 0; b < QB; ++b)
             o_acc[b][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[b], o_acc[b][db], 0, 0, 0);
