@@ -8,8 +8,11 @@
 // 1/T == 0 marks a greedy row.  The product and the sum are rounded separately (no fused
 // multiply-add), as the host reference computes them.
 #include "common.h"
+#include "no_alloc.h"
 
 #include <math.h>
+
+#include <mutex>
 
 __device__ __forceinline__ uint32_t lowbias32(uint32_t x) {
   x ^= x >> 16;
@@ -137,4 +140,58 @@ RLIS_API int rlis_sample_rows(const float* logits, long long row_stride, int row
   }
   RLIS_LAUNCH_CHECK("sample_rows");
   return 0;
+}
+
+// ------------------------------------------------------------ the variant that allocates nothing
+// The per-chunk winners of rlis_sample_rows_static live here: kStaticMaxParts scores followed
+// by as many indices.  In host code this name is only a stand-in for the device array (each GPU
+// has a copy of its own at an address of its own); what kernels and copies get is the address
+// that hipGetSymbolAddress returns for the current device, kept in g_scratch_ptr.
+constexpr int kStaticMaxParts = 16384;
+constexpr int kStaticMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticMaxParts * (sizeof(float) +
+                                                                            sizeof(int))];
+static void* g_scratch_ptr[kStaticMaxDevices];
+static std::mutex g_scratch_mutex;
+
+// The current device's copy of `scratch`; looked up once per device.
+static int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  RLIS_REQUIRE(e == hipSuccess, "sample_rows_static: hipGetDevice failed: %s",
+               hipGetErrorString(e));
+  RLIS_REQUIRE(dev >= 0 && dev < kStaticMaxDevices,
+               "sample_rows_static: device %d is beyond the %d devices it keeps scratch for", dev,
+               kStaticMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    RLIS_REQUIRE(e == hipSuccess && p,
+                 "sample_rows_static: hipGetSymbolAddress failed on device %d: %s", dev,
+                 hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+RLIS_API int rlis_sample_rows_static_max_parts(void) { return kStaticMaxParts; }
+
+RLIS_API int rlis_sample_rows_static(const float* logits, long long row_stride, int rows, int vocab,
+                                     const uint32_t* keys, const float* inv_temps, int* out,
+                                     int chunks, hipStream_t stream) {
+  RLIS_REQUIRE(rows >= 0 && chunks >= 1, "sample_rows_static: bad sizes");
+  RLIS_REQUIRE((long long)rows * chunks <= kStaticMaxParts,
+               "sample_rows_static: %d rows x %d chunks exceed the %d partial results its static "
+               "scratch holds", rows, chunks, kStaticMaxParts);
+  if (chunks == 1 || rows == 0)
+    return rlis_sample_rows(logits, row_stride, rows, vocab, keys, inv_temps, out, 1, nullptr,
+                            nullptr, stream);
+  void* base = nullptr;
+  if (int rc = static_scratch(&base)) return rc;
+  float* part_best = static_cast<float*>(base);
+  int* part_idx = reinterpret_cast<int*>(part_best + kStaticMaxParts);
+  return rlis_sample_rows(logits, row_stride, rows, vocab, keys, inv_temps, out, chunks, part_best,
+                          part_idx, stream);
 }
