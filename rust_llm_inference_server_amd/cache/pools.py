@@ -1,14 +1,19 @@
 """The device side of the cache: one pool of pages per group and one buffer of fixed-size
 per-request state.
 
-A group's pool holds, for every layer slot of the group, ``num_pages`` pages of keys
-``[page][kv head][offset][d]`` and of values ``[page][kv head][d][offset]`` (values transposed
-inside a page, so that both attention kernels read each as it lies).  One page id addresses
-the same page in every layer slot of its group, as one block id addresses every layer in the
-reference (crates/model/src/paged.rs:1-7, 41-60).  Pools are allocated once, zeroed."""
+A group's pool holds, for every layer slot of the group and for every array its cache request
+names, ``num_pages`` pages of that array's page shape.  The attention kind keeps keys
+``[page][kv head][offset][d]`` and values ``[page][kv head][d][offset]`` (values transposed
+inside a page, so that both attention kernels read each as it lies); another mixer names its
+own arrays and gets them the same way.  One page id addresses the same page in every layer
+slot of its group, as one block id addresses every layer in the reference
+(crates/model/src/paged.rs:1-7, 41-60).  Pools are allocated once, zeroed.
+
+One page beyond the manager's is scratch, and one state slot beyond the manager's: padding
+rows of a captured decode step read and write them, so they touch nothing a request owns."""
 from __future__ import annotations
 
-from typing import List, Optional, Sequence
+from typing import Dict, List, Optional, Sequence
 
 import torch
 
@@ -21,45 +26,52 @@ class CachePools:
                  state_bytes: int = 0):
         self.page_size = page_size
         self.dtype = dtype
-        self.k: List[torch.Tensor] = []
-        self.v: List[torch.Tensor] = []
-        # One page beyond the manager's is scratch: padding rows of a captured decode step
-        # read and write it, so they touch nothing a request owns.
+        self.device = device
+        # Per group: array name -> (layer slots, pages + 1, *page shape).
+        self.arrays: List[Dict[str, torch.Tensor]] = []
         self.scratch_page = max(num_pages) if len(num_pages) else 0
         for layout, pages in zip(cache_groups, num_pages):
-            r, n = layout.request, max(1, len(layout.writer_runs))
+            n = max(1, len(layout.writer_runs))
             total = self.scratch_page + 1
-            self.k.append(torch.zeros((n, total, r.num_kv_heads, page_size, r.head_dim),
-                                      dtype=dtype, device=device))
-            self.v.append(torch.zeros((n, total, r.num_kv_heads, r.head_dim, page_size),
-                                      dtype=dtype, device=device))
+            self.arrays.append({
+                a.name: torch.zeros((n, total) + a.page_shape(page_size), dtype=dtype,
+                                    device=device)
+                for a in layout.request.arrays})
         self.state: Optional[torch.Tensor] = None
+        self.scratch_state_slot = num_state_slots
         if state_bytes > 0 and num_state_slots > 0:
-            self.state = torch.zeros((num_state_slots, state_bytes), dtype=torch.uint8,
+            self.state = torch.zeros((num_state_slots + 1, state_bytes), dtype=torch.uint8,
                                      device=device)
 
     def binding(self, rb) -> CacheBinding:
         b = CacheBinding(group=rb.group, writes=rb.writes)
         if rb.group >= 0:
-            b.k_pages = self.k[rb.group][rb.slot]
-            b.v_pages = self.v[rb.group][rb.slot]
+            b.pages = {name: t[rb.slot] for name, t in self.arrays[rb.group].items()}
         if rb.state_bytes and self.state is not None:
             b.state = self.state[:, rb.state_offset:rb.state_offset + rb.state_bytes]
         return b
 
     def copy_pages(self, group: int, src: Sequence[int], dst: Sequence[int]) -> None:
-        """Copy-on-write copies, in every layer slot of the group."""
+        """Copy-on-write copies, in every layer slot and array of the group."""
         from .. import ops
-        dev = self.k[group].device
-        s = torch.tensor(list(src), dtype=torch.int32, device=dev)
-        d = torch.tensor(list(dst), dtype=torch.int32, device=dev)
-        ops.copy_pages(self.k[group], s, d)
-        ops.copy_pages(self.v[group], s, d)
+        s = torch.tensor(list(src), dtype=torch.int32, device=self.device)
+        d = torch.tensor(list(dst), dtype=torch.int32, device=self.device)
+        for t in self.arrays[group].values():
+            ops.copy_pages(t, s, d)
 
     def zero_state(self, slot: int) -> None:
         if self.state is not None:
             self.state[slot].zero_()
 
+    def zero_states(self, slots: Sequence[int]) -> None:
+        """Clear the state of several requests at once (those that start at position 0)."""
+        if self.state is not None and len(slots):
+            self.state[torch.tensor(list(slots), dtype=torch.long, device=self.device)] = 0
+
+    def copy_state(self, src: int, dst: int) -> None:
+        if self.state is not None:
+            self.state[dst].copy_(self.state[src])
+
     def bytes_per_page(self, group: int) -> int:
-        k = self.k[group]
-        return 2 * k.shape[0] * k[0, 0].numel() * k.element_size()
+        return sum(t.shape[0] * t[0, 0].numel() * t.element_size()
+                   for t in self.arrays[group].values())

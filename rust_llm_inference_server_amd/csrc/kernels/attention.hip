@@ -147,7 +147,10 @@ template <> struct Vec16<bf16_t> {
 // Grid (kv head * head chunks, sequence, split); 256 threads.  Head chunk c serves query
 // heads kvh * g + c * G + [0, G) (those beyond the group are computed on a clamped head and
 // dropped).  Partition `split` of a sequence with n visible keys covers
-// [lo + split * part, lo + (split + 1) * part) with part = ceil(n / splits) rounded up to 64.
+// [lo + split * part, lo + (split + 1) * part) with part = decode_part_len(n, part_keys,
+// max_parts): a function of the sequence's own length.  `splits` is the grid's depth and the
+// stride of the partial results, at least the live partitions of the longest sequence;
+// partitions beyond a sequence's own store an empty result (l = 0), which the merge skips.
 // Output per (sequence, head, split): m, l and the unnormalised accumulator (d floats); with
 // splits == 1 the normalised result goes straight to `out`.
 template <typename TX, int G, int DPL>
@@ -156,7 +159,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     float* __restrict__ part_ml, float* __restrict__ part_acc, const TX* __restrict__ k_pages,
     const TX* __restrict__ v_pages, const int* __restrict__ block_tables, int max_pages,
     const int* __restrict__ ctx_lens, const int* __restrict__ token_rows, int nh, int nkv, int d,
-    int page_size, float scale, int window, int splits, int chunks_per_kv) {
+    int page_size, float scale, int window, int splits, int chunks_per_kv, int part_keys,
+    int max_parts) {
   extern __shared__ float smem[];
   float* q_s = smem;                     // G * d
   float* p_s = q_s + G * d;              // 4 waves * G * 64
@@ -174,8 +178,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int* table = block_tables + (long long)seq * max_pages;
   const int lo = (window > 0 && ctx - window > 0) ? ctx - window : 0;
   const int nkeys = ctx - lo;
-  int part = (nkeys + splits - 1) / splits;
-  part = ((part + 63) / 64) * 64;
+  const int part = decode_part_len(nkeys, part_keys, max_parts);
   const int kbeg = lo + split * part;
   const int kend = min(ctx, kbeg + part);
 
@@ -313,7 +316,11 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   }
 }
 
-// Grid (query head, sequence); merges the partitions of one head.  A thread owns output dims
+// Grid (query head, row); merges the partitions of one head of one output row.  The row's
+// sequence is seq_of_row[row0 + row] (the row itself without that table) and the number of its
+// live partitions seq_parts[sequence] (`splits`, the stride of the partial results, without
+// that table); a row with one partition or none was stored by its kernel already and is left
+// alone.  A thread owns output dims
 // j, j + blockDim, ...; the first kReduceAhead partitions' sums for its first dim are loaded
 // together with the maxima, before the weights exp(m_s - max m) are known, so that the whole
 // merge waits for memory once.  The weights go through LDS (`splits` floats); sums run over s
@@ -324,12 +331,19 @@ template <typename TX>
 __global__ void attn_reduce_kernel(TX* __restrict__ out, long long out_stride,
                                    const float* __restrict__ part_ml,
                                    const float* __restrict__ part_acc,
-                                   const int* __restrict__ token_rows, int nh, int d, int splits) {
-  extern __shared__ float reduce_w[];            // splits weights, then 8 floats of scratch
-  float* scratch = reduce_w + splits;
+                                   const int* __restrict__ token_rows, int nh, int d, int stride,
+                                   const int* __restrict__ seq_of_row,
+                                   const int* __restrict__ seq_parts, int row0) {
+  extern __shared__ float reduce_w[];            // stride weights, then 8 floats of scratch
+  float* scratch = reduce_w + stride;
   const int h = blockIdx.x, seq = blockIdx.y;
-  const int row = token_rows ? token_rows[seq] : seq;
-  const long long base = ((long long)seq * nh + h) * splits;
+  const int row = token_rows ? token_rows[seq] : seq + row0;
+  int splits = stride;
+  if (seq_parts) {
+    splits = min(stride, seq_parts[seq_of_row ? seq_of_row[row] : row]);
+    if (splits <= 1) return;
+  }
+  const long long base = ((long long)seq * nh + h) * stride;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, nwaves = blockDim.x / kWave;
   const int j0 = (int)threadIdx.x < d ? (int)threadIdx.x : 0;
   const float* acc0 = part_acc + base * d + j0;
@@ -383,8 +397,34 @@ int rlis_launch_attn_reduce_bf16(void* out, long long out_stride, const float* p
   dim3 grid(nh, S);
   const int threads = d <= 64 ? 64 : (d <= 128 ? 128 : 256);
   attn_reduce_kernel<bf16_t><<<grid, threads, (splits + 8) * sizeof(float), stream>>>(
-      (bf16_t*)out, out_stride, part_ml, part_acc, nullptr, nh, d, splits);
+      (bf16_t*)out, out_stride, part_ml, part_acc, nullptr, nh, d, splits, nullptr, nullptr, 0);
   RLIS_LAUNCH_CHECK("attn_reduce");
+  return 0;
+}
+
+// Merges the key runs of the matrix-core prefill kernel: `rows` output rows from row0 on, whose
+// partial results lie at part_ml (rows, nh, stride, 2) and part_acc (rows, nh, stride, d);
+// row r belongs to sequence seq_of_token[row0 + r], which has seq_runs[sequence] runs (rows
+// of sequences with a single run are already stored and stay untouched).
+RLIS_API int rlis_attn_reduce_rows(void* out, long long out_stride, const float* part_ml,
+                                   const float* part_acc, const int* seq_of_token,
+                                   const int* seq_runs, int row0, int rows, int nh, int d,
+                                   int stride, hipStream_t stream) {
+  RLIS_REQUIRE(rows >= 0 && row0 >= 0 && nh > 0 && d > 0 && stride >= 1 && stride <= 64,
+               "attn_reduce_rows: bad sizes");
+  RLIS_REQUIRE(part_ml && part_acc && seq_of_token && seq_runs,
+               "attn_reduce_rows: partial results and the run counts are needed");
+  RLIS_REQUIRE(rows <= 65535 * 32, "attn_reduce_rows: %d rows are too many", rows);
+  const int threads = d <= 64 ? 64 : (d <= 128 ? 128 : 256);
+  for (int r = 0; r < rows; r += 65535) {
+    const int n = min(65535, rows - r);
+    dim3 grid(nh, n);
+    attn_reduce_kernel<bf16_t><<<grid, threads, (stride + 8) * sizeof(float), stream>>>(
+        (bf16_t*)out, out_stride, part_ml + (long long)r * nh * stride * 2,
+        part_acc + (long long)r * nh * stride * d, nullptr, nh, d, stride, seq_of_token, seq_runs,
+        row0 + r);
+  }
+  RLIS_LAUNCH_CHECK("attn_reduce_rows");
   return 0;
 }
 
@@ -393,7 +433,8 @@ static int launch_decode(const void* q, long long q_stride, void* out, long long
                          float* part_ml, float* part_acc, const void* k_pages,
                          const void* v_pages, const int* block_tables, int max_pages,
                          const int* ctx_lens, const int* token_rows, int S, int nh, int nkv, int d,
-                         int page_size, float scale, int window, int splits, hipStream_t stream) {
+                         int page_size, float scale, int window, int splits, int part_keys,
+                         int max_parts, hipStream_t stream) {
   const int g = nh / nkv;
   const int chunks = ceil_div(g, G);
   dim3 grid(nkv * chunks, S, splits);
@@ -405,7 +446,7 @@ static int launch_decode(const void* q, long long q_stride, void* out, long long
   attn_decode_kernel<TX, G, DPL><<<grid, 256, smem, stream>>>(                                 \
       (const TX*)q, q_stride, (TX*)out, out_stride, part_ml, part_acc, (const TX*)k_pages,     \
       (const TX*)v_pages, block_tables, max_pages, ctx_lens, token_rows, nh, nkv, d, page_size, \
-      scale, window, splits, chunks)
+      scale, window, splits, chunks, part_keys, max_parts)
   if (dpl <= 1) LAUNCH(1);
   else if (dpl <= 2) LAUNCH(2);
   else LAUNCH(4);
@@ -414,15 +455,20 @@ static int launch_decode(const void* q, long long q_stride, void* out, long long
 }
 
 // q rows are token_rows[seq] (or seq when null) of a (T, q_stride) matrix, out likewise.
-// part_ml (S, nh, splits, 2) and part_acc (S, nh, splits, d) float32 are needed when
-// splits > 1.
+// A sequence's visible keys are cut into partitions of decode_part_len(keys, part_keys,
+// max_parts); `splits` must be at least the live partitions of the longest context (at most
+// max_parts).  part_ml (S, nh, splits, 2) and part_acc (S, nh, splits, d) float32 are needed
+// when splits > 1.
 RLIS_API int rlis_attn_decode(const void* q, int dtype, long long q_stride, void* out,
                               long long out_stride, float* part_ml, float* part_acc,
                               const void* k_pages, const void* v_pages, const int* block_tables,
                               int max_pages, const int* ctx_lens, const int* token_rows, int S,
                               int nh, int nkv, int d, int page_size, float scale, int window,
-                              int splits, hipStream_t stream) {
+                              int splits, int part_keys, int max_parts, hipStream_t stream) {
   RLIS_REQUIRE(S >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0, "attn_decode: bad sizes");
+  RLIS_REQUIRE(part_keys >= 64 && part_keys % 64 == 0 && max_parts >= 1 && splits <= max_parts,
+               "attn_decode: partitions of %d keys (a multiple of 64), %d deep of at most %d",
+               part_keys, splits, max_parts);
   RLIS_REQUIRE(nh % nkv == 0, "attn_decode: %d query heads are not a multiple of %d KV heads",
                nh, nkv);
   RLIS_REQUIRE(d <= 256, "attn_decode: head_dim %d is above the limit of 256", d);
@@ -437,19 +483,23 @@ RLIS_API int rlis_attn_decode(const void* q, int dtype, long long q_stride, void
     if (g == 1)                                                                                  \
       rc = launch_decode<TX, 1>(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,        \
                                 v_pages, block_tables, max_pages, ctx_lens, token_rows, S, nh,   \
-                                nkv, d, page_size, scale, window, splits, stream);               \
+                                nkv, d, page_size, scale, window, splits, part_keys, max_parts,       \
+                                stream);               \
     else if (g == 2)                                                                             \
       rc = launch_decode<TX, 2>(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,        \
                                 v_pages, block_tables, max_pages, ctx_lens, token_rows, S, nh,   \
-                                nkv, d, page_size, scale, window, splits, stream);               \
+                                nkv, d, page_size, scale, window, splits, part_keys, max_parts,       \
+                                stream);               \
     else if (g <= 4)                                                                             \
       rc = launch_decode<TX, 4>(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,        \
                                 v_pages, block_tables, max_pages, ctx_lens, token_rows, S, nh,   \
-                                nkv, d, page_size, scale, window, splits, stream);               \
+                                nkv, d, page_size, scale, window, splits, part_keys, max_parts,       \
+                                stream);               \
     else                                                                                         \
       rc = launch_decode<TX, 8>(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,        \
                                 v_pages, block_tables, max_pages, ctx_lens, token_rows, S, nh,   \
-                                nkv, d, page_size, scale, window, splits, stream);               \
+                                nkv, d, page_size, scale, window, splits, part_keys, max_parts,       \
+                                stream);               \
   } while (0)
   if (dtype == RLIS_F32) BY_G(float);
   else if (dtype == RLIS_BF16) BY_G(bf16_t);
@@ -462,10 +512,12 @@ RLIS_API int rlis_attn_decode(const void* q, int dtype, long long q_stride, void
     const int threads = d <= 64 ? 64 : (d <= 128 ? 128 : 256);
     if (dtype == RLIS_F32)
       attn_reduce_kernel<float><<<grid, threads, (splits + 8) * sizeof(float), stream>>>(
-          (float*)out, out_stride, part_ml, part_acc, token_rows, nh, d, splits);
+          (float*)out, out_stride, part_ml, part_acc, token_rows, nh, d, splits, nullptr, nullptr,
+          0);
     else
       attn_reduce_kernel<bf16_t><<<grid, threads, (splits + 8) * sizeof(float), stream>>>(
-          (bf16_t*)out, out_stride, part_ml, part_acc, token_rows, nh, d, splits);
+          (bf16_t*)out, out_stride, part_ml, part_acc, token_rows, nh, d, splits, nullptr, nullptr,
+          0);
     RLIS_LAUNCH_CHECK("attn_reduce");
   }
   return 0;

@@ -13,8 +13,8 @@ typedef int (*DecodeUnit)(const void* q, long long q_stride, void* out, long lon
                           float* part_ml, float* part_acc, const void* k_pages,
                           const void* v_pages, const int* block_tables, int max_pages,
                           const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift,
-                          int window, float scale, int splits, const DecodeRope* rope,
-                          hipStream_t stream);
+                          int window, float scale, int splits, int part_keys, int max_parts,
+                          const DecodeRope* rope, hipStream_t stream);
 
 // The units (attention_mfma.hip compiled for a padded head size of 32, 64, ... 256) are
 // libraries of their own, built and loaded when a model needs them and registered here.
@@ -40,6 +40,8 @@ static int unit_result(const char* name, int rc, int d) {
   else if (rc == 2)
     rlis_set_error("%s: rotation inside the kernel needs head_dim = rotated width = 64, 128 or "
                    "256 (got %d)", name, d);
+  else if (rc == 3)
+    rlis_set_error("%s: partitions must be a multiple of 256 keys", name);
   else if (rc >= 1000)
     rlis_set_error("%s: launch failed: %s", name, hipGetErrorString((hipError_t)(rc - 1000)));
   else rlis_set_error("%s: unit error %d", name, rc);
@@ -50,27 +52,29 @@ int rlis_launch_attn_reduce_bf16(void* out, long long out_stride, const float* p
                                  const float* part_acc, int S, int nh, int d, int splits,
                                  hipStream_t stream);
 
-// splits > 1: the keys of every tile are cut into that many runs, one workgroup each, whose
-// partial results go to part_ml (rows, nh, splits, 2) and part_acc (rows, nh, splits, d)
-// float32 and are merged afterwards; `rows` output rows from row0 on are those that the tiles
-// cover (all of them: a row that no tile covers would be merged from nothing).
+// unit_map lists num_units quadruples (sequence, first new-token index of a tile, run, runs of
+// the sequence): the keys of a tile of a sequence with more than one run are cut into that
+// many runs, one workgroup each, whose partial results go to part_ml (rows, nh, part_stride, 2)
+// and part_acc (rows, nh, part_stride, d) float32, indexed by the row relative to row0, and are
+// merged afterwards by rlis_attn_reduce_rows.  part_stride is at least the largest run count
+// (1: no sequence has runs, nothing is stored there).
 RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out,
                                     long long out_stride, const void* k_pages,
                                     const void* v_pages, const int* block_tables, int max_pages,
                                     const int* cu_seqlens, const int* start_pos,
-                                    const int* tile_map, int num_tiles, int nh, int nkv, int d,
+                                    const int* unit_map, int num_tiles, int nh, int nkv, int d,
                                     int page_size, int window, float scale, int tile_queries,
-                                    int splits, int row0, int rows, float* part_ml,
+                                    int splits, int row0, float* part_ml,
                                     float* part_acc, hipStream_t stream) {
-  // tile_map lists tiles of tile_queries new tokens: 64 (0 means that too) or 128.
+  // unit_map lists tiles of tile_queries new tokens: 64 (0 means that too) or 128.
   if (tile_queries == 0) tile_queries = 64;
   RLIS_REQUIRE(tile_queries == 64 || tile_queries == 128,
                "attn_prefill_mfma: tiles of %d queries, 64 or 128 only", tile_queries);
   RLIS_REQUIRE(num_tiles >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0,
                "attn_prefill_mfma: bad sizes");
   RLIS_REQUIRE(splits >= 1 && splits <= 64, "attn_prefill_mfma: %d key runs, 1 to 64", splits);
-  RLIS_REQUIRE(splits == 1 || (part_ml && part_acc && row0 >= 0 && rows > 0 && d % 4 == 0),
-               "attn_prefill_mfma: key runs need a workspace and the range of rows they cover");
+  RLIS_REQUIRE(splits == 1 || (part_ml && part_acc && row0 >= 0 && d % 4 == 0),
+               "attn_prefill_mfma: key runs need a workspace and the first row they cover");
   RLIS_REQUIRE(scale > 0.f, "attn_prefill_mfma: the score scale must be positive, got %g", scale);
   RLIS_REQUIRE(nh % nkv == 0, "attn_prefill_mfma: %d query heads are not a multiple of %d KV heads",
                nh, nkv);
@@ -85,22 +89,19 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
                "attn_prefill_mfma: operands must be 16-byte aligned with row strides in steps of 8");
   const PrefillUnit unit = prefill_units[unit_index(d)];
   RLIS_REQUIRE(unit != nullptr, "attn_prefill_mfma: the unit for head size %d is not loaded", d);
-  const int rc = unit_result(
+  return unit_result(
       "attn_prefill_mfma",
       unit(q, q_stride, out, out_stride, k_pages, v_pages, block_tables, max_pages, cu_seqlens,
-           start_pos, tile_map, num_tiles, nh, nkv, d, page_shift, window, scale, tile_queries,
+           start_pos, unit_map, num_tiles, nh, nkv, d, page_shift, window, scale, tile_queries,
            splits, row0, part_ml, part_acc, stream),
       d);
-  if (rc) return rc;
-  if (splits > 1 && num_tiles > 0)
-    return rlis_launch_attn_reduce_bf16((bf16_t*)out + (long long)row0 * out_stride, out_stride,
-                                        part_ml, part_acc, rows, nh, d, splits, stream);
-  return 0;
 }
 
 // One query token per sequence (bfloat16): q rows are the sequences themselves.  Needs at most
-// 16 query heads per KV head; part_ml (S, nh, splits, 2) and part_acc (S, nh, splits, d) float32
-// when splits > 1.
+// 16 query heads per KV head.  A sequence's visible keys are cut into partitions of
+// decode_part_len(keys, part_keys, max_parts); `splits` must be at least the live partitions of
+// the longest context (at most max_parts); part_ml (S, nh, splits, 2) and part_acc
+// (S, nh, splits, d) float32 when splits > 1.
 //
 // positions == null: q is rotated and the pages hold the step's keys and values already.
 // Otherwise the kernel does that itself: q rows hold the k heads at column k_off and the v
@@ -112,7 +113,8 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
                                    void* k_pages, void* v_pages,
                                    const int* block_tables, int max_pages, const int* ctx_lens,
                                    int S, int nh, int nkv, int d, int page_size, int window,
-                                   float scale, int splits, const float* cos, const float* sin,
+                                   float scale, int splits, int part_keys, int max_parts,
+                                   const float* cos, const float* sin,
                                    int rot, const int* positions, const int* slots,
                                    long long k_off, long long v_off, hipStream_t stream) {
   DecodeRope rope;
@@ -147,6 +149,8 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
                "attn_decode_mfma: operands must be 16-byte aligned with row strides in steps of 8");
   RLIS_REQUIRE(splits >= 1 && splits <= 8192 && S <= 65535, "attn_decode_mfma: bad grid");
   RLIS_REQUIRE(splits == 1 || (part_ml && part_acc), "attn_decode_mfma: partitions need a workspace");
+  RLIS_REQUIRE(max_parts >= 1 && splits <= max_parts && part_keys > 0,
+               "attn_decode_mfma: %d partitions deep, at most %d", splits, max_parts);
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;
   const DecodeUnit unit = decode_units[unit_index(d)];
@@ -154,7 +158,8 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
   const int rc = unit_result(
       "attn_decode_mfma",
       unit(q, q_stride, out, out_stride, part_ml, part_acc, k_pages, v_pages, block_tables,
-           max_pages, ctx_lens, S, nh, nkv, d, page_shift, window, scale, splits, &rope, stream),
+           max_pages, ctx_lens, S, nh, nkv, d, page_shift, window, scale, splits, part_keys,
+           max_parts, &rope, stream),
       d);
   if (rc) return rc;
   if (splits > 1 && S > 0)

@@ -50,6 +50,7 @@ union Frag8 {
 // return codes (kUnit...), which the dispatcher turns into messages.
 constexpr int kUnitTooManyTiles = 1;
 constexpr int kUnitBadRotation = 2;
+constexpr int kUnitBadPartition = 3;
 constexpr int kUnitLaunchFailed = 1000;       // + the hipError_t
 #define RLIS_UNIT_LAUNCH_CHECK()                                 \
   do {                                                           \
@@ -93,8 +94,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
     const bf16_t* __restrict__ q, long long q_stride, bf16_t* __restrict__ out,
     long long out_stride, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_seqlens,
-    const int* __restrict__ start_pos, const int* __restrict__ tile_map, int nh, int nkv, int d,
-    int page_shift, float scale, int window, int num_tiles, int tiles_per_round, int splits,
+    const int* __restrict__ start_pos, const int* __restrict__ unit_map, int nh, int nkv, int d,
+    int page_shift, float scale, int window, int num_tiles, int tiles_per_round, int part_stride,
     int row0, float* __restrict__ part_ml, float* __restrict__ part_acc) {
   constexpr int BN = tile_keys(QB);
   // V^T tile rows: 64 keys padded to a stride of 32 bytes mod 64; 32 keys unpadded, with the
@@ -106,23 +107,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
 
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int l16 = lane % 16, lq = lane / 16;
-  // Blocks are numbered heads-fastest over the tiles, which arrive sorted by falling work.
-  // One round of blocks (tiles_per_round tiles x all heads) fills the compute units once; every
-  // other round walks its tiles backwards, so that a unit that drew a long tile in one round
-  // draws a short one in the next.
-  // With `splits` > 1 the keys of a tile are cut into that many runs of whole key tiles, one
-  // workgroup each (splits fastest after the heads): few tiles with long walks over cached
-  // keys then still fill the chip.  Such workgroups store unnormalised sums with their maximum
-  // and denominator, which attn_reduce (attention.hip) merges.
+  // Blocks are numbered heads-fastest over the units of work, which arrive sorted by falling
+  // work.  One round of blocks (tiles_per_round units x all heads) fills the compute units once;
+  // every other round walks its units backwards, so that a compute unit that drew a long one in
+  // one round draws a short one in the next.
+  // A unit is (sequence, first new-token index of the tile, run, runs of this sequence): with
+  // more than one run the keys of a tile are cut into that many runs of whole key tiles, one
+  // workgroup each, so that few tiles with long walks over cached keys still fill the chip.
+  // Such workgroups store unnormalised sums with their maximum and denominator, which
+  // attn_reduce (attention.hip) merges.  How many runs a sequence has is decided from its own
+  // lengths, never from what else is in the batch.
   const int h = blockIdx.x % nh;
-  const int split = (blockIdx.x / nh) % splits;
-  int tile = blockIdx.x / nh / splits;
+  int tile = blockIdx.x / nh;
   if (tiles_per_round > 0) {
     const int round = tile / tiles_per_round, within = tile % tiles_per_round;
     const bool whole = (round + 1) * tiles_per_round <= num_tiles;
     if ((round & 1) && whole) tile = round * tiles_per_round + (tiles_per_round - 1 - within);
   }
-  const int seq = tile_map[2 * tile], qb = tile_map[2 * tile + 1];
+  const int seq = unit_map[4 * tile], qb = unit_map[4 * tile + 1];
+  const int split = unit_map[4 * tile + 2], splits = unit_map[4 * tile + 3];
   const int tok_begin = cu_seqlens[seq];
   const int n_new = cu_seqlens[seq + 1] - tok_begin;
   const int P = start_pos[seq];
@@ -430,7 +433,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
           }
         }
       } else {
-        const long long idx = ((row - row0) * nh + h) * splits + split;
+        const long long idx = ((row - row0) * nh + h) * part_stride + split;
         float* arow = part_acc + idx * d;
 #pragma unroll
         for (int db = 0; db < D / 16; ++db) {
@@ -450,8 +453,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
   }
 }
 
-// tile_map holds num_tiles pairs (sequence, first new-token index of a tile of tile_queries =
-// 64 or 128 tokens), sorted by falling number of keys the tile walks.
+// unit_map holds num_units quadruples (sequence, first new-token index of a tile of
+// tile_queries = 64 or 128 tokens, run, runs of the sequence), sorted by falling number of keys
+// the unit walks.  Units of sequences with more than one run store partial results, part_stride
+// of them per (row, head), from row0 on.
 RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
     const void* q, long long q_stride, void* out, long long out_stride, const void* k_pages,
     const void* v_pages, const int* block_tables, int max_pages, const int* cu_seqlens,
@@ -459,10 +464,10 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
     int page_shift, int window, float scale, int tile_queries, int splits, int row0,
     float* part_ml, float* part_acc, hipStream_t stream) {
   if (num_tiles == 0) return 0;
-  const long long blocks = (long long)num_tiles * nh * splits;
+  const long long blocks = (long long)num_tiles * nh;
   if (blocks >= (1ll << 31)) return kUnitTooManyTiles;
-  // 256 compute units: a round is the tiles whose blocks fill them once.
-  const int tiles_per_round = (splits == 1 && nh <= 256 && 256 % nh == 0) ? 256 / nh : 0;
+  // 256 compute units: a round is the units whose blocks fill them once.
+  const int tiles_per_round = (nh <= 256 && 256 % nh == 0) ? 256 / nh : 0;
   if (tile_queries == 2 * BM)
     KERNEL_NAME<2><<<(int)blocks, 256, 0, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,
@@ -489,8 +494,12 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
 //
 // Partitions are laid over key positions aligned to 32: with lo the first visible key and
 // lo32 = lo rounded down to 32, partition s covers [lo32 + s * part, lo32 + (s + 1) * part)
-// cut to [lo, ctx), part = ceil((ctx - lo32) / splits) rounded up to 256.  Page ids of a chunk
-// are fetched one chunk ahead of its keys and values, which are fetched one chunk ahead of use.
+// cut to [lo, ctx), part = decode_part_len(ctx - lo32, part_keys, max_parts): a function of the
+// sequence's own length and of constants, so that a sequence is cut the same way whatever else
+// is in the batch.  `splits` is the grid's depth and the stride of the partial results, at
+// least the live partitions of the longest sequence; partitions beyond a sequence's own store an
+// empty result.  Page ids of a chunk are fetched one chunk ahead of its keys and values, which
+// are fetched one chunk ahead of use.
 //
 // With rope.positions the kernel also does what rope_kv_write does for the step's own tokens
 // (crates/model/src/llama.rs:205-222): every workgroup rotates its queries in registers
@@ -513,8 +522,8 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
     long long out_stride, float* __restrict__ part_ml, float* __restrict__ part_acc,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ ctx_lens,
-    int nh, int nkv, int d, int page_shift, float scale, int window, int splits,
-    const DecodeRope rope) {
+    int nh, int nkv, int d, int page_shift, float scale, int window, int splits, int part_keys,
+    int max_parts, const DecodeRope rope) {
   extern __shared__ float dsm[];           // ml: waves * g * 2 ; acc: waves * g * d
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int l16 = lane % 16, lq = lane / 16;
@@ -525,9 +534,8 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
   const int page_mask = (1 << page_shift) - 1;
   const int lo = (window > 0 && ctx - window > 0) ? ctx - window : 0;
   const int lo32 = lo & ~31;
-  int part = (ctx - lo32 + splits - 1) / splits;
   constexpr int kStride = 32 * kDecodeWaves;       // keys between two chunks of one wave
-  part = ((part + kStride - 1) / kStride) * kStride;
+  const int part = decode_part_len(ctx - lo32, part_keys, max_parts);   // a multiple of kStride
   const int kbeg = lo32 + split * part;
   const int kend = min(ctx, kbeg + part);
 
@@ -763,8 +771,10 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
     const void* q, long long q_stride, void* out, long long out_stride, float* part_ml,
     float* part_acc, const void* k_pages, const void* v_pages, const int* block_tables,
     int max_pages, const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift, int window,
-    float scale, int splits, const DecodeRope* rope, hipStream_t stream) {
+    float scale, int splits, int part_keys, int max_parts, const DecodeRope* rope,
+    hipStream_t stream) {
   if (S == 0) return 0;
+  if (part_keys % (32 * kDecodeWaves) != 0 || part_keys <= 0) return kUnitBadPartition;
   // rotation inside the kernel needs head_dim = rotated width = 64, 128 or 256
   if (rope->positions && rope->cos && !(D % 64 == 0 && rope->rot == D && d == D))
     return kUnitBadRotation;
@@ -774,7 +784,7 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
   DECODE_KERNEL_NAME<<<grid, 64 * kDecodeWaves, smem, stream>>>(
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, part_ml, part_acc,
       (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, max_pages, ctx_lens, nh, nkv, d,
-      page_shift, scale, window, splits, *rope);
+      page_shift, scale, window, splits, part_keys, max_parts, *rope);
   RLIS_UNIT_LAUNCH_CHECK();
   return 0;
 }

@@ -33,6 +33,18 @@ __device__ __forceinline__ float ld(const bf16_t* p) { return bf16_to_f32(*p); }
 __device__ __forceinline__ void st(float* p, float v) { *p = v; }
 __device__ __forceinline__ void st(bf16_t* p, float v) { *p = f32_to_bf16(v); }
 
+// A delta for the residual stream that arrives as `parts` float32 partial sums, part_stride
+// elements apart: they are added in order and, with round16, the sum is rounded to bfloat16 as
+// a delta that arrives whole in bfloat16 was, so that a block's output is rounded once to the
+// activation dtype whichever kernel produced it.
+template <typename TD>
+__device__ __forceinline__ float delta_sum(const TD* d, int parts, long long part_stride,
+                                           int round16) {
+  float s = ld(d);
+  for (int p = 1; p < parts; ++p) s += ld(d + p * part_stride);
+  return round16 ? bf16_to_f32(f32_to_bf16(s)) : s;
+}
+
 // Sum and maximum of a value with its partner 16 or 32 lanes away (lane ^ 16, lane ^ 32): every
 // lane gets the result.  gfx950 swaps 16- and 32-lane halves of two registers in the vector
 // unit (v_permlane16_swap: odd rows of the first with even rows of the second;
@@ -118,6 +130,16 @@ struct DecodeRope {
   long long k_off, v_off;
   int rot;                // rotated width of a head
 };
+
+// Keys per partition of a decode context of n visible keys: part_keys up to max_parts
+// partitions, then the multiple of part_keys that keeps them at max_parts.  It depends on the
+// sequence's own length and on constants only, so a sequence is cut (and its partitions are
+// merged) the same way whatever else is in the batch; ceil(n / length) partitions are live.
+__host__ __device__ inline int decode_part_len(int n, int part_keys, int max_parts) {
+  const int span = part_keys * max_parts;
+  const int mult = (n + span - 1) / span;
+  return part_keys * (mult < 1 ? 1 : mult);
+}
 
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 static inline long long ceil_div_ll(long long a, long long b) { return (a + b - 1) / b; }

@@ -48,28 +48,28 @@ RLIS_API int rlis_embed(float* out, const void* table, int table_dtype, const in
 
 // ------------------------------------------------------------------- residual add
 // delta may come as `parts` partial sums of n elements each, one after the other; they are
-// added in order.
+// added in order (and their sum rounded to bfloat16 first when round_parts is set).
 template <typename TD>
 __global__ void add_residual_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
-                                    long long n, int parts) {
+                                    long long n, int parts, int round_parts) {
   long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   const long long stride = (long long)gridDim.x * blockDim.x;
   for (; i < n; i += stride) {
-    float v = resid[i];
-    for (int s = 0; s < parts; ++s) v += ld(delta + s * n + i);
-    resid[i] = v;
+    resid[i] += delta_sum(delta + i, parts, n, round_parts);
   }
 }
 
 RLIS_API int rlis_add_residual(float* resid, const void* delta, int delta_dtype, long long n,
-                               int parts, hipStream_t stream) {
+                               int parts, int round_parts, hipStream_t stream) {
   RLIS_REQUIRE(parts >= 1, "add_residual: parts=%d", parts);
   if (n <= 0) return 0;
   const int blocks = (int)(ceil_div_ll(n, 256) < 4096 ? ceil_div_ll(n, 256) : 4096);
   if (delta_dtype == RLIS_F32)
-    add_residual_kernel<float><<<blocks, 256, 0, stream>>>(resid, (const float*)delta, n, parts);
+    add_residual_kernel<float><<<blocks, 256, 0, stream>>>(resid, (const float*)delta, n, parts,
+                                                           round_parts);
   else if (delta_dtype == RLIS_BF16)
-    add_residual_kernel<bf16_t><<<blocks, 256, 0, stream>>>(resid, (const bf16_t*)delta, n, parts);
+    add_residual_kernel<bf16_t><<<blocks, 256, 0, stream>>>(resid, (const bf16_t*)delta, n, parts,
+                                                            round_parts);
   else
     RLIS_REQUIRE(false, "add_residual: unknown dtype %d", delta_dtype);
   RLIS_LAUNCH_CHECK("add_residual");
@@ -79,13 +79,15 @@ RLIS_API int rlis_add_residual(float* resid, const void* delta, int delta_dtype,
 // ------------------------------------------------------- residual add + RMSNorm
 // One block per output row r; the source row is rows[r] when rows is given.  The residual is
 // float32; delta (may be null) is added first and, when write_resid is set, the sum is stored
-// back.  delta may come as `parts` partial sums, part_stride elements apart, added in order.
+// back.  delta may come as `parts` partial sums, part_stride elements apart, added in order
+// (their sum rounded to bfloat16 first when round_parts is set).
 // Sum of squares, rsqrt and both multiplies are float32; one rounding at the store.
 template <typename TD, typename TW, typename TO, int NT>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
                                    const TW* __restrict__ weight, TO* __restrict__ out,
                                    const int* __restrict__ rows, int H, float eps,
-                                   int write_resid, int parts, long long part_stride) {
+                                   int write_resid, int parts, long long part_stride,
+                                   int round_parts) {
   __shared__ float red[NT / kWave];
   const int r = blockIdx.x;
   const long long src = rows ? (long long)rows[r] : (long long)r;
@@ -95,7 +97,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
   for (int j = threadIdx.x; j < H; j += NT) {
     float v = x[j];
     if (d) {
-      for (int s = 0; s < parts; ++s) v += ld(d + s * part_stride + j);
+      v += delta_sum(d + j, parts, part_stride, round_parts);
       if (write_resid) x[j] = v;
     }
     ss += v * v;
@@ -106,8 +108,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
   const bool reread_sum = d && !write_resid;
   for (int j = threadIdx.x; j < H; j += NT) {
     float v = x[j];
-    if (reread_sum)
-      for (int s = 0; s < parts; ++s) v += ld(d + s * part_stride + j);
+    if (reread_sum) v += delta_sum(d + j, parts, part_stride, round_parts);
     st(o + j, v * inv * ld(weight + j));
   }
 }
@@ -118,7 +119,7 @@ template <typename TD, typename TW, typename TO, int NT, int VPT>
 __global__ __launch_bounds__(NT) void add_rmsnorm_small_kernel(
     float* __restrict__ resid, const TD* __restrict__ delta, const TW* __restrict__ weight,
     TO* __restrict__ out, const int* __restrict__ rows, int H, float eps, int write_resid,
-    int parts, long long part_stride) {
+    int parts, long long part_stride, int round_parts) {
   __shared__ float red[NT / kWave];
   const int r = blockIdx.x;
   const long long src = rows ? (long long)rows[r] : (long long)r;
@@ -133,8 +134,7 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_small_kernel(
     w[i] = 0.f;
     if (j < H) {
       v[i] = x[j];
-      if (d)
-        for (int s = 0; s < parts; ++s) v[i] += ld(d + s * part_stride + j);
+      if (d) v[i] += delta_sum(d + j, parts, part_stride, round_parts);
       w[i] = ld(weight + j);
     }
     ss += v[i] * v[i];
@@ -236,25 +236,27 @@ static bool launch_add_rmsnorm_bf16x8(float* resid, const void* delta, const voi
 template <typename TD, typename TW, typename TO>
 static void launch_add_rmsnorm(float* resid, const void* delta, const void* weight, void* out,
                                const int* rows, int R, int H, float eps, int write_resid,
-                               int parts, long long part_stride, hipStream_t stream) {
+                               int parts, long long part_stride, int round_parts,
+                               hipStream_t stream) {
   if (H <= 256 * 4)
     add_rmsnorm_small_kernel<TD, TW, TO, 256, 4><<<R, 256, 0, stream>>>(
         resid, (const TD*)delta, (const TW*)weight, (TO*)out, rows, H, eps, write_resid, parts,
-        part_stride);
+        part_stride, round_parts);
   else if (H <= 256 * 16)
     add_rmsnorm_small_kernel<TD, TW, TO, 256, 16><<<R, 256, 0, stream>>>(
         resid, (const TD*)delta, (const TW*)weight, (TO*)out, rows, H, eps, write_resid, parts,
-        part_stride);
+        part_stride, round_parts);
   else
     add_rmsnorm_kernel<TD, TW, TO, 256><<<R, 256, 0, stream>>>(
         resid, (const TD*)delta, (const TW*)weight, (TO*)out, rows, H, eps, write_resid, parts,
-        part_stride);
+        part_stride, round_parts);
 }
 
 RLIS_API int rlis_add_rmsnorm(float* resid, const void* delta, int delta_dtype,
                               const void* weight, int weight_dtype, void* out, int out_dtype,
                               const int* rows, int R, int H, float eps, int write_resid,
-                              int parts, long long part_stride, hipStream_t stream) {
+                              int parts, long long part_stride, int round_parts,
+                              hipStream_t stream) {
   RLIS_REQUIRE(R >= 0 && H > 0, "add_rmsnorm: bad sizes R=%d H=%d", R, H);
   RLIS_REQUIRE(parts >= 1, "add_rmsnorm: parts=%d", parts);
   RLIS_REQUIRE(!(rows && write_resid && delta),
@@ -270,7 +272,7 @@ RLIS_API int rlis_add_rmsnorm(float* resid, const void* delta, int delta_dtype,
 #define CASE(k, TD, TW, TO)                                                                  \
   case k:                                                                                    \
     launch_add_rmsnorm<TD, TW, TO>(resid, delta, weight, out, rows, R, H, eps, write_resid,  \
-                                   parts, part_stride, stream);                              \
+                                   parts, part_stride, round_parts, stream);                 \
     break;
   switch (key) {
     CASE(0, float, float, float)

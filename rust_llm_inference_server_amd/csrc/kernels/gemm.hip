@@ -471,6 +471,7 @@ struct StreamNorm {
   const float* resid;        // (rows, K) float32
   const void* delta;         // null, or `parts` arrays (rows, K), part_stride elements apart
   int delta_f32, parts;
+  int round_parts;           // round the sum of the parts to bfloat16 before it is added
   long long part_stride;
   const void* weight;        // (K)
   int weight_f32;
@@ -590,7 +591,9 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
           load8(nm.resid + at[i], v[i]);
         }
         if (nm.delta) {
-          // two parts per round, so that their loads travel together with the residual's
+          // two parts per round, so that their loads travel together with the residual's; the
+          // parts are summed in order on their own and then join the residual
+          float dsum[kU][8];
           for (int s = 0; s < nm.parts; s += 2) {
             const bool two = s + 1 < nm.parts;
             float d0[kU][8], d1[kU][8];
@@ -610,10 +613,15 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
             for (int i = 0; i < kU; ++i)
 #pragma unroll
               for (int e = 0; e < 8; ++e) {
-                v[i][e] += d0[i][e];
-                if (two) v[i][e] += d1[i][e];
+                dsum[i][e] = s == 0 ? d0[i][e] : dsum[i][e] + d0[i][e];
+                if (two) dsum[i][e] += d1[i][e];
               }
           }
+#pragma unroll
+          for (int i = 0; i < kU; ++i)
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              v[i][e] += nm.round_parts ? bf16_to_f32(f32_to_bf16(dsum[i][e])) : dsum[i][e];
         }
 #pragma unroll
         for (int i = 0; i < kU; ++i) {
@@ -821,7 +829,8 @@ RLIS_API int rlis_gemm_bf16_stream(const void* X, const void* W, void* Y, int y_
 }
 
 // RMSNorm and projection in one pass, for T <= 16 tokens and K <= 4096:
-//   s = resid[row(t)] + sum of the `parts` deltas (delta may be null),
+//   s = resid[row(t)] + sum of the `parts` deltas (delta may be null; with round_parts the
+//       sum of the parts is rounded to bfloat16 before it joins the residual),
 //   y[t] = (s * rsqrt(mean(s^2) + eps) * norm_weight) W^T   (gated as above),
 // where row(t) = rows[t], or t when rows is null.  resid is (R, K) float32 contiguous; each
 // delta part is shaped like it (bfloat16, or float32 for partial sums), part_stride elements
@@ -829,7 +838,8 @@ RLIS_API int rlis_gemm_bf16_stream(const void* X, const void* W, void* Y, int y_
 // workgroups still read that), it receives s.  The normalised row is rounded to bfloat16
 // before the scale by rsqrt is applied rather than after; the scale is exact in float32.
 RLIS_API int rlis_norm_linear_bf16(const float* resid, const void* delta, int delta_dtype,
-                                   int parts, long long part_stride, const void* norm_weight,
+                                   int parts, long long part_stride, int round_parts,
+                                   const void* norm_weight,
                                    int norm_weight_dtype, float eps, const int* rows,
                                    float* resid_out, const void* W, void* Y, int y_dtype, int T,
                                    int N, int K, long long ldw, long long ldy, int gated,
@@ -856,6 +866,7 @@ RLIS_API int rlis_norm_linear_bf16(const float* resid, const void* delta, int de
   nm.delta_f32 = delta_dtype == RLIS_F32;
   nm.parts = delta ? parts : 0;
   nm.part_stride = part_stride;
+  nm.round_parts = round_parts;
   nm.weight = norm_weight;
   nm.weight_f32 = norm_weight_dtype == RLIS_F32;
   nm.eps = eps;

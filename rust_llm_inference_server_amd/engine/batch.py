@@ -5,17 +5,21 @@ The reference builds the same per step in ``PagedBatch::new`` (crates/model/src/
 (llama.rs:252), the write slot ``table[pos / page] * page + pos % page`` of every new token
 (paged.rs:258-263), zero-padded block tables and context lengths (paged.rs:199-213).  Here one
 slot id per token is enough (the write kernel spreads it over heads and dims), and all of it
-goes to the device in one copy."""
+goes to the device in one copy.
+
+What is laid out here is common to every mixer.  What only one kind of mixer needs (the work
+lists of its kernels) comes from that mixer's ``StepPlanner`` and is carried along unseen:
+``build_step`` calls each planner with the step's host-side lengths and packs the arrays it
+returns into the same buffer (``step.plans[key]``)."""
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import List, Optional, Sequence, Tuple
+from typing import Any, Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
 
-PREFILL_TILE = 64     # new tokens per workgroup of the matrix-core prefill attention
-WIDE_TILE = 128       # ... of its form with two query blocks per wave
+from ..stepplan import HostPlan, StepLengths, StepPlan, StepPlanner
 
 
 @dataclass
@@ -48,30 +52,63 @@ class StepContext:
     logit_rows: torch.Tensor          # (R) int32: token rows whose logits are wanted
     num_logit_rows: int
     state_slots: torch.Tensor         # (S) int32
-    tile_map: torch.Tensor            # (num_tiles, 2) int32: (sequence, first new-token index)
-    num_tiles: int
     groups: List[GroupStep]
     max_context: int
     max_new: int
     all_decode: bool
-    decode_splits: Optional[int] = None
     # Sequences that bring a single token come first in the step: sequences (and token rows)
     # [0, num_single) are theirs, so that a decode kernel can take them beside the portions.
     num_single: int = 0
-    max_single_context: int = 0
-    multi_tile_map: Optional[torch.Tensor] = None     # tile_map without the single tokens' tiles
-    num_multi_tiles: int = 0
-    wide_tile_map: Optional[torch.Tensor] = None      # the same two lists in tiles of 128 tokens
-    wide_multi_tile_map: Optional[torch.Tensor] = None
+    # What the mixers' planners made of this step, by planner key.
+    plans: Dict[Any, StepPlan] = field(default_factory=dict)
     # Host copies, for parts that plan on the host.
+    lengths: Optional[StepLengths] = None
     host_start_pos: List[int] = field(default_factory=list)
     host_new: List[int] = field(default_factory=list)
     host_state_slots: List[int] = field(default_factory=list)
     host_order: List[int] = field(default_factory=list)   # entry index of every sequence
 
 
+class MetadataBuffer:
+    """Named int32 arrays packed into one buffer, each starting on a 16-byte boundary, so that
+    a step's metadata reaches the device in one copy.  The eager step builder fills one per
+    step; a captured decode step keeps one of fixed sizes and rewrites it in place."""
+
+    def __init__(self) -> None:
+        self.offsets: Dict[str, Tuple[int, int]] = {}
+        self.size = 0
+        self._chunks: List[np.ndarray] = []
+
+    def put(self, name: str, values) -> None:
+        arr = np.asarray(values, dtype=np.int32).reshape(-1)
+        self.reserve(name, arr.size)
+        self._chunks.append(arr)
+        pad = -arr.size % 4
+        if pad:
+            self._chunks.append(np.zeros(pad, dtype=np.int32))
+
+    def reserve(self, name: str, count: int) -> None:
+        if name in self.offsets:
+            raise KeyError(f"metadata array '{name}' is laid out twice")
+        self.offsets[name] = (self.size, int(count))
+        self.size += -(-int(count) // 4) * 4
+
+    def packed(self) -> torch.Tensor:
+        if not self._chunks:
+            return torch.zeros(0, dtype=torch.int32)
+        return torch.from_numpy(np.concatenate(self._chunks))
+
+    def view(self, buf, name: str):
+        o, n = self.offsets[name]
+        return buf[o:o + n]
+
+
+def plan_name(index: int, array: str) -> str:
+    return f"plan{index}.{array}"
+
+
 def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
-               vocab_size: int) -> StepContext:
+               vocab_size: int, planners: Sequence[StepPlanner] = ()) -> StepContext:
     """Lay out a step.  Every entry's request must hold reserved positions for its tokens.
 
     Inside the step the sequences are ordered single tokens first (``host_order`` maps them back
@@ -88,14 +125,12 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
     ctx_lens: List[int] = []
     state_slots: List[int] = []
     new: List[int] = []
-    tiles: List[Tuple[int, int, int]] = []      # (keys the tile walks, sequence, first index)
-    wide: List[Tuple[int, int, int]] = []       # the same in tiles of WIDE_TILE tokens
     ng = cache.num_groups
     tables: List[List[List[int]]] = [[] for _ in range(ng)]
     slots: List[List[np.ndarray]] = [[] for _ in range(ng)]
     seen = set()
     base_of = [0] * S
-    for s, i in enumerate(order):
+    for i in order:
         e = entries[i]
         n = len(e.tokens)
         if n == 0:
@@ -128,9 +163,6 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
         for w in e.want:
             if not 0 <= int(w) < n:
                 raise ValueError(f"request {e.seq_id}: wanted index {w} is outside its {n} tokens")
-        tiles.extend((computed + min(n, qb + PREFILL_TILE), s, qb)
-                     for qb in range(0, n, PREFILL_TILE))
-        wide.extend((computed + min(n, qb + WIDE_TILE), s, qb) for qb in range(0, n, WIDE_TILE))
         for g in range(ng):
             table = cache.table(e.seq_id, g)
             tables[g].append(table)
@@ -143,63 +175,49 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
     T = cu[-1]
     num_single = sum(1 for n in new if n == 1)
     widths = [max(8, -(-max(len(t) for t in tables[g]) // 8) * 8) for g in range(ng)]
-    chunks: List[np.ndarray] = []
-    offsets = {}
-    filled = 0
+    lengths = StepLengths(np.asarray(start_pos, dtype=np.int64), np.asarray(new, dtype=np.int64),
+                          num_single, ps)
 
-    def put(name, values):
-        nonlocal filled
-        arr = np.asarray(values, dtype=np.int32).reshape(-1)
-        offsets[name] = (filled, arr.size)
-        pad = -arr.size % 4                     # keep every array 16-byte aligned
-        chunks.append(arr)
-        if pad:
-            chunks.append(np.zeros(pad, dtype=np.int32))
-        filled += arr.size + pad
-
-    put("ids", np.concatenate(ids))
-    put("positions", np.concatenate(positions))
-    put("seq_of_token", np.repeat(np.arange(S, dtype=np.int32), new))
-    put("cu", cu)
-    put("start_pos", start_pos)
-    put("ctx_lens", ctx_lens)
-    put("logit_rows", logit_rows)
-    put("state_slots", state_slots)
-    # Longest tiles first: the prefill attention kernel hands them out in this order.
-    tiles.sort(key=lambda t: -t[0])
-    put("tiles", [x for _, s_, qb in tiles for x in (s_, qb)])
-    multi = [t for t in tiles if t[1] >= num_single]
-    put("tiles_multi", [x for _, s_, qb in multi for x in (s_, qb)])
-    wide.sort(key=lambda t: -t[0])
-    put("wide", [x for _, s_, qb in wide for x in (s_, qb)])
-    put("wide_multi", [x for _, s_, qb in wide if s_ >= num_single for x in (s_, qb)])
+    meta = MetadataBuffer()
+    meta.put("ids", np.concatenate(ids))
+    meta.put("positions", np.concatenate(positions))
+    meta.put("seq_of_token", np.repeat(np.arange(S, dtype=np.int32), new))
+    meta.put("cu", cu)
+    meta.put("start_pos", start_pos)
+    meta.put("ctx_lens", ctx_lens)
+    meta.put("logit_rows", logit_rows)
+    meta.put("state_slots", state_slots)
     for g in range(ng):
-        put(f"slots{g}", np.concatenate(slots[g]))
+        meta.put(f"slots{g}", np.concatenate(slots[g]))
         rows = np.zeros((S, widths[g]), dtype=np.int32)
         for r, t in enumerate(tables[g]):
             rows[r, :len(t)] = np.maximum(np.asarray(t, dtype=np.int32), 0)
-        put(f"tables{g}", rows)
-    host = torch.from_numpy(np.concatenate(chunks))
+        meta.put(f"tables{g}", rows)
+    host_plans: List[Tuple[Any, HostPlan]] = []
+    for k, planner in enumerate(planners):
+        plan = planner.plan(lengths)
+        for name, arr in plan.arrays.items():
+            meta.put(plan_name(k, name), arr)
+        host_plans.append((planner.key(), plan))
+    host = meta.packed()
 
     if device.type == "cuda":
         host = host.pin_memory()
     dev = host.to(device, non_blocking=True)
 
     def view(name):
-        o, n = offsets[name]
-        return dev[o:o + n]
+        return meta.view(dev, name)
 
     groups = [GroupStep(page_size=ps, window=cache.groups[g].window,
                         block_tables=view(f"tables{g}").reshape(S, widths[g]),
                         slots=view(f"slots{g}")) for g in range(ng)]
+    plans = {key: StepPlan({name: view(plan_name(k, name)) for name in plan.arrays}, plan.values)
+             for k, (key, plan) in enumerate(host_plans)}
     return StepContext(
         num_tokens=T, num_seqs=S, ids=view("ids"), positions=view("positions"),
         seq_of_token=view("seq_of_token"), cu_seqlens=view("cu"), start_pos=view("start_pos"),
         ctx_lens=view("ctx_lens"), logit_rows=view("logit_rows"), num_logit_rows=len(logit_rows),
-        state_slots=view("state_slots"), tile_map=view("tiles"), num_tiles=len(tiles),
-        groups=groups, max_context=max(ctx_lens), max_new=max(new),
-        all_decode=num_single == S, num_single=num_single,
-        max_single_context=max(ctx_lens[:num_single], default=0),
-        multi_tile_map=view("tiles_multi"), num_multi_tiles=len(multi),
-        wide_tile_map=view("wide"), wide_multi_tile_map=view("wide_multi"),
-        host_start_pos=start_pos, host_new=new, host_state_slots=state_slots, host_order=order)
+        state_slots=view("state_slots"), groups=groups, max_context=max(ctx_lens),
+        max_new=max(new), all_decode=num_single == S, num_single=num_single, plans=plans,
+        lengths=lengths, host_start_pos=start_pos, host_new=new, host_state_slots=state_slots,
+        host_order=order)

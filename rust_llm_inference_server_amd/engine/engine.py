@@ -96,7 +96,7 @@ class Engine:
             num_pages = cfg.num_pages
         else:
             # engine.rs:252-262: pool bytes / (bytes of K and V per token * block size)
-            per_token = sum(2 * len(g.writer_runs) * g.request.num_kv_heads * g.request.head_dim
+            per_token = sum(len(g.writer_runs) * g.request.elements_per_token()
                             for g in model.cache_groups) * elem
             num_pages = int(cfg.kv_cache_gb * (1 << 30)) // max(1, per_token * cfg.block_size)
         if num_pages < 2:

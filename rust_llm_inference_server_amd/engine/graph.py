@@ -7,23 +7,25 @@ int32 buffer (filled on the host by the native page manager, one copy to the dev
 kernels read it through fixed views, and the logits land in a static tensor.
 
 Unused rows of a bucket are padding requests of context 1 that read and write a scratch page
-beyond the manager's pages, so they touch nothing a live request owns.  Nothing in the graph
-depends on the host: partition counts of the decode attention are fixed per bucket and each
-sequence cuts its own context into that many partitions.  Graphs hold no memset nodes (the
-kernels clear nothing) and are checked against the eager step in the tests, replay after
-replay with eager work in between."""
+beyond the manager's pages and a scratch state slot beyond its slots, so they touch nothing a
+live request owns.  Nothing in the graph depends on the host: what a mixer's planner sizes by
+the longest context is fixed per context bucket, and how a sequence's own work is cut follows
+from its own lengths on the device, so a replay computes bit for bit what the eager step does.
+Graphs hold no memset nodes (the kernels clear nothing) and are checked against the eager step
+in the tests, replay after replay with eager work in between."""
 from __future__ import annotations
 
 import contextlib
 import ctypes
 import gc
 import weakref
-from typing import Optional, Sequence
+from typing import Dict, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
 
-from .batch import GroupStep, StepContext
+from ..stepplan import StepPlan
+from .batch import GroupStep, MetadataBuffer, StepContext
 
 
 def bucket_for(n: int, limit: int) -> int:
@@ -51,8 +53,19 @@ def no_collection():
             gc.enable()
 
 
+def context_bucket(context: int, limit: int) -> int:
+    """The smallest of 1024, 2048, 4096, ... that holds ``context`` positions, capped at
+    ``limit``: captured steps are kept per bucket, so that what a planner sizes by the longest
+    context (the depth of a grid) need not be sized for the longest context there could be."""
+    b = 1024
+    while b < context:
+        b *= 2
+    return min(b, limit)
+
+
 class DecodeGraph:
-    """The captured decode step of one batch-size bucket."""
+    """The captured decode steps of one batch-size bucket: one static metadata buffer, and one
+    HIP graph per context bucket."""
 
     def __init__(self, runner, bucket: int):
         self.runner = weakref.proxy(runner)     # the runner owns its graphs: no cycle
@@ -62,102 +75,121 @@ class DecodeGraph:
         ps = cache.page_size
         self.width = W = max(8, -(-(-(-model.max_positions // ps)) // 8) * 8)
         ng = cache.num_groups
-        # ---- static layout ---------------------------------------------------------------
-        names = ["ids", "positions", "seq_of_token", "cu", "start_pos", "ctx_lens", "logit_rows",
-                 "state_slots"]
-        sizes = {n: B for n in names}
-        sizes["cu"] = B + 1
+        # ---- static layout: the step builder's arrays, at their largest --------------------
+        self.meta = meta = MetadataBuffer()
+        for name in ("ids", "positions", "seq_of_token"):
+            meta.reserve(name, B)
+        meta.reserve("cu", B + 1)
+        for name in ("start_pos", "ctx_lens", "logit_rows", "state_slots"):
+            meta.reserve(name, B)
         for g in range(ng):
-            sizes[f"slots{g}"] = B
-            sizes[f"tables{g}"] = B * W
-        self.offsets, total = {}, 0
-        for name, n in sizes.items():
-            self.offsets[name] = (total, n)
-            total += -(-n // 4) * 4
-        self.host = torch.zeros(total, dtype=torch.int32).pin_memory()
+            meta.reserve(f"slots{g}", B)
+            meta.reserve(f"tables{g}", B * W)
+        self.host = torch.zeros(meta.size, dtype=torch.int32).pin_memory()
         self.np = self.host.numpy()
-        self.dev = torch.zeros(total, dtype=torch.int32, device=dev)
+        self.dev = torch.zeros(meta.size, dtype=torch.int32, device=dev)
         self.seq_ids = np.zeros(B, dtype=np.int64)
-
-        def hview(name):
-            o, n = self.offsets[name]
-            return self.np[o:o + n]
-
-        def dview(name):
-            o, n = self.offsets[name]
-            return self.dev[o:o + n]
-
-        self.h = {name: hview(name) for name in sizes}
+        self.h = {name: meta.view(self.np, name) for name in meta.offsets}
         self.h["seq_of_token"][:] = np.arange(B)
         self.h["cu"][:] = np.arange(B + 1)
         self.h["logit_rows"][:] = np.arange(B)
         base = self.host.data_ptr()
-        ptr = lambda name: base + 4 * self.offsets[name][0]
+        ptr = lambda name: base + 4 * meta.offsets[name][0]
         self.ptr_positions, self.ptr_slots = ptr("positions"), ptr("state_slots")
         self.ptr_tables = (ctypes.c_void_p * ng)(*[ptr(f"tables{g}") for g in range(ng)])
         self.ptr_wslots = (ctypes.c_void_p * ng)(*[ptr(f"slots{g}") for g in range(ng)])
         self.scratch_page = runner.pools.scratch_page
-        groups = [GroupStep(page_size=ps, window=cache.groups[g].window,
-                            block_tables=dview(f"tables{g}").reshape(B, W),
-                            slots=dview(f"slots{g}")) for g in range(ng)]
-        self.step = StepContext(
-            num_tokens=B, num_seqs=B, ids=dview("ids"), positions=dview("positions"),
-            seq_of_token=dview("seq_of_token"), cu_seqlens=dview("cu"),
-            start_pos=dview("start_pos"), ctx_lens=dview("ctx_lens"),
-            logit_rows=dview("logit_rows"), num_logit_rows=B, state_slots=dview("state_slots"),
-            tile_map=dview("ids")[:0], num_tiles=0, groups=groups,
-            max_context=model.max_positions, max_new=1, all_decode=True, decode_splits=None)
-        self.graph: Optional[torch.cuda.CUDAGraph] = None
-        self.logits: Optional[torch.Tensor] = None
+        self.scratch_state_slot = runner.pools.scratch_state_slot
+        dview = lambda name: meta.view(self.dev, name)
+        self.groups = [GroupStep(page_size=ps, window=cache.groups[g].window,
+                                 block_tables=dview(f"tables{g}").reshape(B, W),
+                                 slots=dview(f"slots{g}")) for g in range(ng)]
+        self.views = {name: dview(name) for name in meta.offsets}
+        # context bucket -> (graph, its static logits)
+        self.graphs: Dict[int, Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
         self._copied: Optional[torch.cuda.Event] = None
 
+    def step_for(self, context_limit: int) -> StepContext:
+        """The step as the kernels of a captured run see it: static views, and each planner's
+        plan for any contexts up to ``context_limit``."""
+        B, v = self.bucket, self.views
+        runner = self.runner
+        plans = {}
+        for planner in runner.model.step_planners:
+            host = planner.plan_captured(B, context_limit, runner.cache.page_size)
+            if host.arrays:
+                raise ValueError(f"the plan of a captured step may hold values only, "
+                                 f"{type(planner).__name__} returned arrays")
+            plans[planner.key()] = StepPlan({}, host.values)
+        return StepContext(
+            num_tokens=B, num_seqs=B, ids=v["ids"], positions=v["positions"],
+            seq_of_token=v["seq_of_token"], cu_seqlens=v["cu"], start_pos=v["start_pos"],
+            ctx_lens=v["ctx_lens"], logit_rows=v["logit_rows"], num_logit_rows=B,
+            state_slots=v["state_slots"], groups=self.groups, max_context=context_limit,
+            max_new=1, all_decode=True, num_single=B, plans=plans)
+
     # ------------------------------------------------------------------------------------
-    def _fill(self, seq_ids: Sequence[int], tokens: Sequence[int]) -> None:
-        S, B, W = len(seq_ids), self.bucket, self.width
-        h = self.h
-        self.seq_ids[:S] = seq_ids
-        h["ids"][:S] = tokens
-        self.runner.cache.decode_batch(self.seq_ids.ctypes.data, S, W, self.ptr_positions,
-                                       self.ptr_slots, self.ptr_tables, self.ptr_wslots)
-        if S < B:                        # padding requests: context 1 on the scratch page
+    def _pad_from(self, S: int, h: Optional[dict] = None) -> None:
+        """Rows S.. of the bucket: padding requests of context 1 on the scratch page, with the
+        scratch state slot (in the host views ``h``, the live ones by default)."""
+        B, W = self.bucket, self.width
+        h = self.h if h is None else h
+        if S < B:
             h["ids"][S:] = 0
             h["positions"][S:] = 0
-            h["state_slots"][S:] = 0
+            h["state_slots"][S:] = self.scratch_state_slot
             for g in range(len(self.ptr_tables)):
                 h[f"tables{g}"].reshape(B, W)[S:, 0] = self.scratch_page
                 h[f"slots{g}"][S:] = self.scratch_page * self.runner.cache.page_size
         h["start_pos"][:] = h["positions"]
         h["ctx_lens"][:] = h["positions"] + 1
 
-    def run(self, seq_ids: Sequence[int], tokens: Sequence[int]) -> torch.Tensor:
-        """Logits ``(len(seq_ids), vocab)`` of one decode token per request.  The result
-        views a static tensor: it is overwritten by the next call."""
+    def prepare(self, seq_ids: Sequence[int], tokens: Sequence[int]) -> np.ndarray:
+        """Fill the host side of the metadata for one token per request; returns the new
+        tokens' positions.  Nothing is launched or copied to the device yet."""
         if self._copied is not None:
             self._copied.synchronize()       # the host buffer is free to be written again
-        self._fill(seq_ids, tokens)
+        S = len(seq_ids)
+        self.seq_ids[:S] = seq_ids
+        self.h["ids"][:S] = tokens
+        self.runner.cache.decode_batch(self.seq_ids.ctypes.data, S, self.width,
+                                       self.ptr_positions, self.ptr_slots, self.ptr_tables,
+                                       self.ptr_wslots)
+        self._pad_from(S)
+        return self.h["positions"][:S]
+
+    def launch(self, num_seqs: int, context_limit: int) -> torch.Tensor:
+        """Run the prepared step.  Logits ``(num_seqs, vocab)``: a view of a static tensor that
+        the next call for the same context bucket overwrites."""
+        if context_limit not in self.graphs:
+            self._capture(context_limit)
+        graph, logits = self.graphs[context_limit]
         self.dev.copy_(self.host, non_blocking=True)
         if self._copied is None:
             self._copied = torch.cuda.Event()
         self._copied.record()
-        if self.graph is None:
-            self._capture()
-        else:
-            self.graph.replay()
-        return self.logits[:len(seq_ids)]
+        graph.replay()
+        return logits[:num_seqs]
 
-    def _capture(self) -> None:
+    def _capture(self, context_limit: int) -> None:
+        """Capture the step on metadata that is all padding: what the warm-up run and the
+        capture itself compute lands on the scratch page and the scratch state slot, so that no
+        request's cache or state moves before the first replay."""
         runner = self.runner
+        padding = self.host.clone()
+        flat = padding.numpy()
+        self._pad_from(0, {name: self.meta.view(flat, name) for name in self.meta.offsets})
+        self.dev.copy_(padding)
+        step = self.step_for(context_limit)
         # One eager run first: it settles lazy initialisation (library loading, workspace
-        # allocations) that must not happen under capture.  The step is idempotent: it writes
-        # the same keys and values to the same slots.
+        # allocations) that must not happen under capture.
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            runner.model.forward(self.step, runner.pools)
+            runner.model.forward(step, runner.pools)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with no_collection(), torch.cuda.graph(graph):
-            self.logits = runner.model.forward(self.step, runner.pools)
-        self.graph = graph
-        graph.replay()
+            logits = runner.model.forward(step, runner.pools)
+        self.graphs[context_limit] = (graph, logits)

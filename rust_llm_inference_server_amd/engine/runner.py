@@ -116,7 +116,7 @@ class ModelRunner:
         for c in copies:
             by_group.setdefault(c.group, []).append(c)
         for g, cs in by_group.items():
-            if g < len(self.pools.k):
+            if g < len(self.pools.arrays):
                 self.pools.copy_pages(g, [c.src for c in cs], [c.dst for c in cs])
 
     def free(self, seq_id: int) -> None:
@@ -138,14 +138,16 @@ class ModelRunner:
         if self.max_batched_tokens is not None and total > self.max_batched_tokens:
             raise ValueError(f"{total} tokens in one step, max_batched_tokens is "
                              f"{self.max_batched_tokens}")
-        step = build_step(entries, self.cache, self.device, self.vocab_size)
+        step = build_step(entries, self.cache, self.device, self.vocab_size,
+                          self.model.step_planners)
         if step.max_context > self.model.max_positions:
             raise ValueError(f"sequence of {step.max_context} positions exceeds max_seq_len "
                              f"{self.model.max_positions}")
         if self.pools.state is not None:
-            for start, slot in zip(step.host_start_pos, step.host_state_slots):
-                if start == 0:
-                    self.pools.zero_state(slot)      # a fresh (or recomputed) request
+            # a fresh (or recomputed) request starts from cleared state
+            self.pools.zero_states([slot for start, slot in zip(step.host_start_pos,
+                                                                step.host_state_slots)
+                                    if start == 0])
         logits = self.model.forward(step, self.pools)
         for i, start in zip(step.host_order, step.host_start_pos):
             self.cache.advance(entries[i].seq_id, start + len(entries[i].tokens))
@@ -154,7 +156,7 @@ class ModelRunner:
     def _decode_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """A step of one token per request, replayed from the HIP graph of its batch-size
         bucket (captured at first use).  Same kernels, same results as the eager step."""
-        from .graph import DecodeGraph, bucket_for
+        from .graph import DecodeGraph, bucket_for, context_bucket
         S = len(entries)
         seq_ids = [e.seq_id for e in entries]
         if len(set(seq_ids)) != S:
@@ -172,15 +174,20 @@ class ModelRunner:
         graph = self._graphs.get(bucket)
         if graph is None:
             graph = self._graphs[bucket] = DecodeGraph(self, bucket)
-        logits = graph.run(seq_ids, tokens)
-        positions = graph.h["positions"]
-        if int(positions[:S].max()) + 1 > self.model.max_positions:
-            raise ValueError(f"sequence of {int(positions[:S].max()) + 1} positions exceeds "
-                             f"max_seq_len {self.model.max_positions}")
+        positions = graph.prepare(seq_ids, tokens)
+        # Everything that can refuse the step is checked before anything is launched.
+        longest = int(positions.max()) + 1
+        if longest > self.model.max_positions:
+            raise ValueError(f"sequence of {longest} positions exceeds max_seq_len "
+                             f"{self.model.max_positions}")
         if self.pools.state is not None:
-            pass                                   # graph-safe mixers keep no state slots
-        for i, seq in enumerate(seq_ids):
-            self.cache.advance(seq, int(positions[i]) + 1)
+            # a request whose first token this is starts from cleared state
+            self.pools.zero_states([int(graph.h["state_slots"][i]) for i in range(S)
+                                    if positions[i] == 0])
+        ends = [int(p) + 1 for p in positions]
+        logits = graph.launch(S, context_bucket(longest, self.model.max_positions))
+        for seq, end in zip(seq_ids, ends):
+            self.cache.advance(seq, end)
         if rows == list(range(S)):
             return logits
         if not rows:

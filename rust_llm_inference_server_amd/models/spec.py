@@ -114,6 +114,14 @@ class Model:
         self.graph_safe = all(getattr(p, "graph_safe", False)
                               for p in (self.embedding, *self.layers, self.final_norm, self.head))
         self._plan_cache()
+        # The per-step planners of the mixers, one per distinct key.
+        self.step_planners: List[Any] = []
+        seen = set()
+        for layer in self.layers:
+            planner = layer.mixer.step_planner()
+            if planner is not None and planner.key() not in seen:
+                seen.add(planner.key())
+                self.step_planners.append(planner)
 
     # ---------------------------------------------------------------- cache plan
     def _plan_cache(self) -> None:
@@ -150,7 +158,7 @@ class Model:
     def forward(self, step: Any, pools: Any) -> torch.Tensor:
         """Logits float32 ``(R, V)`` at ``step.logit_rows``; K, V and state of the step's
         tokens are left in ``pools``."""
-        stream = ResidualStream(self.embedding.forward(step.ids))
+        stream = ResidualStream(self.embedding.forward(step.ids), self.act_dtype)
         for i, run in enumerate(self.runs):
             self.layers[run.layer].forward(stream, step, pools.binding(self.bindings[i]))
         if step.num_logit_rows == 0:

@@ -11,7 +11,9 @@ from typing import Optional, Tuple
 
 import torch
 
+from ..stepplan import StepPlan
 from . import lib
+from .attention_plan import AttentionPlanner
 from .lib import KernelError
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
@@ -23,15 +25,6 @@ SKINNY_MAX_ROWS = 64
 STREAM_MAX_ROWS = 16
 # Single tokens in a batch that also holds portions of prompts take the decode attention kernel.
 SPLIT_MIXED_ATTENTION = True
-# The prefill attention takes tiles of 128 queries when that makes this many workgroups (5/3 as
-# many up to head size 64), or when contexts are long (4096 positions, or 2048 cached ones);
-# 1 << 30: never.
-PREFILL_WIDE_MIN_GROUPS = 768
-# The prefill attention cuts the keys of its tiles into runs (one workgroup each, merged
-# afterwards) when its tiles leave compute units without work: as many runs as the units hold
-# at once, with at least this many keys a run (0 units: never).
-PREFILL_SPLIT_UNITS = 256
-PREFILL_SPLIT_MIN_KEYS = 1024
 # The norm in front of a projection goes into the streaming kernel where that applies.
 FUSE_NORM_LINEAR = True
 # The matrix-core decode attention rotates q and k and stores the new k, v itself where it can.
@@ -108,20 +101,21 @@ def _delta_parts(resid: torch.Tensor, delta: torch.Tensor, what: str) -> int:
                       f"{tuple(resid.shape)}")
 
 
-def add_residual(resid: torch.Tensor, delta: torch.Tensor) -> None:
-    """``resid += delta`` with the sum formed in float32."""
+def add_residual(resid: torch.Tensor, delta: torch.Tensor, round_parts: bool = False) -> None:
+    """``resid += delta`` with the sum formed in float32.  ``round_parts``: a stack of partial
+    sums is added up and rounded to bfloat16 before it joins the residual."""
     _check(resid, "residual", torch.float32)
     if not resid.is_contiguous():
         raise KernelError("add_residual: residual must be contiguous")
     parts = _delta_parts(resid, delta, "add_residual")
     lib.call("rlis_add_residual", resid.data_ptr(), delta.data_ptr(), _dt(delta), resid.numel(),
-             parts, lib.stream_ptr())
+             parts, int(bool(round_parts) and parts > 1), lib.stream_ptr())
 
 
 def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
                 eps: float, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
-                write_resid: bool = True) -> torch.Tensor:
-    """``norm(resid + delta) * weight`` row by row.
+                write_resid: bool = True, round_parts: bool = False) -> torch.Tensor:
+    """``norm(resid + delta) * weight`` row by row (``round_parts`` as in ``add_residual``).
 
     With ``rows`` only those rows are produced and the residual is left as it is; otherwise
     the sum is stored back into ``resid`` when ``write_resid`` is set."""
@@ -141,7 +135,8 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
     lib.call("rlis_add_rmsnorm", resid.data_ptr(),
              None if delta is None else delta.data_ptr(), 0 if delta is None else _dt(delta),
              weight.data_ptr(), _dt(weight), out.data_ptr(), _DT[out_dtype], rows_ptr, R, H,
-             float(eps), int(bool(write_resid)), parts, T * H, lib.stream_ptr())
+             float(eps), int(bool(write_resid)), parts, T * H,
+             int(bool(round_parts) and parts > 1), lib.stream_ptr())
     return out
 
 
@@ -226,9 +221,10 @@ def can_fuse_norm_linear(resid: torch.Tensor, w: torch.Tensor, rows: Optional[in
 
 def norm_linear(resid: torch.Tensor, delta: Optional[torch.Tensor], norm_weight: torch.Tensor,
                 eps: float, w: torch.Tensor, out_dtype: torch.dtype, gated: bool = False,
-                rows: Optional[torch.Tensor] = None):
+                rows: Optional[torch.Tensor] = None, round_parts: bool = False):
     """RMSNorm of ``resid + delta`` and the product with ``w`` in one kernel (see
-    ``can_fuse_norm_linear``); ``gated`` as ``linear_swiglu``.  Returns ``(y, resid_sum)``:
+    ``can_fuse_norm_linear``); ``gated`` as ``linear_swiglu``, ``round_parts`` as in
+    ``add_residual``.  Returns ``(y, resid_sum)``:
     without ``rows``, ``resid_sum`` is ``resid + delta`` in a new tensor (``resid`` itself when
     there is no delta); with ``rows``, only those rows are produced and ``resid_sum`` is None."""
     _check(resid, "residual", torch.float32, 2)
@@ -256,7 +252,8 @@ def norm_linear(resid: torch.Tensor, delta: Optional[torch.Tensor], norm_weight:
     if R:
         lib.call("rlis_norm_linear_bf16", resid.data_ptr(),
                  None if delta is None else delta.data_ptr(), 0 if delta is None else _dt(delta),
-                 parts, T * K, norm_weight.data_ptr(), _dt(norm_weight), float(eps), rows_ptr,
+                 parts, T * K, int(bool(round_parts) and parts > 1), norm_weight.data_ptr(),
+                 _dt(norm_weight), float(eps), rows_ptr,
                  None if (delta is None or rows is not None) else resid_sum.data_ptr(),
                  w.data_ptr(), y.data_ptr(), _DT[out_dtype], R, N, K, ldw, N, int(bool(gated)),
                  lib.stream_ptr())
@@ -351,36 +348,35 @@ def copy_pages(pages: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> Non
 
 
 # ----------------------------------------------------------------------- attention
-def decode_splits(num_seqs: int, num_kv_heads: int, group: int, max_context: int) -> int:
-    """Partitions per context for the decode kernel (the rule of crates/model/src/
-    paged_attention.rs:21-36 with targets measured on this chip): as many as bring the launch
-    to one workgroup per compute unit, never more than 16 (beyond that the merge costs more
-    than the partitions gain) and at least 256 positions each.  From 32 requests of 8 KV heads
-    on that is one partition, and no merge kernel."""
-    pairs = max(1, num_seqs * num_kv_heads * math.ceil(group / 8))
-    return max(1, min(256 // pairs, 16, math.ceil(max_context / 256)))
-
-
 def _decode_mfma_ok(qkv: torch.Tensor, nh: int, nkv: int, d: int, page_size: int) -> bool:
     """Whether single tokens of this layout can take the matrix-core decode kernel."""
     g = nh // nkv
     return (qkv.dtype == torch.bfloat16 and d % 16 == 0 and d <= 256 and g <= 16
-            and g * (d + 2) * 32 <= 65536
-            and page_size >= 8 and page_size & (page_size - 1) == 0 and qkv.stride(0) % 8 == 0
-            and DECODE_ATTENTION != "vector")
+            and g * (d + 2) * 32 <= 65536 and AttentionPlanner.pages_fit(page_size)
+            and qkv.stride(0) % 8 == 0 and DECODE_ATTENTION != "vector")
+
+
+def _prefill_mfma_ok(qkv: torch.Tensor, d: int, page_size: int) -> bool:
+    return (qkv.dtype == torch.bfloat16 and d % 16 == 0 and d <= 256
+            and AttentionPlanner.pages_fit(page_size) and qkv.stride(0) % 8 == 0)
+
+
+def attention_planner(num_heads: int, num_kv_heads: int, head_dim: int,
+                      dtype: torch.dtype) -> AttentionPlanner:
+    """The planner a mixer that calls ``paged_attention`` / ``rope_attention`` names as its
+    ``step_planner()``."""
+    return AttentionPlanner(num_heads, num_kv_heads, head_dim, matrix=dtype == torch.bfloat16,
+                            singles_apart=SPLIT_MIXED_ATTENTION and DECODE_ATTENTION != "vector")
 
 
 def _attention_kernel(qkv: torch.Tensor, nh: int, nkv: int, d: int, page_size: int, step,
                       force: Optional[str]):
     """(kind, matrix_decode): which attention kernel a batch takes."""
-    q_stride = qkv.stride(0)
     kind = force or FORCE_ATTENTION
     if kind is None:
         if step.all_decode and d % 8 == 0 and d <= 256 and (nh // nkv) * d <= 2048:
             kind = "decode"
-        elif (qkv.dtype == torch.bfloat16 and d % 16 == 0 and d <= 256 and page_size >= 8
-              and page_size & (page_size - 1) == 0 and q_stride % 8 == 0
-              and not step.all_decode):
+        elif _prefill_mfma_ok(qkv, d, page_size) and not step.all_decode:
             kind = "prefill"
         else:
             kind = "generic"
@@ -388,12 +384,24 @@ def _attention_kernel(qkv: torch.Tensor, nh: int, nkv: int, d: int, page_size: i
     return kind, mfma
 
 
+def _plan_now(step, planner: AttentionPlanner, device: torch.device) -> StepPlan:
+    """A plan made on the spot from the step's host lengths (callers outside a model: tests,
+    probes); a model's steps bring theirs, made by the step builder."""
+    lengths = getattr(step, "lengths", None)
+    if lengths is None:
+        raise KernelError("attention: the step brings neither a plan nor its host lengths")
+    host = planner.plan(lengths)
+    arrays = {k: torch.from_numpy(v).to(device) for k, v in host.arrays.items()}
+    return StepPlan(arrays, host.values)
+
+
 def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                    cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
                    positions: torch.Tensor, slots: Optional[torch.Tensor],
                    k_pages: torch.Tensor, v_pages: torch.Tensor, page_size: int,
                    block_tables: torch.Tensor, step, scale: float,
-                   window: Optional[int] = None, write_kv: bool = True) -> torch.Tensor:
+                   window: Optional[int] = None, write_kv: bool = True,
+                   plan: Optional[StepPlan] = None) -> torch.Tensor:
     """``rope_kv_write`` followed by ``paged_attention``.  A decode batch that takes the
     matrix-core decode kernel does both in that kernel when the whole head is rotated and is
     64, 128 or 256 wide (or nothing is rotated); ``qkv`` is then left unrotated."""
@@ -410,26 +418,30 @@ def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
         if write_kv and slots is None:
             raise KernelError("rope_attention: a cache write needs slots")
         return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
-                               scale, window,
+                               scale, window, plan=plan,
                                rope=(cos, sin, positions, slots if write_kv else None))
     rope_kv_write(qkv, nh, nkv, d, cos, sin, positions, slots, k_pages, v_pages, page_size,
                   write_kv=write_kv)
     return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
-                           scale, window)
+                           scale, window, plan=plan)
 
 
 def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                     k_pages: torch.Tensor, v_pages: torch.Tensor, page_size: int,
                     block_tables: torch.Tensor, step, scale: float,
                     window: Optional[int] = None, force: Optional[str] = None,
-                    rope: Optional[tuple] = None) -> torch.Tensor:
+                    rope: Optional[tuple] = None, plan: Optional[StepPlan] = None
+                    ) -> torch.Tensor:
     """Attention of the step's new tokens over the paged cache -> ``(T, nh * d)``.
 
     ``qkv`` holds the rotated queries in its first ``nh * d`` columns; K and V of the new
     tokens are already in the pages.  ``step`` is the ``StepContext`` (token and sequence
-    metadata on the device).  The kernel is chosen from the shape of the batch: every
-    sequence brings one token -> decode kernel; bfloat16 with multi-token sequences ->
-    matrix-core prefill kernel; float32, or sizes those kernels refuse -> generic kernel.
+    metadata on the device), ``plan`` what an ``AttentionPlanner`` made for it (made on the
+    spot from ``step.lengths`` when absent).  The kernel is chosen from the shape of the
+    batch: every sequence brings one token -> decode kernel; bfloat16 with multi-token
+    sequences -> matrix-core prefill kernel (single tokens that lead the step beside them ->
+    decode kernel); float32, or sizes those kernels refuse -> generic kernel.  How a sequence's
+    keys are cut (decode partitions, tile form, key runs) follows from its own lengths alone.
     ``force`` names one of 'generic', 'decode', 'prefill' for tests.  ``rope`` (from
     ``rope_attention`` only): ``(cos, sin, positions, slots)`` for the matrix-core decode kernel
     to rotate and store the step's tokens itself."""
@@ -460,13 +472,27 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     kind, mfma = _attention_kernel(qkv, nh, nkv, d, page_size, step, force)
     if rope is not None and not mfma:
         raise KernelError("attention: only the matrix-core decode kernel rotates and stores")
-    def decode(S: int, max_context: int, matrix: bool, splits: Optional[int]) -> None:
+    if kind == "generic":
+        lib.call("rlis_attn_generic", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(), nh * d,
+                 k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,
+                 _i32(step.seq_of_token, "seq_of_token", T), _i32(step.positions, "positions", T),
+                 T, nh, nkv, d, page_size, float(scale), win, stream)
+        return out
+    if kind not in ("decode", "prefill"):
+        raise KernelError(f"attention: unknown kernel '{kind}'")
+    if plan is None or force == "prefill":
+        planner = AttentionPlanner(nh, nkv, d, matrix=qkv.dtype == torch.bfloat16,
+                                   singles_apart=force is None and SPLIT_MIXED_ATTENTION
+                                   and DECODE_ATTENTION != "vector")
+        plan = _plan_now(step, planner, qkv.device)
+
+    def decode(S: int, depth: int, matrix: bool) -> None:
         """The first S sequences, one token each (their token rows are the first S too)."""
-        splits = splits or decode_splits(S, nkv, nh // nkv, max_context)
+        from . import attention_plan as ap
         part_ml = part_acc = None
-        if splits > 1:
-            part_ml = torch.empty((S, nh, splits, 2), dtype=torch.float32, device=qkv.device)
-            part_acc = torch.empty((S, nh, splits, d), dtype=torch.float32, device=qkv.device)
+        if depth > 1:
+            part_ml = torch.empty((S, nh, depth, 2), dtype=torch.float32, device=qkv.device)
+            part_acc = torch.empty((S, nh, depth, d), dtype=torch.float32, device=qkv.device)
         ml_ptr = None if part_ml is None else part_ml.data_ptr()
         acc_ptr = None if part_acc is None else part_acc.data_ptr()
         if matrix:
@@ -482,76 +508,68 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
             lib.call("rlis_attn_decode_mfma", qkv.data_ptr(), q_stride, out.data_ptr(), nh * d,
                      ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
                      block_tables.data_ptr(), max_pages, _i32(step.ctx_lens, "ctx_lens", S), S,
-                     nh, nkv, d, page_size, win, float(scale), splits, cos_p, sin_p, rot, pos_p,
-                     slots_p, nh * d, (nh + nkv) * d, stream)
+                     nh, nkv, d, page_size, win, float(scale), depth, ap.DECODE_PART_KEYS,
+                     ap.DECODE_MAX_PARTS, cos_p, sin_p, rot, pos_p, slots_p, nh * d,
+                     (nh + nkv) * d, stream)
         else:
             lib.call("rlis_attn_decode", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(),
                      nh * d, ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
                      block_tables.data_ptr(), max_pages, _i32(step.ctx_lens, "ctx_lens", S), None,
-                     S, nh, nkv, d, page_size, float(scale), win, splits, stream)
+                     S, nh, nkv, d, page_size, float(scale), win, depth, ap.DECODE_PART_KEYS,
+                     ap.DECODE_MAX_PARTS, stream)
 
     if kind == "decode":
         if not step.all_decode:
             raise KernelError("attention: the decode kernel needs one token per sequence")
-        decode(step.num_seqs, step.max_context, mfma, step.decode_splits)
-    elif kind == "prefill":
-        if qkv.dtype != torch.bfloat16:
-            raise KernelError("attention: the matrix-core prefill kernel is bfloat16 only")
-        tile_map, num_tiles = step.tile_map, step.num_tiles
-        # Single tokens beside portions of prompts: the step lists them first, and the decode
-        # kernel reads their keys and values once for the whole group of heads, where a
-        # 64-query tile of the prefill kernel would walk the context for one query per head.
-        singles = getattr(step, "num_single", 0) if force is None and SPLIT_MIXED_ATTENTION else 0
-        row0 = 0                      # the first row that the prefill kernel's tiles cover
-        if singles and _decode_mfma_ok(qkv, nh, nkv, d, page_size):
-            decode(singles, step.max_single_context, True, None)
-            tile_map, num_tiles, row0 = step.multi_tile_map, step.num_multi_tiles, singles
-        # Tiles of 128 queries (two query blocks per wave, half the LDS traffic per flop) where
-        # they are plenty, or where the walks over keys are long (few such tiles still fill the
-        # chip then, their keys cut into runs).  The step brings them for the same sequences.
-        tile_queries = 64
-        wide = getattr(step, "wide_multi_tile_map" if tile_map is not step.tile_map
-                       else "wide_tile_map", None)
-        if wide is not None and d <= 128:
-            groups = wide.numel() // 2 * nh
-            cached = step.max_context - getattr(step, "max_new", 0)
-            # (measured: up to head size 64 the smaller tiles hold out to 5/3 as many groups)
-            enough = PREFILL_WIDE_MIN_GROUPS if d > 64 else PREFILL_WIDE_MIN_GROUPS * 5 // 3
-            if groups >= enough or (PREFILL_WIDE_MIN_GROUPS < (1 << 30) and (
-                    step.max_context >= 4096 or cached >= 2048)):
-                tile_map, num_tiles, tile_queries = wide, wide.numel() // 2, 128
-        if num_tiles:
-            lib.ensure_attention_unit(d)
-            # Few tiles with long walks over cached keys (a portion of a long prompt): the keys
-            # of every tile are cut into runs, one workgroup each, and merged afterwards.
-            splits = getattr(step, "prefill_splits", None)
-            if splits is None:
-                # as many runs as keep every compute unit's resident workgroups in one round
-                # (4 of them up to head size 64, 3 with 128-query tiles, 2 beyond)
-                splits, groups = 1, num_tiles * nh
-                if groups <= PREFILL_SPLIT_UNITS:
-                    resident = 2 if d > 64 else (3 if tile_queries == 128 else 4)
-                    splits = max(1, min(PREFILL_SPLIT_UNITS * resident // groups,
-                                        step.max_context // PREFILL_SPLIT_MIN_KEYS, 16))
-            part_ml = part_acc = None
-            if splits > 1:
-                part_ml = torch.empty((T - row0, nh, splits, 2), dtype=torch.float32, device=qkv.device)
-                part_acc = torch.empty((T - row0, nh, splits, d), dtype=torch.float32, device=qkv.device)
-            lib.call("rlis_attn_prefill_mfma", qkv.data_ptr(), q_stride, out.data_ptr(), nh * d,
-                     k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,
-                     _i32(step.cu_seqlens, "cu_seqlens", step.num_seqs + 1),
-                     _i32(step.start_pos, "start_pos", step.num_seqs),
-                     _i32(tile_map, "tile_map", 2 * num_tiles), num_tiles, nh, nkv, d,
-                     page_size, win, float(scale), tile_queries, splits, row0, T - row0,
-                     None if part_ml is None else part_ml.data_ptr(),
-                     None if part_acc is None else part_acc.data_ptr(), stream)
-    elif kind == "generic":
-        lib.call("rlis_attn_generic", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(), nh * d,
+        if plan.value("num_decode") != step.num_seqs:
+            raise KernelError("attention: the plan is not one of a step of single tokens")
+        decode(step.num_seqs, plan.value("decode_depth"), mfma)
+        return out
+    if qkv.dtype != torch.bfloat16:
+        raise KernelError("attention: the matrix-core prefill kernel is bfloat16 only")
+    if not _prefill_mfma_ok(qkv, d, page_size):
+        raise KernelError(f"attention: the matrix-core prefill kernel takes head sizes in steps "
+                          f"of 16 up to 256 and pages of a power of two from 8 on, not head size "
+                          f"{d} with pages of {page_size}")
+    # Single tokens beside portions of prompts: the step lists them first, and the decode
+    # kernel reads their keys and values once for the whole group of heads, where a tile of the
+    # prefill kernel would walk the context for one query per head.
+    singles = plan.value("num_decode")
+    if singles:
+        if not _decode_mfma_ok(qkv, nh, nkv, d, page_size):
+            raise KernelError("attention: the plan sends single tokens to the matrix-core "
+                              "decode kernel, which does not take this layout")
+        decode(singles, plan.value("decode_depth"), True)
+    row0, max_runs = plan.value("tile_row0"), plan.value("max_runs")
+    part_ml = part_acc = None
+    if max_runs > 1:
+        part_ml = torch.empty((T - row0, nh, max_runs, 2), dtype=torch.float32, device=qkv.device)
+        part_acc = torch.empty((T - row0, nh, max_runs, d), dtype=torch.float32, device=qkv.device)
+    ml_ptr = None if part_ml is None else part_ml.data_ptr()
+    acc_ptr = None if part_acc is None else part_acc.data_ptr()
+    launched = False
+    # Tiles of 64 queries, and tiles of 128 (two query blocks per wave, half the LDS traffic per
+    # flop) for the sequences whose own lengths ask for them.
+    for tile, name in ((64, "units64"), (128, "units128")):
+        n = plan.value("num_" + name)
+        if not n:
+            continue
+        lib.ensure_attention_unit(d)
+        launched = True
+        lib.call("rlis_attn_prefill_mfma", qkv.data_ptr(), q_stride, out.data_ptr(), nh * d,
                  k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,
-                 _i32(step.seq_of_token, "seq_of_token", T), _i32(step.positions, "positions", T),
-                 T, nh, nkv, d, page_size, float(scale), win, stream)
-    else:
-        raise KernelError(f"attention: unknown kernel '{kind}'")
+                 _i32(step.cu_seqlens, "cu_seqlens", step.num_seqs + 1),
+                 _i32(step.start_pos, "start_pos", step.num_seqs),
+                 _i32(plan[name], name, 4 * n), n, nh, nkv, d, page_size, win, float(scale), tile,
+                 max_runs, row0, ml_ptr, acc_ptr, stream)
+    if not launched and T > row0:
+        raise KernelError("attention: the plan holds no tiles for the step's portions")
+    if launched and max_runs > 1:
+        # the runs of a sequence's tiles, merged as the decode kernel's partitions are
+        lib.call("rlis_attn_reduce_rows", out.data_ptr(), nh * d, ml_ptr, acc_ptr,
+                 _i32(step.seq_of_token, "seq_of_token", T),
+                 _i32(plan["seq_runs"], "seq_runs", step.num_seqs), row0, T - row0, nh, d,
+                 max_runs, stream)
     return out
 
 
@@ -579,6 +597,6 @@ def sample_rows(logits: torch.Tensor, keys: torch.Tensor, inv_temps: torch.Tenso
     return out
 
 
-__all__ = ["KernelError", "add_residual", "add_rmsnorm", "copy_pages", "decode_splits", "embed",
-           "linear", "linear_swiglu", "norm_linear", "paged_attention", "rope_attention",
-           "rope_kv_write", "sample_rows", "swiglu"]
+__all__ = ["AttentionPlanner", "KernelError", "add_residual", "add_rmsnorm", "attention_planner",
+           "copy_pages", "embed", "linear", "linear_swiglu", "norm_linear", "paged_attention",
+           "rope_attention", "rope_kv_write", "sample_rows", "swiglu"]

@@ -58,8 +58,14 @@ class PagedAttention(Mixer):
         if self.position.rot_dim > self.head_dim:
             raise ValueError("attention: the rotated width exceeds the head size")
 
+        self.planner = ops.attention_planner(self.num_heads, self.num_kv_heads, self.head_dim,
+                                             self.act_dtype)
+
     def cache_request(self) -> CacheRequest:
-        return CacheRequest(self.num_kv_heads, self.head_dim, self.window)
+        return CacheRequest.kv(self.num_kv_heads, self.head_dim, self.window)
+
+    def step_planner(self):
+        return self.planner
 
     def forward(self, x: Any, step: Any, binding: CacheBinding) -> torch.Tensor:
         group = step.groups[binding.group]
@@ -71,5 +77,5 @@ class PagedAttention(Mixer):
                                  self.position.cos, self.position.sin, step.positions,
                                  group.slots, binding.k_pages, binding.v_pages, group.page_size,
                                  group.block_tables, step, self.scale, self.window,
-                                 write_kv=binding.writes)
+                                 write_kv=binding.writes, plan=step.plans.get(self.planner.key()))
         return ops.linear(out, self.w_o, self.act_dtype, partials=True)

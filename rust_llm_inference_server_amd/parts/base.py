@@ -22,6 +22,8 @@ from typing import Any, Callable, Dict, List, Optional, Tuple, Type
 
 import torch
 
+from ..stepplan import HostPlan, StepLengths, StepPlan, StepPlanner  # noqa: F401 (re-exported)
+
 
 # --------------------------------------------------------------------------- specs
 @dataclass(frozen=True)
@@ -41,35 +43,86 @@ class PartSpec:
     params: Dict[str, Any] = field(default_factory=dict)
 
 
+PAGE = -1     # in a PageArray's shape: the axis that is as long as a page has positions
+
+
+@dataclass(frozen=True)
+class PageArray:
+    """One array a mixer keeps per page: its name and the shape of one page, in which ``PAGE``
+    marks the axis of positions.  Keys of 8 heads of 64 are ``("k", (8, PAGE, 64))``; one latent
+    vector of 96 numbers per position is ``("latent", (PAGE, 96))``."""
+
+    name: str
+    shape: Tuple[int, ...]
+
+    def __post_init__(self):
+        if self.shape.count(PAGE) != 1 or any(n <= 0 for n in self.shape if n != PAGE):
+            raise ValueError(f"page array '{self.name}': shape {self.shape} needs positive sizes "
+                             "and the position axis exactly once")
+
+    def page_shape(self, page_size: int) -> Tuple[int, ...]:
+        return tuple(page_size if n == PAGE else n for n in self.shape)
+
+    def elements_per_token(self) -> int:
+        n = 1
+        for x in self.shape:
+            n *= 1 if x == PAGE else x
+        return n
+
+
 @dataclass(frozen=True)
 class CacheRequest:
-    """What a mixer needs from the paged cache: keys and values of ``num_kv_heads`` heads of
-    ``head_dim`` for every earlier position (``window`` None) or for the last ``window``
-    positions only.  Mixers with equal requests share a page group."""
+    """What a mixer keeps in pages for every cached position: a kind of its own, given as the
+    arrays of one page (each in the activation dtype), for every earlier position (``window``
+    None) or for the last ``window`` positions only.  Mixers with equal requests share a page
+    group; the pools are allocated from the request, so a mixer that caches something else than
+    keys and values names its own arrays.  ``CacheRequest.kv`` is the kind attention uses."""
 
-    num_kv_heads: int
-    head_dim: int
+    arrays: Tuple[PageArray, ...]
     window: Optional[int] = None
 
-    def group_key(self) -> Tuple[int, int, Optional[int]]:
-        return (self.num_kv_heads, self.head_dim, self.window)
+    def __post_init__(self):
+        names = [a.name for a in self.arrays]
+        if not names or len(set(names)) != len(names):
+            raise ValueError(f"a cache request needs arrays with distinct names, got {names}")
+
+    @classmethod
+    def kv(cls, num_kv_heads: int, head_dim: int, window: Optional[int] = None) -> "CacheRequest":
+        """Keys ``[kv head][position][d]`` and values ``[kv head][d][position]`` (values
+        transposed inside a page, so that both attention kernels read each as it lies)."""
+        return cls((PageArray("k", (num_kv_heads, PAGE, head_dim)),
+                    PageArray("v", (num_kv_heads, head_dim, PAGE))), window)
+
+    def group_key(self) -> Tuple[Any, ...]:
+        return (self.arrays, self.window)
+
+    def elements_per_token(self) -> int:
+        return sum(a.elements_per_token() for a in self.arrays)
 
 
 @dataclass
 class CacheBinding:
     """Where one run of a mixer keeps its memory of the past.
 
-    ``k_pages``/``v_pages`` are this run's slices of its group's page pool, ``group`` indexes
-    ``StepContext.groups`` (block tables and slots of that group).  ``writes`` is false when
-    the run reads the cache another run has written in the same step.  ``state`` is the
-    run's slice of the fixed-size per-request state buffer, ``(num_slots, state_bytes)``
-    uint8, or None when the mixer asked for none."""
+    ``pages`` maps each array name of the mixer's cache request to this run's slice of its
+    group's pool, ``(num_pages, *page shape)``; ``group`` indexes ``StepContext.groups`` (block
+    tables and slots of that group).  ``writes`` is false when the run reads the cache another
+    run has written in the same step.  ``state`` is the run's slice of the fixed-size
+    per-request state buffer, ``(num_slots, state_bytes)`` uint8, or None when the mixer asked
+    for none."""
 
     group: int = -1
-    k_pages: Optional[torch.Tensor] = None
-    v_pages: Optional[torch.Tensor] = None
+    pages: Dict[str, torch.Tensor] = field(default_factory=dict)
     writes: bool = True
     state: Optional[torch.Tensor] = None
+
+    @property
+    def k_pages(self) -> Optional[torch.Tensor]:
+        return self.pages.get("k")
+
+    @property
+    def v_pages(self) -> Optional[torch.Tensor]:
+        return self.pages.get("v")
 
 
 @dataclass
@@ -223,12 +276,16 @@ class Mixer(Part):
     ``cache_request()`` says what the mixer keeps in pages (None: nothing);
     ``state_bytes()`` how many bytes of fixed-size state it keeps per request (0: none).  A
     mixer with state must leave, after a step, the state as it is after the last token the
-    step brought for that request."""
+    step brought for that request.  ``step_planner()`` names the host-side planning its kernels
+    need per step (None: the common metadata is enough)."""
 
     # True when forward takes ``x`` as a NormedInput (and projects it with ``project``).
     takes_normed_input = False
 
     def cache_request(self) -> Optional[CacheRequest]:
+        return None
+
+    def step_planner(self) -> Optional[StepPlanner]:
         return None
 
     def state_bytes(self) -> int:
@@ -275,14 +332,19 @@ class ResidualStream:
     """The residual sum, kept in 32-bit, plus a delta that has not been added yet.
 
     A block's output is left *pending* so that the next norm can add it and normalise in one
-    pass over the row; the sum itself is always formed and stored in float32."""
+    pass over the row; the sum itself is always formed and stored in float32.  A block's output
+    joins the sum rounded once to the activation dtype: a delta that arrives as a stack of
+    float32 partial sums is added up and, in a bfloat16 model, rounded to bfloat16 first
+    (``round_parts``), as a delta that arrives whole in bfloat16 was by its kernel, so that the
+    rounding does not depend on which kernel a batch's size chose."""
 
-    __slots__ = ("x", "pending")
+    __slots__ = ("x", "pending", "round_parts")
 
-    def __init__(self, x: torch.Tensor):
+    def __init__(self, x: torch.Tensor, act_dtype: torch.dtype = torch.float32):
         assert x.dtype == torch.float32
         self.x = x
         self.pending: Optional[torch.Tensor] = None
+        self.round_parts = act_dtype == torch.bfloat16
 
     def add(self, delta: torch.Tensor) -> None:
         if self.pending is not None:
@@ -293,6 +355,6 @@ class ResidualStream:
         """Fold a pending delta into the residual and return the residual."""
         if self.pending is not None:
             from .. import ops
-            ops.add_residual(self.x, self.pending)
+            ops.add_residual(self.x, self.pending, round_parts=self.round_parts)
             self.pending = None
         return self.x

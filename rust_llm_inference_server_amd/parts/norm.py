@@ -29,11 +29,12 @@ class RMSNorm(Norm):
 
     def forward(self, stream: ResidualStream) -> torch.Tensor:
         delta, stream.pending = stream.pending, None
-        return ops.add_rmsnorm(stream.x, delta, self.weight, self.eps, self.out_dtype)
+        return ops.add_rmsnorm(stream.x, delta, self.weight, self.eps, self.out_dtype,
+                               round_parts=stream.round_parts)
 
     def forward_rows(self, stream: ResidualStream, rows: torch.Tensor) -> torch.Tensor:
         return ops.add_rmsnorm(stream.x, stream.pending, self.weight, self.eps, self.out_dtype,
-                               rows=rows)
+                               rows=rows, round_parts=stream.round_parts)
 
     def fused_linear(self, stream: ResidualStream, w: torch.Tensor, out_dtype: torch.dtype,
                      gated: bool, rows: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
@@ -41,7 +42,7 @@ class RMSNorm(Norm):
         if self.out_dtype != torch.bfloat16 or not ops.can_fuse_norm_linear(stream.x, w, count):
             return None
         y, total = ops.norm_linear(stream.x, stream.pending, self.weight, self.eps, w, out_dtype,
-                                   gated=gated, rows=rows)
+                                   gated=gated, rows=rows, round_parts=stream.round_parts)
         if rows is None:
             stream.x, stream.pending = total, None
         return y

@@ -16,11 +16,12 @@ def embed(ids, table):
     return table[ids.long()].to(torch.float32)
 
 
-def add_residual(resid, delta):
+def add_residual(resid, delta, round_parts=False):
     resid += delta.to(torch.float32)
 
 
-def add_rmsnorm(resid, delta, weight, eps, out_dtype, rows=None, write_resid=True):
+def add_rmsnorm(resid, delta, weight, eps, out_dtype, rows=None, write_resid=True,
+                round_parts=False):
     x = resid if delta is None else resid + delta.to(torch.float32)
     if rows is not None:
         x = x[rows.long()]
@@ -77,12 +78,13 @@ def copy_pages(pages, src, dst):
         pages[:, d] = pages[:, s]
 
 
-def decode_splits(num_seqs, num_kv_heads, group, max_context):
-    return 1
+def attention_planner(num_heads, num_kv_heads, head_dim, dtype):
+    from rust_llm_inference_server_amd.ops.attention_plan import AttentionPlanner
+    return AttentionPlanner(num_heads, num_kv_heads, head_dim, matrix=dtype == torch.bfloat16)
 
 
 def paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, page_size,
-                    block_tables, step, scale, window=None, force=None):
+                    block_tables, step, scale, window=None, force=None, plan=None):
     T = qkv.shape[0]
     nh, nkv, d = num_heads, num_kv_heads, head_dim
     g = nh // nkv
@@ -104,7 +106,8 @@ def paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, pa
 
 
 def rope_attention(qkv, num_heads, num_kv_heads, head_dim, cos, sin, positions, slots, k_pages,
-                   v_pages, page_size, block_tables, step, scale, window=None, write_kv=True):
+                   v_pages, page_size, block_tables, step, scale, window=None, write_kv=True,
+                   plan=None):
     rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, cos, sin, positions, slots, k_pages,
                   v_pages, page_size, write_kv=write_kv)
     return paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, page_size,
@@ -144,6 +147,6 @@ def install(monkeypatch) -> None:
     import rust_llm_inference_server_amd.engine.runner as runner
     for name in ("embed", "add_residual", "add_rmsnorm", "swiglu", "linear", "linear_swiglu",
                  "can_fuse_norm_linear", "rope_kv_write", "rope_attention",
-                 "copy_pages", "decode_splits", "paged_attention", "sample_rows"):
+                 "copy_pages", "attention_planner", "paged_attention", "sample_rows"):
         monkeypatch.setattr(ops, name, globals()[name])
     monkeypatch.setattr(runner, "default_device", lambda: torch.device("cpu"))

@@ -1,12 +1,15 @@
 """Each kernel alone against a plain float32 PyTorch reference of the same op, at sizes other
 than the engine's test models: widths and vocabularies that are no power of two, head sizes
 in steps of 16, odd head counts and groups, page sizes 8 to 64."""
+import contextlib
 import math
 
+import numpy as np
 import pytest
 import torch
 
 import plain_llama as plain
+from rust_llm_inference_server_amd.stepplan import StepLengths
 
 pytestmark = pytest.mark.gpu
 
@@ -362,6 +365,30 @@ class FakeStep:
     pass
 
 
+@contextlib.contextmanager
+def attention_constants(**values):
+    """Run with other constants in the attention planner (partition sizes, tile forms, key
+    runs): every combination must give the same numbers up to rounding."""
+    from rust_llm_inference_server_amd.ops import attention_plan as ap
+    old = {k: getattr(ap, k) for k in values}
+    try:
+        for k, v in values.items():
+            setattr(ap, k, v)
+        yield
+    finally:
+        for k, v in old.items():
+            setattr(ap, k, v)
+
+
+def key_runs(n):
+    """Constants that cut every multi-token sequence's tiles into n runs where it has the keys."""
+    return dict(PREFILL_SPLIT_UNITS=1 << 20, PREFILL_SPLIT_MIN_KEYS=1, PREFILL_MAX_RUNS=n)
+
+
+# partitions of the decode kernels: (keys per partition, most partitions)
+DECODE_CUTS = [(1024, 16), (256, 16), (256, 2)]
+
+
 def paged_case(lens_cached, lens_new, nh, nkv, d, ps, dtype, seed=0, q_scale=1.0):
     """A batch of sequences with scattered pages.  Returns (qkv, k_pages, v_pages, tables,
     step, per-sequence K and V in float32, q in float32)."""
@@ -401,21 +428,16 @@ def paged_case(lens_cached, lens_new, nh, nkv, d, ps, dtype, seed=0, q_scale=1.0
     step.ctx_lens = i32(totals)
     step.positions = i32([c + i for c, n in zip(lens_cached, lens_new) for i in range(n)])
     step.seq_of_token = i32([s for s, n in enumerate(lens_new) for _ in range(n)])
-    tiles = [x for s, n in enumerate(lens_new) for qb in range(0, n, 64) for x in (s, qb)]
-    step.tile_map, step.num_tiles = i32(tiles), len(tiles) // 2
     step.max_context, step.max_new = max(totals), max(lens_new)
     step.all_decode = all(n == 1 for n in lens_new)
-    step.decode_splits = None
-    wide = [x for s, n in enumerate(lens_new) for qb in range(0, n, 128) for x in (s, qb)]
-    step.wide_tile_map = i32(wide)
-    # single tokens that lead the batch, as the engine's steps order them
+    # single tokens that lead the batch, as the engine's steps order them (the kernels' work
+    # lists are planned from these host lengths at the call)
     lead = next((i for i, n in enumerate(lens_new) if n != 1), S)
-    if all(n > 1 for n in lens_new[lead:]):
-        multi = [x for s, n in enumerate(lens_new) if s >= lead for qb in range(0, n, 64) for x in (s, qb)]
-        step.num_single, step.max_single_context = lead, max(totals[:lead], default=0)
-        step.multi_tile_map, step.num_multi_tiles = i32(multi), len(multi) // 2
-        step.wide_multi_tile_map = i32([x for s, n in enumerate(lens_new) if s >= lead
-                                        for qb in range(0, n, 128) for x in (s, qb)])
+    if not all(n > 1 for n in lens_new[lead:]):
+        lead = 0
+    step.num_single = lead
+    step.lengths = StepLengths(np.asarray(lens_cached, dtype=np.int64),
+                               np.asarray(lens_new, dtype=np.int64), lead, ps)
     return (qkv.to(DEV), k_pages.to(DEV), v_pages.to(DEV), bt.to(DEV), step, ks, vs, cu)
 
 
@@ -468,7 +490,7 @@ def test_attention_single_tokens_beside_portions(ops, nh, nkv, d, ps, window):
     new = [1, 1, 1, 1, 33, 70, 2, 129, 64]
     scale = 1.0 / math.sqrt(d)
     qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=nh + 1)
-    assert step.num_single == 4 and step.num_multi_tiles == 8
+    assert step.num_single == 4
     want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, window)
     got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window)
     torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
@@ -498,12 +520,8 @@ def test_attention_prefill_tiles_of_128_queries(ops, nh, nkv, d, ps, window):
     qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=nh + 2)
     want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, window)
     narrow = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window)
-    old = ops.PREFILL_WIDE_MIN_GROUPS
-    try:
-        ops.PREFILL_WIDE_MIN_GROUPS = 0
+    with attention_constants(PREFILL_WIDE_MIN_GROUPS=0):
         got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window)
-    finally:
-        ops.PREFILL_WIDE_MIN_GROUPS = old
     torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
     torch.testing.assert_close(got.float(), narrow.float(), atol=2e-2, rtol=2e-2)
 
@@ -523,17 +541,12 @@ def test_attention_prefill_with_keys_cut_into_runs(ops, nh, nkv, d, ps, window, 
     scale = 1.0 / math.sqrt(d)
     qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=nh + 3)
     want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, window)
-    step.prefill_splits = splits
-    old = ops.PREFILL_WIDE_MIN_GROUPS
-    try:
-        for wide in (False, True):
-            ops.PREFILL_WIDE_MIN_GROUPS = 0 if wide else 1 << 30
+    for wide in (False, True):
+        with attention_constants(PREFILL_WIDE_MIN_GROUPS=0 if wide else 1 << 30, **key_runs(splits)):
             got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window)
             torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
             whole = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window, force="prefill")
             torch.testing.assert_close(whole.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
-    finally:
-        ops.PREFILL_WIDE_MIN_GROUPS = old
 
 
 @pytest.mark.parametrize("kind,dtype", kinds_and_dtypes("generic", "prefill", "decode"))
@@ -558,11 +571,10 @@ def test_attention_decode(ops, dtype, nh, nkv, d, ps, decode_kind):
     scale = 1.0 / math.sqrt(d)
     qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=d)
     want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, None)
-    for splits in (1, 3, 8):
-        step.decode_splits = splits
-        got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, None, force="decode")
+    for part_keys, max_parts in DECODE_CUTS:
+        with attention_constants(DECODE_PART_KEYS=part_keys, DECODE_MAX_PARTS=max_parts):
+            got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, None, force="decode")
         torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
-    step.decode_splits = None
     got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, None)
     torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
 
@@ -589,16 +601,16 @@ def test_rope_attention_decode_in_one_kernel(ops, nh, nkv, d, ps, rotate, window
     slots = torch.tensor([int(tables[s, (l - 1) // ps]) * ps + (l - 1) % ps for s, l in enumerate(lens)],
                          dtype=torch.int32, device=DEV)
     for write_kv in (True, False):
-        for splits in (None, 1, 3, 8):
-            step.decode_splits = splits
+        for part_keys, max_parts in DECODE_CUTS:
             results = []
             for fused in (False, True):
                 q2, k2, v2 = qkv.clone(), kp.clone(), vp.clone()
                 old = ops.FUSE_ROPE_DECODE
                 try:
                     ops.FUSE_ROPE_DECODE = fused
-                    out = ops.rope_attention(q2, nh, nkv, d, cos, sin, step.positions, slots, k2, v2,
-                                             ps, bt, step, scale, window, write_kv=write_kv)
+                    with attention_constants(DECODE_PART_KEYS=part_keys, DECODE_MAX_PARTS=max_parts):
+                        out = ops.rope_attention(q2, nh, nkv, d, cos, sin, step.positions, slots, k2,
+                                                 v2, ps, bt, step, scale, window, write_kv=write_kv)
                 finally:
                     ops.FUSE_ROPE_DECODE = old
                 results.append((out.float().cpu(), k2.float().cpu(), v2.cpu()))
@@ -608,7 +620,6 @@ def test_rope_attention_decode_in_one_kernel(ops, nh, nkv, d, ps, rotate, window
             assert torch.equal(v1, v0)
             if not write_kv:
                 assert torch.equal(k1, kp.float().cpu()) and torch.equal(v1, vp.cpu())
-    step.decode_splits = None
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -621,9 +632,9 @@ def test_attention_decode_long_split(ops, dtype, decode_kind):
     scale = 1.0 / math.sqrt(d)
     qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=9)
     want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, None)
-    for splits in (None, 36):
-        step.decode_splits = splits
-        got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, None, force="decode")
+    for part_keys, max_parts in ((1024, 16), (256, 36), (256, 5)):
+        with attention_constants(DECODE_PART_KEYS=part_keys, DECODE_MAX_PARTS=max_parts):
+            got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, None, force="decode")
         torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
 
 
@@ -790,9 +801,9 @@ def test_pages_past_two_to_the_31_elements(ops, dtype):
     # single tokens: the decode kernels, with and without the rotation and cache write inside
     lens = [c + n for c, n in zip(cached, new)]
     dq, _, _, _, dstep, *_ = paged_case([l - 1 for l in lens], [1] * len(lens), nh, nkv, d, ps, dtype, seed=3)
-    dstep.decode_splits = 3
-    a = ops.paged_attention(dq, nh, nkv, d, kp, vp, ps, bt, dstep, scale, None, force="decode")
-    b = ops.paged_attention(dq, nh, nkv, d, kb, vb, ps, bt_big, dstep, scale, None, force="decode")
+    with attention_constants(DECODE_PART_KEYS=256):
+        a = ops.paged_attention(dq, nh, nkv, d, kp, vp, ps, bt, dstep, scale, None, force="decode")
+        b = ops.paged_attention(dq, nh, nkv, d, kb, vb, ps, bt_big, dstep, scale, None, force="decode")
     assert torch.equal(a, b)
     dslots = torch.tensor([int(tables[s, (l - 1) // ps]) * ps + (l - 1) % ps for s, l in enumerate(lens)],
                           dtype=torch.int32, device=DEV)

@@ -76,17 +76,20 @@ def test_step_layout_puts_single_tokens_first(cpu_ops, tiny_folders):
     runner.step([StepEntry(2, list(range(8)), []), StepEntry(4, [7, 8, 9, 10], [])])
     entries = [StepEntry(1, list(range(10, 43 - 3)), [0, 29]), StepEntry(2, [5], [0]),
                StepEntry(3, list(range(70)), [69]), StepEntry(4, [6], [])]
-    step = build_step(entries, runner.cache, torch.device("cpu"), 256)
+    step = build_step(entries, runner.cache, torch.device("cpu"), 256, model.step_planners)
     assert step.host_order == [1, 3, 0, 2] and step.num_single == 2 and not step.all_decode
     assert step.host_new == [1, 1, 30, 70] and step.host_start_pos == [8, 4, 0, 0]
-    assert step.max_single_context == 9 and step.max_context == 70
+    assert step.max_context == 70
+    assert step.lengths.start.tolist() == [8, 4, 0, 0] and step.lengths.num_single == 2
     assert step.ids.tolist()[:2] == [5, 6] and step.positions.tolist()[:3] == [8, 4, 0]
     assert step.cu_seqlens.tolist() == [0, 1, 2, 32, 102]
     assert step.logit_rows.tolist() == [2, 31, 0, 101]            # entry order, then want order
-    tiles = step.tile_map.reshape(-1, 2).tolist()
-    multi = step.multi_tile_map.reshape(-1, 2).tolist()
-    assert sorted(tiles) == [[0, 0], [1, 0], [2, 0], [3, 0], [3, 64]]
-    assert multi == [[3, 64], [3, 0], [2, 0]] and step.num_multi_tiles == 3
+    # the attention mixer's plan rides along (a float32 model plans no tiles, only the depth of
+    # the decode grid), under the key of its planner
+    (planner,) = model.step_planners
+    plan = step.plans[planner.key()]
+    assert plan.value("num_units64") == 0 and plan.value("decode_depth") == 1
+    assert plan["seq_runs"].tolist() == [1, 1, 1, 1]
     # and the runner's answer does not depend on the order the entries come in
     want = runner.step(entries)
     assert [runner.num_computed(s) for s in (1, 2, 3, 4)] == [30, 9, 70, 5]

@@ -186,8 +186,9 @@ def test_long_prompt_whole_and_in_portions(tmp_path, wide):
         pos += n
     assert pos == len(long_t)
     steps[-1]["end"] = ["r0", "r1"]
-    old, call = ops.PREFILL_WIDE_MIN_GROUPS, ops.lib.call
-    seen = []                                   # (tile_queries, splits) of every prefill launch
+    from rust_llm_inference_server_amd.ops import attention_plan
+    old, call = attention_plan.PREFILL_WIDE_MIN_GROUPS, ops.lib.call
+    seen = []                 # (tile_queries, stride of the runs' results) of every prefill launch
 
     def spy(name, *args):
         if name == "rlis_attn_prefill_mfma":
@@ -195,12 +196,12 @@ def test_long_prompt_whole_and_in_portions(tmp_path, wide):
         return call(name, *args)
 
     try:
-        ops.PREFILL_WIDE_MIN_GROUPS = 0 if wide else 1 << 30
+        attention_plan.PREFILL_WIDE_MIN_GROUPS = 0 if wide else 1 << 30
         ops.lib.call = spy
         runner = make_runner(folder, "bfloat16", 2 * 2624 + 64, page_size=16)
         outputs = traces.replay_in_process(runner, steps)
     finally:
-        ops.PREFILL_WIDE_MIN_GROUPS, ops.lib.call = old, call
+        attention_plan.PREFILL_WIDE_MIN_GROUPS, ops.lib.call = old, call
     assert any(runs > 1 for _, runs in seen) and any(runs == 1 for _, runs in seen)
     assert {tq for tq, _ in seen} == ({128} if wide else {64})
     whole = outputs[0]
