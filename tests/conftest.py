@@ -85,3 +85,14 @@ def tiny_folders(tmp_path_factory):
     for i, (name, cfg) in enumerate(TINY.items()):
         out[name] = make_model_folder(tmp_path_factory.mktemp(f"tiny_{name}"), cfg, seed=i)
     return out
+
+
+@pytest.fixture(scope="session")
+def tiny_folders_bf16(tmp_path_factory):
+    """The same models with weights stored in bfloat16: what a bfloat16 engine computes with,
+    so that the plain float32 implementation can run on exactly those numbers."""
+    out = {}
+    for i, (name, cfg) in enumerate(TINY.items()):
+        out[name] = make_model_folder(tmp_path_factory.mktemp(f"tiny16_{name}"), cfg, seed=i,
+                                      dtype=torch.bfloat16)
+    return out

@@ -262,20 +262,25 @@ def argmax(row: torch.Tensor) -> int:
     return best
 
 
-def sample_row(row: torch.Tensor, key: int, inv_t: float) -> int:
-    """One row of the device sampler's host reference (crates/model/src/sampling.rs:84-100):
-    s = x * inv_t + gumbel(key, v) when inv_t > 0 else x; largest s, ties to the lowest id."""
+def sample_scores(row: torch.Tensor, key: int, inv_t: float):
+    """The scores the device sampler compares (crates/model/src/sampling.rs:84-100):
+    s = x * inv_t + gumbel(key, v) when inv_t > 0 else x, float32."""
     import numpy as np
     x = row.to(torch.float32).numpy()
-    if inv_t > 0:
-        v = np.arange(x.shape[0], dtype=np.uint64)
-        h = (np.uint64(key) ^ ((v * np.uint64(0x9E3779B9)) & np.uint64(0xFFFFFFFF))).astype(np.uint64)
-        h = _lowbias32_np(h)
-        u = (np.float32(1.0 / 8388608.0) * ((h >> np.uint64(9)).astype(np.float32) + np.float32(0.5))).astype(np.float32)
-        g = -np.log(-np.log(u, dtype=np.float32), dtype=np.float32)
-        s = (x * np.float32(inv_t)).astype(np.float32) + g
-    else:
-        s = x
+    if not inv_t > 0:
+        return x
+    v = np.arange(x.shape[0], dtype=np.uint64)
+    h = (np.uint64(key) ^ ((v * np.uint64(0x9E3779B9)) & np.uint64(0xFFFFFFFF))).astype(np.uint64)
+    h = _lowbias32_np(h)
+    u = (np.float32(1.0 / 8388608.0) * ((h >> np.uint64(9)).astype(np.float32) + np.float32(0.5))).astype(np.float32)
+    g = -np.log(-np.log(u, dtype=np.float32), dtype=np.float32)
+    return (x * np.float32(inv_t)).astype(np.float32) + g
+
+
+def sample_row(row: torch.Tensor, key: int, inv_t: float) -> int:
+    """One row of the device sampler's host reference: largest score, ties to the lowest id."""
+    import numpy as np
+    s = sample_scores(row, key, inv_t)
     best, best_v = float("-inf"), 2 ** 32 - 1
     top = np.flatnonzero(s == s.max()) if not np.isnan(s).all() else []
     for v in top:

@@ -1,0 +1,102 @@
+"""The attention kernels' per-step plan (``ops/attention_plan.py``), on the host: what a
+sequence gets (tile form, key runs, the depth of the decode grid) follows from its own lengths
+and from constants, never from its neighbours; every tile of every portion is listed once per
+run; and the kernels' partition rule matches the host's."""
+import numpy as np
+import pytest
+
+from rust_llm_inference_server_amd.ops import attention_plan as ap
+from rust_llm_inference_server_amd.stepplan import StepLengths
+
+
+def lengths(cached, new, page_size=16):
+    single = 0
+    for n in new:
+        if n != 1:
+            break
+        single += 1
+    return StepLengths(np.asarray(cached, dtype=np.int64), np.asarray(new, dtype=np.int64), single,
+                       page_size)
+
+
+def units_of(plan, name):
+    return [tuple(u) for u in plan.arrays[name].reshape(-1, 4).tolist()]
+
+
+def test_every_tile_is_listed_once_per_run_and_longest_first():
+    planner = ap.AttentionPlanner(32, 8, 64)
+    cached, new = [10, 300, 0, 40, 3000, 100], [1, 1, 300, 70, 200, 5000]
+    plan = planner.plan(lengths(cached, new))
+    assert plan.values["num_decode"] == 2 and plan.values["tile_row0"] == 2
+    runs = plan.arrays["seq_runs"].tolist()
+    assert runs[:2] == [1, 1]
+    seen = {}
+    for tile, name in ((64, "units64"), (128, "units128")):
+        units = units_of(plan, name)
+        assert len(units) == plan.values["num_" + name]
+        work = []
+        for s, qb, r, nr in units:
+            assert s >= 2 and nr == runs[s] and 0 <= r < nr and qb % tile == 0 and qb < new[s]
+            assert planner.tile_queries(cached[s], new[s]) == tile
+            seen.setdefault((s, qb), []).append(r)
+            work.append(-(-(cached[s] + min(new[s], qb + tile)) // nr))
+        assert work == sorted(work, reverse=True)
+    for s in range(2, 6):
+        tile = planner.tile_queries(cached[s], new[s])
+        for qb in range(0, new[s], tile):
+            assert sorted(seen.pop((s, qb))) == list(range(runs[s]))
+    assert not seen
+    assert plan.values["max_runs"] == max(runs)
+    # the short portion on a long context is cut into runs, the long prompt is not
+    assert runs[4] > 1 and runs[5] == 1
+    assert planner.tile_queries(3000, 200) == 128 and planner.tile_queries(0, 300) == 64
+
+
+def test_a_sequence_is_planned_the_same_alone_and_among_neighbours():
+    rng = np.random.default_rng(0)
+    for nh, nkv, d in ((32, 8, 64), (24, 8, 128), (6, 2, 32), (16, 2, 256)):
+        planner = ap.AttentionPlanner(nh, nkv, d)
+        for _ in range(20):
+            S = int(rng.integers(1, 9))
+            new = sorted((int(rng.choice([1, 1, 2, 17, 64, 200, 513, 3000])) for _ in range(S)),
+                         key=lambda n: n != 1)
+            cached = [int(rng.choice([0, 5, 1023, 1024, 2047, 2048, 4095, 9000])) for _ in range(S)]
+            both = planner.plan(lengths(cached, new))
+            for s in range(S):
+                if new[s] == 1:
+                    continue
+                one = planner.plan(lengths([cached[s]], [new[s]]))
+                assert one.arrays["seq_runs"].tolist() == [both.arrays["seq_runs"][s]]
+                for name in ("units64", "units128"):
+                    mine = sorted((qb, r, nr) for q, qb, r, nr in units_of(both, name) if q == s)
+                    assert mine == sorted((qb, r, nr) for _, qb, r, nr in units_of(one, name))
+
+
+def test_decode_partitions_follow_the_sequence_alone():
+    assert ap.decode_parts(1) == 1 and ap.decode_parts(1024) == 1 and ap.decode_parts(1025) == 2
+    assert ap.decode_parts(16 * 1024) == 16 and ap.decode_parts(16 * 1024 + 1) == 9
+    assert ap.decode_parts(131072) == 16
+    assert ap.decode_depth(700) == 1 and ap.decode_depth(4096) == 4 and ap.decode_depth(1 << 20) == 16
+    for ctx in (1, 999, 1024, 5000, 16384, 16385, 40000, 131072):
+        assert ap.decode_parts(ctx) <= ap.decode_depth(ctx)
+    planner = ap.AttentionPlanner(32, 8, 64)
+    plan = planner.plan(lengths([0, 4999, 20], [1, 1, 1]))
+    assert plan.values["num_decode"] == 3 and plan.values["decode_depth"] == 5
+    assert plan.values["num_units64"] == plan.values["num_units128"] == 0
+    fixed = planner.plan_captured(8, 2048, 16)
+    assert not fixed.arrays and fixed.values["decode_depth"] == 2 and fixed.values["num_decode"] == 8
+
+
+def test_layouts_the_matrix_kernels_do_not_take_plan_no_tiles():
+    # float32, or pages that are no power of two: only the depth of the decode grid is planned
+    for planner, ps in ((ap.AttentionPlanner(4, 1, 16, matrix=False), 16),
+                        (ap.AttentionPlanner(4, 1, 16), 12),
+                        (ap.AttentionPlanner(4, 1, 24), 16)):
+        plan = planner.plan(lengths([5, 0], [1, 40], ps))
+        assert plan.values["num_units64"] == plan.values["num_units128"] == 0
+        assert plan.values["num_decode"] == 0
+    # 17 query heads per KV head are more than the decode kernel takes: single tokens get tiles
+    wide_group = ap.AttentionPlanner(34, 2, 16)
+    plan = wide_group.plan(lengths([5, 0], [1, 40]))
+    assert plan.values["num_decode"] == 0 and plan.values["num_units64"] == 2
+    assert plan.values["tile_row0"] == 0

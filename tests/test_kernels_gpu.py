@@ -658,6 +658,66 @@ def test_attention_finds_a_far_key(ops, dtype, kind, decode_kind):
     torch.testing.assert_close(got[-1, :d].float().cpu(), vs[0][far, 0, :], **tol(dtype, 1e-4, 2e-2))
 
 
+def alone(step, s, cached, new, bt, qkv, cu, ps):
+    """The step, block table and queries of sequence ``s`` of a batch as a batch of its own (same
+    pages)."""
+    one = FakeStep()
+    n, c = new[s], cached[s]
+    one.num_tokens, one.num_seqs = n, 1
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    one.cu_seqlens, one.start_pos, one.ctx_lens = i32([0, n]), i32([c]), i32([c + n])
+    one.positions, one.seq_of_token = i32(list(range(c, c + n))), i32([0] * n)
+    one.max_context, one.max_new, one.all_decode = c + n, n, n == 1
+    one.num_single = 1 if n == 1 else 0
+    one.lengths = StepLengths(np.asarray([c], dtype=np.int64), np.asarray([n], dtype=np.int64),
+                              one.num_single, ps)
+    return one, bt[s:s + 1].contiguous(), qkv[cu[s]:cu[s + 1]].contiguous()
+
+
+@pytest.mark.parametrize("nh,nkv,d,ps", [(32, 8, 64, 16), (24, 8, 128, 16), (6, 2, 32, 8)])
+@pytest.mark.parametrize("window", [None, 700])
+def test_attention_rows_do_not_depend_on_the_neighbours(ops, nh, nkv, d, ps, window):
+    """bfloat16: the rows of a sequence come out bit for bit the same when it is alone in the
+    step as among others, whatever they bring: decode partitions, tile form and key runs follow
+    from its own lengths.  Long contexts beside short ones, portions that take key runs (few
+    tiles on a long context) beside ones that do not, tiles of 128 queries beside tiles of 64."""
+    dtype = torch.bfloat16
+    scale = 1.0 / math.sqrt(d)
+    # single tokens first, as the engine's steps order them; contexts on both sides of 1024,
+    # 2048 and 4096 positions
+    cached = [0, 1023, 1024, 2500, 4200, 0, 3000, 100, 2047, 4000]
+    new = [1, 1, 1, 1, 1, 300, 200, 700, 70, 130]
+    qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=d + 7)
+    assert step.num_single == 5
+    together = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window)
+    want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, window)
+    torch.testing.assert_close(together.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
+    planner = ops.attention_planner(nh, nkv, d, dtype)
+    forms = {planner.tile_queries(c, n) for c, n in zip(cached[5:], new[5:])}
+    runs = {planner.key_runs(c, n, planner.tile_queries(c, n)) for c, n in zip(cached[5:], new[5:])}
+    if d <= 128:
+        assert forms == {64, 128}
+    assert 1 in runs and max(runs) > 1                      # the batch mixes all of it
+    for s in range(len(new)):
+        one, table, q = alone(step, s, cached, new, bt, qkv, cu, ps)
+        got = ops.paged_attention(q, nh, nkv, d, kp, vp, ps, table, one, scale, window)
+        assert torch.equal(got, together[cu[s]:cu[s + 1]]), f"sequence {s}"
+    # the single tokens as a decode step of their own, and in another order
+    order = [3, 0, 4, 2, 1]
+    sub = FakeStep()
+    sub.num_tokens = sub.num_seqs = sub.num_single = 5
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    sub.cu_seqlens, sub.start_pos = i32(list(range(6))), i32([cached[s] for s in order])
+    sub.ctx_lens = i32([cached[s] + 1 for s in order])
+    sub.positions, sub.seq_of_token = sub.start_pos, i32(list(range(5)))
+    sub.max_context, sub.max_new, sub.all_decode = max(cached[:5]) + 1, 1, True
+    sub.lengths = StepLengths(np.asarray([cached[s] for s in order], dtype=np.int64),
+                              np.ones(5, dtype=np.int64), 5, ps)
+    got = ops.paged_attention(qkv[order].contiguous(), nh, nkv, d, kp, vp, ps,
+                              bt[order].contiguous(), sub, scale, window)
+    assert torch.equal(got, together[order])
+
+
 @pytest.mark.parametrize("kind,dtype", kinds_and_dtypes("generic", "prefill", "decode"))
 @pytest.mark.parametrize("window", [5, 64, 100, 300])
 def test_attention_window_edge(ops, dtype, kind, window, decode_kind):

@@ -241,11 +241,21 @@ def register_toy():
             self.weight = ctx.take(join(prefix, "mix.weight")).float()
             self.decay = float(params["decay"])
             self.act_dtype = ctx.act_dtype
+            # With "on_device" a step of one token per request is device work alone (the
+            # state rows are gathered and scattered by the step's slot ids), so that such steps
+            # may be captured into a graph.
+            self.graph_safe = bool(params.get("on_device", False))
 
         def state_bytes(self):
             return 4 * self.size
 
         def forward(self, x, step, binding):
+            if self.graph_safe and step.all_decode:
+                states = binding.state.view(torch.float32)          # (slots, size)
+                slots = step.state_slots[:x.shape[0]].long()
+                new = states.index_select(0, slots) * self.decay + x.float()
+                states.index_copy_(0, slots, new)
+                return (new @ self.weight.t()).to(self.act_dtype)
             out = torch.empty_like(x, dtype=torch.float32)
             begin = 0
             for n, slot in zip(step.host_new, step.host_state_slots):
@@ -320,6 +330,183 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
             mine = torch.stack([got[k][p] for p in range(len(tokens))])
             assert (mine - ref[k]).abs().max().item() < 2e-4, f"{build.__name__} request {k}"
         assert runner.cache.num_free_slots() == 4
+
+
+def test_toy_mixer_with_state_through_captured_decode_steps(tmp_path):
+    """The same toy mixer doing its single-token steps on the device alone, so that the model's
+    decode steps are captured into HIP graphs: every way of cutting, then requests that start
+    with single tokens on state slots that earlier requests left full.  The captured path must
+    clear the slot of a request that starts, keep padding rows off the live slots, and not
+    advance any state while it captures."""
+    from rust_llm_inference_server_amd.engine import ModelRunner, StepEntry, load_model
+    from rust_llm_inference_server_amd.registry import Architecture, register_architecture
+    from rust_llm_inference_server_amd.weights import write_model_folder
+    register_toy()
+    H = 48
+    kinds = ["toy", "attention", "toy"]
+
+    def build_spec(cfg):
+        blocks = []
+        for kind in cfg["mixers"]:
+            if kind == "toy":
+                blocks.append(layer_spec(H, 1, 1, 16, 64, 1e-5, 1e4, None, mixer="toy_running_sum",
+                                         extra={"hidden_size": H, "decay": 0.9, "on_device": True}))
+            else:
+                blocks.append(layer_spec(H, 3, 1, 16, 64, 1e-5, 1e4, None))
+        return toy_spec(blocks, H=H, V=cfg["vocab_size"])
+
+    register_architecture(Architecture("ToyOnDeviceForCausalLM", parse_config=lambda d: d,
+                                       build_spec=build_spec, config_to_dict=lambda c: c))
+    config = {"architectures": ["ToyOnDeviceForCausalLM"], "vocab_size": 97, "mixers": kinds}
+    folder = str(tmp_path / "toy")
+    write_model_folder(folder, config, build_spec(config).tensor_specs(), seed=9)
+    w = plain.read_weights(folder)
+    reqs = traces.random_requests(97, [30, 4, 70, 11, 45, 2], seed=8)
+    ref = {k: plain_running_sum_model(w, t, kinds) for k, t in reqs.items()}
+    for build in (traces.trace_whole, traces.trace_tail, traces.trace_portions, traces.trace_mixed):
+        steps, max_tokens = build(reqs)
+        model = load_model(folder, "float32", max_positions=128)
+        assert model.graph_safe and model.state_bytes == 2 * 4 * H
+        runner = ModelRunner(model, num_pages=max_tokens // 16, page_size=16, max_num_seqs=4)
+        assert runner.use_graphs
+        got = traces.collect(steps, traces.replay_in_process(runner, steps), 97)
+        if build in (traces.trace_tail, traces.trace_mixed):
+            assert runner._graphs, "no decode step took the graph path"
+        for k, tokens in reqs.items():
+            mine = torch.stack([got[k][p] for p in range(len(tokens))])
+            assert (mine - ref[k]).abs().max().item() < 2e-4, f"{build.__name__} request {k}"
+        assert runner.cache.num_free_slots() == 4
+    # Requests fed one token at a time from position 0, three at once in a bucket of four (one
+    # padding row), on slots that the requests above left full; a fourth joins later, when the
+    # graph exists already.
+    keys = ["r0", "r2", "r4", "r3"]
+    for i, k in enumerate(keys[:3]):
+        runner.reserve(100 + i, 12)
+    runner.reserve(103, 8)
+    for t in range(12):
+        live = [0, 1, 2] + ([3] if t >= 4 else [])
+        entries = [StepEntry(100 + i, [reqs[keys[i]][t - (4 if i == 3 else 0)]], [0]) for i in live]
+        logits = runner.step(entries).float().cpu()
+        for row, i in enumerate(live):
+            pos = t - (4 if i == 3 else 0)
+            assert (logits[row] - ref[keys[i]][pos]).abs().max().item() < 2e-4, (keys[i], pos)
+    assert {1 << 2} <= set(runner._graphs)
+
+
+# ------------------------- a toy mixer that caches one vector per position
+def register_latent_toy():
+    """Defined and registered here, in the test: a mixer whose memory of the past grows with
+    the length but is no pair of keys and values.  It keeps one latent vector of ``rank``
+    numbers per position in pages of its own kind and gives every token the mean of the latents
+    up to and including its own, projected back up."""
+    from rust_llm_inference_server_amd.parts import Mixer, TensorSpec, register
+    from rust_llm_inference_server_amd.parts.base import PAGE, CacheRequest, PageArray, join
+
+    @register("mixer", "toy_latent_mean")
+    class LatentMean(Mixer):
+        @classmethod
+        def tensor_specs(cls, params, prefix):
+            H, r = params["hidden_size"], params["rank"]
+            return [TensorSpec(join(prefix, "down.weight"), (r, H)),
+                    TensorSpec(join(prefix, "up.weight"), (H, r))]
+
+        def __init__(self, params, prefix, ctx):
+            super().__init__(params, prefix, ctx)
+            self.rank = params["rank"]
+            self.down = ctx.take(join(prefix, "down.weight")).float()
+            self.up = ctx.take(join(prefix, "up.weight")).float()
+            self.act_dtype = ctx.act_dtype
+
+        def cache_request(self):
+            return CacheRequest((PageArray("latent", (PAGE, self.rank)),))
+
+        def forward(self, x, step, binding):
+            group = step.groups[binding.group]
+            pages = binding.pages["latent"]                       # (num pages, page, rank)
+            ps = group.page_size
+            flat = pages.view(-1, self.rank)
+            latent = (x.float() @ self.down.t()).to(pages.dtype)
+            if binding.writes:
+                flat.index_copy_(0, group.slots.long(), latent)
+            tables = group.block_tables.cpu()
+            out = torch.empty((x.shape[0], self.rank), dtype=torch.float32, device=x.device)
+            begin = 0
+            for s, (start, n) in enumerate(zip(step.host_start_pos, step.host_new)):
+                pos = torch.arange(start + n)
+                rows = (tables[s, pos // ps].long() * ps + pos % ps).to(x.device)
+                seen = flat.index_select(0, rows).float().cumsum(0)       # read back from the pages
+                count = torch.arange(1, start + n + 1, device=x.device).unsqueeze(1)
+                out[begin:begin + n] = (seen / count)[start:]
+                begin += n
+            return (out @ self.up.t()).to(self.act_dtype)
+
+    return LatentMean
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-4), ("bfloat16", 3e-2)])
+def test_toy_mixer_with_a_cache_kind_of_its_own(tmp_path, dtype, tol):
+    """A mixer that caches one vector per position, registered from the test: the pools are
+    allocated from its cache request (no keys, no values), beside an attention layer's group,
+    and the model runs through every way of cutting with pages used again."""
+    from rust_llm_inference_server_amd.engine import ModelRunner, load_model
+    from rust_llm_inference_server_amd.registry import Architecture, register_architecture
+    from rust_llm_inference_server_amd.weights import write_model_folder
+    register_latent_toy()
+    H, rank = 48, 20
+    kinds = ["latent", "attention", "latent"]
+
+    def build_spec(cfg):
+        blocks = []
+        for kind in cfg["mixers"]:
+            if kind == "latent":
+                blocks.append(layer_spec(H, 1, 1, 16, 64, 1e-5, 1e4, None, mixer="toy_latent_mean",
+                                         extra={"hidden_size": H, "rank": rank}))
+            else:
+                blocks.append(layer_spec(H, 3, 1, 16, 64, 1e-5, 1e4, None))
+        return toy_spec(blocks, H=H, V=cfg["vocab_size"])
+
+    register_architecture(Architecture("ToyLatentForCausalLM", parse_config=lambda d: d,
+                                       build_spec=build_spec, config_to_dict=lambda c: c))
+    config = {"architectures": ["ToyLatentForCausalLM"], "vocab_size": 97, "mixers": kinds}
+    folder = str(tmp_path / "latent")
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    write_model_folder(folder, config, build_spec(config).tensor_specs(), seed=12, dtype=tdt)
+    w = plain.read_weights(folder)
+
+    def plain_model(ids):
+        x = plain.embedding(w["model.embed_tokens.weight"], ids)
+        for li, kind in enumerate(kinds):
+            p = f"model.layers.{li}"
+            h = plain.rms_norm(x, w[f"{p}.input_layernorm.weight"], 1e-5)
+            if kind == "latent":
+                lat = h @ w[f"{p}.self_attn.down.weight"].t()
+                mean = lat.cumsum(0) / torch.arange(1, len(ids) + 1).unsqueeze(1)
+                x = x + mean @ w[f"{p}.self_attn.up.weight"].t()
+            else:
+                cfg = {"num_attention_heads": 3, "num_key_value_heads": 1, "head_dim": 16}
+                x = x + plain.attention_layer(h, w, f"{p}.self_attn", cfg, plain.inv_freqs(16, 1e4, None))
+            h = plain.rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], 1e-5)
+            x = x + plain.swiglu_mlp(h, w, f"{p}.mlp")
+        return plain.linear(plain.rms_norm(x, w["model.norm.weight"], 1e-5), w["lm_head.weight"])
+
+    reqs = traces.random_requests(97, [30, 4, 70, 11, 45, 2], seed=8)
+    ref = {k: plain_model(t) for k, t in reqs.items()}
+    for build in (traces.trace_whole, traces.trace_tail, traces.trace_portions, traces.trace_mixed):
+        steps, max_tokens = build(reqs)
+        model = load_model(folder, dtype, max_positions=128)
+        assert len(model.cache_groups) == 2               # the latents' group and attention's
+        latent_group = [g for g in model.cache_groups if g.request.arrays[0].name == "latent"][0]
+        assert latent_group.request.elements_per_token() == rank and len(latent_group.writer_runs) == 2
+        runner = ModelRunner(model, num_pages=max_tokens // 16, page_size=16, max_num_seqs=4)
+        g = model.cache_groups.index(latent_group)
+        assert set(runner.pools.arrays[g]) == {"latent"}
+        assert runner.pools.arrays[g]["latent"].shape[2:] == (16, rank)
+        got = traces.collect(steps, traces.replay_in_process(runner, steps), 97)
+        for k, tokens in reqs.items():
+            mine = torch.stack([got[k][p] for p in range(len(tokens))])
+            assert (mine - ref[k]).abs().max().item() < tol, f"{build.__name__} request {k}"
+        for gi in range(runner.cache.num_groups):
+            assert runner.cache.num_free_pages(gi) == runner.cache.num_pages(gi)
 
 
 # ------------------------- a toy feed-forward with routing and a toy position encoding
