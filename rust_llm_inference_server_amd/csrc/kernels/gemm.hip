@@ -591,37 +591,46 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
           load8(nm.resid + at[i], v[i]);
         }
         if (nm.delta) {
-          // two parts per round, so that their loads travel together with the residual's; the
-          // parts are summed in order on their own and then join the residual
-          float dsum[kU][8];
-          for (int s = 0; s < nm.parts; s += 2) {
-            const bool two = s + 1 < nm.parts;
-            float d0[kU][8], d1[kU][8];
+          // The first two parts are loaded together, so that their loads travel with the
+          // residual's; the parts are summed in order on their own and then join the residual.
+          const bool two = nm.parts > 1;
+          float acc[kU][8], nxt[kU][8];
+#pragma unroll
+          for (int i = 0; i < kU; ++i) {
+            if (nm.delta_f32) {
+              const float* dp = (const float*)nm.delta + at[i];
+              load8(dp, acc[i]);
+              load8(two ? dp + nm.part_stride : dp, nxt[i]);
+            } else {
+              const bf16_t* dp = (const bf16_t*)nm.delta + at[i];
+              load8(dp, acc[i]);
+              load8(two ? dp + nm.part_stride : dp, nxt[i]);
+            }
+          }
+          if (two) {
+#pragma unroll
+            for (int i = 0; i < kU; ++i)
+#pragma unroll
+              for (int e = 0; e < 8; ++e) acc[i][e] += nxt[i][e];
+          }
+          for (int s = 2; s < nm.parts; ++s) {
 #pragma unroll
             for (int i = 0; i < kU; ++i) {
-              if (nm.delta_f32) {
-                const float* dp = (const float*)nm.delta + s * nm.part_stride + at[i];
-                load8(dp, d0[i]);
-                load8(two ? dp + nm.part_stride : dp, d1[i]);
-              } else {
-                const bf16_t* dp = (const bf16_t*)nm.delta + s * nm.part_stride + at[i];
-                load8(dp, d0[i]);
-                load8(two ? dp + nm.part_stride : dp, d1[i]);
-              }
+              if (nm.delta_f32)
+                load8((const float*)nm.delta + s * nm.part_stride + at[i], nxt[i]);
+              else
+                load8((const bf16_t*)nm.delta + s * nm.part_stride + at[i], nxt[i]);
             }
 #pragma unroll
             for (int i = 0; i < kU; ++i)
 #pragma unroll
-              for (int e = 0; e < 8; ++e) {
-                dsum[i][e] = s == 0 ? d0[i][e] : dsum[i][e] + d0[i][e];
-                if (two) dsum[i][e] += d1[i][e];
-              }
+              for (int e = 0; e < 8; ++e) acc[i][e] += nxt[i][e];
           }
 #pragma unroll
           for (int i = 0; i < kU; ++i)
 #pragma unroll
             for (int e = 0; e < 8; ++e)
-              v[i][e] += nm.round_parts ? bf16_to_f32(f32_to_bf16(dsum[i][e])) : dsum[i][e];
+              v[i][e] += nm.round_parts ? bf16_to_f32(f32_to_bf16(acc[i][e])) : acc[i][e];
         }
 #pragma unroll
         for (int i = 0; i < kU; ++i) {
