@@ -5,7 +5,9 @@ and which state slot a request owns; it holds no GPU memory (``pools.py`` does).
 behaviour follows the reference's ``BlockManager`` (crates/kvcache/src/lib.rs:177-438):
 ``reserve`` is all-or-nothing and returns the copy-on-write copies to perform, ``free``
 returns everything, ``check_invariants`` verifies that no page is lost, held twice or freed
-twice."""
+twice.  A reservation makes positions addressable and the pages from the computed length on
+the request's own, so a request that shares pages after a ``fork`` gets its copies before it
+writes, however far ahead it had reserved."""
 from __future__ import annotations
 
 import ctypes
@@ -29,7 +31,7 @@ def runtime() -> ctypes.CDLL:
             "rlis_cache_destroy": (None, [c_void_p]),
             "rlis_cache_reserve": (c_int, [c_void_p, c_longlong, c_int, PI, c_int, PI]),
             "rlis_cache_advance": (c_int, [c_void_p, c_longlong, c_int]),
-            "rlis_cache_fork": (c_int, [c_void_p, c_longlong, c_longlong]),
+            "rlis_cache_fork": (c_int, [c_void_p, c_longlong, c_longlong, PI]),
             "rlis_cache_free": (c_int, [c_void_p, c_longlong]),
             "rlis_cache_num_free": (c_int, [c_void_p, c_int]),
             "rlis_cache_num_pages": (c_int, [c_void_p, c_int]),
@@ -42,6 +44,9 @@ def runtime() -> ctypes.CDLL:
             "rlis_cache_check": (c_int, [c_void_p, c_char_p, c_int]),
             "rlis_cache_decode_batch": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                 c_void_p, c_void_p, c_void_p]),
+            "rlis_fill_normal": (c_int, [c_void_p, c_longlong, ctypes.c_ulonglong,
+                                         ctypes.c_ulonglong, ctypes.c_double, ctypes.c_double,
+                                         c_int]),
             "rlis_sched_create": (c_void_p, [c_void_p, c_int, c_int, c_int, c_int]),
             "rlis_sched_destroy": (None, [c_void_p]),
             "rlis_sched_add": (c_int, [c_void_p, c_longlong, c_int]),
@@ -180,9 +185,14 @@ class CacheManager:
         if runtime().rlis_cache_advance(self._h, seq, computed) != 0:
             raise ValueError(rt_error())
 
-    def fork(self, parent: int, child: int) -> None:
-        if runtime().rlis_cache_fork(self._h, parent, child) != 0:
+    def fork(self, parent: int, child: int) -> Tuple[int, int]:
+        """``child`` shares the pages of ``parent``'s computed positions (what ``parent`` has
+        reserved beyond them stays its own).  Returns the state slots ``(parent's, child's)``
+        whose contents the device must copy, ``(-1, -1)`` without state slots."""
+        seats = (c_int * 2)()
+        if runtime().rlis_cache_fork(self._h, parent, child, seats) != 0:
             raise ValueError(rt_error())
+        return seats[0], seats[1]
 
     def free(self, seq: int) -> None:
         if runtime().rlis_cache_free(self._h, seq) != 0:

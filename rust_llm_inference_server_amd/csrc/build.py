@@ -38,7 +38,9 @@ HIP_FLAGS = [
     "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wno-unused-command-line-argument",
 ]
-CXX_FLAGS = ["-O2", "-fPIC", "-std=c++17", "-fvisibility=hidden", "-Wall"]
+# (no fused multiply-adds: the seeded weights must come out the same from any compiler)
+CXX_FLAGS = ["-O2", "-fPIC", "-std=c++17", "-fvisibility=hidden", "-Wall", "-pthread",
+             "-ffp-contract=off"]
 
 # Head sizes (rounded up to a multiple of 32) the matrix-core attention unit is built for.
 MFMA_ATTENTION_HEAD_DIMS = (32, 64, 96, 128, 160, 192, 224, 256)
@@ -170,7 +172,7 @@ def build_many(kinds: Sequence[str], jobs: Optional[int] = None) -> List[str]:
         if _is_hip(kind):
             link = [_hipcc(), f"--offload-arch={ARCH}", "-fPIC", "-shared", "-o", tmp, *objs[kind]]
         else:
-            link = [shutil.which("g++") or "g++", "-shared", "-o", tmp, *objs[kind]]
+            link = [shutil.which("g++") or "g++", "-shared", "-pthread", "-o", tmp, *objs[kind]]
         _run(link, f"linking {os.path.basename(out)}")
         os.replace(tmp, out)
         with open(out + ".hash", "w") as f:

@@ -73,8 +73,15 @@ RT_API int rlis_cache_advance(void* h, long long seq, int computed) {
   return 0;
 }
 
-RT_API int rlis_cache_fork(void* h, long long parent, long long child) {
-  GUARD(static_cast<CacheManager*>(h)->fork(parent, child));
+// seats[0..1] = the parent's and the child's state slot (-1, -1 without state slots): the
+// device copies the first onto the second.
+RT_API int rlis_cache_fork(void* h, long long parent, long long child, int* seats) {
+  std::pair<int, int> moved(-1, -1);
+  GUARD(moved = static_cast<CacheManager*>(h)->fork(parent, child));
+  if (seats) {
+    seats[0] = moved.first;
+    seats[1] = moved.second;
+  }
   return 0;
 }
 
@@ -89,28 +96,29 @@ RT_API int rlis_cache_refcount(void* h, int g, int p) { return static_cast<Cache
 RT_API int rlis_cache_num_free_slots(void* h) { return static_cast<CacheManager*>(h)->num_free_slots(); }
 RT_API int rlis_cache_contains(void* h, long long seq) { return static_cast<CacheManager*>(h)->contains(seq); }
 
+// Pages that reserve(seq, total) would take from group g (growth plus copies of shared pages).
 RT_API int rlis_cache_pages_needed(void* h, long long seq, int total, int g) {
-  return static_cast<CacheManager*>(h)->pages_needed(seq, total, g);
+  return static_cast<CacheManager*>(h)->quote(seq, total).pages[g];
 }
 
 // Writes the block table of (seq, group) into out (up to cap entries) and returns its
 // length, or -1 for an unknown request.
 RT_API int rlis_cache_table(void* h, long long seq, int g, int* out, int cap) {
-  const rlis::SeqEntry* e = static_cast<CacheManager*>(h)->entry(seq);
-  if (!e) return -1;
-  const auto& pages = e->pages[g];
-  const int n = (int)pages.size() < cap ? (int)pages.size() : cap;
-  for (int i = 0; i < n; ++i) out[i] = pages[i];
-  return (int)pages.size();
+  const rlis::Lease* l = static_cast<CacheManager*>(h)->lease(seq);
+  if (!l) return -1;
+  const rlis::PageRun& run = l->runs[g];
+  const int n = run.count() < cap ? run.count() : cap;
+  for (int i = 0; i < n; ++i) out[i] = run.at(i);
+  return run.count();
 }
 
 // info[0..2] = reserved tokens, computed tokens, state slot; returns -1 for an unknown request.
 RT_API int rlis_cache_info(void* h, long long seq, int* info) {
-  const rlis::SeqEntry* e = static_cast<CacheManager*>(h)->entry(seq);
-  if (!e) return -1;
-  info[0] = e->num_tokens;
-  info[1] = e->num_computed;
-  info[2] = e->state_slot;
+  const rlis::Lease* l = static_cast<CacheManager*>(h)->lease(seq);
+  if (!l) return -1;
+  info[0] = l->reserved;
+  info[1] = l->computed;
+  info[2] = l->seat;
   return 0;
 }
 
@@ -125,24 +133,25 @@ RT_API int rlis_cache_decode_batch(void* h, const long long* seqs, int n, int wi
   auto* m = static_cast<CacheManager*>(h);
   const int ps = m->page_size();
   for (int i = 0; i < n; ++i) {
-    const rlis::SeqEntry* e = m->entry(seqs[i]);
-    if (!e || e->num_computed + 1 > e->num_tokens) {
+    const rlis::Lease* l = m->lease(seqs[i]);
+    if (!l || l->computed + 1 > l->reserved) {
       g_error = "request " + std::to_string(seqs[i]) + ": position " +
-                std::to_string(e ? e->num_tokens : 0) + " has no page reserved";
+                std::to_string(l ? l->reserved : 0) + " has no page reserved";
       return -1;
     }
-    const int pos = e->num_computed;
+    const int pos = l->computed;
     positions[i] = pos;
-    state_slots[i] = e->state_slot < 0 ? 0 : e->state_slot;
+    state_slots[i] = l->seat < 0 ? 0 : l->seat;
     for (int g = 0; g < m->num_groups(); ++g) {
-      const auto& pages = e->pages[g];
-      if ((int)pages.size() > width) {
+      const rlis::PageRun& run = l->runs[g];
+      if (run.count() > width) {
         g_error = "block table of request " + std::to_string(seqs[i]) + " is wider than the buffer";
         return -1;
       }
       int* row = tables[g] + (long long)i * width;
-      for (size_t p = 0; p < pages.size(); ++p) row[p] = pages[p] < 0 ? 0 : pages[p];
-      const int page = pages[pos / ps];
+      for (int p = 0; p < run.gone; ++p) row[p] = 0;
+      for (size_t p = 0; p < run.live.size(); ++p) row[run.gone + p] = run.live[p];
+      const int page = run.at(pos / ps);
       if (page < 0) {
         g_error = "request " + std::to_string(seqs[i]) + ": position " + std::to_string(pos) +
                   " has no page reserved";
@@ -155,7 +164,7 @@ RT_API int rlis_cache_decode_batch(void* h, const long long* seqs, int n, int wi
 }
 
 RT_API int rlis_cache_check(void* h, char* buf, int cap) {
-  return copy_message(static_cast<CacheManager*>(h)->check_invariants(), buf, cap);
+  return copy_message(static_cast<CacheManager*>(h)->audit(), buf, cap);
 }
 
 // -------------------------------------------------------------------- scheduler

@@ -1,19 +1,27 @@
-// Page bookkeeping of the cache: which physical pages hold which request's positions.
-// Pure host logic, no GPU (as crates/kvcache/src/lib.rs:1-5 of the reference).
+// Page bookkeeping of the cache: which physical pages hold which request's positions, and
+// which seat (slot of fixed-size state) a request sits in.  Pure host logic, no GPU.
 //
-// The reference has one pool whose block ids address every layer (lib.rs:3-5).  Here layers
-// are collected in *groups* with pages of their own: a group keeps either every position of a
-// request or only a window of the latest ones.  Every group has its own pool, and every
-// request one block table per group.  A page of a windowed group is given back as soon as all
-// its positions have left the window; all pages go back when the request is freed.  Beside
-// the pages, a request holds one *state slot* (a fixed-size area for mixers whose memory of
-// the past does not grow) from its first reservation until it is freed.
+// Layers are collected in *groups* with pools of their own: a group keeps every position of a
+// request or only a window of the latest ones.  A request holds one *lease*: per group the
+// run of pages that back its positions (pages that a window has passed are given back while
+// the request lives), the number of positions reserved and of positions computed, and its
+// seat.  Three rules carry everything else:
 //
-// Kept from the reference: reference counts with a LIFO free list that hands out page 0 first
-// (lib.rs:57-82, 123-165), all-or-nothing reservation that grows whole pages (lib.rs:282-336),
-// copy-on-write of a shared, partly filled last page (lib.rs:293-297, 319-328), fork
-// (lib.rs:338-354) and the invariant checker (lib.rs:372-437).  Left out: the hash registry and
-// the evictable set of its prefix cache.
+//  * A reservation is quoted before it is made.  `quote` says what making positions
+//    [0, total) of a request addressable *and writable from its computed length on* would take
+//    from every pool, and whether it takes a seat; `reserve` commits a quote only if every pool
+//    can pay it, so a reservation that fails changes nothing.  The scheduler admits with the
+//    same quote plus its watermark.
+//  * Pages are shared by reference count.  A fork shares the pages of the positions that are
+//    computed and nothing beyond; whoever then reserves a range that touches a shared page
+//    gets a copy of it first (the copy is returned for the device to perform) and lets go of
+//    the original.
+//  * Pools hand out the page that was returned last (page 0 first in a fresh pool), so pages
+//    are used again at once and stale contents are what the next request finds.
+//
+// What this must do is the reference's BlockManager contract (crates/kvcache/src/lib.rs:
+// 177-438: all-or-nothing reserve, copy-on-write, fork, free, invariants); groups, windows,
+// seats, the quote and the computed length are this engine's.
 #pragma once
 #include <cstdint>
 #include <string>
@@ -30,20 +38,25 @@ struct PageCopy {
   int dst;
 };
 
-class PageAllocator {
+// One group's pages: a reference count per page and the free pages as a stack threaded
+// through `below_`.
+class PagePool {
  public:
-  explicit PageAllocator(int num_pages);
-  int num_pages() const { return (int)refcounts_.size(); }
-  int num_free() const { return (int)free_.size(); }
-  int refcount(int p) const { return refcounts_[p]; }
-  int allocate();            // -1 when none is free
-  void incref(int p);
-  void decref(int p);        // throws on a page that is already free
-  const std::vector<int>& free_list() const { return free_; }
+  explicit PagePool(int num_pages);
+  int size() const { return (int)refs_.size(); }
+  int free_count() const { return free_count_; }
+  int refs(int p) const { return refs_[p]; }
+  int take();                  // the page on top of the stack, now held once; -1 when empty
+  void share(int p);           // one more holder
+  void drop(int p);            // one holder fewer; the page goes back on the stack at zero
+  // Pages on the free stack from the top down (for the audit).
+  std::vector<int> free_pages() const;
 
  private:
-  std::vector<int> refcounts_;
-  std::vector<int> free_;    // LIFO
+  std::vector<int> refs_;
+  std::vector<int> below_;     // for a free page: the free page under it, -1 at the bottom
+  int top_ = -1;
+  int free_count_ = 0;
 };
 
 struct GroupSpec {
@@ -51,12 +64,26 @@ struct GroupSpec {
   int num_pages;
 };
 
-struct SeqEntry {
-  // Per group: physical page of logical page i, or -1 once the window has passed it.
-  std::vector<std::vector<int>> pages;
-  int num_tokens = 0;     // positions with a slot reserved
-  int num_computed = 0;   // positions whose keys and values are written
-  int state_slot = -1;
+// The pages of one group that back a request: logical page i is gone (returned, a window has
+// passed it) for i < gone, else live[i - gone].
+struct PageRun {
+  int gone = 0;
+  std::vector<int> live;
+  int count() const { return gone + (int)live.size(); }
+  int at(int i) const { return i < gone ? -1 : live[i - gone]; }
+};
+
+struct Lease {
+  std::vector<PageRun> runs;   // one per group
+  int reserved = 0;            // positions with a place in the pages
+  int computed = 0;            // positions whose contents are written
+  int seat = -1;               // state slot, -1 when the model keeps no state
+};
+
+// What a reservation would take.
+struct Quote {
+  std::vector<int> pages;      // per group: pages to grow by plus shared pages to copy
+  bool seat = false;           // a seat too (the request is new and seats exist)
 };
 
 enum ReserveResult { kReserved = 0, kOutOfPages = 1, kOutOfSlots = 2 };
@@ -67,41 +94,44 @@ class CacheManager {
 
   int page_size() const { return page_size_; }
   int num_groups() const { return (int)groups_.size(); }
-  int num_pages(int g) const { return alloc_[g].num_pages(); }
-  int num_free(int g) const { return alloc_[g].num_free(); }
-  int refcount(int g, int p) const { return alloc_[g].refcount(p); }
+  int num_pages(int g) const { return pools_[g].size(); }
+  int num_free(int g) const { return pools_[g].free_count(); }
+  int refcount(int g, int p) const { return pools_[g].refs(p); }
   int window(int g) const { return groups_[g].window; }
-  int num_state_slots() const { return num_state_slots_; }
-  int num_free_slots() const { return (int)free_slots_.size(); }
+  int num_state_slots() const { return num_seats_; }
+  int num_free_slots() const { return (int)free_seats_.size(); }
   int pages_for(int tokens) const { return (tokens + page_size_ - 1) / page_size_; }
 
-  bool contains(SeqId s) const { return seqs_.count(s) != 0; }
-  const SeqEntry* entry(SeqId s) const;
+  bool contains(SeqId s) const { return leases_.count(s) != 0; }
+  const Lease* lease(SeqId s) const;
 
-  // Pages `reserve(s, total)` would take from group g, a copy-on-write included.
-  int pages_needed(SeqId s, int total_tokens, int g) const;
-  // Makes positions up to total_tokens addressable in every group; creates the request on
-  // first use (and takes a state slot).  All or nothing: on failure nothing changes.
+  Quote quote(SeqId s, int total_tokens) const;
+  // Whether every pool can pay the quote and still keep `spare` pages free, and a seat is
+  // there if the quote takes one.  `short_of_seats` (may be null) says which of the two failed.
+  bool affordable(const Quote& q, int spare, bool* short_of_seats = nullptr) const;
+  // Makes positions [0, total_tokens) of s addressable in every group and the pages from its
+  // computed length on its own; creates the request on first use (and seats it).  All or
+  // nothing.  Copies to perform on the device are appended to `copies`.
   ReserveResult reserve(SeqId s, int total_tokens, std::vector<PageCopy>* copies);
-  // Positions [0, computed) are written; windowed groups give back pages no later query
-  // can see.
+  // Positions [0, computed) are written; windowed groups give back pages no later query sees.
   void advance(SeqId s, int computed);
-  void fork(SeqId parent, SeqId child);
+  // child shares parent's computed positions.  Returns the seats (parent's, child's) whose
+  // state the device must copy, both -1 when there are no seats.
+  std::pair<int, int> fork(SeqId parent, SeqId child);
   void free_seq(SeqId s);
 
-  // Empty when every invariant holds, else a description of the first violation.
-  std::string check_invariants() const;
+  // Empty when the books balance, else the first thing that does not.
+  std::string audit() const;
 
  private:
-  bool needs_cow(const SeqEntry& e, int g) const;
-  int first_live_page(int computed, int g) const;
+  int first_visible_page(int computed, int g) const;
 
   int page_size_;
   std::vector<GroupSpec> groups_;
-  std::vector<PageAllocator> alloc_;
-  int num_state_slots_;
-  std::vector<int> free_slots_;   // LIFO
-  std::unordered_map<SeqId, SeqEntry> seqs_;
+  std::vector<PagePool> pools_;
+  int num_seats_;
+  std::vector<int> free_seats_;   // a stack: the seat returned last is taken next
+  std::unordered_map<SeqId, Lease> leases_;
 };
 
 }  // namespace rlis

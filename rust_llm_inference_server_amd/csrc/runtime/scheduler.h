@@ -1,23 +1,26 @@
-// Iteration-level scheduling over the paged cache: continuous batching with chunked prefill
-// and preemption by recompute, as crates/engine/src/scheduler.rs of the reference decides it.
+// What each step computes: continuous batching with chunked prefill under a token budget, and
+// preemption by recompute when pages run out.  The decisions are the reference's
+// (crates/engine/src/scheduler.rs:1-8, 193-306); the book-keeping is this engine's.
 //
-// A request is `num_tokens` (prompt plus generated) and `num_computed` (positions whose keys
-// and values are cached); every step computes the next portion of the gap.  That one rule is
-// prefill (gap = prompt), chunked prefill (gap above the token budget), decode (gap = 1) and
-// recompute after preemption (gap = everything) (scheduler.rs:1-8).
+// Every request sits in one *roster*, ordered by arrival, with a standing: queued (never ran),
+// parked (preempted: it holds nothing and will recompute), or running (it holds a lease).  A
+// request is `tokens` (prompt plus generated) and `computed` (positions in the cache); a step
+// computes the next portion of the gap between the two, which is prefill, chunked prefill,
+// decode or recompute depending only on how large the gap is.
 //
-//  * Running requests go first, oldest first, within max_batched_tokens (scheduler.rs:207-226).
-//  * When a running request needs a page and none is free, the newest running request is
-//    preempted: its pages and state slot are freed, it recomputes later (scheduler.rs:227-246).
-//  * Admission is first come, first served: preempted requests (oldest first) before new ones,
-//    only while the whole known length fits with `watermark` pages to spare in every group;
-//    the head of the line is never skipped; no admission in a step that preempted
-//    (scheduler.rs:193-205, 253-306).
-//  * The static policy admits only when nothing is running, and ignores the token budget
-//    then (scheduler.rs:197-200, 254-255).
-// Left out: forked requests and the prefix cache.
+// A step is planned in two passes over the roster:
+//  1. Running requests, oldest first, each take min(gap, budget left) tokens.  When the cache
+//     cannot give a request its pages, the *youngest* running request is parked (it returns its
+//     lease and starts over later); that may be the request that asked, which then waits.
+//  2. Admission, unless the first pass parked someone (static policy: only when nothing runs):
+//     the oldest parked request, or else the oldest queued one, is admitted while a seat among
+//     max_num_seqs is free, budget is left (the static policy ignores the budget) and the cache
+//     can pay for the whole known length with `watermark` pages to spare in every group.  The
+//     head of the line is never skipped; an admitted request reserves its whole known length
+//     at once, so that later admissions cannot overcommit the pools.
 #pragma once
-#include <deque>
+#include <map>
+#include <unordered_map>
 #include <vector>
 
 #include "cache_manager.h"
@@ -49,7 +52,8 @@ class Scheduler {
  public:
   Scheduler(SchedulerConfig cfg, CacheManager* cache);
 
-  // Longest request (prompt plus output) that can ever be admitted (scheduler.rs:48-53).
+  // Longest request (prompt plus output) that can ever be admitted: what the smallest pool
+  // holds beyond the watermark.
   int max_seq_tokens() const;
   void add(SeqId id, int prompt_len);
   Schedule schedule();
@@ -57,31 +61,36 @@ class Scheduler {
   void append_token(SeqId id);
   bool is_caught_up(SeqId id) const;
   void remove(SeqId id);
-  bool has_work() const { return !(running_.empty() && waiting_.empty() && preempted_.empty()); }
-  int num_running() const { return (int)running_.size(); }
-  int num_waiting() const { return (int)(waiting_.size() + preempted_.size()); }
+  bool has_work() const { return !roster_.empty(); }
+  int num_running() const { return standing_count_[kRunning]; }
+  int num_waiting() const { return standing_count_[kQueued] + standing_count_[kParked]; }
   long long num_preemptions() const { return num_preemptions_; }
   int num_tokens(SeqId id) const;
   int num_computed(SeqId id) const;
   std::string check() const;
 
  private:
-  struct SeqState {
+  enum Standing { kQueued = 0, kParked = 1, kRunning = 2 };
+  struct Member {
     SeqId id;
-    long long arrival;
-    int num_tokens;
-    int num_computed;
+    int tokens;
+    int computed;
+    Standing standing;
   };
-  void schedule_running(Schedule* out, int* budget);
-  void admit(Schedule* out, int* budget);
-  void preempt(SeqState s, Schedule* out);
-  const SeqState* find(SeqId id) const;
+  using Roster = std::map<long long, Member>;   // by arrival
+
+  Member* find(SeqId id);
+  const Member* find(SeqId id) const;
+  void stand(Member& m, Standing s);
+  void take_portion(Member& m, int* budget, Schedule* plan);
+  Roster::iterator youngest_running();
+  Roster::iterator next_in_line();
 
   SchedulerConfig cfg_;
   CacheManager* cache_;
-  std::deque<SeqState> waiting_;
-  std::deque<SeqState> preempted_;   // sorted by arrival
-  std::vector<SeqState> running_;    // sorted by arrival; the last one is the victim
+  Roster roster_;
+  std::unordered_map<SeqId, long long> arrival_of_;
+  int standing_count_[3] = {0, 0, 0};
   long long next_arrival_ = 0;
   long long num_preemptions_ = 0;
 };

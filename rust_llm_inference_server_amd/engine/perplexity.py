@@ -47,9 +47,11 @@ def perplexity(runner: ModelRunner, tokens: Sequence[int], bos: int, ctx: int,
         chunk = [int(t) for t in tokens[w * ctx:(w + 1) * ctx]]
         chunk[0] = int(bos)
         runner.reserve(seq_id, ctx)
-        # Rows first .. ctx-2 predict tokens first+1 .. ctx-1; the last row has no target.
-        logits = runner.step([StepEntry(seq_id, chunk, list(range(first, ctx - 1)))])
-        runner.free(seq_id)
+        try:
+            # Rows first .. ctx-2 predict tokens first+1 .. ctx-1; the last row has no target.
+            logits = runner.step([StepEntry(seq_id, chunk, list(range(first, ctx - 1)))])
+        finally:
+            runner.free(seq_id)       # also when the step raises: the next call starts clean
         targets = torch.tensor(chunk[first + 1:], device=logits.device).reshape(-1, 1)
         logp = torch.log_softmax(logits.double(), dim=-1).gather(1, targets).reshape(-1)
         nll = (-logp).cpu()

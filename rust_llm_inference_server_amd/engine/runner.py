@@ -119,6 +119,14 @@ class ModelRunner:
             if g < len(self.pools.arrays):
                 self.pools.copy_pages(g, [c.src for c in cs], [c.dst for c in cs])
 
+    def fork(self, parent: int, child: int) -> None:
+        """``child`` continues from what ``parent`` has computed: it shares those pages (the
+        first of the two to write into a shared page gets its own copy, made when it reserves)
+        and starts from a copy of the parent's state."""
+        src, dst = self.cache.fork(parent, child)
+        if src >= 0 and dst >= 0:
+            self.pools.copy_state(src, dst)
+
     def free(self, seq_id: int) -> None:
         self.cache.free(seq_id)
 

@@ -42,10 +42,13 @@ def test_out_of_pages_changes_nothing():
 
 
 def test_fork_shares_and_writes_copy_on_write():
+    """lib.rs:470-502, with the positions computed (a fork shares what is computed)."""
     m = CacheManager(4, [GroupSpec(8)])
     m.reserve(1, 6)
-    m.fork(1, 2)
+    m.advance(1, 6)
+    assert m.fork(1, 2) == (-1, -1)                 # no state slots to copy
     assert m.num_free_pages() == 6                  # fork allocates nothing
+    assert m.num_tokens(2) == 6 and m.num_computed(2) == 6
     shared_last = m.table(1)[1]
     copies = m.reserve(2, 7)                        # writes into the shared, half-full last page
     mine = m.table(2)[1]
@@ -58,9 +61,33 @@ def test_fork_shares_and_writes_copy_on_write():
 def test_full_shared_pages_need_no_copy():
     m = CacheManager(4, [GroupSpec(8)])
     m.reserve(1, 8)
+    m.advance(1, 8)
     m.fork(1, 2)
     assert m.reserve(2, 9) == []
     assert m.pages_needed(1, 9) == 1
+
+
+def test_fork_of_a_request_that_reserved_ahead():
+    """The scheduler reserves a request's whole known length at admission, far ahead of what is
+    computed.  A fork shares the computed positions only; the page both will write next is
+    copied for whichever of the two reserves a range that touches it, the parent included,
+    although the parent had that page reserved all along."""
+    m = CacheManager(4, [GroupSpec(8)], num_state_slots=3)
+    m.reserve(1, 14)                                # pages 0..3
+    m.advance(1, 6)
+    parent_slot = m.state_slot(1)
+    assert m.fork(1, 2) == (parent_slot, m.state_slot(2)) and m.state_slot(2) != parent_slot
+    assert m.table(2) == m.table(1)[:2] and m.num_tokens(2) == 6
+    assert m.refcount(0, m.table(1)[1]) == 2 and m.refcount(0, m.table(1)[2]) == 1
+    assert m.pages_needed(1, 7) == 1                # the parent's next write lands in a shared page
+    before = m.table(1)
+    copies = m.reserve(1, 7)                        # within what it had reserved: still a copy
+    assert copies == [PageCopy(0, before[1], m.table(1)[1])] and m.num_tokens(1) == 14
+    assert m.reserve(2, 9) == [] and len(m.table(2)) == 3      # the child's page is its own now
+    m.check_invariants()
+    m.free(1)
+    m.free(2)
+    assert m.num_free_pages() == 8 and m.num_free_slots() == 3
 
 
 def test_window_group_gives_pages_back_as_the_window_passes():

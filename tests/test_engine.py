@@ -247,6 +247,28 @@ def test_perplexity_matches_the_plain_implementation(backend, tiny_folders):
         perplexity(runner, tokens[:10], bos=1, ctx=16)
 
 
+def test_perplexity_gives_its_pages_back_when_a_step_fails(backend, tiny_folders):
+    from rust_llm_inference_server_amd.engine import ModelRunner
+    from rust_llm_inference_server_amd.engine.perplexity import perplexity
+    folder = tiny_folders["a"]
+    tokens = prompts_for(256, [40], seed=3)[0]
+    runner = ModelRunner(load(folder, backend, max_positions=128), num_pages=4, page_size=8, max_num_seqs=2)
+    real, calls = runner.step, []
+
+    def failing(entries):
+        calls.append(1)
+        if len(calls) == 2:
+            raise RuntimeError("the device said no")
+        return real(entries)
+
+    runner.step = failing
+    with pytest.raises(RuntimeError, match="the device said no"):
+        perplexity(runner, tokens, bos=1, ctx=16)
+    assert runner.cache.num_free_pages() == 4 and not runner.cache.contains(-1)
+    runner.step = real
+    assert perplexity(runner, tokens, bos=1, ctx=16).windows == 2
+
+
 def test_pool_size_watermark_and_budget_follow_the_references_rules(backend, tiny_folders):
     """crates/engine/src/engine.rs:252-280: pages = pool bytes / (bytes of K and V per token *
     block size); watermark = max(1, pages / 100); the budget is at least max_num_seqs; the

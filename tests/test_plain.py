@@ -46,9 +46,11 @@ def test_inv_freq_matches_the_reference_vector(fn):
 def test_inv_freq_matches_the_reference_fixture(fn):
     """The parity fixture the reference ships holds the same vector as a tensor
     (scripts/parity/dump_reference.py:116-119); read with the safetensors package."""
-    path = "/root/reference/tests/fixtures/parity/reference.safetensors"
+    root = os.environ.get("RLIS_REFERENCE_DIR", "/root/reference")
+    path = os.path.join(root, "tests/fixtures/parity/reference.safetensors")
     if not os.path.exists(path):
-        pytest.skip("the reference's fixture is not mounted")
+        pytest.skip(f"the reference's fixture is not at {path} (set RLIS_REFERENCE_DIR to the "
+                    "reference checkout); the same 32 values are pinned from rope.rs:146-156 above")
     from safetensors import safe_open
     with safe_open(path, framework="pt") as f:
         want = f.get_tensor("inv_freq")
@@ -256,3 +258,48 @@ def test_perplexity_of_uniform_logits_is_the_vocabulary_size():
     assert abs(out["ppl"] - cfg["vocab_size"]) < 1e-6 * cfg["vocab_size"]
     assert out["ppl_stderr"] < 1e-4
     assert plain.perplexity(w, c, tokens, bos=1, ctx=16, max_windows=2)["windows"] == 2
+
+
+def test_perplexity_replaces_each_windows_first_token_and_scores_its_second_half(tiny_folders):
+    """crates/engine/src/perplexity.rs:44-59 written out by hand on a model whose logits depend on
+    the tokens: windows of ctx tokens, the first token of each replaced by BOS, rows ctx/2 ..
+    ctx-2 scored against the tokens that follow them.  What pins it: the value does not change
+    with the token that BOS replaces, it does change with BOS (the later rows see it through
+    attention), and it is neither the all-rows nor the unreplaced value."""
+    w, c = plain.read_weights(tiny_folders["a"]), plain.read_config(tiny_folders["a"])
+    g = torch.Generator().manual_seed(11)
+    tokens = torch.randint(0, c["vocab_size"], (47,), generator=g).tolist()
+    ctx, bos = 10, 7
+
+    def by_hand(toks, first_row, replace):
+        nll = []
+        for wi in range(len(toks) // ctx):
+            chunk = list(toks[wi * ctx:(wi + 1) * ctx])
+            if replace:
+                chunk[0] = bos
+            logits = plain.forward(w, c, chunk).double()
+            for row in range(first_row, ctx - 1):
+                nll.append(float(torch.logsumexp(logits[row], 0) - logits[row][chunk[row + 1]]))
+        return nll
+
+    nll = by_hand(tokens, ctx // 2, True)
+    assert len(nll) == 4 * 4                       # 4 windows (7 tokens left over), rows 5..8
+    mean = sum(nll) / len(nll)
+    out = plain.perplexity(w, c, tokens, bos=bos, ctx=ctx)
+    assert out["windows"] == 4 and out["tokens_scored"] == 16
+    assert abs(out["mean_nll"] - mean) < 1e-12 and abs(out["ppl"] - math.exp(mean)) < 1e-9
+    var = sum(x * x for x in nll) / len(nll) - mean * mean
+    assert abs(out["ppl_stderr"] - math.exp(mean) * math.sqrt(var / len(nll))) < 1e-9
+    # the replaced tokens do not matter, BOS does
+    other = list(tokens)
+    for wi in range(4):
+        other[wi * ctx] = (other[wi * ctx] + 1) % c["vocab_size"]
+    assert plain.perplexity(w, c, other, bos=bos, ctx=ctx)["mean_nll"] == out["mean_nll"]
+    assert abs(plain.perplexity(w, c, tokens, bos=bos + 1, ctx=ctx)["mean_nll"] - mean) > 1e-6
+    # plausible mistakes give other numbers
+    for wrong in (by_hand(tokens, ctx // 2, False), by_hand(tokens, 0, True),
+                  by_hand(tokens, ctx // 2 + 1, True)):
+        assert abs(sum(wrong) / len(wrong) - mean) > 1e-6
+    # odd window length: rows 6 .. 11 of 13
+    odd = plain.perplexity(w, c, tokens, bos=bos, ctx=13, max_windows=2)
+    assert odd["windows"] == 2 and odd["tokens_scored"] == 2 * (13 - 1 - 13 // 2)

@@ -156,6 +156,48 @@ def test_first_tokens_of_a_sequence(case, dtype):
         assert runner.cache.num_free_pages(0) == runner.cache.num_pages(0)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_fork_then_both_decode(case, dtype):
+    """A request that has reserved far ahead (as the scheduler does at admission) is forked in
+    the middle of a page; parent and child go on with different tokens, side by side in the
+    same steps, across the next page's edge.  Each must see the shared past and its own
+    continuation only: the first write of either into the shared page goes to a copy."""
+    from rust_llm_inference_server_amd.engine import StepEntry
+    name, cfg, per_dtype = case
+    folder, reqs, ref = per_dtype[dtype]
+    page = 8 if name == "b" else 16
+    tokens = reqs["r3"]                               # 100 tokens (fewer where positions are)
+    split = page * 2 + 3                              # in the middle of the third page
+    tail = min(len(tokens) - split, page + 6)         # past that page's end
+    w, c = plain.read_weights(folder), plain.read_config(folder)
+    other = [(t + 1) % cfg["vocab_size"] for t in tokens[split:split + tail]]
+    want_parent = ref["r3"]
+    want_child = plain.forward(w, c, tokens[:split] + other)
+    runner = make_runner(folder, dtype, 4 * 128, page_size=page)
+    runner.reserve(0, split + tail)                   # the whole known length at once
+    runner.step([StepEntry(0, tokens[:split], [])])
+    free_before = runner.cache.num_free_pages(0)
+    runner.fork(0, 1)
+    assert runner.cache.num_free_pages(0) == free_before          # a fork allocates nothing
+    shared = runner.cache.table(0)[:3]
+    assert runner.cache.table(1) == shared
+    for t in range(tail):
+        runner.reserve(0, split + t + 1)
+        runner.reserve(1, split + t + 1)
+        if t == 0:
+            # the parent got a copy of the half-full page, the child keeps the original alone
+            assert runner.cache.table(0)[2] != shared[2] and runner.cache.table(1)[2] == shared[2]
+            assert runner.cache.table(0)[:2] == runner.cache.table(1)[:2] == shared[:2]
+        logits = runner.step([StepEntry(0, [tokens[split + t]], [0]),
+                              StepEntry(1, [other[t]], [0])]).float().cpu()
+        assert (logits[0] - want_parent[split + t]).abs().max().item() < TOL[dtype], f"parent at {t}"
+        assert (logits[1] - want_child[split + t]).abs().max().item() < TOL[dtype], f"child at {t}"
+    runner.cache.check_invariants()
+    runner.free(0)
+    runner.free(1)
+    assert runner.cache.num_free_pages(0) == runner.cache.num_pages(0)
+
+
 LONG = {
     "architectures": ["LlamaForCausalLM"], "hidden_size": 128, "intermediate_size": 176,
     "num_hidden_layers": 2, "num_attention_heads": 8, "num_key_value_heads": 2, "head_dim": 64,

@@ -120,6 +120,52 @@ def test_random_weights_are_seeded_and_have_the_stated_distributions():
     assert torch.equal(h["lm_head.weight"], a["lm_head.weight"].to(torch.bfloat16))
 
 
+def test_random_values_are_a_function_of_seed_tensor_and_element():
+    """The generator written out a second time, in plain Python integers and ``math``: value i
+    of tensor t under seed s is Box-Muller of two splitmix64 hashes of (s, t, i // 2).  The
+    native code must give the same float32 values (to the last bit, give or take a library's
+    last digit of log and cos in double precision: one float32 step at most, and next to never),
+    on one thread as on many."""
+    import math
+    from rust_llm_inference_server_amd.weights.random_init import normal_fill
+    mask = (1 << 64) - 1
+
+    def mix(x):
+        x = (x + 0x9E3779B97F4A7C15) & mask
+        x = ((x ^ (x >> 30)) * 0xBF58476D1CE4E5B9) & mask
+        x = ((x ^ (x >> 27)) * 0x94D049BB133111EB) & mask
+        return x ^ (x >> 31)
+
+    def twin(n, seed, tensor, mean, std):
+        key = mix(seed ^ mix(tensor))
+        out = []
+        for j in range((n + 1) // 2):
+            u1 = ((mix((key + 2 * j) & mask) >> 11) + 0.5) / 2.0 ** 53
+            u2 = ((mix((key + 2 * j + 1) & mask) >> 11) + 0.5) / 2.0 ** 53
+            r = math.sqrt(-2.0 * math.log(u1))
+            out += [mean + std * (r * math.cos(2 * math.pi * u2)),
+                    mean + std * (r * math.sin(2 * math.pi * u2))]
+        return torch.tensor(out[:n], dtype=torch.float64).to(torch.float32)
+
+    for n, seed, tensor, mean, std in ((1, 0, 0, 0.0, 0.02), (7, 5, 3, 1.0, 0.02), (4001, 2 ** 63 + 9, 146, 0.0, 1.0)):
+        got = normal_fill(n, seed, tensor, mean, std, threads=1)
+        want = twin(n, seed, tensor, mean, std)
+        step = torch.maximum(want.abs(), torch.tensor(1e-30)) * 2.0 ** -23
+        assert ((got - want).abs() <= step).all()
+        assert (got != want).sum().item() <= 1
+    # any number of threads, the same bits; a long tensor is cut among them
+    big = normal_fill(300001, 7, 2, 0.0, 0.02, threads=1)
+    for threads in (2, 3, 16, 0):
+        assert torch.equal(normal_fill(300001, 7, 2, 0.0, 0.02, threads=threads), big)
+    assert abs(big.mean().item()) < 2e-4 and abs(big.std().item() - 0.02) < 2e-4
+    # a prefix of a tensor is the tensor's beginning; another tensor index, other values
+    assert torch.equal(normal_fill(1000, 7, 2, 0.0, 0.02), big[:1000])
+    assert not torch.equal(normal_fill(1000, 7, 3, 0.0, 0.02), big[:1000])
+    # the normal's tails are there and nothing is off the scale
+    z = big / 0.02
+    assert 3.5 < z.abs().max().item() < 6.5 and abs((z.abs() < 1).float().mean().item() - 0.6827) < 0.005
+
+
 def test_written_folder_loads_back(tmp_path):
     folder = make_model_folder(tmp_path / "m", TINY_B, 3)
     assert sorted(os.listdir(folder)) == ["config.json", "model.safetensors"]
