@@ -562,7 +562,9 @@ def register_toy_router_and_position():
             self.max_positions = ctx.max_positions
 
 
-def plain_router_model(w, ids, H, nh, nkv, d, rot, step_size, experts, eps=1e-5):
+def plain_router_model(w, ids, H, nh, nkv, d, rot, step_size, experts, eps=1e-5, margins=None):
+    """``margins`` (a list) receives every row's gap between its two largest router
+    probabilities."""
     x = plain.embedding(w["model.embed_tokens.weight"], ids)
     T = len(ids)
     for li in range(2):
@@ -580,6 +582,9 @@ def plain_router_model(w, ids, H, nh, nkv, d, rot, step_size, experts, eps=1e-5)
             x = x + plain.linear(o.transpose(0, 1).reshape(T, nh * d), w[f"{p}.self_attn.o_proj.weight"])
             h = plain.rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], eps)
             prob = torch.softmax(plain.linear(h, w[f"{p}.mlp.router.weight"]), dim=-1)
+            if margins is not None:
+                top2 = prob.topk(2, dim=-1).values
+                margins += (top2[:, 0] - top2[:, 1]).tolist()
             rows = []
             for t in range(T):
                 e = int(prob[t].argmax())
@@ -618,11 +623,20 @@ def test_toy_routed_feed_forward_and_toy_position_encoding(tmp_path, dtype, tol)
                                        build_spec=build_spec, config_to_dict=lambda c: c))
     config = {"architectures": ["ToyRoutedForCausalLM"], "vocab_size": 97, "step": 0.05}
     spec = build_spec(config)
-    folder = str(tmp_path / "toy_routed")
-    write_model_folder(folder, config, spec.tensor_specs(), seed=12)
-    w = plain.read_weights(folder)
     reqs = traces.random_requests(97, [30, 4, 70, 11], seed=10)
-    ref = {k: plain_router_model(w, t, H, nh, nkv, d, rot, 0.05, E) for k, t in reqs.items()}
+    # Weights for which no row's routing is a near-tie: a row whose two best experts are a hair
+    # apart goes to either in bfloat16, and the other expert's output is another number
+    # altogether.  The first seed whose closest call is clear of that is taken.
+    for seed in range(12, 60):
+        folder = str(tmp_path / f"toy_routed_{seed}")
+        write_model_folder(folder, config, spec.tensor_specs(), seed=seed)
+        w = plain.read_weights(folder)
+        margins = []
+        ref = {k: plain_router_model(w, t, H, nh, nkv, d, rot, 0.05, E, margins=margins)
+               for k, t in reqs.items()}
+        if min(margins) > 2e-3:
+            break
+    assert min(margins) > 2e-3, "no seed gave clear routing"
     for build in (traces.trace_whole, traces.trace_tail, traces.trace_portions, traces.trace_mixed):
         steps, max_tokens = build(reqs)
         model = load_model(folder, dtype, max_positions=128)
