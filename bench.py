@@ -1,4 +1,5 @@
-"""Decode and prefill throughput of the Llama-3.2-1B shape on one MI355X.
+"""Decode and prefill throughput of the Llama-3.2-1B shape on one MI355X, and the larger
+workloads beside it.
 
     python bench.py --gpus 1 --steps K --warmup W
 
@@ -7,19 +8,32 @@ benchmark context (4,096 positions): W untimed decode steps, then exactly K time
 the engine (schedule, forward from the paged cache, on-device greedy sampling, token fed
 back), bracketed by device synchronisation.  On the same line: a 2,048-token prefill with its
 fraction of the bf16 matrix peak, the decode step's achieved fraction of the HBM roofline
-(bytes that must be read: every weight once plus the live requests' cache), and decode
-throughput at batch 1 and 64 after 512-token prompts.  Weights are random (N(0, 0.02)),
-prompts are uniform random token ids.
+(bytes that must be read: every weight once plus the live requests' cache), and under
+``points`` decode throughput at batch 1, 8 and 64 after 512-token prompts (each with its
+fraction of the HBM roofline, ``..._frac``) and, while the time budget lasts (``--extra-seconds``;
+``--skip-extra`` leaves them out), two more workloads, each in a fresh model:
+
+* ``serve_3b_...``: 64 requests with prompts of 128 to 2,048 tokens through the engine under
+  continuous batching with a token budget of 512 (chunked prefill), 256 new tokens each, at the
+  Llama-3.2-3B shape: generated tokens per second from the first arrival to the last end;
+* ``long_8b_...``: 32 requests of 8,192 prompt tokens and 128 new tokens each at the
+  Llama-3.1-8B shape: the same, plus tokens per second and HBM fraction of the steps that only
+  decode (context about 8,256), and the prompt tokens per second of the steps before them.
+
+Each of the two runs as a child process (the second command below, and the third): a failure
+there is reported on stderr and leaves the headline as it is.
+Weights are random (N(0, 0.02)), prompts are uniform random token ids.
 
     python bench.py --serve --model llama-3.2-3b --max-batched-tokens 512
+    python bench.py --serve --model llama-3.1-8b --requests 32 --min-prompt 8192 \\
+        --max-prompt 8192 --new-tokens 128 --max-batched-tokens 8192
 
-measures another workload instead (its own JSON line): R requests with prompts of uniform
-random length under continuous batching with chunked prefill, N new tokens each with seeded
-temperature sampling, timed from the first request's arrival to the last one's end."""
+run one of those workloads alone and print its own JSON line."""
 import argparse
 import copy
 import json
 import os
+import subprocess
 import sys
 import time
 
@@ -28,6 +42,116 @@ sys.path.insert(0, ROOT)
 
 HBM_GBPS = 8000.0            # MI355X HBM3E, published
 PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}
+PAGE = 16
+
+
+def say(msg: str) -> None:
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+class Shape:
+    """Sizes of a preset and the bytes and flops that follow from them."""
+
+    def __init__(self, cfg: dict, elem: int):
+        self.cfg = cfg
+        self.L, self.H, self.I = cfg["num_hidden_layers"], cfg["hidden_size"], cfg["intermediate_size"]
+        self.nh, self.nkv, self.d = (cfg["num_attention_heads"], cfg["num_key_value_heads"],
+                                     cfg["head_dim"])
+        self.V = cfg["vocab_size"]
+        self.layer_params = ((self.nh + 2 * self.nkv) * self.d * self.H + self.H * self.nh * self.d
+                             + 3 * self.H * self.I + 2 * self.H)
+        tied = cfg["tie_word_embeddings"]
+        self.weight_bytes = (self.L * self.layer_params + self.V * self.H + self.H
+                             + (0 if tied else self.V * self.H)) * elem
+        self.kv_bytes_per_token = 2 * self.L * self.nkv * self.d * elem
+
+    def decode_step_bytes(self, batch: int, mean_context: float) -> float:
+        """What a decode step has to read: every weight once and the live requests' cache."""
+        return self.weight_bytes + batch * mean_context * self.kv_bytes_per_token
+
+    def prefill_flops(self, T: int) -> float:
+        linear = 2.0 * T * self.L * (self.layer_params - 2 * self.H)
+        attention = 4.0 * self.L * self.nh * self.d * T * (T + 1) / 2
+        return linear + attention + 2.0 * self.V * self.H
+
+
+def build_model(name: str, dtype: str, layers, longest: int):
+    import torch
+    from rust_llm_inference_server_amd.config import preset_dict
+    from rust_llm_inference_server_amd.engine import random_model
+    cfg = preset_dict(name)
+    full_layers = cfg["num_hidden_layers"]
+    if layers:
+        cfg["num_hidden_layers"] = layers
+    cfg["max_position_embeddings"] = min(cfg["max_position_embeddings"], longest + 64)
+    t0 = time.time()
+    model = random_model(cfg, seed=0, dtype=dtype, max_positions=cfg["max_position_embeddings"])
+    torch.cuda.synchronize()
+    say(f"{name} ready in {time.time() - t0:.1f}s")
+    return model, cfg, full_layers
+
+
+def run_requests(model, shape: Shape, reqs, new_tokens: int, budget: int, trials: int = 2) -> dict:
+    """``reqs`` through the engine under continuous batching with a token budget of ``budget``
+    (chunked prefill), ``new_tokens`` each with seeded temperature sampling; timed from the
+    first arrival to the last end (best of ``trials``: the first also captures the graphs).
+    Steps that only decode, with every request live, are also timed on their own."""
+    import torch
+    from rust_llm_inference_server_amd.config import EngineConfig
+    from rust_llm_inference_server_amd.engine import Engine
+    from rust_llm_inference_server_amd.sampling import SamplingParams
+    lens = [len(r) for r in reqs]
+    pages = sum(-(-(n + new_tokens) // PAGE) + 1 for n in lens) + 64
+    sp = SamplingParams(max_tokens=new_tokens, ignore_eos=True, temperature=0.8, seed=1)
+    best = None
+    for trial in range(trials):
+        engine = Engine(model, EngineConfig(
+            max_num_seqs=len(reqs), max_batched_tokens=max(budget, len(reqs)), num_pages=pages,
+            block_size=PAGE, max_seq_len=max(lens) + new_tokens + 8))
+        for r in reqs:
+            engine.add_request(r, sp)
+        decode_s = prefill_s = 0.0
+        decode_steps = decode_tokens = 0
+        context_sum = 0.0
+        torch.cuda.synchronize()
+        t0 = last = time.perf_counter()
+        while engine.has_work():
+            before = copy.copy(engine.stats())
+            running = engine.scheduler.num_running
+            engine.step()                      # ends with the sampled tokens on the host
+            now = time.perf_counter()
+            after = engine.stats()
+            made = after.generated_tokens - before.generated_tokens
+            if after.prefill_tokens != before.prefill_tokens:
+                prefill_s += now - last
+            elif running == len(reqs) and made == len(reqs):
+                decode_s += now - last
+                decode_steps += 1
+                decode_tokens += made
+                context_sum += (sum(lens) + after.generated_tokens) / len(reqs)
+            last = now
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        stats = engine.stats()
+        generated = stats.generated_tokens
+        say(f"  run {trial}: {dt:.3f}s, {stats.steps} steps, {stats.preemptions} preemptions")
+        result = {
+            "seconds": dt, "generated": generated, "prompt_tokens": sum(lens), "steps": stats.steps,
+            "preemptions": stats.preemptions, "tok_s": generated / dt,
+            "total_tok_s": (generated + sum(lens)) / dt,
+            "prefill_tok_s": stats.prefill_tokens / prefill_s if prefill_s else 0.0,
+            "decode_steps": decode_steps,
+            "decode_tok_s": decode_tokens / decode_s if decode_s else 0.0,
+            "decode_ms": decode_s / decode_steps * 1e3 if decode_steps else 0.0,
+        }
+        if decode_steps:
+            step_bytes = shape.decode_step_bytes(len(reqs), context_sum / decode_steps)
+            result["decode_context"] = context_sum / decode_steps
+            result["decode_frac"] = step_bytes / (decode_s / decode_steps) / 1e9 / HBM_GBPS
+        if best is None or result["seconds"] < best["seconds"]:
+            best = result
+        del engine
+    return best
 
 
 def main() -> int:
@@ -44,10 +168,14 @@ def main() -> int:
     ap.add_argument("--points-context", type=int, default=512)
     ap.add_argument("--skip-points", action="store_true")
     ap.add_argument("--skip-prefill", action="store_true")
+    ap.add_argument("--skip-extra", action="store_true",
+                    help="leave out the 3B serving run and the 8B long-context run")
+    ap.add_argument("--extra-seconds", type=float, default=150.0,
+                    help="an extra workload starts only while the run is younger than this")
     ap.add_argument("--max-batched-tokens", type=int, default=8192,
                     help="token budget of the engine steps that prefill the decode runs")
     ap.add_argument("--serve", action="store_true",
-                    help="time a batch of requests through Engine.generate instead")
+                    help="time a batch of requests through the engine instead")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--min-prompt", type=int, default=128)
     ap.add_argument("--max-prompt", type=int, default=2048)
@@ -56,58 +184,76 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (single-GPU engine)")
         return 2
+    started = time.time()
 
     import torch
-    from rust_llm_inference_server_amd.config import EngineConfig, preset_dict
-    from rust_llm_inference_server_amd.engine import Engine, ModelRunner, StepEntry, random_model
+    from rust_llm_inference_server_amd.config import EngineConfig
+    from rust_llm_inference_server_amd.engine import Engine, ModelRunner, StepEntry
     from rust_llm_inference_server_amd.ops import lib
     from rust_llm_inference_server_amd.sampling import SamplingParams
 
     torch.cuda.set_device(0)
     lib.load()
-    cfg = preset_dict(args.model)
-    full_layers = cfg["num_hidden_layers"]
-    if args.layers:
-        cfg["num_hidden_layers"] = args.layers
-    # room for the timed steps themselves when they are more than the context holds
-    longest = max(args.context, args.prefill_tokens, 4096, args.steps + args.warmup + 128)
-    if args.serve:
-        longest = max(longest, args.max_prompt + args.new_tokens)
-    cfg["max_position_embeddings"] = min(cfg["max_position_embeddings"], longest + 64)
-    page = 16
     K, W = args.steps, args.warmup
     elem = 2 if args.dtype == "bfloat16" else 4
-    t_load = time.time()
-    model = random_model(cfg, seed=0, dtype=args.dtype, max_positions=cfg["max_position_embeddings"])
-    torch.cuda.synchronize()
-    print(f"[bench] model ready in {time.time() - t_load:.1f}s", file=sys.stderr, flush=True)
-    L, H, I = cfg["num_hidden_layers"], cfg["hidden_size"], cfg["intermediate_size"]
-    nh, nkv, d, V = (cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"],
-                     cfg["vocab_size"])
-    layer_params = (nh + 2 * nkv) * d * H + H * nh * d + 3 * H * I + 2 * H
-    weight_bytes = (L * layer_params + V * H + H + (0 if cfg["tie_word_embeddings"] else V * H)) * elem
-    kv_bytes_per_token = 2 * L * nkv * d * elem
     g = torch.Generator().manual_seed(0)
 
-    def prompts(n, length):
-        return [torch.randint(0, V, (length,), generator=g).tolist() for _ in range(n)]
+    def prompts(n, length, vocab):
+        return [torch.randint(0, vocab, (length,), generator=g).tolist() for _ in range(n)]
+
+    def random_requests(n, lo, hi, vocab):
+        lens = torch.randint(lo, hi + 1, (n,), generator=g).tolist()
+        return [torch.randint(0, vocab, (m,), generator=g).tolist() for m in lens]
+
+    if args.serve:
+        # ---- one workload of requests through the engine, alone ------------------------------
+        model, cfg, full_layers = build_model(args.model, args.dtype, args.layers,
+                                              args.max_prompt + args.new_tokens)
+        shape = Shape(cfg, elem)
+        reqs = random_requests(args.requests, args.min_prompt, args.max_prompt, shape.V)
+        r = run_requests(model, shape, reqs, args.new_tokens, args.max_batched_tokens)
+        print(json.dumps({
+            "metric": f"served tok/s, {args.requests} requests ({args.model} shape)",
+            "value": round(r["tok_s"], 1), "unit": "generated tokens/s", "n_gpus": 1,
+            "seconds": round(r["seconds"], 4), "higher_is_better": True,
+            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
+            "config": {"model": args.model, "layers": shape.L, "layers_full": full_layers,
+                       "requests": args.requests, "min_prompt": args.min_prompt,
+                       "max_prompt": args.max_prompt, "new_tokens": args.new_tokens,
+                       "max_batched_tokens": args.max_batched_tokens, "page_size": PAGE,
+                       "prompt_tokens": r["prompt_tokens"], "generated_tokens": r["generated"],
+                       "steps": r["steps"], "preemptions": r["preemptions"]},
+            "total_tokens_per_s": round(r["total_tok_s"], 1),
+            "prefill_tokens_per_s": round(r["prefill_tok_s"], 1),
+            "decode": {"steps": r["decode_steps"], "tokens_per_s": round(r["decode_tok_s"], 1),
+                       "ms_per_step": round(r["decode_ms"], 4),
+                       "context": round(r.get("decode_context", 0.0), 1),
+                       "hbm_frac": round(r.get("decode_frac", 0.0), 4)},
+        }))
+        return 0
+
+    # room for the timed steps themselves when they are more than the context holds
+    longest = max(args.context, args.prefill_tokens, 4096, K + W + 128)
+    model, cfg, full_layers = build_model(args.model, args.dtype, args.layers, longest)
+    shape = Shape(cfg, elem)
 
     def decode_run(batch, context, steps, warmup):
-        """tokens/s and ms/step of `steps` decode steps of `batch` requests, none of which goes
-        beyond `context`.  Prompts are prefilled in portions under the engine's token budget
-        while earlier requests already decode, so every request is given room for the steps
-        that the prefill of the others takes; the timed steps are pure decode steps."""
+        """tokens/s, ms/step and mean context of `steps` decode steps of `batch` requests, none
+        of which goes beyond `context`.  Prompts are prefilled in portions under the engine's
+        token budget while earlier requests already decode, so every request is given room for
+        the steps that the prefill of the others takes; the timed steps are pure decode steps."""
         budget = max(args.max_batched_tokens, batch)
         prefill_steps = -(-batch * context // budget) + 1
         new_tokens = steps + warmup + prefill_steps + 1
         context = max(context, new_tokens + 16)           # more steps than the context holds
         prompt_len = context - new_tokens
-        pages = batch * (-(-context // page) + 1) + 8
+        pages = batch * (-(-context // PAGE) + 1) + 8
         engine = Engine(model, EngineConfig(max_num_seqs=max(batch, 1), max_batched_tokens=budget,
-                                            num_pages=pages, block_size=page,
+                                            num_pages=pages, block_size=PAGE,
                                             max_seq_len=context + 8, watermark_pages=0))
         sp = SamplingParams(max_tokens=new_tokens, ignore_eos=True)
-        for p in prompts(batch, prompt_len):
+        for p in prompts(batch, prompt_len, shape.V):
             engine.add_request(p, sp)
         while engine.stats().prefill_tokens < batch * prompt_len or engine.stats().waiting:
             engine.step()                                     # prefill, in portions
@@ -128,48 +274,10 @@ def main() -> int:
         mean_ctx = prompt_len + (before.generated_tokens + after.generated_tokens) / 2 / batch
         return batch * steps / dt, dt / steps * 1e3, mean_ctx
 
-    if args.serve:
-        # ---- continuous batching: R requests, chunked prefill under the token budget ---------
-        lens = torch.randint(args.min_prompt, args.max_prompt + 1, (args.requests,), generator=g).tolist()
-        reqs = [torch.randint(0, V, (n,), generator=g).tolist() for n in lens]
-        pages = sum(-(-(n + args.new_tokens) // page) + 1 for n in lens) + 64
-        sp = SamplingParams(max_tokens=args.new_tokens, ignore_eos=True, temperature=0.8, seed=1)
-        best = None
-        for trial in range(2):                       # the first run also captures the graphs
-            engine = Engine(model, EngineConfig(
-                max_num_seqs=args.requests, max_batched_tokens=max(args.max_batched_tokens, args.requests),
-                num_pages=pages, block_size=page, max_seq_len=args.max_prompt + args.new_tokens + 8))
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            outs = engine.generate(reqs, sp)
-            torch.cuda.synchronize()
-            dt = time.perf_counter() - t0
-            best = dt if best is None else min(best, dt)
-            stats = engine.stats()
-            print(f"[bench] serve run {trial}: {dt:.3f}s, {stats.steps} steps, "
-                  f"{stats.preemptions} preemptions", file=sys.stderr, flush=True)
-        generated = sum(len(o.token_ids) for o in outs)
-        print(json.dumps({
-            "metric": f"served tok/s, {args.requests} requests ({args.model} shape)",
-            "value": round(generated / best, 1), "unit": "generated tokens/s", "n_gpus": 1,
-            "seconds": round(best, 4), "higher_is_better": True,
-            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-            "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
-            "config": {"model": args.model, "layers": L, "layers_full": full_layers,
-                       "requests": args.requests, "min_prompt": args.min_prompt,
-                       "max_prompt": args.max_prompt, "new_tokens": args.new_tokens,
-                       "max_batched_tokens": args.max_batched_tokens, "page_size": page,
-                       "prompt_tokens": sum(lens), "generated_tokens": generated,
-                       "steps": stats.steps, "mean_ttft_ms": round(
-                           sum(o.ttft for o in outs) / len(outs) * 1e3, 1)},
-            "total_tokens_per_s": round((generated + sum(lens)) / best, 1),
-        }))
-        return 0
-
     # ---- prefill: one prompt of T tokens in one step, last-row logits ------------------
     T = args.prefill_tokens
-    runner = ModelRunner(model, num_pages=-(-T // page) + 1, page_size=page, max_num_seqs=1)
-    prompt = prompts(1, T)[0]
+    runner = ModelRunner(model, num_pages=-(-T // PAGE) + 1, page_size=PAGE, max_num_seqs=1)
+    prompt = prompts(1, T, shape.V)[0]
     times = []
     for i in range(1 if args.skip_prefill else 4):
         runner.reserve(0, T)
@@ -180,32 +288,65 @@ def main() -> int:
         times.append(time.perf_counter() - t0)
         runner.free(0)
     prefill_s = min(times[1:] or times)
-    linear_flops = 2.0 * T * L * (layer_params - 2 * H)
-    attn_flops = 4.0 * L * nh * d * T * (T + 1) / 2
-    head_flops = 2.0 * V * H
-    prefill_flops = linear_flops + attn_flops + head_flops
     prefill = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
-               "frac": round(prefill_flops / prefill_s / (PEAK_TFLOPS[args.dtype] * 1e12), 4)}
+               "frac": round(shape.prefill_flops(T) / prefill_s / (PEAK_TFLOPS[args.dtype] * 1e12), 4)}
     del runner
-    print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
+    say(f"prefill {prefill}")
 
     # ---- headline: batch B near the benchmark context ------------------------------------
     value, ms_per_step, mean_ctx = decode_run(args.batch, args.context, K, W)
-    step_bytes = weight_bytes + args.batch * mean_ctx * kv_bytes_per_token
-    achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
+    achieved = shape.decode_step_bytes(args.batch, mean_ctx) / (ms_per_step * 1e-3) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_GBPS, 4)}
-    print(f"[bench] decode b{args.batch}: {value:.0f} tok/s, {ms_per_step:.3f} ms/step",
-          file=sys.stderr, flush=True)
+    say(f"decode b{args.batch}: {value:.0f} tok/s, {ms_per_step:.3f} ms/step, "
+        f"{roofline['frac']:.3f} of HBM")
 
     points = {}
     if not args.skip_points:
-        for b in (1, 64):
+        # the metric's own workload: 512-token prompts, then decode at batch 1, 8 and 64
+        for b in (1, 8, 64):
             steps = min(K, 128)
             ctx = args.points_context + steps + W
-            v, ms, _ = decode_run(b, ctx, steps, W)
-            points[f"decode_b{b}"] = round(v, 1)
-            print(f"[bench] decode b{b}: {v:.0f} tok/s, {ms:.3f} ms/step", file=sys.stderr, flush=True)
+            v, ms, mean = decode_run(b, ctx, steps, W)
+            frac = shape.decode_step_bytes(b, mean) / (ms * 1e-3) / 1e9 / HBM_GBPS
+            name = f"decode_b{b}" if b != args.batch else f"decode_b{b}_ctx{args.points_context}"
+            points[name] = round(v, 1)
+            points[name + "_frac"] = round(frac, 4)
+            say(f"decode b{b} after {args.points_context}-token prompts: {v:.0f} tok/s, "
+                f"{ms:.3f} ms/step, {frac:.3f} of HBM")
+
+    # ---- the larger workloads, each in a model of its own ------------------------------------
+    extras = [] if args.skip_extra or args.skip_points or args.layers else [
+        ("serve_3b", "llama-3.2-3b", dict(n=64, lo=128, hi=2048, new=256, budget=512)),
+        ("long_8b", "llama-3.1-8b", dict(n=32, lo=8192, hi=8192, new=128, budget=8192)),
+    ]
+    for key, name, wl in extras:
+        if time.time() - started > args.extra_seconds:
+            say(f"{key}: left out, the run is older than {args.extra_seconds:.0f}s")
+            continue
+        # A process of its own: whatever happens there, the headline below is printed.
+        cmd = [sys.executable, os.path.abspath(__file__), "--serve", "--model", name, "--dtype",
+               args.dtype, "--requests", str(wl["n"]), "--min-prompt", str(wl["lo"]), "--max-prompt",
+               str(wl["hi"]), "--new-tokens", str(wl["new"]), "--max-batched-tokens",
+               str(wl["budget"])]
+        try:
+            child = subprocess.run(cmd, stdout=subprocess.PIPE, text=True, timeout=240)
+            line = (child.stdout.strip().splitlines() or [""])[-1]
+            if child.returncode != 0 or not line.startswith("{"):
+                raise RuntimeError(f"exit code {child.returncode}")
+            r = json.loads(line)
+            points[f"{key}_tok_s"] = r["value"]
+            points[f"{key}_total_tok_s"] = r["total_tokens_per_s"]
+            points[f"{key}_prefill_tok_s"] = r["prefill_tokens_per_s"]
+            points[f"{key}_decode_tok_s"] = r["decode"]["tokens_per_s"]
+            points[f"{key}_decode_ms"] = r["decode"]["ms_per_step"]
+            points[f"{key}_decode_frac"] = r["decode"]["hbm_frac"]
+            say(f"{key}: {r['value']:.0f} generated tok/s in {r['seconds']:.2f}s; decode steps "
+                f"{r['decode']['ms_per_step']:.2f} ms, {r['decode']['tokens_per_s']:.0f} tok/s, "
+                f"{r['decode']['hbm_frac']:.3f} of HBM at context {r['decode']['context']:.0f}; "
+                f"prompts {r['prefill_tokens_per_s']:.0f} tok/s")
+        except Exception as exc:
+            say(f"{key} failed: {type(exc).__name__}: {exc}")
 
     print(json.dumps({
         "metric": f"decode tok/s at batch {args.batch} ({args.model} shape)", "value": round(value, 1),
@@ -213,11 +354,11 @@ def main() -> int:
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
-        "config": {"model": args.model, "layers": L, "layers_full": full_layers, "hidden": H,
-                   "heads": nh, "kv_heads": nkv, "head_dim": d, "intermediate": I, "vocab": V,
-                   "global_batch": args.batch, "seq_len": args.context, "page_size": page,
-                   "prefill_tokens": T, "points_context": args.points_context,
-                   "parallelism": "single GPU"},
+        "config": {"model": args.model, "layers": shape.L, "layers_full": full_layers,
+                   "hidden": shape.H, "heads": shape.nh, "kv_heads": shape.nkv, "head_dim": shape.d,
+                   "intermediate": shape.I, "vocab": shape.V, "global_batch": args.batch,
+                   "seq_len": args.context, "page_size": PAGE, "prefill_tokens": T,
+                   "points_context": args.points_context, "parallelism": "single GPU"},
         "prefill": prefill, "roofline": roofline, "points": points,
     }))
     return 0

@@ -595,3 +595,59 @@ RLIS_API int rlis_copy_pages(void* pages, int dtype, int num_layers, long long n
   RLIS_LAUNCH_CHECK("copy_pages");
   return 0;
 }
+
+// ------------------------------------------------------------- seeded random weights
+// The generator of runtime/random_fill.cpp on the device: value i of a tensor is a function of
+// (seed, tensor index, i) alone: two splitmix64 hashes of the pair index give two uniforms,
+// Box-Muller in double precision turns them into the pair's two normals, rounded once to
+// float32 (and, for a bfloat16 destination, once more).  The host's and the device's log, cos
+// and sin may differ in the last digit of a double, which the rounding to float32 hides but for
+// a value in a few hundred million.
+__device__ __forceinline__ uint64_t splitmix64(uint64_t x) {
+  x += 0x9E3779B97F4A7C15ull;
+  x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+  x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+  return x ^ (x >> 31);
+}
+
+template <typename TO>
+__global__ void fill_normal_kernel(TO* __restrict__ out, long long n, uint64_t key, double mean,
+                                   double std_dev) {
+  const long long pairs = (n + 1) / 2;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long j = (long long)blockIdx.x * blockDim.x + threadIdx.x; j < pairs; j += stride) {
+    const uint64_t a = splitmix64(key + 2 * (uint64_t)j), b = splitmix64(key + 2 * (uint64_t)j + 1);
+    const double u1 = ((double)(a >> 11) + 0.5) * (1.0 / 9007199254740992.0);
+    const double u2 = ((double)(b >> 11) + 0.5) * (1.0 / 9007199254740992.0);
+    const double r = sqrt(-2.0 * log(u1));
+    const double angle = 6.283185307179586476925286766559 * u2;
+    st(out + 2 * j, (float)(mean + std_dev * (r * cos(angle))));
+    if (2 * j + 1 < n) st(out + 2 * j + 1, (float)(mean + std_dev * (r * sin(angle))));
+  }
+}
+
+// out[0 .. n) = mean + std * N(0, 1) keyed by (seed, tensor); out is float32 or bfloat16.
+RLIS_API int rlis_fill_normal_device(void* out, int out_dtype, long long n, unsigned long long seed,
+                                     unsigned long long tensor, double mean, double std_dev,
+                                     hipStream_t stream) {
+  RLIS_REQUIRE(n >= 0 && out, "fill_normal: bad arguments");
+  if (n == 0) return 0;
+  // host side of the same hash
+  auto mix = [](uint64_t x) {
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+  };
+  const uint64_t key = mix((uint64_t)seed ^ mix((uint64_t)tensor));
+  const long long pairs = (n + 1) / 2;
+  const int blocks = (int)(ceil_div_ll(pairs, 256) < 8192 ? ceil_div_ll(pairs, 256) : 8192);
+  if (out_dtype == RLIS_F32)
+    fill_normal_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, n, key, mean, std_dev);
+  else if (out_dtype == RLIS_BF16)
+    fill_normal_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, n, key, mean, std_dev);
+  else
+    RLIS_REQUIRE(false, "fill_normal: unknown dtype %d", out_dtype);
+  RLIS_LAUNCH_CHECK("fill_normal");
+  return 0;
+}

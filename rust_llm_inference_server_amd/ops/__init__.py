@@ -597,6 +597,18 @@ def sample_rows(logits: torch.Tensor, keys: torch.Tensor, inv_temps: torch.Tenso
     return out
 
 
+def fill_normal(out: torch.Tensor, seed: int, tensor_index: int, mean: float, std: float) -> None:
+    """Fill ``out`` (float32 or bfloat16, contiguous, on the GPU) with ``mean + std * N(0, 1)``
+    keyed by (seed, tensor index, element index): the generator of ``weights/random_init.py``,
+    run on the device."""
+    _check(out, "fill_normal out")
+    if not out.is_contiguous():
+        raise KernelError("fill_normal: the tensor must be contiguous")
+    mask = (1 << 64) - 1
+    lib.call("rlis_fill_normal_device", out.data_ptr(), _dt(out), out.numel(), int(seed) & mask,
+             int(tensor_index) & mask, float(mean), float(std), lib.stream_ptr())
+
+
 __all__ = ["AttentionPlanner", "KernelError", "add_residual", "add_rmsnorm", "attention_planner",
-           "copy_pages", "embed", "linear", "linear_swiglu", "norm_linear", "paged_attention",
+           "copy_pages", "embed", "fill_normal", "linear", "linear_swiglu", "norm_linear", "paged_attention",
            "rope_attention", "rope_kv_write", "sample_rows", "swiglu"]

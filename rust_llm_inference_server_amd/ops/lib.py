@@ -35,6 +35,8 @@ _SIGNATURES = {
                                P],
     "rlis_attn_reduce_rows": [P, L, P, P, P, P, I, I, I, I, I, P],
     "rlis_sample_rows": [P, L, I, I, P, P, P, I, P, P, P],
+    "rlis_fill_normal_device": [P, I, L, ctypes.c_ulonglong, ctypes.c_ulonglong, ctypes.c_double,
+                                ctypes.c_double, P],
 }
 
 

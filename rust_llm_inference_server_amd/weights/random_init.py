@@ -39,7 +39,15 @@ def normal_fill(numel: int, seed: int, tensor_index: int, mean: float, std: floa
 def random_tensor(spec: TensorSpec, seed: int, dtype: torch.dtype,
                   device: torch.device = torch.device("cpu"), index: int = 0) -> torch.Tensor:
     """The tensor ``spec`` describes, ``index`` being its place in the specification's list.
-    Values are made in float32 on the host, then rounded to ``dtype`` and moved."""
+    Values are made in float32 on the host, then rounded to ``dtype`` and moved; for a tensor
+    that is to live on the GPU they are made there, by the same formula (a model of billions of
+    weights is then ready in a moment)."""
+    if device.type == "cuda" and spec.init in ("normal", "ones_normal"):
+        from .. import ops
+        with torch.cuda.device(device):
+            t = torch.empty(tuple(spec.shape), dtype=dtype, device=device)
+            ops.fill_normal(t, seed, index, 1.0 if spec.init == "ones_normal" else 0.0, spec.std)
+        return t
     numel = 1
     for n in spec.shape:
         numel *= int(n)

@@ -118,8 +118,29 @@ def test_bench_line_has_the_agreed_fields():
     assert set(rec["prefill"]) == {"value", "tokens", "ms", "frac"} and rec["prefill"]["tokens"] == 2048
     assert rec["roofline"]["bound"] == "hbm" and rec["roofline"]["peak"] == 8000.0
     assert abs(rec["roofline"]["frac"] - rec["roofline"]["achieved"] / 8000.0) < 1e-3
-    assert set(rec["points"]) == {"decode_b1", "decode_b64"}
+    assert {"decode_b1", "decode_b64", "decode_b8_ctx512"} <= set(rec["points"])
+    assert all(isinstance(v, (int, float)) for v in rec["points"].values())
+    for name in ("decode_b1", "decode_b64", "decode_b8_ctx512"):
+        assert 0 < rec["points"][name + "_frac"] < 1
     assert abs(rec["value"] - 8 / rec["ms_per_step"] * 1e3) < 0.01 * rec["value"]
+
+
+@pytest.mark.gpu
+def test_bench_serves_a_batch_of_requests():
+    """The mode that the larger workloads run in (as child processes of the default run): a
+    few requests through the engine, one JSON line with the decode steps timed on their own."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--serve", "--layers", "2",
+                        "--requests", "6", "--min-prompt", "20", "--max-prompt", "90",
+                        "--new-tokens", "24", "--max-batched-tokens", "64"],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if l.startswith("{")]
+    assert len(lines) == 1
+    rec = json.loads(lines[0])
+    assert rec["config"]["generated_tokens"] == 6 * 24 and rec["config"]["requests"] == 6
+    assert rec["value"] > 0 and rec["total_tokens_per_s"] > rec["value"]
+    assert rec["decode"]["steps"] > 0 and 0 < rec["decode"]["hbm_frac"] < 1
+    assert 20 < rec["decode"]["context"] < 90 + 24
 
 
 @pytest.mark.gpu

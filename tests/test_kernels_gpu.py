@@ -882,6 +882,25 @@ def test_pages_past_two_to_the_31_elements(ops, dtype):
     assert torch.equal(pool[0, 2], far) and torch.equal(pool[0, big - 1], first)
 
 
+def test_seeded_weights_made_on_the_device_are_the_hosts(ops):
+    """The seeded generator on the device against the host's (one formula, twice written): the
+    float32 values agree to the bit but for a library's last digit of log and cos in double
+    precision (one float32 step, next to never); bfloat16 is the float32 value rounded."""
+    from rust_llm_inference_server_amd.weights.random_init import normal_fill
+    for n, seed, tensor, mean, std in ((1, 0, 0, 0.0, 0.02), (7, 5, 3, 1.0, 0.02),
+                                       (300001, 2 ** 63 + 9, 146, 0.0, 0.02)):
+        want = normal_fill(n, seed, tensor, mean, std)
+        got = torch.empty(n, dtype=torch.float32, device=DEV)
+        ops.fill_normal(got, seed, tensor, mean, std)
+        got = got.cpu()
+        step = torch.maximum(want.abs(), torch.tensor(1e-30)) * 2.0 ** -23
+        assert ((got - want).abs() <= step).all()
+        assert (got != want).sum().item() <= max(1, n // 100000)
+        half = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+        ops.fill_normal(half, seed, tensor, mean, std)
+        assert (half.cpu() != got.to(torch.bfloat16)).sum().item() == 0
+
+
 # ----------------------------------------------------------------- refusals
 def test_kernels_refuse_what_they_cannot_do(ops):
     with pytest.raises(ops.KernelError):
