@@ -233,6 +233,88 @@ static bool launch_add_rmsnorm_bf16x8(float* resid, const void* delta, const voi
   return true;
 }
 
+// The delta as a stack of float32 partial sums (what the split-k and the streaming products
+// leave for their consumer), rows of a multiple of 4 and at most 256 * 4 * CH elements: four
+// elements per thread and chunk, 16-byte accesses, four parts in flight at a time; the parts
+// are added in order and their sum rounded to bfloat16 when round_parts is set.
+template <typename TW, typename TO, int CH>
+__global__ __launch_bounds__(256) void add_rmsnorm_stack_kernel(
+    float* __restrict__ resid, const float* __restrict__ delta, const TW* __restrict__ weight,
+    TO* __restrict__ out, const int* __restrict__ rows, int H, float eps, int write_resid,
+    int parts, long long part_stride, int round_parts) {
+  __shared__ float red[256 / kWave];
+  const int r = blockIdx.x;
+  const long long src = rows ? (long long)rows[r] : (long long)r;
+  float* x = resid + src * H;
+  const float* d = delta + src * H;
+  float v[CH][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int ch = 0; ch < CH; ++ch) {
+    const int j = (threadIdx.x + ch * 256) * 4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[ch][e] = 0.f;
+    if (j < H) {
+      const float4 xr = *(const float4*)(x + j);
+      float4 s = *(const float4*)(d + j);
+      int p = 1;
+      for (; p + 3 < parts; p += 4) {
+        const float4 a = *(const float4*)(d + (p + 0) * part_stride + j);
+        const float4 b = *(const float4*)(d + (p + 1) * part_stride + j);
+        const float4 c = *(const float4*)(d + (p + 2) * part_stride + j);
+        const float4 e4 = *(const float4*)(d + (p + 3) * part_stride + j);
+        s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
+        s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
+        s.x += c.x; s.y += c.y; s.z += c.z; s.w += c.w;
+        s.x += e4.x; s.y += e4.y; s.z += e4.z; s.w += e4.w;
+      }
+      for (; p < parts; ++p) {
+        const float4 a = *(const float4*)(d + p * part_stride + j);
+        s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
+      }
+      if (round_parts) {
+        s.x = bf16_to_f32(f32_to_bf16(s.x)); s.y = bf16_to_f32(f32_to_bf16(s.y));
+        s.z = bf16_to_f32(f32_to_bf16(s.z)); s.w = bf16_to_f32(f32_to_bf16(s.w));
+      }
+      v[ch][0] = xr.x + s.x; v[ch][1] = xr.y + s.y; v[ch][2] = xr.z + s.z; v[ch][3] = xr.w + s.w;
+      if (write_resid) *(float4*)(x + j) = make_float4(v[ch][0], v[ch][1], v[ch][2], v[ch][3]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss += v[ch][e] * v[ch][e];
+    }
+  }
+  ss = block_sum<256>(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+  TO* o = out + (long long)r * H;
+#pragma unroll
+  for (int ch = 0; ch < CH; ++ch) {
+    const int j = (threadIdx.x + ch * 256) * 4;
+    if (j < H) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) st(o + j + e, v[ch][e] * inv * ld(weight + j + e));
+    }
+  }
+}
+
+// True when the kernel for stacks of float32 partial sums took the call.
+template <typename TW, typename TO>
+static bool launch_add_rmsnorm_stack(float* resid, const void* delta, const void* weight,
+                                     void* out, const int* rows, int R, int H, float eps,
+                                     int write_resid, int parts, long long part_stride,
+                                     int round_parts, hipStream_t stream) {
+  if (H % 4 != 0 || H > 256 * 4 * 8 || part_stride % 4 != 0) return false;
+  if (((uintptr_t)resid | (uintptr_t)delta) % 16) return false;
+#define LAUNCH(CH)                                                                            \
+  add_rmsnorm_stack_kernel<TW, TO, CH><<<R, 256, 0, stream>>>(                                \
+      resid, (const float*)delta, (const TW*)weight, (TO*)out, rows, H, eps, write_resid,     \
+      parts, part_stride, round_parts)
+  if (H <= 256 * 4) LAUNCH(1);
+  else if (H <= 256 * 8) LAUNCH(2);
+  else if (H <= 256 * 16) LAUNCH(4);
+  else LAUNCH(8);
+#undef LAUNCH
+  return true;
+}
+
 template <typename TD, typename TW, typename TO>
 static void launch_add_rmsnorm(float* resid, const void* delta, const void* weight, void* out,
                                const int* rows, int R, int H, float eps, int write_resid,
@@ -267,6 +349,25 @@ RLIS_API int rlis_add_rmsnorm(float* resid, const void* delta, int delta_dtype,
                                 stream)) {
     RLIS_LAUNCH_CHECK("add_rmsnorm");
     return 0;
+  }
+  if (delta && delta_dtype == RLIS_F32 && parts > 1) {
+    bool took = false;
+    if (weight_dtype == RLIS_BF16 && out_dtype == RLIS_BF16)
+      took = launch_add_rmsnorm_stack<bf16_t, bf16_t>(resid, delta, weight, out, rows, R, H, eps,
+                                                      write_resid, parts, part_stride, round_parts,
+                                                      stream);
+    else if (weight_dtype == RLIS_F32 && out_dtype == RLIS_BF16)
+      took = launch_add_rmsnorm_stack<float, bf16_t>(resid, delta, weight, out, rows, R, H, eps,
+                                                     write_resid, parts, part_stride, round_parts,
+                                                     stream);
+    else if (weight_dtype == RLIS_F32 && out_dtype == RLIS_F32)
+      took = launch_add_rmsnorm_stack<float, float>(resid, delta, weight, out, rows, R, H, eps,
+                                                    write_resid, parts, part_stride, round_parts,
+                                                    stream);
+    if (took) {
+      RLIS_LAUNCH_CHECK("add_rmsnorm");
+      return 0;
+    }
   }
   const int key = (delta ? delta_dtype : out_dtype) * 4 + weight_dtype * 2 + out_dtype;
 #define CASE(k, TD, TW, TO)                                                                  \

@@ -429,6 +429,154 @@ RLIS_API int rlis_gemm_bf16_skinny_swiglu(const void* X, const void* W, void* Y,
   return 0;
 }
 
+// ==================================================== split-k product for 17 to 64 rows
+// y (T <= 64, N) = x W^T as float32 partial sums, one (T, N) array per k slice, for the
+// projections whose result joins the residual stream (its next consumer adds the slices in
+// order).  A workgroup of four waves owns 64 weight rows and one k slice of KS (256 or 512): the
+// rows of x of that slice lie in LDS for all four waves (tokens beyond T and k beyond K as
+// zeros), each wave loads its 16 weight rows of the slice straight into operand layout, all of
+// them at once (16 rows x 64 bytes per instruction, KS / 32 instructions in flight per lane),
+// and multiplies them with the four token groups from LDS (v_mfma_f32_16x16x32_bf16, weight
+// rows as the M side).  Every weight is read once, x once per 64 weight rows through the L2.
+// Which k a slice covers depends on K and N alone, so a row's sums do not depend on T.
+constexpr int kSplitRows = 64;          // weight rows per workgroup
+constexpr int kSplitPad = 16;           // bf16 elements between rows of x in LDS: 32 bytes mod 64
+
+template <int KS, int NT>
+__global__ __launch_bounds__(256, 2) void gemm_bf16_splitk_kernel(const bf16_t* __restrict__ X,
+                                                               const bf16_t* __restrict__ W,
+                                                               float* __restrict__ Y, int T, int N,
+                                                               int K, long long ldx, long long ldw,
+                                                               long long part_stride) {
+  extern __shared__ __attribute__((aligned(16))) bf16_t splitk_x[];   // [NT * 16][KS + pad]
+  constexpr int XS = KS + kSplitPad;
+  constexpr int STEPS = KS / 32;
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int l16 = lane % 16, lq = lane / 16;
+  const int slice = blockIdx.y;
+  const int k0 = slice * KS;
+  const int n0 = blockIdx.x * kSplitRows + wave * 16;
+
+  // This wave's weight rows, in operand layout: lane l holds row l % 16 and the 8 k at
+  // (l / 16) * 8 of every step.  Loads are never predicated off: a row past N reads row N - 1
+  // (its products are not stored), a k past K reads k = 0 (it meets a zero of x).
+  const int row = min(n0 + l16, N - 1);
+  const bf16_t* wrow = W + (long long)row * ldw;
+  Frag8 a[STEPS];
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    const int k = k0 + s * 32 + lq * 8;
+    a[s].u = *(const uint4*)(wrow + (k < K ? k : 0));
+  }
+  // The slice of x into LDS: 16-byte pieces, rows of tokens (zeros past T and past K).  All of a
+  // thread's pieces are loaded before the first is stored, so that they travel together (and
+  // with the weights); the loads are unconditional from a safe address, the value is selected.
+  constexpr int PIECES = KS / 8;
+  constexpr int XIT = NT * 16 * PIECES / 256;
+  uint4 xv[XIT];
+#pragma unroll
+  for (int j = 0; j < XIT; ++j) {
+    const int i = tid + j * 256;
+    const int tok = i / PIECES, k = k0 + (i % PIECES) * 8;
+    const bool ok = tok < T && k < K;
+    const uint4 v = *(const uint4*)(X + (ok ? (long long)tok * ldx + k : 0));
+    xv[j] = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+  }
+#pragma unroll
+  for (int j = 0; j < XIT; ++j) {
+    const int i = tid + j * 256;
+    *(uint4*)(splitk_x + (i / PIECES) * XS + (i % PIECES) * 8) = xv[j];
+  }
+  __syncthreads();
+
+  f32x4 acc[NT];
+#pragma unroll
+  for (int tg = 0; tg < NT; ++tg) acc[tg] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+#pragma unroll
+    for (int tg = 0; tg < NT; ++tg) {
+      Frag8 b;
+      b.u = *(const uint4*)(splitk_x + (tg * 16 + l16) * XS + s * 32 + lq * 8);
+      acc[tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s].v, b.v, acc[tg], 0, 0, 0);
+    }
+  }
+  // The accumulator holds token l % 16 of its group and weight rows (l / 16) * 4 + r.
+  float* y = Y + (long long)slice * part_stride;
+  const int col = n0 + lq * 4;
+#pragma unroll
+  for (int tg = 0; tg < NT; ++tg) {
+    const int tok = tg * 16 + l16;
+    if (tok >= T) continue;
+    float* dst = y + (long long)tok * N + col;
+    if (col + 3 < N && (N % 4) == 0 && (part_stride % 4) == 0) {
+      *(float4*)dst = make_float4(acc[tg][0], acc[tg][1], acc[tg][2], acc[tg][3]);
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (col + r < N) dst[r] = acc[tg][r];
+    }
+  }
+}
+
+// The k slice length rlis_gemm_bf16_splitk uses for a product with N weight rows over K: 512,
+// or 256 where that is needed to give every compute unit a workgroup.  Functions of N and K
+// alone; the number of slices (and of partial results) is ceil(K / slice).
+static int splitk_slice(int N, int K) {
+  const long long groups = ceil_div(N, kSplitRows);
+  return groups * ceil_div(K, 512) >= 256 ? 512 : 256;
+}
+RLIS_API int rlis_gemm_bf16_splitk_slices(int N, int K) { return ceil_div(K, splitk_slice(N, K)); }
+
+// Y receives rlis_gemm_bf16_splitk_slices(N, K) partial results (T, N) float32 contiguous,
+// part_stride elements apart, to be added in order.  17 <= T <= 64 is what it is for; fewer
+// rows work too.  bfloat16 operands, K a multiple of 8.
+RLIS_API int rlis_gemm_bf16_splitk(const void* X, const void* W, void* Y, int T, int N, int K,
+                                   long long ldx, long long ldw, long long part_stride,
+                                   hipStream_t stream) {
+  RLIS_REQUIRE(T >= 0 && T <= 64, "gemm_bf16_splitk: T=%d rows, at most 64", T);
+  RLIS_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldx >= K && ldw >= K,
+               "gemm_bf16_splitk: bad sizes N=%d K=%d ldx=%lld ldw=%lld", N, K, ldx, ldw);
+  RLIS_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)Y % 16) == 0,
+               "gemm_bf16_splitk: operands must be 16-byte aligned");
+  RLIS_REQUIRE(part_stride >= (long long)T * N,
+               "gemm_bf16_splitk: partial results %lld elements apart do not hold (T, N)",
+               part_stride);
+  if (T == 0) return 0;
+  const int ks = splitk_slice(N, K);
+  const int slices = ceil_div(K, ks);
+  const int nt = ceil_div(T, 16);
+  dim3 grid(ceil_div(N, kSplitRows), slices);
+  RLIS_REQUIRE(slices <= 65535, "gemm_bf16_splitk: K=%d is too long", K);
+  const size_t smem = (size_t)nt * 16 * (ks + kSplitPad) * sizeof(bf16_t);
+#define GO(KS, NT)                                                                          \
+  {                                                                                         \
+    static bool raised = false;                                                             \
+    if (!raised && smem > 48 * 1024) {                                                      \
+      hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_splitk_kernel<KS, NT>,      \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,        \
+                                         (int)smem);                                        \
+      RLIS_REQUIRE(e == hipSuccess, "gemm_bf16_splitk: cannot raise the LDS limit: %s",     \
+                   hipGetErrorString(e));                                                   \
+      raised = true;                                                                        \
+    }                                                                                       \
+    gemm_bf16_splitk_kernel<KS, NT><<<grid, 256, smem, stream>>>(                           \
+        (const bf16_t*)X, (const bf16_t*)W, (float*)Y, T, N, K, ldx, ldw, part_stride);     \
+  }
+#define BY_NT(KS)                        \
+  switch (nt) {                          \
+    case 1: GO(KS, 1) break;             \
+    case 2: GO(KS, 2) break;             \
+    case 3: GO(KS, 3) break;             \
+    default: GO(KS, 4) break;            \
+  }
+  if (ks == 512) BY_NT(512) else BY_NT(256)
+#undef BY_NT
+#undef GO
+  RLIS_LAUNCH_CHECK("gemm_bf16_splitk");
+  return 0;
+}
+
 // ============================================================ streaming skinny product
 // y (T <= 16, N) = x W^T at the speed of the weight stream.
 //

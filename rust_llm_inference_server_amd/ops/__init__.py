@@ -23,6 +23,9 @@ _DT = {torch.float32: 0, torch.bfloat16: 1}
 SKINNY_MAX_ROWS = 64
 # ... and with at most this many rows the streaming kernel (16 at most; 0 switches it off).
 STREAM_MAX_ROWS = 16
+# A product whose result joins the residual stream as partial sums (``partials=True``) takes the
+# split-k kernel from 17 rows up to this many (64 at most; 0 switches it off).
+SPLITK_MAX_ROWS = 64
 # Single tokens in a batch that also holds portions of prompts take the decode attention kernel.
 SPLIT_MIXED_ATTENTION = True
 # The norm in front of a projection goes into the streaming kernel where that applies.
@@ -103,13 +106,14 @@ def _delta_parts(resid: torch.Tensor, delta: torch.Tensor, what: str) -> int:
 
 def add_residual(resid: torch.Tensor, delta: torch.Tensor, round_parts: bool = False) -> None:
     """``resid += delta`` with the sum formed in float32.  ``round_parts``: a stack of partial
-    sums is added up and rounded to bfloat16 before it joins the residual."""
+    sums (of one slice or of many) is added up and rounded to bfloat16 before it joins the
+    residual."""
     _check(resid, "residual", torch.float32)
     if not resid.is_contiguous():
         raise KernelError("add_residual: residual must be contiguous")
     parts = _delta_parts(resid, delta, "add_residual")
     lib.call("rlis_add_residual", resid.data_ptr(), delta.data_ptr(), _dt(delta), resid.numel(),
-             parts, int(bool(round_parts) and parts > 1), lib.stream_ptr())
+             parts, int(bool(round_parts) and delta.dim() > resid.dim()), lib.stream_ptr())
 
 
 def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
@@ -136,7 +140,8 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
              None if delta is None else delta.data_ptr(), 0 if delta is None else _dt(delta),
              weight.data_ptr(), _dt(weight), out.data_ptr(), _DT[out_dtype], rows_ptr, R, H,
              float(eps), int(bool(write_resid)), parts, T * H,
-             int(bool(round_parts) and parts > 1), lib.stream_ptr())
+             int(bool(round_parts) and delta is not None and delta.dim() > resid.dim()),
+             lib.stream_ptr())
     return out
 
 
@@ -168,8 +173,9 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     rows and the hand-written matrix-core GEMM beyond.
 
     ``partials``: the caller hands the result to the residual stream and takes it as a stack
-    ``(S, T, N)`` of float32 partial sums too (one per k slice of the streaming kernel, added in
-    order by ``add_rmsnorm`` / ``add_residual``) where that saves a pass."""
+    ``(S, T, N)`` of float32 partial sums too (one per k slice of the streaming kernel, or of
+    the split-k kernel that 17 to 64 rows take, added in order by ``add_rmsnorm`` /
+    ``add_residual``) where that saves a pass."""
     ldx = _rows_contig(x, "linear x")
     ldw = _rows_contig(w, "linear weight")
     T, K = x.shape
@@ -181,6 +187,12 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     bf16 = x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
     aligned = (K % 8 == 0 and ldx % 8 == 0 and ldw % 8 == 0
                and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+    if bf16 and aligned and partials and STREAM_MAX_ROWS < T <= SPLITK_MAX_ROWS:
+        slices = lib.load().rlis_gemm_bf16_splitk_slices(N, K)
+        y = torch.empty((slices, T, N), dtype=torch.float32, device=x.device)
+        lib.call("rlis_gemm_bf16_splitk", x.data_ptr(), w.data_ptr(), y.data_ptr(), T, N, K, ldx,
+                 ldw, T * N, stream)
+        return y
     if bf16 and aligned and T > STREAM_MAX_ROWS and BF16_GEMM == "library":
         if out_dtype == torch.bfloat16:
             return torch.matmul(x, w.t())
@@ -252,7 +264,9 @@ def norm_linear(resid: torch.Tensor, delta: Optional[torch.Tensor], norm_weight:
     if R:
         lib.call("rlis_norm_linear_bf16", resid.data_ptr(),
                  None if delta is None else delta.data_ptr(), 0 if delta is None else _dt(delta),
-                 parts, T * K, int(bool(round_parts) and parts > 1), norm_weight.data_ptr(),
+                 parts, T * K,
+                 int(bool(round_parts) and delta is not None and delta.dim() > resid.dim()),
+                 norm_weight.data_ptr(),
                  _dt(norm_weight), float(eps), rows_ptr,
                  None if (delta is None or rows is not None) else resid_sum.data_ptr(),
                  w.data_ptr(), y.data_ptr(), _DT[out_dtype], R, N, K, ldw, N, int(bool(gated)),

@@ -84,6 +84,36 @@ def test_add_rmsnorm(ops, out_dtype, w_dtype, T, H, eps):
     torch.testing.assert_close(out3.float().cpu(), want[[T - 1, 0]], **tol(out_dtype, 2e-5))
 
 
+@pytest.mark.parametrize("out_dtype,w_dtype", [(torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32),
+                                               (torch.float32, torch.float32)])
+@pytest.mark.parametrize("T,H,parts", [(64, 2048, 16), (3, 100, 2), (17, 4096, 7), (5, 8192, 28), (2, 8196, 3),
+                                       (9, 130, 5)])
+def test_add_rmsnorm_of_a_stack_of_partial_sums(ops, out_dtype, w_dtype, T, H, parts):
+    """The delta as a stack of float32 partial sums: they are added in order, their sum is
+    rounded to bfloat16 when asked, then it joins the residual; with all rows and with a
+    selection of rows; widths that take the vectorised kernel and widths that do not."""
+    resid = rnd(T, H, seed=1) * 3
+    stack = rnd(parts, T, H, seed=2)
+    w = (1 + rnd(H, seed=3) * 0.1).to(w_dtype)
+    for rounding in (False, True):
+        total = stack[0].clone()
+        for s in range(1, parts):
+            total += stack[s]
+        if rounding:
+            total = total.to(torch.bfloat16).float()
+        want_resid = resid + total
+        want = plain.rms_norm(want_resid.cpu(), w.float().cpu(), 1e-5)
+        r = resid.clone()
+        out = ops.add_rmsnorm(r, stack, w, 1e-5, out_dtype, round_parts=rounding)
+        assert torch.equal(r, want_resid)
+        torch.testing.assert_close(out.float().cpu(), want, **tol(out_dtype, 2e-5))
+        rows = torch.tensor([T - 1, 0], dtype=torch.int32, device=DEV)
+        r3 = resid.clone()
+        out3 = ops.add_rmsnorm(r3, stack, w, 1e-5, out_dtype, rows=rows, round_parts=rounding)
+        assert torch.equal(r3, resid)
+        torch.testing.assert_close(out3.float().cpu(), want[[T - 1, 0]], **tol(out_dtype, 2e-5))
+
+
 def test_rmsnorm_unit_mean_square(ops):
     # with w = 1 and eps = 0 every row has unit mean square; scaling the input changes nothing
     x = rnd(4, 300, seed=5) * 7
@@ -185,6 +215,34 @@ def test_linear_streaming_kernel(ops, out_dtype, T, N, K):
         want_g = (torch.nn.functional.silu(g) * u).float()
         torch.testing.assert_close(gated.float(), want_g, atol=max(1.0, want_g.abs().max().item()) / 64,
                                    rtol=2e-2)
+
+
+@pytest.mark.parametrize("T,N,K", [(17, 2048, 2048), (64, 2048, 8192), (33, 3072, 2048), (24, 130, 96),
+                                   (64, 331, 104), (48, 17, 14336), (19, 1001, 4608), (40, 16, 8),
+                                   (64, 4096, 14336), (50, 3072, 3072)])
+def test_linear_split_k_kernel(ops, T, N, K):
+    """The split-k kernel that 17 to 64 rows take where the result joins the residual stream:
+    float32 partial sums per k slice against float64 products of the same bf16-rounded
+    operands; sizes that end inside a slice, inside a block of weight rows and inside a token
+    group.  A row's sums are the same bits with 17 rows in the call as with 64."""
+    x, w = rnd(T, K, dtype=torch.bfloat16, seed=3), rnd(N, K, dtype=torch.bfloat16, seed=4, scale=0.05)
+    want = (x.double() @ w.double().t()).float()
+    parts = ops.linear(x, w, partials=True)
+    assert parts.dim() == 3 and parts.shape[1:] == (T, N) and parts.dtype == torch.float32
+    assert parts.shape[0] == -(-K // 512) or parts.shape[0] == -(-K // 256)
+    got = parts.sum(dim=0)
+    scale = max(1.0, want.abs().max().item())
+    torch.testing.assert_close(got, want, atol=2e-5 * scale * math.sqrt(K / 64), rtol=1e-4)
+    fewer = ops.linear(x[:17].contiguous(), w, partials=True)
+    assert torch.equal(fewer, parts[:, :17])
+    # the residual stream's consumers add the slices in order and round once
+    resid = rnd(T, N, seed=5)
+    summed = resid.clone()
+    ops.add_residual(summed, parts, round_parts=True)
+    rounded = parts[0].clone()
+    for s in range(1, parts.shape[0]):
+        rounded += parts[s]
+    assert torch.equal(summed, resid + rounded.to(torch.bfloat16).float())
 
 
 @pytest.mark.parametrize("T,N,K,parts,rows", [(1, 2048, 2048, 0, False), (8, 3072, 2048, 1, False),
