@@ -303,3 +303,24 @@ def test_perplexity_replaces_each_windows_first_token_and_scores_its_second_half
     # odd window length: rows 6 .. 11 of 13
     odd = plain.perplexity(w, c, tokens, bos=bos, ctx=13, max_windows=2)
     assert odd["windows"] == 2 and odd["tokens_scored"] == 2 * (13 - 1 - 13 // 2)
+
+
+@pytest.mark.parametrize("name", ["a", "b", "c", "d"])
+def test_the_two_plain_implementations_agree(tiny_folders, name):
+    """The torch twin and the scalar-loop host implementation (plain_llama_host.cpp) were written
+    apart from the same formulas: whole sequences through both, every logit within 1e-4 (the
+    reference's own gate for its tiny model, crates/model/src/llama.rs:355).  A reading mistake
+    would have to be made twice, the same way, to pass."""
+    import plain_host
+    if not plain_host.available():
+        pytest.skip("g++ is not on the PATH")
+    folder = tiny_folders[name]
+    w, c = plain.read_weights(folder), plain.read_config(folder)
+    g = torch.Generator().manual_seed(21)
+    for n in (1, 2, 37):
+        ids = torch.randint(0, c["vocab_size"], (n,), generator=g).tolist()
+        a, b = plain.forward(w, c, ids), plain_host.forward(w, c, ids)
+        assert a.shape == b.shape == (n, c["vocab_size"])
+        assert (a - b).abs().max().item() < 1e-4
+    # the llama3 bands of the two agree too (tiny b and d scale their frequencies)
+    assert abs(b).max().item() > 0.05

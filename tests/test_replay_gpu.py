@@ -74,6 +74,23 @@ def test_replay_families(case, dtype, family):
     assert runner.cache.num_free_pages(0) == runner.cache.num_pages(0)
 
 
+def test_engine_matches_the_second_plain_implementation(case):
+    """The engine's float32 logits, prefill and decoded tail, against the scalar-loop host
+    implementation (plain_llama_host.cpp), which shares no code with the torch twin either."""
+    import plain_host
+    if not plain_host.available():
+        pytest.skip("g++ is not on the PATH")
+    name, cfg, per_dtype = case
+    folder, reqs, _ = per_dtype["float32"]
+    w, c = plain.read_weights(folder), plain.read_config(folder)
+    some = {k: reqs[k] for k in ("r0", "r3", "r5")}            # 5, 100 and 1 tokens
+    ref = {k: plain_host.forward(w, c, t) for k, t in some.items()}
+    steps, max_tokens = traces.trace_tail(some)
+    runner = make_runner(folder, "float32", max_tokens, page_size=8 if name == "b" else 16)
+    outputs = traces.replay_in_process(runner, steps)
+    check(steps, outputs, some, ref, cfg["vocab_size"], TOL["float32"])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_captured_decode_steps_match_eager_ones(case, dtype):
     """Steps of one token per request run from a captured HIP graph.  Replayed many times with
