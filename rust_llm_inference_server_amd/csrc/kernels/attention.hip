@@ -9,7 +9,10 @@
 // Math as in the reference's attention_block (crates/model/src/attention.rs:204-223) and its
 // decode kernel (crates/model/src/paged_attention.metal:56-198): query head h uses KV head
 // h / group; score = (q . k) * scale; a query at position p sees keys at positions <= p
-// (attention.rs:225-233) and, when a window w is given, > p - w; softmax statistics (running
+// (attention.rs:225-233) and, when a window w is given, > p - w; a position encoding that works
+// on the scores gives `slopes` (one float per query head; the reference has none): the score of
+// key position u for a query at position p then gets slope * (u - p) added, in float32, before
+// the softmax; softmax statistics (running
 // maximum m, denominator l, unnormalised accumulator) are float32; partitions of a long
 // context are merged with weights e^(m_i - max m) over the non-empty ones (metal:276-304).
 //
@@ -28,7 +31,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
     const TX* __restrict__ k_pages, const TX* __restrict__ v_pages,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ seq_of_token,
     const int* __restrict__ positions, int nh, int nkv, int d, int page_size, float scale,
-    int window) {
+    int window, const float* __restrict__ slopes) {
   extern __shared__ float smem[];
   float* q_s = smem;                          // d
   float* p_s = smem + d;                      // 64
@@ -37,6 +40,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
   const int seq = seq_of_token[t];
   const int pos = positions[t];
   const int kvh = h / (nh / nkv);
+  const float slope = slopes ? slopes[h] : 0.f;
   const int* table = block_tables + (long long)seq * max_pages;
   for (int j = lane; j < d; j += 64) q_s[j] = ld(q + (long long)t * q_stride + h * d + j) * scale;
   __syncthreads();
@@ -56,7 +60,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
       const TX* kp = k_pages + ((page * nkv + kvh) * page_size + off) * d;
       float dot = 0.f;
       for (int j = 0; j < d; ++j) dot = fmaf(q_s[j], ld(kp + j), dot);
-      s = dot;
+      s = dot + slope * (float)(kpos - pos);
       vbase = (page * nkv + kvh) * (long long)d * page_size + off;
     }
     const float m_new = fmaxf(m, wave_max(s));
@@ -92,7 +96,8 @@ RLIS_API int rlis_attn_generic(const void* q, int dtype, long long q_stride, voi
                                long long out_stride, const void* k_pages, const void* v_pages,
                                const int* block_tables, int max_pages, const int* seq_of_token,
                                const int* positions, int T, int nh, int nkv, int d, int page_size,
-                               float scale, int window, hipStream_t stream) {
+                               float scale, int window, const float* slopes,
+                               hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0, "attn_generic: bad sizes");
   RLIS_REQUIRE(nh % nkv == 0, "attn_generic: %d query heads are not a multiple of %d KV heads",
                nh, nkv);
@@ -105,7 +110,8 @@ RLIS_API int rlis_attn_generic(const void* q, int dtype, long long q_stride, voi
 #define LAUNCH(TX, DPL)                                                                        \
   attn_generic_kernel<TX, DPL><<<grid, 64, smem, stream>>>(                                    \
       (const TX*)q, q_stride, (TX*)out, out_stride, (const TX*)k_pages, (const TX*)v_pages,    \
-      block_tables, max_pages, seq_of_token, positions, nh, nkv, d, page_size, scale, window)
+      block_tables, max_pages, seq_of_token, positions, nh, nkv, d, page_size, scale, window,  \
+      slopes)
 #define BY_DPL(TX)                         \
   do {                                     \
     if (dpl <= 1) LAUNCH(TX, 1);           \
@@ -160,7 +166,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     const TX* __restrict__ v_pages, const int* __restrict__ block_tables, int max_pages,
     const int* __restrict__ ctx_lens, const int* __restrict__ token_rows, int nh, int nkv, int d,
     int page_size, float scale, int window, int splits, int chunks_per_kv, int part_keys,
-    int max_parts) {
+    int max_parts, const float* __restrict__ slopes) {
   extern __shared__ float smem[];
   float* q_s = smem;                     // G * d
   float* p_s = q_s + G * d;              // 4 waves * G * 64
@@ -196,6 +202,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 #pragma unroll
     for (int i = 0; i < DPL; ++i) acc[hh][i] = 0.f;
   }
+  float slope[G];
+#pragma unroll
+  for (int hh = 0; hh < G; ++hh) slope[hh] = slopes ? slopes[h0 + min(hh, gn - 1)] : 0.f;
   float* my_p = p_s + wave * G * 64;
   long long* my_vbase = vbase_s + wave * 64;
   constexpr int VN = Vec16<TX>::N;
@@ -233,7 +242,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     float corr[G];
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) {
-      const float sv = valid ? s[hh] : -INFINITY;
+      const float sv = valid ? s[hh] + slope[hh] * (float)(kpos - (ctx - 1)) : -INFINITY;
       const float m_new = fmaxf(m[hh], wave_max(sv));
       const float p = valid ? expf(sv - m_new) : 0.f;
       corr[hh] = (m[hh] == -INFINITY) ? 0.f : expf(m[hh] - m_new);
@@ -434,7 +443,7 @@ static int launch_decode(const void* q, long long q_stride, void* out, long long
                          const void* v_pages, const int* block_tables, int max_pages,
                          const int* ctx_lens, const int* token_rows, int S, int nh, int nkv, int d,
                          int page_size, float scale, int window, int splits, int part_keys,
-                         int max_parts, hipStream_t stream) {
+                         int max_parts, const float* slopes, hipStream_t stream) {
   const int g = nh / nkv;
   const int chunks = ceil_div(g, G);
   dim3 grid(nkv * chunks, S, splits);
@@ -446,7 +455,7 @@ static int launch_decode(const void* q, long long q_stride, void* out, long long
   attn_decode_kernel<TX, G, DPL><<<grid, 256, smem, stream>>>(                                 \
       (const TX*)q, q_stride, (TX*)out, out_stride, part_ml, part_acc, (const TX*)k_pages,     \
       (const TX*)v_pages, block_tables, max_pages, ctx_lens, token_rows, nh, nkv, d, page_size, \
-      scale, window, splits, chunks, part_keys, max_parts)
+      scale, window, splits, chunks, part_keys, max_parts, slopes)
   if (dpl <= 1) LAUNCH(1);
   else if (dpl <= 2) LAUNCH(2);
   else LAUNCH(4);
@@ -464,7 +473,8 @@ RLIS_API int rlis_attn_decode(const void* q, int dtype, long long q_stride, void
                               const void* k_pages, const void* v_pages, const int* block_tables,
                               int max_pages, const int* ctx_lens, const int* token_rows, int S,
                               int nh, int nkv, int d, int page_size, float scale, int window,
-                              int splits, int part_keys, int max_parts, hipStream_t stream) {
+                              int splits, int part_keys, int max_parts, const float* slopes,
+                              hipStream_t stream) {
   RLIS_REQUIRE(S >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0, "attn_decode: bad sizes");
   RLIS_REQUIRE(part_keys >= 64 && part_keys % 64 == 0 && max_parts >= 1 && splits <= max_parts,
                "attn_decode: partitions of %d keys (a multiple of 64), %d deep of at most %d",
@@ -484,22 +494,22 @@ RLIS_API int rlis_attn_decode(const void* q, int dtype, long long q_stride, void
       rc = launch_decode<TX, 1>(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,        \
                                 v_pages, block_tables, max_pages, ctx_lens, token_rows, S, nh,   \
                                 nkv, d, page_size, scale, window, splits, part_keys, max_parts,       \
-                                stream);               \
+                                slopes, stream);               \
     else if (g == 2)                                                                             \
       rc = launch_decode<TX, 2>(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,        \
                                 v_pages, block_tables, max_pages, ctx_lens, token_rows, S, nh,   \
                                 nkv, d, page_size, scale, window, splits, part_keys, max_parts,       \
-                                stream);               \
+                                slopes, stream);               \
     else if (g <= 4)                                                                             \
       rc = launch_decode<TX, 4>(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,        \
                                 v_pages, block_tables, max_pages, ctx_lens, token_rows, S, nh,   \
                                 nkv, d, page_size, scale, window, splits, part_keys, max_parts,       \
-                                stream);               \
+                                slopes, stream);               \
     else                                                                                         \
       rc = launch_decode<TX, 8>(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,        \
                                 v_pages, block_tables, max_pages, ctx_lens, token_rows, S, nh,   \
                                 nkv, d, page_size, scale, window, splits, part_keys, max_parts,       \
-                                stream);               \
+                                slopes, stream);               \
   } while (0)
   if (dtype == RLIS_F32) BY_G(float);
   else if (dtype == RLIS_BF16) BY_G(bf16_t);

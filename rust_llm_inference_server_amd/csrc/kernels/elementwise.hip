@@ -458,7 +458,8 @@ RLIS_API int rlis_swiglu(void* out, const void* gu, int dtype, int T, int I, hip
 // ------------------------------------------------ rotary encoding + K/V page write
 // qkv (T, row_stride): q heads at columns [0, nh*d), k heads at [k_off, k_off + nkv*d), v heads
 // at [v_off, v_off + nkv*d).  The first rot_dim dims of every q and k head are rotated
-// (rotate-half: dim j pairs with j + rot_dim/2), the rest pass through.  q is rotated in
+// (rotate-half: dim j pairs with j + rot_dim/2; or, `interleaved`, dim 2j pairs with 2j + 1;
+// either way with the j-th angle of the position's row), the rest pass through.  q is rotated in
 // place.  When write_kv is set, rotated k goes to k_pages[page][kv head][offset][d] and v to
 // v_pages[page][kv head][d][offset] (v is stored transposed inside a page), with
 // page = slot / page_size, offset = slot % page_size; rotated k is not stored back to qkv.
@@ -469,7 +470,8 @@ __global__ void rope_kv_write_kernel(TX* __restrict__ qkv, long long row_stride,
                                      const float* __restrict__ sin_t,
                                      const int* __restrict__ positions,
                                      const int* __restrict__ slots, TX* __restrict__ k_pages,
-                                     TX* __restrict__ v_pages, int page_size, int write_kv) {
+                                     TX* __restrict__ v_pages, int page_size, int write_kv,
+                                     int interleaved) {
   const int t = blockIdx.x;
   TX* row = qkv + (long long)t * row_stride;
   const int pos = positions[t];
@@ -480,10 +482,11 @@ __global__ void rope_kv_write_kernel(TX* __restrict__ qkv, long long row_stride,
   for (int i = threadIdx.x; i < nh * half; i += blockDim.x) {
     const int h = i / half, j = i - h * half;
     TX* p = row + h * d;
-    const float x1 = ld(p + j), x2 = ld(p + j + half);
+    const int a = interleaved ? 2 * j : j, b = interleaved ? 2 * j + 1 : j + half;
+    const float x1 = ld(p + a), x2 = ld(p + b);
     const float cc = c[j], sn = s[j];
-    st(p + j, x1 * cc - x2 * sn);
-    st(p + j + half, x2 * cc + x1 * sn);
+    st(p + a, x1 * cc - x2 * sn);
+    st(p + b, x2 * cc + x1 * sn);
   }
   if (!write_kv) return;
   const int slot = slots[t];
@@ -494,11 +497,12 @@ __global__ void rope_kv_write_kernel(TX* __restrict__ qkv, long long row_stride,
   for (int i = threadIdx.x; i < nkv * half; i += blockDim.x) {
     const int h = i / half, j = i - h * half;
     const TX* p = row + k_off + h * d;
-    const float x1 = ld(p + j), x2 = ld(p + j + half);
+    const int a = interleaved ? 2 * j : j, b = interleaved ? 2 * j + 1 : j + half;
+    const float x1 = ld(p + a), x2 = ld(p + b);
     const float cc = c[j], sn = s[j];
     TX* dst = k_pages + ((page * nkv + h) * page_size + off) * d;
-    st(dst + j, x1 * cc - x2 * sn);
-    st(dst + j + half, x2 * cc + x1 * sn);
+    st(dst + a, x1 * cc - x2 * sn);
+    st(dst + b, x2 * cc + x1 * sn);
   }
   const int tail = d - rot_dim;
   for (int i = threadIdx.x; i < nkv * tail; i += blockDim.x) {
@@ -633,14 +637,14 @@ RLIS_API int rlis_rope_kv_write(void* qkv, int dtype, long long row_stride, int 
                                 int T, int nh, int nkv, int d, int rot_dim, const float* cos_t,
                                 const float* sin_t, const int* positions, const int* slots,
                                 void* k_pages, void* v_pages, int page_size, int write_kv,
-                                hipStream_t stream) {
+                                int interleaved, hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && d > 0, "rope_kv_write: bad sizes");
   RLIS_REQUIRE(rot_dim >= 0 && rot_dim <= d && rot_dim % 2 == 0,
                "rope_kv_write: rot_dim %d must be even and at most head_dim %d", rot_dim, d);
   RLIS_REQUIRE(!write_kv || (page_size > 0 && k_pages && v_pages && slots),
                "rope_kv_write: cache write asked for without pages");
   if (T == 0) return 0;
-  const bool by8 = dtype == RLIS_BF16 && d % 8 == 0 && rot_dim % 16 == 0 && row_stride % 8 == 0 &&
+  const bool by8 = !interleaved && dtype == RLIS_BF16 && d % 8 == 0 && rot_dim % 16 == 0 && row_stride % 8 == 0 &&
                    k_off % 8 == 0 && v_off % 8 == 0 && ((uintptr_t)qkv % 16) == 0 &&
                    ((uintptr_t)cos_t % 16) == 0 && ((uintptr_t)sin_t % 16) == 0 &&
                    (!write_kv || (((uintptr_t)k_pages % 16) == 0 && T <= (1 << 30)));
@@ -656,11 +660,11 @@ RLIS_API int rlis_rope_kv_write(void* qkv, int dtype, long long row_stride, int 
   if (dtype == RLIS_F32)
     rope_kv_write_kernel<float><<<T, 256, 0, stream>>>(
         (float*)qkv, row_stride, k_off, v_off, nh, nkv, d, rot_dim, cos_t, sin_t, positions,
-        slots, (float*)k_pages, (float*)v_pages, page_size, write_kv);
+        slots, (float*)k_pages, (float*)v_pages, page_size, write_kv, interleaved);
   else if (dtype == RLIS_BF16)
     rope_kv_write_kernel<bf16_t><<<T, 256, 0, stream>>>(
         (bf16_t*)qkv, row_stride, k_off, v_off, nh, nkv, d, rot_dim, cos_t, sin_t, positions,
-        slots, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, write_kv);
+        slots, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, write_kv, interleaved);
   else
     RLIS_REQUIRE(false, "rope_kv_write: unknown dtype %d", dtype);
   RLIS_LAUNCH_CHECK("rope_kv_write");

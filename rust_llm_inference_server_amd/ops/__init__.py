@@ -310,9 +310,11 @@ def rope_kv_write(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
                   cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
                   positions: torch.Tensor, slots: Optional[torch.Tensor],
                   k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor],
-                  page_size: int, write_kv: bool = True) -> None:
+                  page_size: int, write_kv: bool = True, interleaved: bool = False) -> None:
     """Rotate the q and k heads of ``qkv (T, (nh + 2 nkv) d)`` by their positions (q in
     place) and, when ``write_kv``, store rotated k and v into the pages at ``slots``.
+    The rotation pairs dim ``j`` with ``j + rot/2`` (rotate-half, the reference's), or with
+    ``interleaved`` dim ``2j`` with ``2j + 1``.
 
     ``cos``/``sin`` are float32 ``(max_positions, rot_dim / 2)``; None means no rotation.
     ``k_pages (pages, nkv, page, d)``, ``v_pages (pages, nkv, d, page)``."""
@@ -345,7 +347,7 @@ def rope_kv_write(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
         kp, vp, sp = k_pages.data_ptr(), v_pages.data_ptr(), _i32(slots, "slots", T)
     lib.call("rlis_rope_kv_write", qkv.data_ptr(), _dt(qkv), stride, nh * d, (nh + nkv) * d, T,
              nh, nkv, d, rot, cos_ptr, sin_ptr, _i32(positions, "positions", T), sp, kp, vp,
-             page_size, int(bool(write_kv)), lib.stream_ptr())
+             page_size, int(bool(write_kv)), int(bool(interleaved)), lib.stream_ptr())
 
 
 def copy_pages(pages: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
@@ -376,25 +378,27 @@ def _prefill_mfma_ok(qkv: torch.Tensor, d: int, page_size: int) -> bool:
 
 
 def attention_planner(num_heads: int, num_kv_heads: int, head_dim: int,
-                      dtype: torch.dtype) -> AttentionPlanner:
+                      dtype: torch.dtype, biased: bool = False) -> AttentionPlanner:
     """The planner a mixer that calls ``paged_attention`` / ``rope_attention`` names as its
-    ``step_planner()``."""
-    return AttentionPlanner(num_heads, num_kv_heads, head_dim, matrix=dtype == torch.bfloat16,
+    ``step_planner()``; ``biased``: it will pass ``bias_slopes`` (no matrix-core kernels then)."""
+    return AttentionPlanner(num_heads, num_kv_heads, head_dim,
+                            matrix=dtype == torch.bfloat16 and not biased,
                             singles_apart=SPLIT_MIXED_ATTENTION and DECODE_ATTENTION != "vector")
 
 
 def _attention_kernel(qkv: torch.Tensor, nh: int, nkv: int, d: int, page_size: int, step,
-                      force: Optional[str]):
-    """(kind, matrix_decode): which attention kernel a batch takes."""
+                      force: Optional[str], biased: bool = False):
+    """(kind, matrix_decode): which attention kernel a batch takes.  A bias on the scores is
+    taken by the vector-unit kernels only (the generic one and the vector decode kernel)."""
     kind = force or FORCE_ATTENTION
     if kind is None:
         if step.all_decode and d % 8 == 0 and d <= 256 and (nh // nkv) * d <= 2048:
             kind = "decode"
-        elif _prefill_mfma_ok(qkv, d, page_size) and not step.all_decode:
+        elif _prefill_mfma_ok(qkv, d, page_size) and not step.all_decode and not biased:
             kind = "prefill"
         else:
             kind = "generic"
-    mfma = kind == "decode" and _decode_mfma_ok(qkv, nh, nkv, d, page_size)
+    mfma = kind == "decode" and not biased and _decode_mfma_ok(qkv, nh, nkv, d, page_size)
     return kind, mfma
 
 
@@ -415,14 +419,17 @@ def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
                    k_pages: torch.Tensor, v_pages: torch.Tensor, page_size: int,
                    block_tables: torch.Tensor, step, scale: float,
                    window: Optional[int] = None, write_kv: bool = True,
-                   plan: Optional[StepPlan] = None) -> torch.Tensor:
+                   plan: Optional[StepPlan] = None, interleaved: bool = False,
+                   bias_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``rope_kv_write`` followed by ``paged_attention``.  A decode batch that takes the
-    matrix-core decode kernel does both in that kernel when the whole head is rotated and is
-    64, 128 or 256 wide (or nothing is rotated); ``qkv`` is then left unrotated."""
+    matrix-core decode kernel does both in that kernel when the whole head is rotated
+    (rotate-half) and is 64, 128 or 256 wide (or nothing is rotated); ``qkv`` is then left
+    unrotated.  ``interleaved`` and ``bias_slopes`` as in ``rope_kv_write`` and
+    ``paged_attention``."""
     nh, nkv, d = num_heads, num_kv_heads, head_dim
     _rows_contig(qkv, "qkv")
-    kind, mfma = _attention_kernel(qkv, nh, nkv, d, page_size, step, None)
-    fusable = cos is None or (2 * cos.shape[1] == d and d in (64, 128, 256))
+    kind, mfma = _attention_kernel(qkv, nh, nkv, d, page_size, step, None, bias_slopes is not None)
+    fusable = cos is None or (2 * cos.shape[1] == d and d in (64, 128, 256) and not interleaved)
     if mfma and fusable and FUSE_ROPE_DECODE and qkv.shape[1] == (nh + 2 * nkv) * d:
         if cos is not None:
             _check(cos, "cos", torch.float32, 2)
@@ -435,17 +442,17 @@ def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
                                scale, window, plan=plan,
                                rope=(cos, sin, positions, slots if write_kv else None))
     rope_kv_write(qkv, nh, nkv, d, cos, sin, positions, slots, k_pages, v_pages, page_size,
-                  write_kv=write_kv)
+                  write_kv=write_kv, interleaved=interleaved)
     return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
-                           scale, window, plan=plan)
+                           scale, window, plan=plan, bias_slopes=bias_slopes)
 
 
 def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                     k_pages: torch.Tensor, v_pages: torch.Tensor, page_size: int,
                     block_tables: torch.Tensor, step, scale: float,
                     window: Optional[int] = None, force: Optional[str] = None,
-                    rope: Optional[tuple] = None, plan: Optional[StepPlan] = None
-                    ) -> torch.Tensor:
+                    rope: Optional[tuple] = None, plan: Optional[StepPlan] = None,
+                    bias_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of the step's new tokens over the paged cache -> ``(T, nh * d)``.
 
     ``qkv`` holds the rotated queries in its first ``nh * d`` columns; K and V of the new
@@ -456,6 +463,9 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     sequences -> matrix-core prefill kernel (single tokens that lead the step beside them ->
     decode kernel); float32, or sizes those kernels refuse -> generic kernel.  How a sequence's
     keys are cut (decode partitions, tile form, key runs) follows from its own lengths alone.
+    ``bias_slopes`` (float32, one per query head; the reference has no such thing): the score of
+    key position ``u`` for a query at position ``p`` gets ``slope * (u - p)`` added before the
+    softmax; the vector-unit kernels take it, so such a batch goes to them.
     ``force`` names one of 'generic', 'decode', 'prefill' for tests.  ``rope`` (from
     ``rope_attention`` only): ``(cos, sin, positions, slots)`` for the matrix-core decode kernel
     to rotate and store the step's tokens itself."""
@@ -483,19 +493,28 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     win = int(window) if window else 0
     out = torch.empty((T, nh * d), dtype=qkv.dtype, device=qkv.device)
     stream = lib.stream_ptr()
-    kind, mfma = _attention_kernel(qkv, nh, nkv, d, page_size, step, force)
+    slopes_ptr = None
+    if bias_slopes is not None:
+        _check(bias_slopes, "bias_slopes", torch.float32, 1)
+        if bias_slopes.numel() != nh or not bias_slopes.is_contiguous():
+            raise KernelError(f"attention: {bias_slopes.numel()} bias slopes for {nh} heads")
+        slopes_ptr = bias_slopes.data_ptr()
+    kind, mfma = _attention_kernel(qkv, nh, nkv, d, page_size, step, force, slopes_ptr is not None)
     if rope is not None and not mfma:
         raise KernelError("attention: only the matrix-core decode kernel rotates and stores")
+    if slopes_ptr is not None and kind == "prefill":
+        raise KernelError("attention: the matrix-core prefill kernel takes no bias on the scores")
     if kind == "generic":
         lib.call("rlis_attn_generic", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(), nh * d,
                  k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,
                  _i32(step.seq_of_token, "seq_of_token", T), _i32(step.positions, "positions", T),
-                 T, nh, nkv, d, page_size, float(scale), win, stream)
+                 T, nh, nkv, d, page_size, float(scale), win, slopes_ptr, stream)
         return out
     if kind not in ("decode", "prefill"):
         raise KernelError(f"attention: unknown kernel '{kind}'")
     if plan is None or force == "prefill":
-        planner = AttentionPlanner(nh, nkv, d, matrix=qkv.dtype == torch.bfloat16,
+        planner = AttentionPlanner(nh, nkv, d,
+                                   matrix=qkv.dtype == torch.bfloat16 and slopes_ptr is None,
                                    singles_apart=force is None and SPLIT_MIXED_ATTENTION
                                    and DECODE_ATTENTION != "vector")
         plan = _plan_now(step, planner, qkv.device)
@@ -530,7 +549,7 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                      nh * d, ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
                      block_tables.data_ptr(), max_pages, _i32(step.ctx_lens, "ctx_lens", S), None,
                      S, nh, nkv, d, page_size, float(scale), win, depth, ap.DECODE_PART_KEYS,
-                     ap.DECODE_MAX_PARTS, stream)
+                     ap.DECODE_MAX_PARTS, slopes_ptr, stream)
 
     if kind == "decode":
         if not step.all_decode:

@@ -19,7 +19,7 @@ _SIGNATURES = {
     "rlis_add_residual": [P, P, I, L, I, I, P],
     "rlis_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, I, L, I, P],
     "rlis_swiglu": [P, P, I, I, I, P],
-    "rlis_rope_kv_write": [P, I, L, I, I, I, I, I, I, I, P, P, P, P, P, P, I, I, P],
+    "rlis_rope_kv_write": [P, I, L, I, I, I, I, I, I, I, P, P, P, P, P, P, I, I, I, P],
     "rlis_copy_pages": [P, I, I, L, L, P, P, I, P],
     "rlis_gemm_plain": [P, I, P, I, P, I, I, I, I, L, L, L, P],
     "rlis_gemm_bf16_mfma": [P, P, P, I, I, I, I, L, L, L, P],
@@ -28,8 +28,8 @@ _SIGNATURES = {
     "rlis_gemm_bf16_stream": [P, P, P, I, I, I, I, L, L, L, L, I, P],
     "rlis_gemm_bf16_splitk": [P, P, P, I, I, I, L, L, L, P],
     "rlis_norm_linear_bf16": [P, P, I, I, L, I, P, I, F, P, P, P, P, I, I, I, I, L, L, I, P],
-    "rlis_attn_generic": [P, I, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
-    "rlis_attn_decode": [P, I, L, P, L, P, P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, I, I, P],
+    "rlis_attn_generic": [P, I, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P, P],
+    "rlis_attn_decode": [P, I, L, P, L, P, P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, I, I, P, P],
     "rlis_attn_decode_mfma": [P, L, P, L, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, I, I, P, P, I,
                               P, P, L, L, P],
     "rlis_attn_prefill_mfma": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, I, P, P,

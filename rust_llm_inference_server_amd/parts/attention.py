@@ -22,7 +22,13 @@ from .rope import shared_position
 @register("mixer", "attention")
 class PagedAttention(Mixer):
     """Parameters: ``hidden_size``, ``num_heads``, ``num_kv_heads``, ``head_dim``, ``scale``,
-    ``window`` (None: all earlier positions), ``position`` (a PartSpec)."""
+    ``window`` (None: all earlier positions), ``position`` (a PartSpec).
+
+    What the position part may carry: ``rot_dim``, ``cos``, ``sin`` (float32 tables, a rotation
+    of the first ``rot_dim`` dims of every q and k head; rot_dim 0: none), ``interleaved``
+    (the rotation pairs dim 2j with 2j + 1 instead of j with j + rot/2), ``bias_slopes``
+    (float32, one per query head: slope * (key position - query position) is added to the
+    scores).  The reference's Llama uses the first three (crates/model/src/rope.rs:61-117)."""
 
     graph_safe = True
     takes_normed_input = True
@@ -58,8 +64,9 @@ class PagedAttention(Mixer):
         if self.position.rot_dim > self.head_dim:
             raise ValueError("attention: the rotated width exceeds the head size")
 
-        self.planner = ops.attention_planner(self.num_heads, self.num_kv_heads, self.head_dim,
-                                             self.act_dtype)
+        self.planner = ops.attention_planner(
+            self.num_heads, self.num_kv_heads, self.head_dim, self.act_dtype,
+            biased=getattr(self.position, "bias_slopes", None) is not None)
 
     def cache_request(self) -> CacheRequest:
         return CacheRequest.kv(self.num_kv_heads, self.head_dim, self.window)
@@ -77,5 +84,7 @@ class PagedAttention(Mixer):
                                  self.position.cos, self.position.sin, step.positions,
                                  group.slots, binding.k_pages, binding.v_pages, group.page_size,
                                  group.block_tables, step, self.scale, self.window,
-                                 write_kv=binding.writes, plan=step.plans.get(self.planner.key()))
+                                 write_kv=binding.writes, plan=step.plans.get(self.planner.key()),
+                                 interleaved=bool(getattr(self.position, "interleaved", False)),
+                                 bias_slopes=getattr(self.position, "bias_slopes", None))
         return ops.linear(out, self.w_o, self.act_dtype, partials=True)

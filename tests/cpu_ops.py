@@ -50,7 +50,8 @@ def can_fuse_norm_linear(resid, w, rows=None):
 
 
 def rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, cos, sin, positions, slots, k_pages,
-                  v_pages, page_size, write_kv=True):
+                  v_pages, page_size, write_kv=True, interleaved=False):
+    assert not interleaved, "the test double rotates halves only"
     T = qkv.shape[0]
     nh, nkv, d = num_heads, num_kv_heads, head_dim
     x = qkv.float()
@@ -78,13 +79,15 @@ def copy_pages(pages, src, dst):
         pages[:, d] = pages[:, s]
 
 
-def attention_planner(num_heads, num_kv_heads, head_dim, dtype):
+def attention_planner(num_heads, num_kv_heads, head_dim, dtype, biased=False):
     from rust_llm_inference_server_amd.ops.attention_plan import AttentionPlanner
     return AttentionPlanner(num_heads, num_kv_heads, head_dim, matrix=dtype == torch.bfloat16)
 
 
 def paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, page_size,
-                    block_tables, step, scale, window=None, force=None, plan=None):
+                    block_tables, step, scale, window=None, force=None, plan=None,
+                    bias_slopes=None):
+    assert bias_slopes is None, "the test double adds no bias"
     T = qkv.shape[0]
     nh, nkv, d = num_heads, num_kv_heads, head_dim
     g = nh // nkv
@@ -107,7 +110,7 @@ def paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, pa
 
 def rope_attention(qkv, num_heads, num_kv_heads, head_dim, cos, sin, positions, slots, k_pages,
                    v_pages, page_size, block_tables, step, scale, window=None, write_kv=True,
-                   plan=None):
+                   plan=None, interleaved=False, bias_slopes=None):
     rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, cos, sin, positions, slots, k_pages,
                   v_pages, page_size, write_kv=write_kv)
     return paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, page_size,

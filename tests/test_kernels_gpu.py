@@ -809,6 +809,94 @@ def test_attention_window_edge(ops, dtype, kind, window, decode_kind):
     torch.testing.assert_close(seen, vs[0][p - window + 1, 0, :], **tol(dtype, 1e-4, 2e-2))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,ps", [(6, 2, 32, 8), (5, 5, 48, 16), (32, 8, 64, 16)])
+def test_attention_with_a_bias_on_the_scores(ops, dtype, nh, nkv, d, ps):
+    """slope[h] * (key position - query position) added to the scores before the softmax (a
+    position encoding that works on the scores; the reference has none): portions beside single
+    tokens through the generic kernel, single tokens through the vector decode kernel, with and
+    without a window, against the plain attention with the bias as an additive mask.  A slope
+    so steep that only the query's own position counts returns that position's value."""
+    scale = 1.0 / math.sqrt(d)
+    slopes = torch.tensor([0.5 ** (1 + h % 5) for h in range(nh)], dtype=torch.float32)
+
+    def reference(qkv, ks, vs, cu, cached, new, sl, window):
+        outs = []
+        q_all = qkv.float().cpu()[:, :nh * d]
+        for s, (c, n) in enumerate(zip(cached, new)):
+            q = q_all[cu[s]:cu[s + 1]].reshape(n, nh, d).transpose(0, 1)
+            k, v = ks[s].transpose(0, 1), vs[s].transpose(0, 1)
+            dist = torch.arange(c + n).reshape(1, -1) - torch.arange(c, c + n).reshape(-1, 1)
+            mask = plain.causal_mask(n, c, window)
+            o = torch.stack([plain.gqa_attention(q[h:h + 1], k[h // (nh // nkv):h // (nh // nkv) + 1],
+                                                 v[h // (nh // nkv):h // (nh // nkv) + 1],
+                                                 mask + sl[h] * dist, scale)[0] for h in range(nh)])
+            outs.append(o.transpose(0, 1).reshape(n, nh * d))
+        return torch.cat(outs)
+
+    for cached, new in (([0, 5, 40, 130, 17], [33, 1, 70, 2, 64]), ([4, 99, 0, 640], [1, 1, 1, 1])):
+        for window in (None, 50):
+            qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=nh + 9)
+            got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window,
+                                      bias_slopes=slopes.to(DEV))
+            want = reference(qkv, ks, vs, cu, cached, new, slopes, window)
+            torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
+            plainly = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window)
+            assert (got.float() - plainly.float()).abs().max().item() > 1e-2       # the bias matters
+    steep = torch.full((nh,), 1000.0, dtype=torch.float32, device=DEV)
+    qkv, kp, vp, bt, step, ks, vs, cu = paged_case([30, 7], [1, 1], nh, nkv, d, ps, dtype, seed=3)
+    got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, None, bias_slopes=steep)
+    for s, last in enumerate((30, 7)):
+        for h in range(nh):
+            torch.testing.assert_close(got[s, h * d:(h + 1) * d].float().cpu(), vs[s][last, h // (nh // nkv)],
+                                       **tol(dtype, 1e-5, 1e-2))
+    qkv, kp, vp, bt, step, *_ = paged_case([0], [40], 4, 2, 32, 8, torch.bfloat16)
+    with pytest.raises(ops.KernelError, match="no bias"):
+        ops.paged_attention(qkv, 4, 2, 32, kp, vp, 8, bt, step, 1.0, None, force="prefill",
+                            bias_slopes=torch.ones(4, device=DEV))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rope_interleaved_layout(ops, dtype):
+    """The rotation that pairs dim 2j with 2j + 1 (the reference rotates halves): against the
+    formula, over part of the head, into the pages; position 0 is the identity."""
+    T, nh, nkv, d, rot, ps = 9, 3, 1, 48, 32, 8
+    inv = plain.inv_freqs(rot, 10000.0, None)
+    positions = torch.tensor([0, 1, 5, 63, 17, 2, 3, 40, 8], dtype=torch.int32)
+    cos, sin = plain.rope_tables(inv, positions.tolist())
+    cos_all, sin_all = plain.rope_tables(inv, range(64))
+    qkv = rnd(T, (nh + 2 * nkv) * d, dtype=dtype, seed=12)
+    src = qkv.float().cpu()
+    slots = torch.arange(T, dtype=torch.int32) + 3
+    kp = torch.zeros(4, nkv, ps, d, dtype=dtype, device=DEV)
+    vp = torch.zeros(4, nkv, d, ps, dtype=dtype, device=DEV)
+    ops.rope_kv_write(qkv, nh, nkv, d, cos_all.to(DEV), sin_all.to(DEV), positions.to(DEV), slots.to(DEV),
+                      kp, vp, ps, interleaved=True)
+
+    def rotated(x):                                  # x (T, heads, d)
+        out = x.clone()
+        a, b = x[..., 0:rot:2], x[..., 1:rot:2]
+        c, s = cos.unsqueeze(1), sin.unsqueeze(1)
+        out[..., 0:rot:2] = a * c - b * s
+        out[..., 1:rot:2] = b * c + a * s
+        return out
+
+    want_q = rotated(src[:, :nh * d].reshape(T, nh, d)).reshape(T, nh * d)
+    torch.testing.assert_close(qkv[:, :nh * d].float().cpu(), want_q, **tol(dtype, 1e-5, 2e-2))
+    want_k = rotated(src[:, nh * d:(nh + nkv) * d].reshape(T, nkv, d))
+    for t in range(T):
+        slot = int(slots[t])
+        torch.testing.assert_close(kp[slot // ps, :, slot % ps, :].float().cpu(), want_k[t],
+                                   **tol(dtype, 1e-5, 2e-2))
+    assert torch.equal(qkv[0, :nh * d].float().cpu(), src[0, :nh * d])         # position 0
+    # not the rotation of halves
+    halves = qkv.clone()
+    halves[:] = rnd(T, (nh + 2 * nkv) * d, dtype=dtype, seed=12)
+    ops.rope_kv_write(halves, nh, nkv, d, cos_all.to(DEV), sin_all.to(DEV), positions.to(DEV), None, None,
+                      None, ps, write_kv=False)
+    assert (halves[1:, :nh * d].float() - qkv[1:, :nh * d].float()).abs().max().item() > 0.1
+
+
 def test_attention_one_key_returns_its_value(ops):
     nh, nkv, d, ps = 4, 2, 32, 8
     for kind in ("generic", "decode"):

@@ -656,6 +656,106 @@ def test_toy_routed_feed_forward_and_toy_position_encoding(tmp_path, dtype, tol)
     assert len(used) >= 2
 
 
+def register_toy_biased_position():
+    """Defined and registered here, in the test: a position encoding that does both things the
+    built-in one does not: its rotation pairs neighbouring dims (2j with 2j + 1) over a part of
+    the head, and it adds slope * (key position - query position) to every score."""
+    from rust_llm_inference_server_amd.parts import PositionEncoding, register
+
+    @register("position", "toy_interleaved_with_bias")
+    class InterleavedWithBias(PositionEncoding):
+        def __init__(self, params, prefix, ctx):
+            super().__init__(params, prefix, ctx)
+            self.rot_dim = int(params["rot_dim"])
+            self.interleaved = True
+            inv = plain.inv_freqs(self.rot_dim, float(params["theta"]), None)
+            angles = torch.arange(ctx.max_positions, dtype=torch.float32).reshape(-1, 1) * inv
+            self.cos = torch.cos(angles).to(ctx.device).contiguous()
+            self.sin = torch.sin(angles).to(ctx.device).contiguous()
+            self.bias_slopes = torch.tensor(params["slopes"], dtype=torch.float32, device=ctx.device)
+            self.max_positions = ctx.max_positions
+
+    return InterleavedWithBias
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-4), ("bfloat16", 4e-2)])
+def test_toy_position_encoding_with_another_layout_and_a_score_bias(tmp_path, dtype, tol):
+    """The attention mixer with a position part, registered from the test, that rotates
+    neighbouring dims over half of the head and biases the scores by distance: the first layer
+    of a model whose second layer is the ordinary one, through every way of cutting.  The bias
+    is strong enough that leaving it out would show."""
+    from rust_llm_inference_server_amd.engine import ModelRunner, load_model
+    from rust_llm_inference_server_amd.parts import PartSpec
+    from rust_llm_inference_server_amd.registry import Architecture, register_architecture
+    from rust_llm_inference_server_amd.weights import write_model_folder
+    register_toy_biased_position()
+    H, nh, nkv, d, rot = 48, 4, 2, 32, 16
+    slopes = [0.5, 0.25, 0.125, 0.0625]
+
+    def build_spec(cfg):
+        first = layer_spec(H, nh, nkv, d, 64, 1e-5, 1e4, None)
+        first.params["mixer"].params["position"] = PartSpec(
+            "toy_interleaved_with_bias", {"rot_dim": rot, "theta": 1e4, "slopes": cfg["slopes"]})
+        return toy_spec([first, layer_spec(H, nh, nkv, d, 64, 1e-5, 1e4, None)], H=H, V=cfg["vocab_size"])
+
+    register_architecture(Architecture("ToyBiasedForCausalLM", parse_config=lambda c: c,
+                                       build_spec=build_spec, config_to_dict=lambda c: c))
+    config = {"architectures": ["ToyBiasedForCausalLM"], "vocab_size": 97, "slopes": slopes}
+    folder = str(tmp_path / "toy_biased")
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    write_model_folder(folder, config, build_spec(config).tensor_specs(), seed=14, dtype=tdt)
+    w = plain.read_weights(folder)
+
+    def plain_model(ids, with_bias=True):
+        x = plain.embedding(w["model.embed_tokens.weight"], ids)
+        T = len(ids)
+        for li in range(2):
+            p = f"model.layers.{li}"
+            h = plain.rms_norm(x, w[f"{p}.input_layernorm.weight"], 1e-5)
+            if li == 0:
+                inv = plain.inv_freqs(rot, 1e4, None)
+                cos, sin = plain.rope_tables(inv, range(T))
+
+                def rotate(t):                      # (heads, T, d): pairs (2j, 2j + 1) below rot
+                    out = t.clone()
+                    a, b = t[..., 0:rot:2], t[..., 1:rot:2]
+                    out[..., 0:rot:2] = a * cos - b * sin
+                    out[..., 1:rot:2] = b * cos + a * sin
+                    return out
+
+                q = rotate(plain.linear(h, w[f"{p}.self_attn.q_proj.weight"]).reshape(T, nh, d).transpose(0, 1))
+                k = rotate(plain.linear(h, w[f"{p}.self_attn.k_proj.weight"]).reshape(T, nkv, d).transpose(0, 1))
+                v = plain.linear(h, w[f"{p}.self_attn.v_proj.weight"]).reshape(T, nkv, d).transpose(0, 1)
+                dist = (torch.arange(T).reshape(1, -1) - torch.arange(T).reshape(-1, 1)).float()
+                heads = []
+                for hh in range(nh):
+                    mask = plain.causal_mask(T, 0, None) + (slopes[hh] * dist if with_bias else 0.0)
+                    kv = hh // (nh // nkv)
+                    heads.append(plain.gqa_attention(q[hh:hh + 1], k[kv:kv + 1], v[kv:kv + 1], mask)[0])
+                o = torch.stack(heads)
+                x = x + plain.linear(o.transpose(0, 1).reshape(T, nh * d), w[f"{p}.self_attn.o_proj.weight"])
+            else:
+                cfg = {"num_attention_heads": nh, "num_key_value_heads": nkv, "head_dim": d}
+                x = x + plain.attention_layer(h, w, f"{p}.self_attn", cfg, plain.inv_freqs(d, 1e4, None))
+            h = plain.rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], 1e-5)
+            x = x + plain.swiglu_mlp(h, w, f"{p}.mlp")
+        return plain.linear(plain.rms_norm(x, w["model.norm.weight"], 1e-5), w["lm_head.weight"])
+
+    reqs = traces.random_requests(97, [30, 4, 70, 11], seed=10)
+    ref = {k: plain_model(t) for k, t in reqs.items()}
+    assert (ref["r2"] - plain_model(reqs["r2"], with_bias=False)).abs().max().item() > 4 * tol
+    for build in (traces.trace_whole, traces.trace_tail, traces.trace_portions, traces.trace_mixed):
+        steps, max_tokens = build(reqs)
+        model = load_model(folder, dtype, max_positions=128)
+        runner = ModelRunner(model, num_pages=max_tokens // 16, page_size=16, max_num_seqs=4)
+        got = traces.collect(steps, traces.replay_in_process(runner, steps), 97)
+        for k, tokens in reqs.items():
+            mine = torch.stack([got[k][p] for p in range(len(tokens))])
+            diff = (mine - ref[k]).abs().max(dim=-1).values
+            assert diff.max().item() < tol, (f"{build.__name__} request {k}: first wrong position "
+                                             f"{int((diff >= tol).nonzero()[0])}")
+
+
 def test_long_decoding_stays_on_the_plain_path(tiny_folders):
     """A short prompt, then 230 tokens one by one (teacher-forced), across many page edges."""
     from rust_llm_inference_server_amd.engine import ModelRunner, StepEntry, load_model
