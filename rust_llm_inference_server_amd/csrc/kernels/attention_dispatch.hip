@@ -14,7 +14,7 @@ typedef int (*DecodeUnit)(const void* q, long long q_stride, void* out, long lon
                           const void* v_pages, const int* block_tables, int max_pages,
                           const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift,
                           int window, float scale, int splits, int part_keys, int max_parts,
-                          const DecodeRope* rope, hipStream_t stream);
+                          int merge_inside, const DecodeRope* rope, hipStream_t stream);
 
 // The units (attention_mfma.hip compiled for a padded head size of 32, 64, ... 256) are
 // libraries of their own, built and loaded when a model needs them and registered here.
@@ -42,6 +42,8 @@ static int unit_result(const char* name, int rc, int d) {
                    "256 (got %d)", name, d);
   else if (rc == 3)
     rlis_set_error("%s: partitions must be a multiple of 256 keys", name);
+  else if (rc == 4)
+    rlis_set_error("%s: too many sequences and KV heads to merge inside the kernel", name);
   else if (rc >= 1000)
     rlis_set_error("%s: launch failed: %s", name, hipGetErrorString((hipError_t)(rc - 1000)));
   else rlis_set_error("%s: unit error %d", name, rc);
@@ -108,13 +110,18 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
 // heads at v_off; with cos/sin (float32 (max positions, rot / 2), rot = d = 64, 128 or 256) q
 // and the new k are rotated by positions[s], without them nothing is; with slots the new k and
 // v go to the pages at slots[s] (page * page_size + offset).
+//
+// merge_inside != 0: the partitions of a sequence are merged by the last of their workgroups to
+// finish, counted in device memory that the library owns, instead of by a second kernel (which
+// still runs for more than 65,536 sequences times KV heads).  Same sums in the same order
+// either way.  Launches that overlap in time on one device must pass 0.
 RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
                                    long long out_stride, float* part_ml, float* part_acc,
                                    void* k_pages, void* v_pages,
                                    const int* block_tables, int max_pages, const int* ctx_lens,
                                    int S, int nh, int nkv, int d, int page_size, int window,
                                    float scale, int splits, int part_keys, int max_parts,
-                                   const float* cos, const float* sin,
+                                   int merge_inside, const float* cos, const float* sin,
                                    int rot, const int* positions, const int* slots,
                                    long long k_off, long long v_off, hipStream_t stream) {
   DecodeRope rope;
@@ -155,14 +162,15 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
   while ((1 << page_shift) < page_size) ++page_shift;
   const DecodeUnit unit = decode_units[unit_index(d)];
   RLIS_REQUIRE(unit != nullptr, "attn_decode_mfma: the unit for head size %d is not loaded", d);
+  const int inside = merge_inside && splits > 1 && (long long)S * nkv <= 65536;
   const int rc = unit_result(
       "attn_decode_mfma",
       unit(q, q_stride, out, out_stride, part_ml, part_acc, k_pages, v_pages, block_tables,
            max_pages, ctx_lens, S, nh, nkv, d, page_shift, window, scale, splits, part_keys,
-           max_parts, &rope, stream),
+           max_parts, inside, &rope, stream),
       d);
   if (rc) return rc;
-  if (splits > 1 && S > 0)
+  if (splits > 1 && S > 0 && !inside)
     return rlis_launch_attn_reduce_bf16(out, out_stride, part_ml, part_acc, S, nh, d, splits, stream);
   return 0;
 }

@@ -51,6 +51,7 @@ union Frag8 {
 constexpr int kUnitTooManyTiles = 1;
 constexpr int kUnitBadRotation = 2;
 constexpr int kUnitBadPartition = 3;
+constexpr int kUnitTooManyArrivals = 4;
 constexpr int kUnitLaunchFailed = 1000;       // + the hipError_t
 #define RLIS_UNIT_LAUNCH_CHECK()                                 \
   do {                                                           \
@@ -517,13 +518,35 @@ __device__ __forceinline__ void load8f(const float* p, float (&v)[8]) {
 
 constexpr int kDecodeWaves = 8;
 
+// Arrival counts of the partitions of one (sequence, KV head), for merging inside the kernel:
+// zero when the library is loaded, and set back to zero by the workgroup that merges, so every
+// launch finds zeros.  Each device holds its own copy.  Launches that overlap on one device
+// (two streams) would count into each other's slots: such callers merge outside.
+constexpr int kArrivalSlots = 65536;
+constexpr int kMergeAhead = 8;           // partitions whose results the merge loads at once
+static __device__ unsigned decode_arrivals[kArrivalSlots];
+
+// Partial results pass between workgroups of one launch, which may run on different compute
+// dies, each with a cache of its own between it and memory.  They are therefore stored and
+// loaded as device-scope atomics (relaxed): such a store goes through to where every die sees
+// it, and has arrived there once the wave's store counter has drained (which is what the
+// barrier in front of the arrival count waits for); such a load does not take a stale line.
+// That keeps the whole-cache write-backs and invalidations of device-scope fences out of the
+// kernel: 256 workgroups fencing cost more than the second kernel they were to save.
+__device__ __forceinline__ void store_shared_result(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_shared_result(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
     const bf16_t* __restrict__ q, long long q_stride, bf16_t* __restrict__ out,
     long long out_stride, float* __restrict__ part_ml, float* __restrict__ part_acc,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ ctx_lens,
     int nh, int nkv, int d, int page_shift, float scale, int window, int splits, int part_keys,
-    int max_parts, const DecodeRope rope) {
+    int max_parts, int merge_inside, const DecodeRope rope) {
   extern __shared__ float dsm[];           // ml: waves * g * 2 ; acc: waves * g * d
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int l16 = lane % 16, lq = lane / 16;
@@ -538,6 +561,10 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
   const int part = decode_part_len(ctx - lo32, part_keys, max_parts);   // a multiple of kStride
   const int kbeg = lo32 + split * part;
   const int kend = min(ctx, kbeg + part);
+  // Merging inside: only the partitions that hold keys of this sequence run, and the last of
+  // them to finish merges them all; a sequence with one such partition stores its result itself.
+  const int own = merge_inside ? max(1, min(splits, (ctx - lo32 + part - 1) / part)) : splits;
+  if (split >= own) return;
 
   const int pos = rope.positions ? rope.positions[seq] : 0;
   if (rope.positions && rope.slots && kbeg < ctx && kend == ctx) {
@@ -753,17 +780,81 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
       a += aw[w] * e;
     }
     const int h = kvh * g + hh;
-    if (splits == 1) {
+    if (own == 1) {
       out[(long long)seq * out_stride + h * d + j] = f32_to_bf16(a / lsum);
     } else {
       const long long idx = ((long long)seq * nh + h) * splits + split;
-      part_acc[idx * d + j] = a;
+      store_shared_result(part_acc + idx * d + j, a);
       if (j == 0) {
         // attn_reduce works with natural-log maxima: m * ln 2
-        part_ml[idx * 2] = big * 0.6931471805599453f;
-        part_ml[idx * 2 + 1] = lsum;
+        store_shared_result(part_ml + idx * 2, big * 0.6931471805599453f);
+        store_shared_result(part_ml + idx * 2 + 1, lsum);
       }
     }
+  }
+  if (!merge_inside || own == 1) return;
+
+  // ---- the last partition of (sequence, KV head) to arrive merges them all -------------
+  // Every thread's stores have arrived before it passes the barrier; thread 0 then counts this
+  // workgroup in.  The sums run over the partitions in order, with the arithmetic of
+  // attn_reduce_kernel, so the result does not depend on which workgroup came last.
+  __shared__ int merges;
+  __builtin_amdgcn_s_waitcnt(0);         // all counters at zero: this wave's stores have arrived
+  __syncthreads();
+  if (tid == 0) {
+    unsigned* slot = decode_arrivals + (seq * nkv + kvh);
+    const bool last = __hip_atomic_fetch_add(slot, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+                      (unsigned)(own - 1);
+    if (last) __hip_atomic_store(slot, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    merges = last;
+  }
+  __syncthreads();
+  if (!merges) return;
+  for (int i = tid; i < g * d; i += 64 * kDecodeWaves) {
+    const int hh = i / d, j = i % d;
+    const int h = kvh * g + hh;
+    const long long base = ((long long)seq * nh + h) * splits;
+    // The first kMergeAhead partitions are loaded at once (a partition past the sequence's own
+    // reads its last one and counts as empty), any further ones one after the other.
+    float mv[kMergeAhead], lv[kMergeAhead], av[kMergeAhead];
+#pragma unroll
+    for (int s = 0; s < kMergeAhead; ++s) {
+      const long long idx = base + min(s, own - 1);
+      mv[s] = load_shared_result(part_ml + idx * 2);
+      lv[s] = load_shared_result(part_ml + idx * 2 + 1);
+      av[s] = load_shared_result(part_acc + idx * d + j);
+    }
+    float big = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < kMergeAhead; ++s) {
+      if (s >= own) lv[s] = 0.f;
+      if (lv[s] > 0.f) big = fmaxf(big, mv[s]);
+    }
+    for (int s = kMergeAhead; s < own; ++s) {
+      const float m = load_shared_result(part_ml + (base + s) * 2);
+      const float l = load_shared_result(part_ml + (base + s) * 2 + 1);
+      if (l > 0.f) big = fmaxf(big, m);
+    }
+    float lsum = 0.f, a = 0.f;
+#pragma unroll
+    for (int s = 0; s < kMergeAhead; ++s) {
+      const float e = lv[s] > 0.f ? expf(mv[s] - big) : 0.f;
+      if (e > 0.f) {
+        lsum += lv[s] * e;
+        a += av[s] * e;
+      }
+    }
+    for (int s = kMergeAhead; s < own; ++s) {
+      const float m = load_shared_result(part_ml + (base + s) * 2);
+      const float l = load_shared_result(part_ml + (base + s) * 2 + 1);
+      const float v = load_shared_result(part_acc + (base + s) * d + j);
+      const float e = l > 0.f ? expf(m - big) : 0.f;
+      if (e > 0.f) {
+        lsum += l * e;
+        a += v * e;
+      }
+    }
+    out[(long long)seq * out_stride + h * d + j] = f32_to_bf16(a / lsum);
   }
 }
 
@@ -771,10 +862,11 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
     const void* q, long long q_stride, void* out, long long out_stride, float* part_ml,
     float* part_acc, const void* k_pages, const void* v_pages, const int* block_tables,
     int max_pages, const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift, int window,
-    float scale, int splits, int part_keys, int max_parts, const DecodeRope* rope,
-    hipStream_t stream) {
+    float scale, int splits, int part_keys, int max_parts, int merge_inside,
+    const DecodeRope* rope, hipStream_t stream) {
   if (S == 0) return 0;
   if (part_keys % (32 * kDecodeWaves) != 0 || part_keys <= 0) return kUnitBadPartition;
+  if (merge_inside && (long long)S * nkv > kArrivalSlots) return kUnitTooManyArrivals;
   // rotation inside the kernel needs head_dim = rotated width = 64, 128 or 256
   if (rope->positions && rope->cos && !(D % 64 == 0 && rope->rot == D && d == D))
     return kUnitBadRotation;
@@ -784,7 +876,7 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
   DECODE_KERNEL_NAME<<<grid, 64 * kDecodeWaves, smem, stream>>>(
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, part_ml, part_acc,
       (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, max_pages, ctx_lens, nh, nkv, d,
-      page_shift, scale, window, splits, part_keys, max_parts, *rope);
+      page_shift, scale, window, splits, part_keys, max_parts, merge_inside, *rope);
   RLIS_UNIT_LAUNCH_CHECK();
   return 0;
 }

@@ -41,6 +41,11 @@ FORCE_ATTENTION: Optional[str] = None
 # "matrix": bfloat16 decode attention on the matrix cores where it applies; "vector": always
 # the vector-unit decode kernel (tests compare the two).
 DECODE_ATTENTION = "matrix"
+# The matrix-core decode attention merges a sequence's partitions in the workgroup that finishes
+# last instead of in a second kernel (the same sums either way; tests compare the two).  The
+# arrival counts are the library's, one set per device: a caller whose launches overlap on one
+# device (several streams) switches this off.
+MERGE_DECODE_INSIDE = True
 
 
 def _dt(t: torch.Tensor) -> int:
@@ -542,8 +547,8 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                      ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
                      block_tables.data_ptr(), max_pages, _i32(step.ctx_lens, "ctx_lens", S), S,
                      nh, nkv, d, page_size, win, float(scale), depth, ap.DECODE_PART_KEYS,
-                     ap.DECODE_MAX_PARTS, cos_p, sin_p, rot, pos_p, slots_p, nh * d,
-                     (nh + nkv) * d, stream)
+                     ap.DECODE_MAX_PARTS, int(MERGE_DECODE_INSIDE), cos_p, sin_p, rot, pos_p,
+                     slots_p, nh * d, (nh + nkv) * d, stream)
         else:
             lib.call("rlis_attn_decode", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(),
                      nh * d, ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),

@@ -696,6 +696,38 @@ def test_attention_decode_long_split(ops, dtype, decode_kind):
         torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
 
 
+@pytest.mark.parametrize("nh,nkv,d,ps", [(32, 8, 64, 16), (24, 8, 128, 16), (16, 2, 256, 16), (5, 5, 48, 16),
+                                         (9, 3, 112, 16)])
+@pytest.mark.parametrize("window", [None, 700])
+def test_attention_decode_partitions_merged_inside_the_kernel(ops, nh, nkv, d, ps, window):
+    """The matrix-core decode kernel merging a sequence's partitions itself (the last workgroup
+    to finish does it) against the same kernel followed by the merge kernel: bit for bit the
+    same, whichever workgroup comes last, and again on every further call (the arrival counts
+    go back to zero by themselves).  Sequences with one partition beside ones with many, and a
+    grid deeper than most sequences need."""
+    dtype = torch.bfloat16
+    lens = [1, 5, 300, 1024, 1025, 2100, 4000, 9000, 255, 256, 257, 3, 2048, 2049]
+    cached, new = [l - 1 for l in lens], [1] * len(lens)
+    scale = 1.0 / math.sqrt(d)
+    qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=d + 3)
+    want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, window)
+    old = ops.MERGE_DECODE_INSIDE
+    try:
+        for part_keys, max_parts in ((1024, 16), (256, 36), (256, 5), (512, 2)):
+            with attention_constants(DECODE_PART_KEYS=part_keys, DECODE_MAX_PARTS=max_parts):
+                ops.MERGE_DECODE_INSIDE = False
+                outside = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window,
+                                              force="decode")
+                torch.testing.assert_close(outside.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
+                ops.MERGE_DECODE_INSIDE = True
+                for call in range(3):
+                    inside = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale,
+                                                 window, force="decode")
+                    assert torch.equal(inside, outside), f"cut {part_keys} x {max_parts}, call {call}"
+    finally:
+        ops.MERGE_DECODE_INSIDE = old
+
+
 @pytest.mark.parametrize("kind,dtype", kinds_and_dtypes("generic", "prefill", "decode"))
 def test_attention_finds_a_far_key(ops, dtype, kind, decode_kind):
     """One key among hundreds is made to stand out (its key vector equals the scaled query
