@@ -234,63 +234,80 @@ static bool launch_add_rmsnorm_bf16x8(float* resid, const void* delta, const voi
 }
 
 // The delta as a stack of float32 partial sums (what the split-k and the streaming products
-// leave for their consumer), rows of a multiple of 4 and at most 256 * 4 * CH elements: four
-// elements per thread and chunk, 16-byte accesses, four parts in flight at a time; the parts
-// are added in order and their sum rounded to bfloat16 when round_parts is set.
-template <typename TW, typename TO, int CH>
-__global__ __launch_bounds__(256) void add_rmsnorm_stack_kernel(
+// leave for their consumer), rows of a multiple of 4 and at most NT * 4 * CH elements: four
+// elements per thread and chunk, 16-byte accesses.  Such stacks come with few rows (64 at most)
+// and up to dozens of parts, so a row gets a wide workgroup (NT threads, as many as the row has
+// groups of four, up to 1024) and every thread keeps four parts of all its chunks in flight;
+// the parts are added in order and their sum rounded to bfloat16 when round_parts is set.
+template <typename TW, typename TO, int CH, int NT>
+__global__ __launch_bounds__(NT) void add_rmsnorm_stack_kernel(
     float* __restrict__ resid, const float* __restrict__ delta, const TW* __restrict__ weight,
     TO* __restrict__ out, const int* __restrict__ rows, int H, float eps, int write_resid,
     int parts, long long part_stride, int round_parts) {
-  __shared__ float red[256 / kWave];
+  __shared__ float red[NT / kWave];
   const int r = blockIdx.x;
   const long long src = rows ? (long long)rows[r] : (long long)r;
   float* x = resid + src * H;
   const float* d = delta + src * H;
+  // A chunk past the row reads the row's first elements instead (and stores nothing).
+  int col[CH];
+  bool live[CH];
+  float4 xr[CH], s[CH];
+#pragma unroll
+  for (int ch = 0; ch < CH; ++ch) {
+    const int j = (threadIdx.x + ch * NT) * 4;
+    live[ch] = j < H;
+    col[ch] = live[ch] ? j : 0;
+    xr[ch] = *(const float4*)(x + col[ch]);
+    s[ch] = *(const float4*)(d + col[ch]);
+  }
+  int p = 1;
+  for (; p + 3 < parts; p += 4) {
+    float4 a[CH][4];
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) a[ch][q] = *(const float4*)(d + (p + q) * part_stride + col[ch]);
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        s[ch].x += a[ch][q].x; s[ch].y += a[ch][q].y; s[ch].z += a[ch][q].z; s[ch].w += a[ch][q].w;
+      }
+  }
+  for (; p < parts; ++p) {
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch) {
+      const float4 a = *(const float4*)(d + p * part_stride + col[ch]);
+      s[ch].x += a.x; s[ch].y += a.y; s[ch].z += a.z; s[ch].w += a.w;
+    }
+  }
   float v[CH][4];
   float ss = 0.f;
 #pragma unroll
   for (int ch = 0; ch < CH; ++ch) {
-    const int j = (threadIdx.x + ch * 256) * 4;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) v[ch][e] = 0.f;
-    if (j < H) {
-      const float4 xr = *(const float4*)(x + j);
-      float4 s = *(const float4*)(d + j);
-      int p = 1;
-      for (; p + 3 < parts; p += 4) {
-        const float4 a = *(const float4*)(d + (p + 0) * part_stride + j);
-        const float4 b = *(const float4*)(d + (p + 1) * part_stride + j);
-        const float4 c = *(const float4*)(d + (p + 2) * part_stride + j);
-        const float4 e4 = *(const float4*)(d + (p + 3) * part_stride + j);
-        s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
-        s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
-        s.x += c.x; s.y += c.y; s.z += c.z; s.w += c.w;
-        s.x += e4.x; s.y += e4.y; s.z += e4.z; s.w += e4.w;
-      }
-      for (; p < parts; ++p) {
-        const float4 a = *(const float4*)(d + p * part_stride + j);
-        s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
-      }
-      if (round_parts) {
-        s.x = bf16_to_f32(f32_to_bf16(s.x)); s.y = bf16_to_f32(f32_to_bf16(s.y));
-        s.z = bf16_to_f32(f32_to_bf16(s.z)); s.w = bf16_to_f32(f32_to_bf16(s.w));
-      }
-      v[ch][0] = xr.x + s.x; v[ch][1] = xr.y + s.y; v[ch][2] = xr.z + s.z; v[ch][3] = xr.w + s.w;
-      if (write_resid) *(float4*)(x + j) = make_float4(v[ch][0], v[ch][1], v[ch][2], v[ch][3]);
+    if (round_parts) {
+      s[ch].x = bf16_to_f32(f32_to_bf16(s[ch].x)); s[ch].y = bf16_to_f32(f32_to_bf16(s[ch].y));
+      s[ch].z = bf16_to_f32(f32_to_bf16(s[ch].z)); s[ch].w = bf16_to_f32(f32_to_bf16(s[ch].w));
+    }
+    v[ch][0] = xr[ch].x + s[ch].x; v[ch][1] = xr[ch].y + s[ch].y;
+    v[ch][2] = xr[ch].z + s[ch].z; v[ch][3] = xr[ch].w + s[ch].w;
+    if (live[ch]) {
+      if (write_resid)
+        *(float4*)(x + col[ch]) = make_float4(v[ch][0], v[ch][1], v[ch][2], v[ch][3]);
 #pragma unroll
       for (int e = 0; e < 4; ++e) ss += v[ch][e] * v[ch][e];
     }
   }
-  ss = block_sum<256>(ss, red);
+  ss = block_sum<NT>(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)H + eps);
   TO* o = out + (long long)r * H;
 #pragma unroll
   for (int ch = 0; ch < CH; ++ch) {
-    const int j = (threadIdx.x + ch * 256) * 4;
-    if (j < H) {
+    if (live[ch]) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) st(o + j + e, v[ch][e] * inv * ld(weight + j + e));
+      for (int e = 0; e < 4; ++e)
+        st(o + col[ch] + e, v[ch][e] * inv * ld(weight + col[ch] + e));
     }
   }
 }
@@ -301,16 +318,17 @@ static bool launch_add_rmsnorm_stack(float* resid, const void* delta, const void
                                      void* out, const int* rows, int R, int H, float eps,
                                      int write_resid, int parts, long long part_stride,
                                      int round_parts, hipStream_t stream) {
-  if (H % 4 != 0 || H > 256 * 4 * 8 || part_stride % 4 != 0) return false;
+  if (H % 4 != 0 || H > 1024 * 4 * 4 || part_stride % 4 != 0) return false;
   if (((uintptr_t)resid | (uintptr_t)delta) % 16) return false;
-#define LAUNCH(CH)                                                                            \
-  add_rmsnorm_stack_kernel<TW, TO, CH><<<R, 256, 0, stream>>>(                                \
+#define LAUNCH(CH, NT)                                                                        \
+  add_rmsnorm_stack_kernel<TW, TO, CH, NT><<<R, NT, 0, stream>>>(                             \
       resid, (const float*)delta, (const TW*)weight, (TO*)out, rows, H, eps, write_resid,     \
       parts, part_stride, round_parts)
-  if (H <= 256 * 4) LAUNCH(1);
-  else if (H <= 256 * 8) LAUNCH(2);
-  else if (H <= 256 * 16) LAUNCH(4);
-  else LAUNCH(8);
+  if (H <= 256 * 4) LAUNCH(1, 256);
+  else if (H <= 512 * 4) LAUNCH(1, 512);
+  else if (H <= 1024 * 4) LAUNCH(1, 1024);
+  else if (H <= 1024 * 8) LAUNCH(2, 1024);
+  else LAUNCH(4, 1024);
 #undef LAUNCH
   return true;
 }

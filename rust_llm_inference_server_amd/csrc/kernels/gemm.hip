@@ -442,19 +442,18 @@ RLIS_API int rlis_gemm_bf16_skinny_swiglu(const void* X, const void* W, void* Y,
 constexpr int kSplitRows = 64;          // weight rows per workgroup
 constexpr int kSplitPad = 16;           // bf16 elements between rows of x in LDS: 32 bytes mod 64
 
-template <int KS, int NT>
+template <int KS, int NT, bool WALK>
 __global__ __launch_bounds__(256, 2) void gemm_bf16_splitk_kernel(const bf16_t* __restrict__ X,
                                                                const bf16_t* __restrict__ W,
                                                                float* __restrict__ Y, int T, int N,
                                                                int K, long long ldx, long long ldw,
-                                                               long long part_stride) {
+                                                               long long part_stride, int subs) {
   extern __shared__ __attribute__((aligned(16))) bf16_t splitk_x[];   // [NT * 16][KS + pad]
   constexpr int XS = KS + kSplitPad;
   constexpr int STEPS = KS / 32;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int l16 = lane % 16, lq = lane / 16;
   const int slice = blockIdx.y;
-  const int k0 = slice * KS;
   const int n0 = blockIdx.x * kSplitRows + wave * 16;
 
   // This wave's weight rows, in operand layout: lane l holds row l % 16 and the 8 k at
@@ -462,43 +461,65 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_splitk_kernel(const bf16_t* 
   // (its products are not stored), a k past K reads k = 0 (it meets a zero of x).
   const int row = min(n0 + l16, N - 1);
   const bf16_t* wrow = W + (long long)row * ldw;
-  Frag8 a[STEPS];
-#pragma unroll
-  for (int s = 0; s < STEPS; ++s) {
-    const int k = k0 + s * 32 + lq * 8;
-    a[s].u = *(const uint4*)(wrow + (k < K ? k : 0));
-  }
-  // The slice of x into LDS: 16-byte pieces, rows of tokens (zeros past T and past K).  All of a
-  // thread's pieces are loaded before the first is stored, so that they travel together (and
-  // with the weights); the loads are unconditional from a safe address, the value is selected.
+  // The slice of x goes into LDS in 16-byte pieces, rows of tokens (zeros past T and past K).
+  // All of a thread's pieces are loaded before the first is stored, so that they travel
+  // together (and with the weights); the loads are unconditional from a safe address, the value
+  // is selected.
   constexpr int PIECES = KS / 8;
   constexpr int XIT = NT * 16 * PIECES / 256;
+  Frag8 a[STEPS], ahead[WALK ? STEPS : 1];
   uint4 xv[XIT];
+  auto load = [&](int k0, Frag8 (&w)[STEPS]) __attribute__((always_inline)) {
 #pragma unroll
-  for (int j = 0; j < XIT; ++j) {
-    const int i = tid + j * 256;
-    const int tok = i / PIECES, k = k0 + (i % PIECES) * 8;
-    const bool ok = tok < T && k < K;
-    const uint4 v = *(const uint4*)(X + (ok ? (long long)tok * ldx + k : 0));
-    xv[j] = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
-  }
+    for (int s = 0; s < STEPS; ++s) {
+      const int k = k0 + s * 32 + lq * 8;
+      w[s].u = *(const uint4*)(wrow + (k < K ? k : 0));
+    }
 #pragma unroll
-  for (int j = 0; j < XIT; ++j) {
-    const int i = tid + j * 256;
-    *(uint4*)(splitk_x + (i / PIECES) * XS + (i % PIECES) * 8) = xv[j];
-  }
-  __syncthreads();
+    for (int j = 0; j < XIT; ++j) {
+      const int i = tid + j * 256;
+      const int tok = i / PIECES, k = k0 + (i % PIECES) * 8;
+      const bool ok = tok < T && k < K;
+      const uint4 v = *(const uint4*)(X + (ok ? (long long)tok * ldx + k : 0));
+      xv[j] = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+    }
+  };
 
   f32x4 acc[NT];
 #pragma unroll
   for (int tg = 0; tg < NT; ++tg) acc[tg] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  // A workgroup walks over `subs` pieces of KS of its slice (WALK; one piece otherwise), the
+  // next piece's weights and x on their way while the current one is multiplied.
+  if (!WALK) subs = 1;
+  int k0 = slice * subs * KS;
+  load(k0, a);
+  for (int sub = 0; sub < subs; ++sub) {
+    if (sub) __syncthreads();             // the last piece's x has been read by every wave
 #pragma unroll
-  for (int s = 0; s < STEPS; ++s) {
+    for (int j = 0; j < XIT; ++j) {
+      const int i = tid + j * 256;
+      *(uint4*)(splitk_x + (i / PIECES) * XS + (i % PIECES) * 8) = xv[j];
+    }
+    __syncthreads();
+    k0 += KS;
+    bool more = false;
+    if constexpr (WALK) {
+      more = sub + 1 < subs && k0 < K;
+      if (more) load(k0, ahead);
+    }
 #pragma unroll
-    for (int tg = 0; tg < NT; ++tg) {
-      Frag8 b;
-      b.u = *(const uint4*)(splitk_x + (tg * 16 + l16) * XS + s * 32 + lq * 8);
-      acc[tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s].v, b.v, acc[tg], 0, 0, 0);
+    for (int s = 0; s < STEPS; ++s) {
+#pragma unroll
+      for (int tg = 0; tg < NT; ++tg) {
+        Frag8 b;
+        b.u = *(const uint4*)(splitk_x + (tg * 16 + l16) * XS + s * 32 + lq * 8);
+        acc[tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s].v, b.v, acc[tg], 0, 0, 0);
+      }
+    }
+    if (!more) break;
+    if constexpr (WALK) {
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) a[s] = ahead[s];
     }
   }
   // The accumulator holds token l % 16 of its group and weight rows (l / 16) * 4 + r.
@@ -519,14 +540,30 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_splitk_kernel(const bf16_t* 
   }
 }
 
-// The k slice length rlis_gemm_bf16_splitk uses for a product with N weight rows over K: 512,
-// or 256 where that is needed to give every compute unit a workgroup.  Functions of N and K
-// alone; the number of slices (and of partial results) is ceil(K / slice).
-static int splitk_slice(int N, int K) {
+// How rlis_gemm_bf16_splitk cuts a product with N weight rows over K: pieces of 512 k, or of
+// 256 where that is needed to give every compute unit a workgroup, and two pieces per workgroup
+// where one would make more than two workgroups per compute unit (measured on 4096 x 14336 with
+// 32 rows: one piece 29 us and 28 partial results for the consumer to add, two 30 us and 14,
+// four 34 us and 7; the consumer gains more from 14 than the product loses).  Functions of N and
+// K alone; the number of slices (and of partial results) is ceil(K / (piece * pieces per
+// workgroup)).
+struct SplitkCut {
+  int piece, subs, slices;
+};
+static SplitkCut splitk_cut(int N, int K) {
   const long long groups = ceil_div(N, kSplitRows);
-  return groups * ceil_div(K, 512) >= 256 ? 512 : 256;
+  const long long pieces512 = ceil_div(K, 512);
+  SplitkCut c;
+  c.piece = groups * pieces512 >= 256 ? 512 : 256;
+  c.subs = 1;
+  if (c.piece == 512) {
+    const long long per = ceil_div_ll(groups * pieces512, 512);
+    c.subs = per > 1 ? 2 : 1;
+  }
+  c.slices = ceil_div(K, c.piece * c.subs);
+  return c;
 }
-RLIS_API int rlis_gemm_bf16_splitk_slices(int N, int K) { return ceil_div(K, splitk_slice(N, K)); }
+RLIS_API int rlis_gemm_bf16_splitk_slices(int N, int K) { return splitk_cut(N, K).slices; }
 
 // Y receives rlis_gemm_bf16_splitk_slices(N, K) partial results (T, N) float32 contiguous,
 // part_stride elements apart, to be added in order.  17 <= T <= 64 is what it is for; fewer
@@ -543,34 +580,37 @@ RLIS_API int rlis_gemm_bf16_splitk(const void* X, const void* W, void* Y, int T,
                "gemm_bf16_splitk: partial results %lld elements apart do not hold (T, N)",
                part_stride);
   if (T == 0) return 0;
-  const int ks = splitk_slice(N, K);
-  const int slices = ceil_div(K, ks);
+  const SplitkCut cut = splitk_cut(N, K);
+  const int ks = cut.piece, slices = cut.slices;
   const int nt = ceil_div(T, 16);
   dim3 grid(ceil_div(N, kSplitRows), slices);
   RLIS_REQUIRE(slices <= 65535, "gemm_bf16_splitk: K=%d is too long", K);
   const size_t smem = (size_t)nt * 16 * (ks + kSplitPad) * sizeof(bf16_t);
-#define GO(KS, NT)                                                                          \
+#define GO(KS, NT, WALK)                                                                    \
   {                                                                                         \
     static bool raised = false;                                                             \
     if (!raised && smem > 48 * 1024) {                                                      \
-      hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_splitk_kernel<KS, NT>,      \
+      hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_splitk_kernel<KS, NT, WALK>, \
                                          hipFuncAttributeMaxDynamicSharedMemorySize,        \
                                          (int)smem);                                        \
       RLIS_REQUIRE(e == hipSuccess, "gemm_bf16_splitk: cannot raise the LDS limit: %s",     \
                    hipGetErrorString(e));                                                   \
       raised = true;                                                                        \
     }                                                                                       \
-    gemm_bf16_splitk_kernel<KS, NT><<<grid, 256, smem, stream>>>(                           \
-        (const bf16_t*)X, (const bf16_t*)W, (float*)Y, T, N, K, ldx, ldw, part_stride);     \
+    gemm_bf16_splitk_kernel<KS, NT, WALK><<<grid, 256, smem, stream>>>(                     \
+        (const bf16_t*)X, (const bf16_t*)W, (float*)Y, T, N, K, ldx, ldw, part_stride,      \
+        cut.subs);                                                                          \
   }
-#define BY_NT(KS)                        \
-  switch (nt) {                          \
-    case 1: GO(KS, 1) break;             \
-    case 2: GO(KS, 2) break;             \
-    case 3: GO(KS, 3) break;             \
-    default: GO(KS, 4) break;            \
+#define BY_NT(KS, WALK)                        \
+  switch (nt) {                                \
+    case 1: GO(KS, 1, WALK) break;             \
+    case 2: GO(KS, 2, WALK) break;             \
+    case 3: GO(KS, 3, WALK) break;             \
+    default: GO(KS, 4, WALK) break;            \
   }
-  if (ks == 512) BY_NT(512) else BY_NT(256)
+  if (ks == 512 && cut.subs > 1) BY_NT(512, true)
+  else if (ks == 512) BY_NT(512, false)
+  else BY_NT(256, false)
 #undef BY_NT
 #undef GO
   RLIS_LAUNCH_CHECK("gemm_bf16_splitk");

@@ -44,8 +44,12 @@ DECODE_ATTENTION = "matrix"
 # The matrix-core decode attention merges a sequence's partitions in the workgroup that finishes
 # last instead of in a second kernel (the same sums either way; tests compare the two).  The
 # arrival counts are the library's, one set per device: a caller whose launches overlap on one
-# device (several streams) switches this off.
+# device (several streams) switches this off.  It pays while the kernel is short: every
+# workgroup ends with a round trip to memory in which it streams nothing, about 3 % of a long
+# kernel's time, against the 5 us of the second kernel; so it is used up to this many bytes of
+# keys and values under the grid (partitions x partition length x 2 x head size x 2 bytes).
 MERGE_DECODE_INSIDE = True
+MERGE_DECODE_INSIDE_MAX_BYTES = 512 << 20
 
 
 def _dt(t: torch.Tensor) -> int:
@@ -543,11 +547,13 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                 slots_p = None if slots is None else _i32(slots, "slots", S)
                 if cos is not None:
                     cos_p, sin_p, rot = cos.data_ptr(), sin.data_ptr(), 2 * cos.shape[1]
+            inside = MERGE_DECODE_INSIDE and (S * nkv * depth * ap.DECODE_PART_KEYS * d * 4
+                                              <= MERGE_DECODE_INSIDE_MAX_BYTES)
             lib.call("rlis_attn_decode_mfma", qkv.data_ptr(), q_stride, out.data_ptr(), nh * d,
                      ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
                      block_tables.data_ptr(), max_pages, _i32(step.ctx_lens, "ctx_lens", S), S,
                      nh, nkv, d, page_size, win, float(scale), depth, ap.DECODE_PART_KEYS,
-                     ap.DECODE_MAX_PARTS, int(MERGE_DECODE_INSIDE), cos_p, sin_p, rot, pos_p,
+                     ap.DECODE_MAX_PARTS, int(inside), cos_p, sin_p, rot, pos_p,
                      slots_p, nh * d, (nh + nkv) * d, stream)
         else:
             lib.call("rlis_attn_decode", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(),

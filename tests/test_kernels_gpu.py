@@ -219,7 +219,8 @@ def test_linear_streaming_kernel(ops, out_dtype, T, N, K):
 
 @pytest.mark.parametrize("T,N,K", [(17, 2048, 2048), (64, 2048, 8192), (33, 3072, 2048), (24, 130, 96),
                                    (64, 331, 104), (48, 17, 14336), (19, 1001, 4608), (40, 16, 8),
-                                   (64, 4096, 14336), (50, 3072, 3072)])
+                                   (64, 4096, 14336), (50, 3072, 3072), (64, 3072, 8192),
+                                   (32, 4096, 14344), (48, 8192, 3000), (17, 6144, 1536)])
 def test_linear_split_k_kernel(ops, T, N, K):
     """The split-k kernel that 17 to 64 rows take where the result joins the residual stream:
     float32 partial sums per k slice against float64 products of the same bf16-rounded
@@ -229,7 +230,10 @@ def test_linear_split_k_kernel(ops, T, N, K):
     want = (x.double() @ w.double().t()).float()
     parts = ops.linear(x, w, partials=True)
     assert parts.dim() == 3 and parts.shape[1:] == (T, N) and parts.dtype == torch.float32
-    assert parts.shape[0] == -(-K // 512) or parts.shape[0] == -(-K // 256)
+    # pieces of 512 k (256 where the product is small), one or two of them per workgroup
+    groups, pieces = -(-N // 64), -(-K // 512)
+    per_group = 2 if groups * pieces > 512 else 1
+    assert parts.shape[0] == (-(-K // 256) if groups * pieces < 256 else -(-K // (512 * per_group)))
     got = parts.sum(dim=0)
     scale = max(1.0, want.abs().max().item())
     torch.testing.assert_close(got, want, atol=2e-5 * scale * math.sqrt(K / 64), rtol=1e-4)
@@ -711,8 +715,9 @@ def test_attention_decode_partitions_merged_inside_the_kernel(ops, nh, nkv, d, p
     scale = 1.0 / math.sqrt(d)
     qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=d + 3)
     want = reference_attention(qkv, ks, vs, cu, cached, new, nh, nkv, d, scale, window)
-    old = ops.MERGE_DECODE_INSIDE
+    old = ops.MERGE_DECODE_INSIDE, ops.MERGE_DECODE_INSIDE_MAX_BYTES
     try:
+        ops.MERGE_DECODE_INSIDE_MAX_BYTES = 1 << 50          # whatever the size of the grid
         for part_keys, max_parts in ((1024, 16), (256, 36), (256, 5), (512, 2)):
             with attention_constants(DECODE_PART_KEYS=part_keys, DECODE_MAX_PARTS=max_parts):
                 ops.MERGE_DECODE_INSIDE = False
@@ -725,7 +730,7 @@ def test_attention_decode_partitions_merged_inside_the_kernel(ops, nh, nkv, d, p
                                                  window, force="decode")
                     assert torch.equal(inside, outside), f"cut {part_keys} x {max_parts}, call {call}"
     finally:
-        ops.MERGE_DECODE_INSIDE = old
+        ops.MERGE_DECODE_INSIDE, ops.MERGE_DECODE_INSIDE_MAX_BYTES = old
 
 
 @pytest.mark.parametrize("kind,dtype", kinds_and_dtypes("generic", "prefill", "decode"))
