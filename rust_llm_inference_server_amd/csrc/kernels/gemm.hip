@@ -581,7 +581,11 @@ RLIS_API int rlis_gemm_bf16_splitk(const void* X, const void* W, void* Y, int T,
                part_stride);
   if (T == 0) return 0;
   const SplitkCut cut = splitk_cut(N, K);
-  const int ks = cut.piece, slices = cut.slices;
+  // A workgroup that walks takes its slice in pieces of 256 (the registers of a piece are held
+  // twice then): the same k in the same order as pieces of 512 would give.
+  const int walk = cut.subs > 1;
+  const int ks = walk ? 256 : cut.piece, slices = cut.slices;
+  const int subs = cut.piece * cut.subs / ks;
   const int nt = ceil_div(T, 16);
   dim3 grid(ceil_div(N, kSplitRows), slices);
   RLIS_REQUIRE(slices <= 65535, "gemm_bf16_splitk: K=%d is too long", K);
@@ -599,7 +603,7 @@ RLIS_API int rlis_gemm_bf16_splitk(const void* X, const void* W, void* Y, int T,
     }                                                                                       \
     gemm_bf16_splitk_kernel<KS, NT, WALK><<<grid, 256, smem, stream>>>(                     \
         (const bf16_t*)X, (const bf16_t*)W, (float*)Y, T, N, K, ldx, ldw, part_stride,      \
-        cut.subs);                                                                          \
+        subs);                                                                              \
   }
 #define BY_NT(KS, WALK)                        \
   switch (nt) {                                \
@@ -608,7 +612,7 @@ RLIS_API int rlis_gemm_bf16_splitk(const void* X, const void* W, void* Y, int T,
     case 3: GO(KS, 3, WALK) break;             \
     default: GO(KS, 4, WALK) break;            \
   }
-  if (ks == 512 && cut.subs > 1) BY_NT(512, true)
+  if (walk) BY_NT(256, true)
   else if (ks == 512) BY_NT(512, false)
   else BY_NT(256, false)
 #undef BY_NT
