@@ -1,0 +1,162 @@
+// bfloat16 products with more than 64 rows (and the ones of 17 to 64 rows that do not join the
+// residual stream) are the library's: hipBLASLt, called here directly.  The reference uses a
+// library matmul for every projection (crates/model/src/layers.rs:30-46, candle's matmul).
+//
+// Why not through the tensor library's matmul: a step that mixes a portion of a prompt with
+// decoding requests launches four products per layer, and 20 us of host time per call (operator
+// dispatch, output allocation, a heuristics lookup) against 5 us here decide whether the host
+// keeps ahead of the device at 500 tokens a step.
+//
+// The library is not linked: the process already holds one copy (the tensor library's own),
+// and a second copy with its own kernels would answer the same symbols.  rlis_lt_open takes
+// the path of the copy to use, opens it and looks the entry points up.  A plan (operation and
+// layout descriptors, the algorithm the library's heuristics rank first) is made once per
+// shape and kept.
+#include <dlfcn.h>
+#include <hipblaslt/hipblaslt.h>
+
+#include <map>
+#include <mutex>
+#include <tuple>
+
+#include "common.h"
+
+namespace {
+
+struct LtApi {
+  void* lib = nullptr;
+  decltype(&hipblasLtCreate) create = nullptr;
+  decltype(&hipblasLtMatmulDescCreate) desc_create = nullptr;
+  decltype(&hipblasLtMatmulDescSetAttribute) desc_set = nullptr;
+  decltype(&hipblasLtMatrixLayoutCreate) layout_create = nullptr;
+  decltype(&hipblasLtMatmulPreferenceCreate) pref_create = nullptr;
+  decltype(&hipblasLtMatmulPreferenceSetAttribute) pref_set = nullptr;
+  decltype(&hipblasLtMatmulPreferenceDestroy) pref_destroy = nullptr;
+  decltype(&hipblasLtMatmulAlgoGetHeuristic) heuristic = nullptr;
+  decltype(&hipblasLtMatmul) matmul = nullptr;
+};
+
+struct LtPlan {
+  hipblasLtMatmulDesc_t op = nullptr;
+  hipblasLtMatrixLayout_t a = nullptr, b = nullptr, c = nullptr;
+  hipblasLtMatmulAlgo_t algo;
+  size_t workspace = 0;
+};
+
+// (device, T, N, K, ldx, ldw, ldy, float32 result, workspace limit)
+using LtKey = std::tuple<int, int, int, int, long long, long long, long long, int, size_t>;
+
+std::mutex lt_mutex;
+LtApi lt;
+std::map<int, hipblasLtHandle_t> lt_handles;      // per device
+std::map<LtKey, LtPlan> lt_plans;
+
+template <typename F>
+bool lookup(F& fn, const char* name) {
+  fn = (F)dlsym(lt.lib, name);
+  return fn != nullptr;
+}
+
+}  // namespace
+
+// Opens the copy of hipBLASLt at `path` (the one the process has loaded already, if it has) and
+// finds its entry points.  Calling it again is harmless.
+RLIS_API int rlis_lt_open(const char* path) {
+  std::lock_guard<std::mutex> lock(lt_mutex);
+  if (lt.lib) return 0;
+  RLIS_REQUIRE(path && *path, "lt_open: no path to the library");
+  void* lib = dlopen(path, RTLD_NOW | RTLD_LOCAL | RTLD_NOLOAD);
+  if (!lib) lib = dlopen(path, RTLD_NOW | RTLD_LOCAL);
+  RLIS_REQUIRE(lib != nullptr, "lt_open: cannot open %s: %s", path, dlerror());
+  lt.lib = lib;
+  const bool ok = lookup(lt.create, "hipblasLtCreate") &&
+                  lookup(lt.desc_create, "hipblasLtMatmulDescCreate") &&
+                  lookup(lt.desc_set, "hipblasLtMatmulDescSetAttribute") &&
+                  lookup(lt.layout_create, "hipblasLtMatrixLayoutCreate") &&
+                  lookup(lt.pref_create, "hipblasLtMatmulPreferenceCreate") &&
+                  lookup(lt.pref_set, "hipblasLtMatmulPreferenceSetAttribute") &&
+                  lookup(lt.pref_destroy, "hipblasLtMatmulPreferenceDestroy") &&
+                  lookup(lt.heuristic, "hipblasLtMatmulAlgoGetHeuristic") &&
+                  lookup(lt.matmul, "hipblasLtMatmul");
+  if (!ok) {
+    lt = LtApi();
+    rlis_set_error("lt_open: %s lacks an entry point of hipBLASLt", path);
+    return 1;
+  }
+  return 0;
+}
+
+RLIS_API int rlis_lt_is_open() {
+  std::lock_guard<std::mutex> lock(lt_mutex);
+  return lt.lib != nullptr;
+}
+
+// y (T, N) = x (T, K) W^T for W (N, K), all row-major with rows ldx, ldw, ldy elements apart;
+// x and W bfloat16, y bfloat16 or float32 (out_f32), float32 accumulation.  `workspace` is
+// device memory of workspace_bytes that the caller keeps for these calls (none: 0).
+RLIS_API int rlis_lt_gemm_bf16(const void* X, const void* W, void* Y, int out_f32, int T, int N,
+                               int K, long long ldx, long long ldw, long long ldy,
+                               void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  RLIS_REQUIRE(T >= 0 && N > 0 && K > 0 && ldx >= K && ldw >= K && ldy >= N,
+               "lt_gemm: bad sizes T=%d N=%d K=%d ldx=%lld ldw=%lld ldy=%lld", T, N, K, ldx, ldw,
+               ldy);
+  RLIS_REQUIRE(workspace || workspace_bytes == 0, "lt_gemm: a workspace size without a workspace");
+  if (T == 0) return 0;
+  int device = 0;
+  hipError_t he = hipGetDevice(&device);
+  RLIS_REQUIRE(he == hipSuccess, "lt_gemm: %s", hipGetErrorString(he));
+  hipblasLtHandle_t handle = nullptr;
+  LtPlan plan;
+  {
+    std::lock_guard<std::mutex> lock(lt_mutex);
+    RLIS_REQUIRE(lt.lib != nullptr, "lt_gemm: the library has not been opened");
+    auto h = lt_handles.find(device);
+    if (h == lt_handles.end()) {
+      hipblasLtHandle_t made = nullptr;
+      RLIS_REQUIRE(lt.create(&made) == HIPBLAS_STATUS_SUCCESS, "lt_gemm: cannot create a handle");
+      h = lt_handles.emplace(device, made).first;
+    }
+    handle = h->second;
+    const LtKey key(device, T, N, K, ldx, ldw, ldy, out_f32 ? 1 : 0, workspace_bytes);
+    auto p = lt_plans.find(key);
+    if (p == lt_plans.end()) {
+      // Column-major view: y^T (N, T) = W^T-as-stored transposed (N, K) times x-as-stored (K, T).
+      LtPlan made;
+      const hipDataType out_type = out_f32 ? HIP_R_32F : HIP_R_16BF;
+      bool ok = lt.desc_create(&made.op, HIPBLAS_COMPUTE_32F, HIP_R_32F) == HIPBLAS_STATUS_SUCCESS;
+      const int32_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
+      ok = ok && lt.desc_set(made.op, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta)) == HIPBLAS_STATUS_SUCCESS;
+      ok = ok && lt.desc_set(made.op, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof(tb)) == HIPBLAS_STATUS_SUCCESS;
+      ok = ok && lt.layout_create(&made.a, HIP_R_16BF, K, N, ldw) == HIPBLAS_STATUS_SUCCESS;
+      ok = ok && lt.layout_create(&made.b, HIP_R_16BF, K, T, ldx) == HIPBLAS_STATUS_SUCCESS;
+      ok = ok && lt.layout_create(&made.c, out_type, N, T, ldy) == HIPBLAS_STATUS_SUCCESS;
+      RLIS_REQUIRE(ok, "lt_gemm: cannot describe the product T=%d N=%d K=%d", T, N, K);
+      hipblasLtMatmulPreference_t pref = nullptr;
+      ok = lt.pref_create(&pref) == HIPBLAS_STATUS_SUCCESS;
+      const uint64_t limit = workspace_bytes;
+      ok = ok && lt.pref_set(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &limit, sizeof(limit)) ==
+                     HIPBLAS_STATUS_SUCCESS;
+      hipblasLtMatmulHeuristicResult_t found;
+      int count = 0;
+      ok = ok && lt.heuristic(handle, made.op, made.a, made.b, made.c, made.c, pref, 1, &found,
+                              &count) == HIPBLAS_STATUS_SUCCESS;
+      if (pref) lt.pref_destroy(pref);
+      RLIS_REQUIRE(ok && count > 0 && found.state == HIPBLAS_STATUS_SUCCESS,
+                   "lt_gemm: the library has no algorithm for T=%d N=%d K=%d", T, N, K);
+      RLIS_REQUIRE(found.workspaceSize <= workspace_bytes,
+                   "lt_gemm: the algorithm wants %zu bytes of workspace, %zu are there",
+                   found.workspaceSize, workspace_bytes);
+      made.algo = found.algo;
+      made.workspace = found.workspaceSize;
+      p = lt_plans.emplace(key, made).first;
+    }
+    plan = p->second;
+  }
+  const float one = 1.f, zero = 0.f;
+  const hipblasStatus_t st =
+      lt.matmul(handle, plan.op, &one, W, plan.a, X, plan.b, &zero, Y, plan.c, Y, plan.c,
+                &plan.algo, workspace, workspace_bytes, stream);
+  RLIS_REQUIRE(st == HIPBLAS_STATUS_SUCCESS, "lt_gemm: the product T=%d N=%d K=%d failed (%d)", T,
+               N, K, (int)st);
+  return 0;
+}

@@ -35,6 +35,10 @@ FUSE_ROPE_DECODE = True
 # "library": bf16 products with more rows than the streaming kernel takes go to torch
 # (hipBLASLt); "own": they take the hand-written skinny and matrix-core kernels.
 BF16_GEMM = "library"
+# The library's products are called directly (hipBLASLt's own entry points, a plan kept per
+# shape) rather than through torch.matmul: the same library and algorithm, a quarter of the
+# host time per call.
+LIBRARY_GEMM_DIRECT = True
 # None: attention kernels are chosen from the batch; "generic": the generic kernel always
 # (what the command line's --attention v1 asks for).
 FORCE_ATTENTION: Optional[str] = None
@@ -203,6 +207,13 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
                  ldw, T * N, stream)
         return y
     if bf16 and aligned and T > STREAM_MAX_ROWS and BF16_GEMM == "library":
+        ws = lib.library_workspace(x.device) if LIBRARY_GEMM_DIRECT else None
+        if ws is not None and out_dtype in (torch.bfloat16, torch.float32):
+            y = torch.empty((T, N), dtype=out_dtype, device=x.device)
+            lib.call("rlis_lt_gemm_bf16", x.data_ptr(), w.data_ptr(), y.data_ptr(),
+                     int(out_dtype == torch.float32), T, N, K, ldx, ldw, N, ws.data_ptr(),
+                     ws.numel(), stream)
+            return y
         if out_dtype == torch.bfloat16:
             return torch.matmul(x, w.t())
         return torch.mm(x, w.t(), out_dtype=torch.float32)    # float32 accumulation and result

@@ -38,6 +38,8 @@ _SIGNATURES = {
     "rlis_sample_rows": [P, L, I, I, P, P, P, I, P, P, P],
     "rlis_fill_normal_device": [P, I, L, ctypes.c_ulonglong, ctypes.c_ulonglong, ctypes.c_double,
                                 ctypes.c_double, P],
+    "rlis_lt_open": [c_char_p],
+    "rlis_lt_gemm_bf16": [P, P, P, I, I, I, I, L, L, L, P, ctypes.c_size_t, P],
 }
 
 
@@ -74,7 +76,44 @@ def load() -> ctypes.CDLL:
     lib.rlis_norm_linear_max_k.restype = c_int
     lib.rlis_norm_linear_max_k.argtypes = []
     _LIB = lib
+    library_workspace(torch.device("cuda", torch.cuda.current_device()))
     return lib
+
+
+# ---------------------------------------------------------------- the library's products
+# Workspace that hipBLASLt may use for a product, per device (what the tensor library grants it
+# on this family of chips).  Allocated when the kernels are loaded and at the first product on
+# any other device, never while a stream is capturing.
+LT_WORKSPACE_BYTES = 76 << 20
+_LT_OPEN: Optional[bool] = None
+_LT_WORKSPACES: dict = {}
+
+
+def _hipblaslt_path() -> str:
+    """The copy of hipBLASLt that this process has loaded already: the tensor library's own."""
+    import os
+    own = os.path.join(os.path.dirname(torch.__file__), "lib", "libhipblaslt.so")
+    return own if os.path.exists(own) else "libhipblaslt.so"
+
+
+def library_workspace(device: torch.device) -> Optional[torch.Tensor]:
+    """The device's workspace for ``rlis_lt_gemm_bf16``, or None when the library's products
+    cannot be called directly (its entry points were not found, or the workspace would have
+    to be allocated under a capturing stream): the caller then goes through ``torch.matmul``,
+    which reaches the same library."""
+    global _LT_OPEN
+    if _LT_OPEN is None:
+        _LT_OPEN = load().rlis_lt_open(_hipblaslt_path().encode()) == 0
+    if not _LT_OPEN:
+        return None
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    ws = _LT_WORKSPACES.get(index)
+    if ws is None:
+        if torch.cuda.is_current_stream_capturing():
+            return None
+        ws = torch.empty(LT_WORKSPACE_BYTES, dtype=torch.uint8, device=torch.device("cuda", index))
+        _LT_WORKSPACES[index] = ws
+    return ws
 
 
 _UNITS: dict = {}      # padded head size -> the loaded unit library

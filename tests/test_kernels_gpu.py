@@ -249,6 +249,39 @@ def test_linear_split_k_kernel(ops, T, N, K):
     assert torch.equal(summed, resid + rounded.to(torch.bfloat16).float())
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16], ids=["f32out", "bf16out"])
+@pytest.mark.parametrize("T,N,K", [(17, 3072, 2048), (64, 16384, 2048), (100, 2048, 8192), (575, 5120, 3072),
+                                   (2048, 2048, 2048), (33, 331, 104), (300, 1001, 776), (65, 8, 8)])
+def test_library_product_called_directly(ops, out_dtype, T, N, K):
+    """bfloat16 products beyond the hand-written kernels' row counts go to hipBLASLt through its
+    own entry points: against float64 products of the same operands, against the same library
+    through torch.matmul, strided operands, and twice (the second call takes the kept plan)."""
+    from rust_llm_inference_server_amd.ops import lib
+    assert lib.library_workspace(torch.device(DEV)) is not None, "hipBLASLt's entry points were not found"
+    x, w = rnd(T, K, dtype=torch.bfloat16, seed=3), rnd(N, K, dtype=torch.bfloat16, seed=4, scale=0.05)
+    want = (x.double() @ w.double().t()).float()
+    scale = max(1.0, want.abs().max().item())
+    tol_ = dict(atol=(2e-5 if out_dtype == torch.float32 else 8e-3) * scale * math.sqrt(K / 64), rtol=1e-2)
+    old = ops.LIBRARY_GEMM_DIRECT
+    try:
+        ops.LIBRARY_GEMM_DIRECT = False
+        through_torch = ops.linear(x, w, out_dtype)
+        ops.LIBRARY_GEMM_DIRECT = True
+        for _ in range(2):
+            got = ops.linear(x, w, out_dtype)
+            assert got.dtype == out_dtype and got.shape == (T, N)
+            torch.testing.assert_close(got.float(), want, **tol_)
+            torch.testing.assert_close(got.float(), through_torch.float(), **tol_)
+        # rows of x and of the weight inside wider arrays
+        wide_x = rnd(T, K + 24, dtype=torch.bfloat16, seed=5)
+        wide_w = rnd(N, K + 8, dtype=torch.bfloat16, seed=6, scale=0.05)
+        got = ops.linear(wide_x[:, 8:8 + K], wide_w[:, :K], out_dtype)
+        want = (wide_x[:, 8:8 + K].double() @ wide_w[:, :K].double().t()).float()
+        torch.testing.assert_close(got.float(), want, **tol_)
+    finally:
+        ops.LIBRARY_GEMM_DIRECT = old
+
+
 @pytest.mark.parametrize("T,N,K,parts,rows", [(1, 2048, 2048, 0, False), (8, 3072, 2048, 1, False),
                                               (16, 344, 104, 2, False), (5, 1001, 4096, 1, False),
                                               (3, 128256, 256, 1, True), (7, 64, 776, 3, True),
