@@ -44,6 +44,11 @@ def runtime() -> ctypes.CDLL:
             "rlis_cache_check": (c_int, [c_void_p, c_char_p, c_int]),
             "rlis_cache_decode_batch": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                 c_void_p, c_void_p, c_void_p]),
+            "rlis_cache_step_layout": (c_longlong, [c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                                                    c_void_p, c_void_p, c_void_p, c_void_p,
+                                                    c_void_p]),
+            "rlis_cache_step_fill": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                                             c_void_p, c_void_p, c_int, c_void_p, c_longlong]),
             "rlis_fill_normal": (c_int, [c_void_p, c_longlong, ctypes.c_ulonglong,
                                          ctypes.c_ulonglong, ctypes.c_double, ctypes.c_double,
                                          c_int]),
@@ -205,6 +210,27 @@ class CacheManager:
         are ctypes arrays of one pointer per group."""
         if runtime().rlis_cache_decode_batch(self._h, seqs_ptr, n, width, positions_ptr,
                                              state_slots_ptr, tables_ptrs, slots_ptrs) != 0:
+            raise ValueError(rt_error())
+
+    def step_layout(self, n: int, seqs_ptr: int, counts_ptr: int, tokens_ptr: int,
+                    want_counts_ptr: int, wants_ptr: int, info_ptr: int, offsets_ptr: int,
+                    order_ptr: int) -> int:
+        """Sizes, array offsets and sequence order of a step's common metadata (see
+        ``rlis_cache_step_layout``); returns the buffer's size in int32 elements."""
+        total = runtime().rlis_cache_step_layout(self._h, n, seqs_ptr, counts_ptr, tokens_ptr,
+                                                 want_counts_ptr, wants_ptr, info_ptr, offsets_ptr,
+                                                 order_ptr)
+        if total < 0:
+            raise ValueError(rt_error())
+        return total
+
+    def step_fill(self, n: int, seqs_ptr: int, counts_ptr: int, tokens_ptr: int,
+                  want_counts_ptr: int, wants_ptr: int, vocab_size: int, buf_ptr: int,
+                  capacity: int) -> None:
+        """Fill a step's common metadata into a caller-owned int32 buffer."""
+        if runtime().rlis_cache_step_fill(self._h, n, seqs_ptr, counts_ptr, tokens_ptr,
+                                          want_counts_ptr, wants_ptr, vocab_size, buf_ptr,
+                                          capacity) != 0:
             raise ValueError(rt_error())
 
     def check_invariants(self) -> None:

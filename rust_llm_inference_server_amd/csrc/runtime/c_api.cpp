@@ -7,6 +7,7 @@
 
 #include "cache_manager.h"
 #include "scheduler.h"
+#include "step_builder.h"
 
 #define RT_API extern "C" __attribute__((visibility("default")))
 
@@ -159,6 +160,60 @@ RT_API int rlis_cache_decode_batch(void* h, const long long* seqs, int n, int wi
       }
       slots[g][i] = page * ps + pos % ps;
     }
+  }
+  return 0;
+}
+
+// A step's common metadata (step_builder.h).  The entries come as parallel arrays: request
+// ids, token counts, all tokens in one array, counts of wanted indices and all of those in one
+// array.  rlis_cache_step_layout writes info = {tokens, sequences, wanted rows, single-token
+// sequences, longest context, most new tokens, then the table width of every group}, the
+// offsets of the arrays (8 + 2 per group), the entry index of every sequence of the step, and
+// returns the buffer's size in ints; rlis_cache_step_fill fills a buffer of that size.  Both
+// return a negative value with a message for a step that cannot run.
+static std::vector<rlis::StepEntryView> entry_views(int n, const long long* seqs, const int* counts,
+                                                    const long long* tokens, const int* want_counts,
+                                                    const int* wants) {
+  std::vector<rlis::StepEntryView> v(n > 0 ? n : 0);
+  long long t = 0, w = 0;
+  for (int i = 0; i < n; ++i) {
+    v[i] = {seqs[i], tokens + t, counts[i], wants + w, want_counts[i]};
+    t += counts[i] > 0 ? counts[i] : 0;
+    w += want_counts[i] > 0 ? want_counts[i] : 0;
+  }
+  return v;
+}
+
+RT_API long long rlis_cache_step_layout(void* h, int n, const long long* seqs, const int* counts,
+                                        const long long* tokens, const int* want_counts,
+                                        const int* wants, int* info, long long* offsets,
+                                        int* order) {
+  auto* m = static_cast<CacheManager*>(h);
+  rlis::StepLayout lay;
+  GUARD(lay = rlis::plan_step(*m, entry_views(n, seqs, counts, tokens, want_counts, wants)));
+  const int head[6] = {lay.tokens, lay.seqs, lay.wanted, lay.num_single, lay.max_context, lay.max_new};
+  std::copy(head, head + 6, info);
+  std::copy(lay.widths.begin(), lay.widths.end(), info + 6);
+  std::copy(lay.offsets.begin(), lay.offsets.end(), offsets);
+  std::copy(lay.order.begin(), lay.order.end(), order);
+  return lay.total;
+}
+
+RT_API int rlis_cache_step_fill(void* h, int n, const long long* seqs, const int* counts,
+                                const long long* tokens, const int* want_counts, const int* wants,
+                                int vocab_size, int* buf, long long cap) {
+  auto* m = static_cast<CacheManager*>(h);
+  try {
+    const auto entries = entry_views(n, seqs, counts, tokens, want_counts, wants);
+    const rlis::StepLayout lay = rlis::plan_step(*m, entries);
+    if (lay.total > cap) {
+      g_error = "the step's metadata does not fit the buffer";
+      return -1;
+    }
+    rlis::fill_step(*m, entries, lay, vocab_size, buf);
+  } catch (const std::exception& e) {
+    g_error = e.what();
+    return -1;
   }
   return 0;
 }

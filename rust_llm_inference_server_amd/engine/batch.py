@@ -7,12 +7,15 @@ The reference builds the same per step in ``PagedBatch::new`` (crates/model/src/
 slot id per token is enough (the write kernel spreads it over heads and dims), and all of it
 goes to the device in one copy.
 
-What is laid out here is common to every mixer.  What only one kind of mixer needs (the work
-lists of its kernels) comes from that mixer's ``StepPlanner`` and is carried along unseen:
-``build_step`` calls each planner with the step's host-side lengths and packs the arrays it
-returns into the same buffer (``step.plans[key]``)."""
+What is laid out here is common to every mixer, and the host runtime does it (one pass in C++
+over the requests' leases, ``csrc/runtime/step_builder.cpp``; ``build_step_in_python`` is its
+twin).  What only one kind of mixer needs (the work lists of its kernels) comes from that
+mixer's ``StepPlanner`` and is carried along unseen: ``build_step`` calls each planner with the
+step's host-side lengths and packs the arrays it returns into the same buffer
+(``step.plans[key]``)."""
 from __future__ import annotations
 
+import itertools
 from dataclasses import dataclass, field
 from typing import Any, Dict, List, Optional, Sequence, Tuple
 
@@ -107,12 +110,126 @@ def plan_name(index: int, array: str) -> str:
     return f"plan{index}.{array}"
 
 
+# Names of the arrays that every step carries, in the order of the host runtime's layout
+# (csrc/runtime/step_builder.h); each page group adds its write slots and block tables.
+_FIXED_ARRAYS = ("ids", "positions", "seq_of_token", "cu", "start_pos", "ctx_lens", "logit_rows",
+                 "state_slots")
+
+
+def _common_native(entries: Sequence[StepEntry], cache, vocab_size: int, spare: int):
+    """The common arrays laid out by the host runtime (one pass in C++ over the requests'
+    leases).  Returns (pinned buffer with ``spare`` ints of room behind the layout, offsets by
+    name as (offset, count), info) with info = (T, S, R, single-token sequences, longest
+    context, most new tokens, widths per group, order)."""
+    n = len(entries)
+    ng = cache.num_groups
+    counts = np.fromiter((len(e.tokens) for e in entries), dtype=np.int32, count=n)
+    want_counts = np.fromiter((len(e.want) for e in entries), dtype=np.int32, count=n)
+    seqs = np.fromiter((e.seq_id for e in entries), dtype=np.int64, count=n)
+    try:
+        tokens = np.fromiter(itertools.chain.from_iterable(e.tokens for e in entries),
+                             dtype=np.int64, count=int(counts.sum()))
+        wants = np.fromiter(itertools.chain.from_iterable(e.want for e in entries),
+                            dtype=np.int32, count=int(want_counts.sum()))
+    except (TypeError, ValueError):
+        raise ValueError("a request's tokens and wanted indices must be flat lists of integers") \
+            from None
+    info = np.zeros(6 + ng, dtype=np.int32)
+    offsets = np.zeros(len(_FIXED_ARRAYS) + 2 * ng, dtype=np.int64)
+    order = np.zeros(n, dtype=np.int32)
+    args = (n, seqs.ctypes.data, counts.ctypes.data, tokens.ctypes.data, want_counts.ctypes.data,
+            wants.ctypes.data)
+    total = cache.step_layout(*args, info.ctypes.data, offsets.ctypes.data, order.ctypes.data)
+    host = torch.empty(total + spare, dtype=torch.int32, pin_memory=torch.cuda.is_available())
+    cache.step_fill(*args, vocab_size, host.data_ptr(), total)
+    T, S, R = int(info[0]), int(info[1]), int(info[2])
+    widths = [int(w) for w in info[6:]]
+    sizes = [T, T, T, S + 1, S, S, R, S]
+    names = list(_FIXED_ARRAYS)
+    for g in range(ng):
+        names += [f"slots{g}", f"tables{g}"]
+        sizes += [T, S * widths[g]]
+    layout = {name: (int(o), int(c)) for name, o, c in zip(names, offsets, sizes)}
+    return host, total, layout, (T, S, R, int(info[3]), int(info[4]), int(info[5]), widths,
+                                 order.tolist())
+
+
 def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
-               vocab_size: int, planners: Sequence[StepPlanner] = ()) -> StepContext:
+               vocab_size: int, planners: Sequence[StepPlanner] = (),
+               native: Optional[bool] = None) -> StepContext:
     """Lay out a step.  Every entry's request must hold reserved positions for its tokens.
 
     Inside the step the sequences are ordered single tokens first (``host_order`` maps them back
-    to the entries); ``logit_rows`` keeps the order of the entries and of their ``want``."""
+    to the entries); ``logit_rows`` keeps the order of the entries and of their ``want``.
+
+    The common arrays are laid out by the host runtime where the cache manager is the runtime's
+    (``native``; None: if it is); ``build_step_in_python`` does the same here, for caches of
+    another kind and as the twin that tests hold the runtime's layout against."""
+    if native is None:
+        native = hasattr(cache, "step_fill")
+    if not native:
+        return build_step_in_python(entries, cache, device, vocab_size, planners)
+    if not entries:
+        raise ValueError("a step needs at least one request")
+    # what the planners add is not known before the lengths are; their arrays go behind the
+    # common ones, into room asked for up front (a second buffer when a plan outgrows it)
+    spare = 64 + 16 * len(entries) * max(1, len(planners))
+    host, used, layout, info = _common_native(entries, cache, vocab_size, spare)
+    T, S, R, num_single, max_context, max_new, widths, order = info
+    ps = cache.page_size
+    view_host = host.numpy()
+
+    def host_view(name):
+        o, c = layout[name]
+        return view_host[o:o + c]
+
+    start_pos = host_view("start_pos")
+    new = np.diff(host_view("cu"))
+    lengths = StepLengths(start_pos.astype(np.int64), new.astype(np.int64), num_single, ps)
+    host_plans: List[Tuple[Any, HostPlan]] = []
+    extra: List[Tuple[str, np.ndarray]] = []
+    at = used
+    for k, planner in enumerate(planners):
+        plan = planner.plan(lengths)
+        for name, arr in plan.arrays.items():
+            arr = np.asarray(arr, dtype=np.int32).reshape(-1)
+            layout[plan_name(k, name)] = (at, arr.size)
+            extra.append((plan_name(k, name), arr))
+            at += -(-arr.size // 4) * 4
+        host_plans.append((planner.key(), plan))
+    if at > host.numel():
+        grown = torch.empty(at, dtype=torch.int32, pin_memory=host.is_pinned())
+        grown[:used] = host[:used]
+        host, view_host = grown, grown.numpy()
+    for name, arr in extra:
+        o, c = layout[name]
+        view_host[o:o + c] = arr
+    dev = host[:at].to(device, non_blocking=True)
+
+    def view(name):
+        o, c = layout[name]
+        return dev[o:o + c]
+
+    ng = cache.num_groups
+    groups = [GroupStep(page_size=ps, window=cache.groups[g].window,
+                        block_tables=view(f"tables{g}").reshape(S, widths[g]),
+                        slots=view(f"slots{g}")) for g in range(ng)]
+    plans = {key: StepPlan({name: view(plan_name(k, name)) for name in plan.arrays}, plan.values)
+             for k, (key, plan) in enumerate(host_plans)}
+    return StepContext(
+        num_tokens=T, num_seqs=S, ids=view("ids"), positions=view("positions"),
+        seq_of_token=view("seq_of_token"), cu_seqlens=view("cu"), start_pos=view("start_pos"),
+        ctx_lens=view("ctx_lens"), logit_rows=view("logit_rows"), num_logit_rows=R,
+        state_slots=view("state_slots"), groups=groups, max_context=max_context,
+        max_new=max_new, all_decode=num_single == S, num_single=num_single, plans=plans,
+        lengths=lengths, host_start_pos=start_pos.tolist(), host_new=new.tolist(),
+        host_state_slots=host_view("state_slots").tolist(), host_order=order)
+
+
+def build_step_in_python(entries: Sequence[StepEntry], cache, device: torch.device,
+                         vocab_size: int, planners: Sequence[StepPlanner] = ()) -> StepContext:
+    """``build_step`` with the common arrays laid out here, through the cache's ``table`` and
+    ``_get_info`` alone."""
     if not entries:
         raise ValueError("a step needs at least one request")
     order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens) != 1)

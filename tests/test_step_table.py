@@ -87,3 +87,66 @@ def test_the_references_step_table(device, tmp_path):
     used = sorted(TABLES[0][:3] + TABLES[1][:2])          # 11 and 5 positions of 4 a page
     written = [p for p in range(16) if k[p].abs().sum().item() > 0]
     assert written == used
+
+
+def test_the_runtimes_step_layout_is_the_python_twins():
+    """The host runtime lays a step's common arrays out exactly as ``build_step_in_python``
+    does: random steps (single tokens among portions, windows that have given pages back, state
+    slots, wanted rows in the entries' order) over two page groups, array by array; and the same
+    complaints about steps that cannot run."""
+    import numpy as np
+    from rust_llm_inference_server_amd.cache.manager import CacheManager, GroupSpec
+    from rust_llm_inference_server_amd.engine import StepEntry, build_step
+    from rust_llm_inference_server_amd.ops.attention_plan import AttentionPlanner
+    rng = np.random.default_rng(7)
+    cache = CacheManager(8, [GroupSpec(400, None), GroupSpec(400, 24)], num_state_slots=16)
+    cpu = torch.device("cpu")
+    planners = [AttentionPlanner(4, 2, 16)]
+    lengths = {}
+    for trial in range(40):
+        live = list(lengths)
+        for seq in rng.permutation(live)[:rng.integers(0, 3)]:
+            cache.free(int(seq))
+            del lengths[int(seq)]
+        while len(lengths) < 6:
+            lengths[int(rng.integers(0, 10_000))] = 0
+        entries = []
+        for seq in rng.permutation(list(lengths))[:rng.integers(1, 6)]:
+            seq = int(seq)
+            n = int(rng.choice([1, 1, 1, 2, 5, 17, 40]))
+            cache.reserve(seq, lengths[seq] + n)
+            want = sorted({int(w) for w in rng.integers(0, n, size=rng.integers(0, 3))})
+            entries.append(StepEntry(seq, rng.integers(0, 97, size=n).tolist(), want))
+        a = build_step(entries, cache, cpu, 97, planners, native=True)
+        b = build_step(entries, cache, cpu, 97, planners, native=False)
+        for name in ("ids", "positions", "seq_of_token", "cu_seqlens", "start_pos", "ctx_lens",
+                     "logit_rows", "state_slots"):
+            assert torch.equal(getattr(a, name), getattr(b, name)), (trial, name)
+        for ga, gb in zip(a.groups, b.groups):
+            assert torch.equal(ga.block_tables, gb.block_tables) and torch.equal(ga.slots, gb.slots)
+            assert (ga.page_size, ga.window) == (gb.page_size, gb.window)
+        for field in ("num_tokens", "num_seqs", "num_logit_rows", "max_context", "max_new",
+                      "all_decode", "num_single", "host_start_pos", "host_new",
+                      "host_state_slots", "host_order"):
+            assert getattr(a, field) == getattr(b, field), (trial, field)
+        assert a.plans.keys() == b.plans.keys()
+        for key in a.plans:
+            assert a.plans[key].values == b.plans[key].values
+            for name in a.plans[key].arrays:
+                assert torch.equal(a.plans[key][name], b.plans[key][name]), (trial, name)
+        for e in entries:
+            lengths[e.seq_id] += len(e.tokens)
+            cache.advance(e.seq_id, lengths[e.seq_id])
+    seq = next(iter(lengths))
+    cache.reserve(seq, lengths[seq] + 4)
+    for native in (True, False):
+        for bad, message in (([], "at least one request"),
+                             ([StepEntry(seq, [], [])], "empty sequence"),
+                             ([StepEntry(123456, [1], [])], "no page reserved"),
+                             ([StepEntry(seq, [1] * 5, [])], "no page reserved"),
+                             ([StepEntry(seq, [1, 97], [])], "outside the vocabulary"),
+                             ([StepEntry(seq, [1, -1], [])], "outside the vocabulary"),
+                             ([StepEntry(seq, [1, 2], [2])], "wanted index"),
+                             ([StepEntry(seq, [1], []), StepEntry(seq, [2], [])], "appears twice")):
+            with pytest.raises(ValueError, match=message):
+                build_step(bad, cache, cpu, 97, planners, native=native)
