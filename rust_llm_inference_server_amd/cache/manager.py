@@ -58,6 +58,7 @@ def runtime() -> ctypes.CDLL:
             "rlis_sched_schedule": (c_int, [c_void_p, PL, c_int, PI, PL, c_int, PI, PI, c_int, PI]),
             "rlis_sched_advance": (c_int, [c_void_p, c_longlong, c_int]),
             "rlis_sched_append_token": (c_int, [c_void_p, c_longlong]),
+            "rlis_sched_append_tokens": (c_int, [c_void_p, PL, c_int]),
             "rlis_sched_is_caught_up": (c_int, [c_void_p, c_longlong]),
             "rlis_sched_remove": (c_int, [c_void_p, c_longlong]),
             "rlis_sched_has_work": (c_int, [c_void_p]),

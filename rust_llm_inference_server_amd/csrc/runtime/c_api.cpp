@@ -278,6 +278,12 @@ RT_API int rlis_sched_append_token(void* h, long long id) {
   GUARD(static_cast<Scheduler*>(h)->append_token(id));
   return 0;
 }
+// One more token each for the n requests of ids (what rlis_sched_append_token does one by one).
+RT_API int rlis_sched_append_tokens(void* h, const long long* ids, int n) {
+  auto* s = static_cast<Scheduler*>(h);
+  for (int i = 0; i < n; ++i) GUARD(s->append_token(ids[i]));
+  return 0;
+}
 RT_API int rlis_sched_is_caught_up(void* h, long long id) { return static_cast<Scheduler*>(h)->is_caught_up(id); }
 RT_API int rlis_sched_remove(void* h, long long id) {
   GUARD(static_cast<Scheduler*>(h)->remove(id));

@@ -173,9 +173,19 @@ class Engine:
             entries.append(StepEntry(seq_id, seq.tokens[start:end],
                                      [end - start - 1] if last else []))
             final.append(last)
+        # A step in which every request brings one token and the device kernel can sample for
+        # all of them runs as one captured graph, sampling included; the bookkeeping below goes
+        # on while it runs, and only then are the tokens waited for.
+        modes, wait = None, None
+        if all(final) and all(end - start == 1 for _, start, end in sched.seqs):
+            modes = [self._seqs[seq_id].sampler.device_mode(end) for seq_id, _, end in sched.seqs]
+            if any(m is None for m in modes):
+                modes = None
         try:
             self.runner.apply_copies(sched.copies)
-            logits = self.runner.step(entries)
+            if modes is not None:
+                wait = self.runner.step_sampled(entries, modes)
+            logits = self.runner.step(entries) if wait is None else None
         except Exception as exc:
             # engine.rs:523-528: a failed step fails its own requests and no others; their
             # pages are free again and the engine goes on with the rest.
@@ -191,7 +201,7 @@ class Engine:
             seq = self._seqs[seq_id]
             # prompt tokens of this portion (recomputed ones after a preemption count again)
             self.stats_.prefill_tokens += max(0, min(end, seq.prompt_len) - start)
-            if not last:
+            if not last or wait is not None:
                 continue
             mode = seq.sampler.device_mode(len(seq.tokens))
             if mode is not None:
@@ -201,6 +211,13 @@ class Engine:
                 host_rows.append((row, seq_id))
             row += 1
         picked: Dict[int, int] = {}
+        if wait is not None:
+            try:
+                picked = {seq_id: tok for (seq_id, _, _), tok in zip(sched.seqs, wait())}
+            except Exception as exc:
+                for seq_id, _, _ in sched.seqs:
+                    self._finish(self._seqs[seq_id], "error", error=f"{type(exc).__name__}: {exc}")
+                raise
         if device_rows:
             idx = [r for r, _ in device_rows]
             sub = logits if len(idx) == logits.shape[0] else logits[
@@ -213,17 +230,21 @@ class Engine:
             for (_, seq_id), lrow in zip(host_rows, host_logits):
                 seq = self._seqs[seq_id]
                 picked[seq_id] = seq.sampler.sample(lrow, seq.tokens, len(seq.tokens))
-        out = []
+        out, grown = [], []
+        now = time.perf_counter()
         for (seq_id, _, _), last in zip(sched.seqs, final):
             if last:
-                out.append(self._accept(self._seqs[seq_id], picked[seq_id]))
+                out.append(self._accept(self._seqs[seq_id], picked[seq_id], now, grown))
+        self.scheduler.append_tokens(grown)
         self.stats_.running = self.scheduler.num_running
         self.stats_.waiting = self.scheduler.num_waiting
         self.stats_.pages_used = self.stats_.pages_total - self.runner.cache.num_free_pages(0)
         return out
 
-    def _accept(self, seq: _Sequence, token: int) -> Tuple[int, Optional[int], bool]:
-        now = time.perf_counter()
+    def _accept(self, seq: _Sequence, token: int, now: float, grown: List[int]
+                ) -> Tuple[int, Optional[int], bool]:
+        """Take a request's sampled token at time ``now``; a request that goes on is added to
+        ``grown`` (the scheduler hears of those in one call)."""
         if seq.first_token_at is None:
             seq.first_token_at = now
         seq.last_token_at = now
@@ -237,7 +258,7 @@ class Engine:
         if seq.output_len >= seq.params.max_tokens:
             self._finish(seq, "length")
             return (seq.id, token, True)
-        self.scheduler.append_token(seq.id)
+        grown.append(seq.id)
         return (seq.id, token, False)
 
     def _finish(self, seq: _Sequence, reason: str, error: Optional[str] = None) -> None:

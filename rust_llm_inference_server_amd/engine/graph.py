@@ -3,8 +3,11 @@
 A step in which every request brings one token launches well over a hundred small kernels;
 at batch 1 their launch cost exceeds their run time.  Such steps are therefore captured once
 per batch-size bucket into a HIP graph and replayed: the step's metadata lives in one static
-int32 buffer (filled on the host by the native page manager, one copy to the device), the
-kernels read it through fixed views, and the logits land in a static tensor.
+int32 buffer (filled on the host by the native page manager; the graph begins with its copy to
+the device), the kernels read it through fixed views, and the logits land in a static tensor.
+A second kind of graph goes on where the first ends: the sampling kernel on those logits (keys
+and temperatures travel with the metadata) and the copy of the tokens to pinned host memory,
+so that between two decode steps the host launches one graph and waits for one event.
 
 Unused rows of a bucket are padding requests of context 1 that read and write a scratch page
 beyond the manager's pages and a scratch state slot beyond its slots, so they touch nothing a
@@ -85,6 +88,10 @@ class DecodeGraph:
         for g in range(ng):
             meta.reserve(f"slots{g}", B)
             meta.reserve(f"tables{g}", B * W)
+        # what the sampling kernel needs per row (bit patterns; 1/T = 0: greedy), for the steps
+        # that sample inside the graph
+        meta.reserve("sample_keys", B)
+        meta.reserve("sample_inv_t", B)
         self.host = torch.zeros(meta.size, dtype=torch.int32).pin_memory()
         self.np = self.host.numpy()
         self.dev = torch.zeros(meta.size, dtype=torch.int32, device=dev)
@@ -105,9 +112,11 @@ class DecodeGraph:
                                  block_tables=dview(f"tables{g}").reshape(B, W),
                                  slots=dview(f"slots{g}")) for g in range(ng)]
         self.views = {name: dview(name) for name in meta.offsets}
-        # context bucket -> (graph, its static logits)
-        self.graphs: Dict[int, Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
-        self._copied: Optional[torch.cuda.Event] = None
+        # (context bucket, sampled) -> (graph, its static logits or sampled tokens)
+        self.graphs: Dict[Tuple[int, bool], Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
+        # where a sampling graph leaves its tokens for the host
+        self.tokens_host = torch.zeros(B, dtype=torch.int32).pin_memory()
+        self._done: Optional[torch.cuda.Event] = None
 
     def step_for(self, context_limit: int) -> StepContext:
         """The step as the kernels of a captured run see it: static views, and each planner's
@@ -144,14 +153,22 @@ class DecodeGraph:
         h["start_pos"][:] = h["positions"]
         h["ctx_lens"][:] = h["positions"] + 1
 
-    def prepare(self, seq_ids: Sequence[int], tokens: Sequence[int]) -> np.ndarray:
-        """Fill the host side of the metadata for one token per request; returns the new
-        tokens' positions.  Nothing is launched or copied to the device yet."""
-        if self._copied is not None:
-            self._copied.synchronize()       # the host buffer is free to be written again
+    def prepare(self, seq_ids: Sequence[int], tokens: Sequence[int],
+                modes: Optional[Sequence[Tuple[int, float]]] = None) -> np.ndarray:
+        """Fill the host side of the metadata for one token per request (``modes``: each row's
+        (key, 1/T) for a step that samples inside the graph); returns the new tokens'
+        positions.  Nothing is launched yet."""
+        if self._done is not None:
+            self._done.synchronize()         # the last replay has read the host buffer
         S = len(seq_ids)
         self.seq_ids[:S] = seq_ids
         self.h["ids"][:S] = tokens
+        if modes is not None:
+            self.h["sample_keys"][:S] = np.asarray([k for k, _ in modes], dtype=np.uint32).view(np.int32)
+            self.h["sample_inv_t"][:S] = np.asarray([t for _, t in modes],
+                                                    dtype=np.float32).view(np.int32)
+            self.h["sample_keys"][S:] = 0
+            self.h["sample_inv_t"][S:] = 0
         self.runner.cache.decode_batch(self.seq_ids.ctypes.data, S, self.width,
                                        self.ptr_positions, self.ptr_slots, self.ptr_tables,
                                        self.ptr_wslots)
@@ -161,35 +178,62 @@ class DecodeGraph:
     def launch(self, num_seqs: int, context_limit: int) -> torch.Tensor:
         """Run the prepared step.  Logits ``(num_seqs, vocab)``: a view of a static tensor that
         the next call for the same context bucket overwrites."""
-        if context_limit not in self.graphs:
-            self._capture(context_limit)
-        graph, logits = self.graphs[context_limit]
-        self.dev.copy_(self.host, non_blocking=True)
-        if self._copied is None:
-            self._copied = torch.cuda.Event()
-        self._copied.record()
-        graph.replay()
-        return logits[:num_seqs]
+        return self._replay(context_limit, False)[:num_seqs]
 
-    def _capture(self, context_limit: int) -> None:
-        """Capture the step on metadata that is all padding: what the warm-up run and the
-        capture itself compute lands on the scratch page and the scratch state slot, so that no
-        request's cache or state moves before the first replay."""
+    def launch_sampled(self, num_seqs: int, context_limit: int):
+        """Run the prepared step with the sampling inside.  Returns a function that waits for
+        the step and returns the requests' tokens."""
+        self._replay(context_limit, True)
+        done, tokens = self._done, self.tokens_host
+
+        def wait() -> list:
+            done.synchronize()
+            return tokens[:num_seqs].tolist()
+        return wait
+
+    def _replay(self, context_limit: int, sampled: bool) -> torch.Tensor:
+        key = (context_limit, sampled)
+        if key not in self.graphs:
+            self._capture(context_limit, sampled)
+        graph, result = self.graphs[key]
+        graph.replay()          # begins with the copy of the metadata to the device
+        if self._done is None:
+            self._done = torch.cuda.Event()
+        self._done.record()
+        return result
+
+    def _capture(self, context_limit: int, sampled: bool) -> None:
+        """Capture the step: the copy of the host's metadata to the device, the model, and with
+        ``sampled`` the sampling kernel and the copy of its tokens to the host.  The warm-up
+        run works on metadata that is all padding: what it computes lands on the scratch page
+        and the scratch state slot, so that no request's cache or state moves before the first
+        replay (the capture itself runs nothing)."""
+        from .. import ops
         runner = self.runner
         padding = self.host.clone()
         flat = padding.numpy()
         self._pad_from(0, {name: self.meta.view(flat, name) for name in self.meta.offsets})
         self.dev.copy_(padding)
         step = self.step_for(context_limit)
+        keys = self.views["sample_keys"]
+        inv_t = self.views["sample_inv_t"].view(torch.float32)
+
+        def run():
+            logits = runner.model.forward(step, runner.pools)
+            return ops.sample_rows(logits, keys, inv_t) if sampled else logits
+
         # One eager run first: it settles lazy initialisation (library loading, workspace
         # allocations) that must not happen under capture.
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            runner.model.forward(step, runner.pools)
+            run()
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with no_collection(), torch.cuda.graph(graph):
-            logits = runner.model.forward(step, runner.pools)
-        self.graphs[context_limit] = (graph, logits)
+            self.dev.copy_(self.host, non_blocking=True)
+            result = run()
+            if sampled:
+                self.tokens_host.copy_(result, non_blocking=True)
+        self.graphs[(context_limit, sampled)] = (graph, result)

@@ -9,7 +9,7 @@ program, the perplexity tool and the benchmark all call it.  Its contract is the
 crates/model/src/paged.rs:154-161, 255-296)."""
 from __future__ import annotations
 
-from typing import Dict, List, Optional, Sequence, Union
+from typing import Callable, Dict, List, Optional, Sequence, Tuple, Union
 
 import torch
 
@@ -161,9 +161,26 @@ class ModelRunner:
             self.cache.advance(entries[i].seq_id, start + len(entries[i].tokens))
         return logits
 
-    def _decode_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step_sampled(self, entries: Sequence[StepEntry],
+                     modes: Sequence[Tuple[int, float]]) -> Optional[Callable[[], List[int]]]:
+        """A step of one token per request with the sampling kernel inside the captured step:
+        ``modes`` holds each request's (key, 1/T) as ``Sampler.device_mode`` gives them.
+        The step is launched and a function comes back that waits for it and returns the
+        sampled tokens in the order of the entries (what the host has to do meanwhile it does
+        before calling it); None when this runner cannot run the step that way (no captured
+        steps, or entries that are no single tokens with their logits wanted): then nothing has
+        happened and ``step`` is to be called."""
+        if not self.use_graphs or not entries or len(entries) > self.max_num_seqs:
+            return None
+        if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
+            return None
+        return self._decode_step(entries, modes)
+
+    def _decode_step(self, entries: Sequence[StepEntry],
+                     modes: Optional[Sequence[Tuple[int, float]]] = None):
         """A step of one token per request, replayed from the HIP graph of its batch-size
-        bucket (captured at first use).  Same kernels, same results as the eager step."""
+        bucket (captured at first use).  Same kernels, same results as the eager step.  With
+        ``modes`` the graph samples too and the tokens come back instead of the logits."""
         from .graph import DecodeGraph, bucket_for, context_bucket
         S = len(entries)
         seq_ids = [e.seq_id for e in entries]
@@ -182,7 +199,7 @@ class ModelRunner:
         graph = self._graphs.get(bucket)
         if graph is None:
             graph = self._graphs[bucket] = DecodeGraph(self, bucket)
-        positions = graph.prepare(seq_ids, tokens)
+        positions = graph.prepare(seq_ids, tokens, modes)
         # Everything that can refuse the step is checked before anything is launched.
         longest = int(positions.max()) + 1
         if longest > self.model.max_positions:
@@ -193,6 +210,11 @@ class ModelRunner:
             self.pools.zero_states([int(graph.h["state_slots"][i]) for i in range(S)
                                     if positions[i] == 0])
         ends = [int(p) + 1 for p in positions]
+        if modes is not None:
+            wait = graph.launch_sampled(S, context_bucket(longest, self.model.max_positions))
+            for seq, end in zip(seq_ids, ends):
+                self.cache.advance(seq, end)
+            return wait
         logits = graph.launch(S, context_bucket(longest, self.model.max_positions))
         for seq, end in zip(seq_ids, ends):
             self.cache.advance(seq, end)

@@ -6,7 +6,7 @@ from __future__ import annotations
 import ctypes
 from ctypes import c_int, c_longlong
 from dataclasses import dataclass, field
-from typing import List, Tuple
+from typing import List, Sequence, Tuple
 
 from ..cache.manager import CacheManager, PageCopy, rt_error, runtime
 
@@ -74,6 +74,12 @@ class Scheduler:
 
     def append_token(self, seq_id: int) -> None:
         runtime().rlis_sched_append_token(self._h, seq_id)
+
+    def append_tokens(self, seq_ids: Sequence[int]) -> None:
+        """One more token each for ``seq_ids``, in one call."""
+        n = len(seq_ids)
+        if n and runtime().rlis_sched_append_tokens(self._h, (c_longlong * n)(*seq_ids), n) != 0:
+            raise ValueError(rt_error())
 
     def is_caught_up(self, seq_id: int) -> bool:
         return bool(runtime().rlis_sched_is_caught_up(self._h, seq_id))

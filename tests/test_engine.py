@@ -147,6 +147,40 @@ def test_seeded_temperature_ignores_the_neighbours(backend, dtype, folders):
     assert len(set(among[3])) > 1
 
 
+def test_steps_that_sample_inside_the_graph_pick_the_eager_steps_tokens(backend, dtype, folders):
+    """Decode steps whose every request the device kernel can sample for run as one captured
+    graph, metadata copy, model, sampling kernel and the tokens' way to the host included: the
+    same tokens as the engine without captured steps, greedy and with seeded temperature, for
+    requests that arrive and end at different steps; a request with a host-side sampler in the
+    batch sends the step down the other path, to the same tokens again."""
+    if backend.type != "cuda":
+        pytest.skip("captured steps exist on the GPU only")
+    model = load(folders["b"], backend, dtype)
+    prompts = prompts_for(384, [3, 17, 40, 9, 1], seed=8)
+    params = [SamplingParams.greedy(14), SamplingParams(temperature=0.7, seed=5, max_tokens=9),
+              SamplingParams(temperature=1.1, seed=6, max_tokens=14), SamplingParams.greedy(3),
+              SamplingParams(temperature=0.9, seed=7, max_tokens=11)]
+    runs = {}
+    for graphs in (True, False):
+        engine = engine_for(model, use_graphs=graphs, max_batched_tokens=32)
+        assert engine.runner.use_graphs == graphs
+        sampled_steps = []
+        if graphs:
+            real = engine.runner.step_sampled
+            engine.runner.step_sampled = lambda e, m: sampled_steps.append(len(e)) or real(e, m)
+        runs[graphs] = [o.token_ids for o in engine.generate(prompts, params)]
+        if graphs:
+            assert len(sampled_steps) >= 10 and max(sampled_steps) == 5
+    assert runs[True] == runs[False]
+    mixed = params[:4] + [SamplingParams(temperature=0.9, top_k=50, seed=7, max_tokens=11)]
+    with_host = {}
+    for graphs in (True, False):
+        engine = engine_for(model, use_graphs=graphs, max_batched_tokens=32)
+        with_host[graphs] = [o.token_ids for o in engine.generate(prompts, mixed)]
+    assert with_host[True] == with_host[False]
+    assert with_host[True][:4] == runs[True][:4]
+
+
 def test_host_sampler_modes_run_and_are_reproducible(backend, tiny_folders):
     model = load(tiny_folders["b"], backend)
     prompts = prompts_for(384, [7, 21], seed=5)
