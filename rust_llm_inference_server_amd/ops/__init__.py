@@ -51,9 +51,11 @@ DECODE_ATTENTION = "matrix"
 # device (several streams) switches this off.  It pays while the kernel is short: every
 # workgroup ends with a round trip to memory in which it streams nothing, about 3 % of a long
 # kernel's time, against the 5 us of the second kernel; so it is used up to this many bytes of
-# keys and values under the grid (partitions x partition length x 2 x head size x 2 bytes).
+# keys and values under the grid (partitions x partition length x 2 x head size x 2 bytes: an
+# upper bound, since a captured step's grid is as deep as its context bucket's longest context
+# needs and most sequences are shorter).
 MERGE_DECODE_INSIDE = True
-MERGE_DECODE_INSIDE_MAX_BYTES = 512 << 20
+MERGE_DECODE_INSIDE_MAX_BYTES = 2 << 30
 
 
 def _dt(t: torch.Tensor) -> int:
