@@ -166,26 +166,26 @@ class Engine:
                     self.cancel(seq_id)
                 raise RuntimeError("scheduler made no progress")
             return []
-        entries, final = [], []
-        for seq_id, start, end in sched.seqs:
-            seq = self._seqs[seq_id]
-            last = end == len(seq.tokens)
-            entries.append(StepEntry(seq_id, seq.tokens[start:end],
-                                     [end - start - 1] if last else []))
-            final.append(last)
         # A step in which every request brings one token and the device kernel can sample for
-        # all of them runs as one captured graph, sampling included; the bookkeeping below goes
+        # all of them runs as one captured graph, sampling included; the book-keeping below goes
         # on while it runs, and only then are the tokens waited for.
-        modes, wait = None, None
-        if all(final) and all(end - start == 1 for _, start, end in sched.seqs):
-            modes = [self._seqs[seq_id].sampler.device_mode(end) for seq_id, _, end in sched.seqs]
-            if any(m is None for m in modes):
-                modes = None
+        wait = None
+        singles = self._single_tokens(sched)
         try:
             self.runner.apply_copies(sched.copies)
-            if modes is not None:
-                wait = self.runner.step_sampled(entries, modes)
-            logits = self.runner.step(entries) if wait is None else None
+            if singles is not None:
+                wait = self.runner.step_sampled(*singles)
+            if wait is None:
+                entries, final = [], []
+                for seq_id, start, end in sched.seqs:
+                    seq = self._seqs[seq_id]
+                    last = end == len(seq.tokens)
+                    entries.append(StepEntry(seq_id, seq.tokens[start:end],
+                                             [end - start - 1] if last else []))
+                    final.append(last)
+                logits = self.runner.step(entries)
+            else:
+                final = [True] * len(sched.seqs)
         except Exception as exc:
             # engine.rs:523-528: a failed step fails its own requests and no others; their
             # pages are free again and the engine goes on with the rest.
@@ -240,6 +240,23 @@ class Engine:
         self.stats_.waiting = self.scheduler.num_waiting
         self.stats_.pages_used = self.stats_.pages_total - self.runner.cache.num_free_pages(0)
         return out
+
+    def _single_tokens(self, sched) -> Optional[Tuple[List[int], List[int], List[Tuple[int, float]]]]:
+        """(request ids, their tokens, their (key, 1/T)) when every request of the schedule brings
+        its last known token alone and the device kernel can sample for it; else None."""
+        ids, tokens, modes = [], [], []
+        seqs = self._seqs
+        for seq_id, start, end in sched.seqs:
+            seq = seqs[seq_id]
+            if end - start != 1 or end != len(seq.tokens):
+                return None
+            mode = seq.sampler.device_mode(end)
+            if mode is None:
+                return None
+            ids.append(seq_id)
+            tokens.append(seq.tokens[start])
+            modes.append(mode)
+        return ids, tokens, modes
 
     def _accept(self, seq: _Sequence, token: int, now: float, grown: List[int]
                 ) -> Tuple[int, Optional[int], bool]:

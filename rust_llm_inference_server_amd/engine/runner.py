@@ -161,40 +161,46 @@ class ModelRunner:
             self.cache.advance(entries[i].seq_id, start + len(entries[i].tokens))
         return logits
 
-    def step_sampled(self, entries: Sequence[StepEntry],
+    def step_sampled(self, seq_ids: Sequence[int], tokens: Sequence[int],
                      modes: Sequence[Tuple[int, float]]) -> Optional[Callable[[], List[int]]]:
         """A step of one token per request with the sampling kernel inside the captured step:
-        ``modes`` holds each request's (key, 1/T) as ``Sampler.device_mode`` gives them.
-        The step is launched and a function comes back that waits for it and returns the
-        sampled tokens in the order of the entries (what the host has to do meanwhile it does
-        before calling it); None when this runner cannot run the step that way (no captured
-        steps, or entries that are no single tokens with their logits wanted): then nothing has
-        happened and ``step`` is to be called."""
-        if not self.use_graphs or not entries or len(entries) > self.max_num_seqs:
+        request ``seq_ids[i]`` brings ``tokens[i]``, and ``modes[i]`` is its (key, 1/T) as
+        ``Sampler.device_mode`` gives them.  The step is launched and a function comes back
+        that waits for it and returns the sampled tokens in the order of the requests (what the
+        host has to do meanwhile it does before calling it); None when this runner has no
+        captured steps: then nothing has happened and ``step`` is to be called."""
+        if not self.use_graphs or not seq_ids or len(seq_ids) > self.max_num_seqs:
             return None
-        if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
-            return None
-        return self._decode_step(entries, modes)
+        return self._decode_lists(seq_ids, tokens, modes)
 
-    def _decode_step(self, entries: Sequence[StepEntry],
-                     modes: Optional[Sequence[Tuple[int, float]]] = None):
+    def _decode_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """A step of one token per request, replayed from the HIP graph of its batch-size
-        bucket (captured at first use).  Same kernels, same results as the eager step.  With
-        ``modes`` the graph samples too and the tokens come back instead of the logits."""
-        from .graph import DecodeGraph, bucket_for, context_bucket
+        bucket (captured at first use).  Same kernels, same results as the eager step."""
         S = len(entries)
-        seq_ids = [e.seq_id for e in entries]
-        if len(set(seq_ids)) != S:
-            raise ValueError("a request appears twice in one step")
-        tokens = [int(e.tokens[0]) for e in entries]
-        if min(tokens) < 0 or max(tokens) >= self.vocab_size:
-            raise ValueError(f"a token id is outside the vocabulary of {self.vocab_size}")
         rows: List[int] = []
         for i, e in enumerate(entries):
             for w in e.want:
                 if int(w) != 0:
                     raise ValueError(f"request {e.seq_id}: wanted index {w} is outside its 1 tokens")
                 rows.append(i)
+        logits = self._decode_lists([e.seq_id for e in entries],
+                                    [int(e.tokens[0]) for e in entries], None)
+        if rows == list(range(S)):
+            return logits
+        if not rows:
+            return logits[:0]
+        return logits[torch.tensor(rows, device=logits.device)]
+
+    def _decode_lists(self, seq_ids: Sequence[int], tokens: Sequence[int],
+                      modes: Optional[Sequence[Tuple[int, float]]]):
+        """The captured step for requests ``seq_ids`` bringing ``tokens``: the logits of all of
+        them, or with ``modes`` (the graph samples too) the function that waits for the tokens."""
+        from .graph import DecodeGraph, bucket_for, context_bucket
+        S = len(seq_ids)
+        if len(set(seq_ids)) != S:
+            raise ValueError("a request appears twice in one step")
+        if min(tokens) < 0 or max(tokens) >= self.vocab_size:
+            raise ValueError(f"a token id is outside the vocabulary of {self.vocab_size}")
         bucket = bucket_for(S, self.max_num_seqs)
         graph = self._graphs.get(bucket)
         if graph is None:
@@ -209,17 +215,9 @@ class ModelRunner:
             # a request whose first token this is starts from cleared state
             self.pools.zero_states([int(graph.h["state_slots"][i]) for i in range(S)
                                     if positions[i] == 0])
-        ends = [int(p) + 1 for p in positions]
-        if modes is not None:
-            wait = graph.launch_sampled(S, context_bucket(longest, self.model.max_positions))
-            for seq, end in zip(seq_ids, ends):
-                self.cache.advance(seq, end)
-            return wait
-        logits = graph.launch(S, context_bucket(longest, self.model.max_positions))
+        ends = (positions + 1).tolist()
+        limit = context_bucket(longest, self.model.max_positions)
+        result = graph.launch_sampled(S, limit) if modes is not None else graph.launch(S, limit)
         for seq, end in zip(seq_ids, ends):
             self.cache.advance(seq, end)
-        if rows == list(range(S)):
-            return logits
-        if not rows:
-            return logits[:0]
-        return logits[torch.tensor(rows, device=logits.device)]
+        return result

@@ -167,7 +167,7 @@ def test_steps_that_sample_inside_the_graph_pick_the_eager_steps_tokens(backend,
         sampled_steps = []
         if graphs:
             real = engine.runner.step_sampled
-            engine.runner.step_sampled = lambda e, m: sampled_steps.append(len(e)) or real(e, m)
+            engine.runner.step_sampled = lambda i, t, m: sampled_steps.append(len(i)) or real(i, t, m)
         runs[graphs] = [o.token_ids for o in engine.generate(prompts, params)]
         if graphs:
             assert len(sampled_steps) >= 10 and max(sampled_steps) == 5
