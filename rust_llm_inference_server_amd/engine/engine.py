@@ -213,7 +213,7 @@ class Engine:
         picked: Dict[int, int] = {}
         if wait is not None:
             try:
-                picked = {seq_id: tok for (seq_id, _, _), tok in zip(sched.seqs, wait())}
+                picked = dict(zip(singles[0], wait()))
             except Exception as exc:
                 for seq_id, _, _ in sched.seqs:
                     self._finish(self._seqs[seq_id], "error", error=f"{type(exc).__name__}: {exc}")

@@ -8,6 +8,8 @@ from ctypes import c_int, c_longlong
 from dataclasses import dataclass, field
 from typing import List, Sequence, Tuple
 
+import numpy as np
+
 from ..cache.manager import CacheManager, PageCopy, rt_error, runtime
 
 
@@ -61,9 +63,12 @@ class Scheduler:
             self._copies, len(self._copies) // 3, n_c)
         if rc != 0:
             raise RuntimeError(rt_error())
-        s, c = self._seqs, self._copies
+        c = self._copies
+        # (read through a numpy view: element by element a ctypes array costs more than the
+        # scheduling itself at 64 requests)
+        triples = np.frombuffer(self._seqs, dtype=np.int64, count=3 * n_s.value)
         return Schedule(
-            seqs=[(s[3 * i], s[3 * i + 1], s[3 * i + 2]) for i in range(n_s.value)],
+            seqs=[tuple(t) for t in triples.reshape(-1, 3).tolist()],
             copies=[PageCopy(c[3 * i], c[3 * i + 1], c[3 * i + 2]) for i in range(n_c.value)],
             preempted=list(self._pre[:n_p.value]),
         )
