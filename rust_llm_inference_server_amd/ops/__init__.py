@@ -36,7 +36,7 @@ FUSE_ROPE_DECODE = True
 # (hipBLASLt); "own": they take the hand-written skinny and matrix-core kernels.
 BF16_GEMM = "library"
 # The library's products are called directly (hipBLASLt's own entry points, a plan kept per
-# shape) rather than through torch.matmul: the same library and algorithm, a quarter of the
+# shape) rather than through torch.matmul: the same library and algorithm, two thirds of the
 # host time per call.
 LIBRARY_GEMM_DIRECT = True
 # None: attention kernels are chosen from the batch; "generic": the generic kernel always
@@ -184,8 +184,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
 
     A float32 weight (or float32 ``x``) takes the plain FMA kernel, the true 32-bit product.
     bfloat16 operands take the streaming kernel up to 16 rows; more rows go to the library's
-    GEMM (hipBLASLt through torch), or with ``BF16_GEMM = "own"`` to the skinny kernel up to 64
-    rows and the hand-written matrix-core GEMM beyond.
+    GEMM (hipBLASLt, through its own entry points), or with ``BF16_GEMM = "own"`` to the skinny
+    kernel up to 64 rows and the hand-written matrix-core GEMM beyond.
 
     ``partials``: the caller hands the result to the residual stream and takes it as a stack
     ``(S, T, N)`` of float32 partial sums too (one per k slice of the streaming kernel, or of
