@@ -411,6 +411,69 @@ int rlis_launch_attn_reduce_bf16(void* out, long long out_stride, const float* p
   return 0;
 }
 
+// The same merge for the key runs of a prefill step, where the rows are many (every new token
+// of a portion, times the heads) and the runs few: one wave per (row, head), four of them to a
+// workgroup, no LDS and no barrier.  Every lane reads the runs' maxima and denominators for
+// itself (the same addresses across the wave) and owns dims lane, lane + 64, ...; the first
+// kRowRuns runs are loaded at once.  Same sums in the same order as attn_reduce_kernel.
+constexpr int kRowRuns = 8;
+
+__global__ __launch_bounds__(256) void attn_reduce_rows_kernel(
+    bf16_t* __restrict__ out, long long out_stride, const float* __restrict__ part_ml,
+    const float* __restrict__ part_acc, int nh, int d, int stride,
+    const int* __restrict__ seq_of_row, const int* __restrict__ seq_parts, int row0,
+    long long pairs) {
+  const long long pair = (long long)blockIdx.x * 4 + threadIdx.x / kWave;
+  if (pair >= pairs) return;
+  const int lane = threadIdx.x % kWave;
+  const int r = (int)(pair / nh), h = (int)(pair % nh);
+  const int row = row0 + r;
+  const int splits = min(stride, seq_parts[seq_of_row[row]]);
+  if (splits <= 1) return;
+  const long long base = (pair)*stride;
+  float mv[kRowRuns], lv[kRowRuns];
+#pragma unroll
+  for (int s = 0; s < kRowRuns; ++s) {
+    const long long idx = base + min(s, splits - 1);
+    mv[s] = part_ml[idx * 2];
+    lv[s] = s < splits ? part_ml[idx * 2 + 1] : 0.f;
+  }
+  float big = -INFINITY;
+#pragma unroll
+  for (int s = 0; s < kRowRuns; ++s)
+    if (lv[s] > 0.f) big = fmaxf(big, mv[s]);
+  for (int s = kRowRuns; s < splits; ++s)
+    if (part_ml[(base + s) * 2 + 1] > 0.f) big = fmaxf(big, part_ml[(base + s) * 2]);
+  float ev[kRowRuns];
+  float lsum = 0.f;
+#pragma unroll
+  for (int s = 0; s < kRowRuns; ++s) {
+    ev[s] = lv[s] > 0.f ? expf(mv[s] - big) : 0.f;
+    if (ev[s] > 0.f) lsum += lv[s] * ev[s];
+  }
+  for (int s = kRowRuns; s < splits; ++s) {
+    const float l = part_ml[(base + s) * 2 + 1];
+    const float e = l > 0.f ? expf(part_ml[(base + s) * 2] - big) : 0.f;
+    if (e > 0.f) lsum += l * e;
+  }
+  for (int j = lane; j < d; j += kWave) {
+    const float* acc = part_acc + base * d + j;
+    float av[kRowRuns];
+#pragma unroll
+    for (int s = 0; s < kRowRuns; ++s) av[s] = acc[(long long)min(s, splits - 1) * d];
+    float a = 0.f;
+#pragma unroll
+    for (int s = 0; s < kRowRuns; ++s)
+      if (ev[s] > 0.f) a += av[s] * ev[s];
+    for (int s = kRowRuns; s < splits; ++s) {
+      const float l = part_ml[(base + s) * 2 + 1];
+      const float e = l > 0.f ? expf(part_ml[(base + s) * 2] - big) : 0.f;
+      if (e > 0.f) a += acc[(long long)s * d] * e;
+    }
+    out[(long long)row * out_stride + h * d + j] = f32_to_bf16(a / lsum);
+  }
+}
+
 // Merges the key runs of the matrix-core prefill kernel: `rows` output rows from row0 on, whose
 // partial results lie at part_ml (rows, nh, stride, 2) and part_acc (rows, nh, stride, d);
 // row r belongs to sequence seq_of_token[row0 + r], which has seq_runs[sequence] runs (rows
@@ -424,15 +487,12 @@ RLIS_API int rlis_attn_reduce_rows(void* out, long long out_stride, const float*
   RLIS_REQUIRE(part_ml && part_acc && seq_of_token && seq_runs,
                "attn_reduce_rows: partial results and the run counts are needed");
   RLIS_REQUIRE(rows <= 65535 * 32, "attn_reduce_rows: %d rows are too many", rows);
-  const int threads = d <= 64 ? 64 : (d <= 128 ? 128 : 256);
-  for (int r = 0; r < rows; r += 65535) {
-    const int n = min(65535, rows - r);
-    dim3 grid(nh, n);
-    attn_reduce_kernel<bf16_t><<<grid, threads, (stride + 8) * sizeof(float), stream>>>(
-        (bf16_t*)out, out_stride, part_ml + (long long)r * nh * stride * 2,
-        part_acc + (long long)r * nh * stride * d, nullptr, nh, d, stride, seq_of_token, seq_runs,
-        row0 + r);
-  }
+  const long long pairs = (long long)rows * nh;
+  RLIS_REQUIRE((pairs + 3) / 4 <= 0x7fffffffLL, "attn_reduce_rows: %d rows are too many", rows);
+  if (pairs > 0)
+    attn_reduce_rows_kernel<<<(unsigned)((pairs + 3) / 4), 256, 0, stream>>>(
+        (bf16_t*)out, out_stride, part_ml, part_acc, nh, d, stride, seq_of_token, seq_runs, row0,
+        pairs);
   RLIS_LAUNCH_CHECK("attn_reduce_rows");
   return 0;
 }
