@@ -552,7 +552,36 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
   const int l16 = lane % 16, lq = lane / 16;
   const int kvh = blockIdx.x, seq = blockIdx.y, split = blockIdx.z;
   const int g = nh / nkv;
+  // ---- first round trip to memory: what depends on the workgroup's place alone ---------
+  // The context length, the token's position and slot, the raw q rows, and this KV head's new
+  // key and value (element tid of each, with the key's rotation partner; d is at most 256, the
+  // workgroup has 512 threads) are all asked for before anything is waited for.
+  const bool rotates = rope.positions != nullptr;
+  const bool stores_kv = rotates && rope.slots != nullptr;
   const int ctx = ctx_lens[seq];
+  const int pos = rotates ? rope.positions[seq] : 0;
+  const int slot = stores_kv ? rope.slots[seq] : -1;
+  Frag8 qf[D / 32];
+#pragma unroll
+  for (int ks = 0; ks < D / 32; ++ks) {
+    const int dim = ks * 32 + lq * 8;
+    const bool ok = l16 < g && dim < d;
+    const uint4 v = *(const uint4*)(q + (long long)seq * q_stride + (ok ? (kvh * g + l16) * d + dim : 0));
+    qf[ks].u = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+  }
+  const int half = rope.rot / 2;
+  const bool kv_thread = stores_kv && tid < d;
+  const bool k_turns = kv_thread && rope.cos && tid < rope.rot;
+  bf16_t new_k = 0, new_partner = 0, new_v = 0;
+  if (kv_thread) {
+    const bf16_t* krow = q + (long long)seq * q_stride + rope.k_off + kvh * d;
+    const bf16_t* vrow = q + (long long)seq * q_stride + rope.v_off + kvh * d;
+    new_k = krow[tid];
+    new_v = vrow[tid];
+    if (k_turns) new_partner = krow[tid < half ? tid + half : tid - half];
+  }
+
+  // ---- what follows from the context length ---------------------------------------------
   const int* table = block_tables + (long long)seq * max_pages;
   const int page_mask = (1 << page_shift) - 1;
   const int lo = (window > 0 && ctx - window > 0) ? ctx - window : 0;
@@ -566,67 +595,6 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
   const int own = merge_inside ? max(1, min(splits, (ctx - lo32 + part - 1) / part)) : splits;
   if (split >= own) return;
 
-  const int pos = rope.positions ? rope.positions[seq] : 0;
-  if (rope.positions && rope.slots && kbeg < ctx && kend == ctx) {
-    // This workgroup's partition ends with the step's own key.
-    const int slot = rope.slots[seq];
-    if (slot >= 0) {
-      const long long page = slot >> page_shift;
-      const int off = slot & page_mask;
-      const bf16_t* krow = q + (long long)seq * q_stride + rope.k_off + kvh * d;
-      const bf16_t* vrow = q + (long long)seq * q_stride + rope.v_off + kvh * d;
-      bf16_t* kdst = const_cast<bf16_t*>(k_pages) + (((page * nkv + kvh) << page_shift) + off) * d;
-      bf16_t* vdst = const_cast<bf16_t*>(v_pages) + (((page * nkv + kvh) * d) << page_shift) + off;
-      const int half = rope.rot / 2;
-      for (int i = tid; i < d; i += 64 * kDecodeWaves) {
-        bf16_t kv = krow[i];
-        if (rope.cos && i < rope.rot) {
-          const int j = i < half ? i : i - half;
-          const float c = rope.cos[(long long)pos * half + j], s = rope.sin[(long long)pos * half + j];
-          const float x = bf16_to_f32(kv);
-          const float y = bf16_to_f32(i < half ? krow[i + half] : krow[i - half]);
-          kv = f32_to_bf16(i < half ? x * c - y * s : x * c + y * s);
-        }
-        kdst[i] = kv;
-        vdst[(long long)i << page_shift] = vrow[i];
-      }
-    }
-    __syncthreads();       // the stores are visible to the whole workgroup from here on
-  }
-
-  Frag8 qf[D / 32];
-#pragma unroll
-  for (int ks = 0; ks < D / 32; ++ks) {
-    const int dim = ks * 32 + lq * 8;
-    const bool ok = l16 < g && dim < d;
-    const uint4 v = *(const uint4*)(q + (long long)seq * q_stride + (ok ? (kvh * g + l16) * d + dim : 0));
-    qf[ks].u = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
-  }
-  if constexpr (D % 64 == 0) {
-    if (rope.positions && rope.cos) {         // the dispatcher has checked rot == d == D
-      constexpr int HS = D / 64;              // fragments between a dim and its partner
-      const float* cs = rope.cos + (long long)pos * (D / 2);
-      const float* sn = rope.sin + (long long)pos * (D / 2);
-#pragma unroll
-      for (int ks = 0; ks < HS; ++ks) {
-        float c[8], s[8];
-        load8f(cs + ks * 32 + lq * 8, c);
-        load8f(sn + ks * 32 + lq * 8, s);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float x1 = (float)qf[ks].v[e], x2 = (float)qf[ks + HS].v[e];
-          qf[ks].v[e] = (__bf16)(x1 * c[e] - x2 * s[e]);
-          qf[ks + HS].v[e] = (__bf16)(x2 * c[e] + x1 * s[e]);
-        }
-      }
-    }
-  }
-  float m_run = -INFINITY, l_run = 0.f;
-  f32x4 o_acc[D / 16];
-#pragma unroll
-  for (int db = 0; db < D / 16; ++db) o_acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  const float scale2 = scale * 1.4426950408889634f;
-
   // A wave takes its chunks two at a time: the page ids of both, then all their keys and
   // values, are on their way before the first product, and the page ids of the next two follow
   // at once.  The loads are unconditional, so that the compiler can count them: a key past the
@@ -634,7 +602,7 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
   // probability exactly zero; values past the end inside a group of 4 keys are whatever the
   // page holds, and the pages only ever hold zeros or values that a model wrote); a dim past d
   // reads one below d (it meets a zero of q, or a row of O^T that is not stored).
-  const int last_key = kend - 1, last_quad = (kend - 1) & ~3;
+  const int last_key = max(kend - 1, 0), last_quad = last_key & ~3;
   int k_dim[D / 32], v_dim[D / 16];
 #pragma unroll
   for (int ks = 0; ks < D / 32; ++ks) k_dim[ks] = min(ks * 32 + lq * 8, d - 8);
@@ -671,6 +639,73 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
           VF[db].h[hf] = *(const uint2*)(vp_ + ((unsigned)v_dim[db] << page_shift));            \
     }                                                                                           \
   }
+
+  // ---- second round trip: the page ids of this wave's first chunks and the rotation's
+  // angles, which need the context length and the position ------------------------------
+  int c0 = kbeg + wave * 32;
+  constexpr bool kPairs = D <= 128;      // wider heads have no registers for two chunks
+  const bool one_by_one = part <= kStride || !kPairs;
+  RLIS_DEC_PAGES(c0, pk_a, pv_a);
+  if constexpr (kPairs) {
+    if (!one_by_one) RLIS_DEC_PAGES(c0 + kStride, pk_b, pv_b);
+  }
+  constexpr int HS = D % 64 == 0 ? D / 64 : 1;     // fragments between a dim and its partner
+  const bool q_turns = D % 64 == 0 && rotates && rope.cos;   // the dispatcher: rot == d == D
+  float q_cos[HS][8], q_sin[HS][8];
+  if (q_turns) {
+    const float* cs = rope.cos + (long long)pos * (D / 2);
+    const float* sn = rope.sin + (long long)pos * (D / 2);
+#pragma unroll
+    for (int ks = 0; ks < HS; ++ks) {
+      load8f(cs + ks * 32 + lq * 8, q_cos[ks]);
+      load8f(sn + ks * 32 + lq * 8, q_sin[ks]);
+    }
+  }
+  float k_cos = 1.f, k_sin = 0.f;
+  if (k_turns) {
+    const int j = tid < half ? tid : tid - half;
+    k_cos = rope.cos[(long long)pos * half + j];
+    k_sin = rope.sin[(long long)pos * half + j];
+  }
+
+  // ---- the step's own key and value go to the pages before anyone reads them back --------
+  if (stores_kv && kbeg < ctx && kend == ctx) {
+    // This workgroup's partition ends with the step's own key.
+    if (slot >= 0 && kv_thread) {
+      const long long page = slot >> page_shift;
+      const int off = slot & page_mask;
+      bf16_t* kdst = const_cast<bf16_t*>(k_pages) + (((page * nkv + kvh) << page_shift) + off) * d;
+      bf16_t* vdst = const_cast<bf16_t*>(v_pages) + (((page * nkv + kvh) * d) << page_shift) + off;
+      bf16_t kv = new_k;
+      if (k_turns) {
+        const float x = bf16_to_f32(new_k), y = bf16_to_f32(new_partner);
+        kv = f32_to_bf16(tid < half ? x * k_cos - y * k_sin : x * k_cos + y * k_sin);
+      }
+      kdst[tid] = kv;
+      vdst[(long long)tid << page_shift] = new_v;
+    }
+    __syncthreads();       // the stores are visible to the whole workgroup from here on
+  }
+
+  if constexpr (D % 64 == 0) {
+    if (q_turns) {
+#pragma unroll
+      for (int ks = 0; ks < HS; ++ks) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float x1 = (float)qf[ks].v[e], x2 = (float)qf[ks + HS].v[e];
+          qf[ks].v[e] = (__bf16)(x1 * q_cos[ks][e] - x2 * q_sin[ks][e]);
+          qf[ks + HS].v[e] = (__bf16)(x2 * q_cos[ks][e] + x1 * q_sin[ks][e]);
+        }
+      }
+    }
+  }
+  float m_run = -INFINITY, l_run = 0.f;
+  f32x4 o_acc[D / 16];
+#pragma unroll
+  for (int db = 0; db < D / 16; ++db) o_acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  const float scale2 = scale * 1.4426950408889634f;
+
   auto compute = [&](int c0, const Frag8 (&kf)[2][D / 32], const Frag8 (&vf)[D / 16])
                      __attribute__((always_inline)) {
     f32x4 s[2];
@@ -715,20 +750,14 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
     }
   };
 
-  int c0 = kbeg + wave * 32;
-  constexpr bool kPairs = D <= 128;      // wider heads have no registers for two chunks
-  if (part <= kStride || !kPairs) {
+  if (one_by_one) {
     // One chunk at a time: at most one for every wave of the workgroup, or a wide head.
     for (; c0 < kend; c0 += kStride) {
-      RLIS_DEC_PAGES(c0, pk_a, pv_a);
       RLIS_DEC_CHUNK(c0, pk_a, pv_a, k_a, v_a);
+      RLIS_DEC_PAGES(c0 + kStride, pk_a, pv_a);
       compute(c0, k_a, v_a);
     }
   } else if constexpr (kPairs) {
-    if (c0 < kend) {
-      RLIS_DEC_PAGES(c0, pk_a, pv_a);
-      RLIS_DEC_PAGES(c0 + kStride, pk_b, pv_b);
-    }
     for (; c0 < kend; c0 += 2 * kStride) {
       RLIS_DEC_CHUNK(c0, pk_a, pv_a, k_a, v_a);
       RLIS_DEC_CHUNK(c0 + kStride, pk_b, pv_b, k_b, v_b);
