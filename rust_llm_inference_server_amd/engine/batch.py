@@ -173,7 +173,8 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
         raise ValueError("a step needs at least one request")
     # what the planners add is not known before the lengths are; their arrays go behind the
     # common ones, into room asked for up front (a second buffer when a plan outgrows it)
-    spare = 64 + 16 * len(entries) * max(1, len(planners))
+    spare = 256 + (16 * len(entries) + sum(len(e.tokens) for e in entries) // 4) \
+        * max(1, len(planners))
     host, used, layout, info = _common_native(entries, cache, vocab_size, spare)
     T, S, R, num_single, max_context, max_new, widths, order = info
     ps = cache.page_size
