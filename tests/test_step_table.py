@@ -98,10 +98,23 @@ def test_the_runtimes_step_layout_is_the_python_twins():
     from rust_llm_inference_server_amd.cache.manager import CacheManager, GroupSpec
     from rust_llm_inference_server_amd.engine import StepEntry, build_step
     from rust_llm_inference_server_amd.ops.attention_plan import AttentionPlanner
+    from rust_llm_inference_server_amd.stepplan import HostPlan, StepPlanner
+
+    class Wordy(StepPlanner):
+        """A planner whose arrays outgrow the room the builder keeps for plans."""
+
+        def key(self):
+            return "wordy"
+
+        def plan(self, lengths):
+            n = int(lengths.new.sum())
+            return HostPlan({"many": np.arange(5000 + n, dtype=np.int32),
+                             "few": np.asarray(lengths.start, dtype=np.int32)}, {"n": n})
+
     rng = np.random.default_rng(7)
     cache = CacheManager(8, [GroupSpec(400, None), GroupSpec(400, 24)], num_state_slots=16)
     cpu = torch.device("cpu")
-    planners = [AttentionPlanner(4, 2, 16)]
+    planners = [AttentionPlanner(4, 2, 16), Wordy()]
     lengths = {}
     for trial in range(40):
         live = list(lengths)
