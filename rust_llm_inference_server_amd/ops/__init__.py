@@ -54,8 +54,8 @@ DECODE_ATTENTION = "matrix"
 # keys and values under the grid (partitions x partition length x 2 x head size x 2 bytes: an
 # upper bound, since a captured step's grid is as deep as its context bucket's longest context
 # needs and most sequences are shorter; 64 requests of the 3B shape with contexts up to 2,300,
-# 1.07 GB by this count, gain 3 % of their step inside, 32 requests of the 8B shape at 8,300,
-# 1.2 GB, lose 0.7 %).
+# 1.07 GB by this count, gain 3 % of their step inside; 32 requests of the 8B shape at 8,300,
+# 1.125 GB, take the same time either way).
 MERGE_DECODE_INSIDE = True
 MERGE_DECODE_INSIDE_MAX_BYTES = 9 << 27        # 1.125 GB
 
