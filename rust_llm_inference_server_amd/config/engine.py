@@ -21,6 +21,9 @@ class EngineConfig:
     # (engine.rs:263-271: max(1, num_blocks / 100)); None means that rule.
     watermark_pages: Optional[int] = None
     use_graphs: bool = True
+    # Decode steps are launched one ahead of the tokens that the host has seen, where the next
+    # step does not depend on them (False: every step waits for the one before).
+    launch_ahead: bool = True
 
     def validate(self) -> None:
         if self.max_num_seqs <= 0:

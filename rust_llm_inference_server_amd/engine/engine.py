@@ -15,7 +15,7 @@ from __future__ import annotations
 
 import time
 from dataclasses import dataclass
-from typing import Dict, Iterable, List, Optional, Sequence, Tuple, Union
+from typing import Callable, Dict, Iterable, List, Optional, Sequence, Tuple, Union
 
 import torch
 
@@ -61,6 +61,15 @@ class EngineStats:
     waiting: int = 0
     pages_used: int = 0
     pages_total: int = 0
+
+
+@dataclass
+class _Flight:
+    """A launched step of one token per request whose tokens the host has not taken yet."""
+    ids: List[int]                     # the requests, in the order of the step's rows
+    wait: Callable[[], List[int]]      # waits for the step, returns their tokens
+    side: int                          # which of the runner's two host buffers it used
+    appended: bool = False             # the scheduler has been told of its tokens already
 
 
 class _Sequence:
@@ -118,6 +127,7 @@ class Engine:
         self.eos_token_ids = set(int(t) for t in eos_token_ids)
         self._seqs: Dict[int, _Sequence] = {}
         self._finished: Dict[int, Completion] = {}
+        self._flight: Optional[_Flight] = None
         self._next_id = 0
         self.stats_ = EngineStats(pages_total=num_pages)
 
@@ -156,7 +166,30 @@ class Engine:
         """One scheduled batch.  Returns ``(request id, token or None, finished)`` for every
         request that produced a token (``None`` with ``finished``: it stopped at an EOS).
         If the model step raises, the requests of that batch finish with reason ``error``
-        and the exception goes on to the caller; requests outside the batch are untouched."""
+        and the exception goes on to the caller; requests outside the batch are untouched.
+
+        Decoding runs one step ahead where it can: when every request of a step brings one
+        token and will bring one more whatever it samples (no request waits for admission,
+        none reaches its ``max_tokens``, pages are at hand), the next step is launched on the
+        tokens as they lie on the device before the host has seen them, and this call returns
+        the tokens of the step before.  A request that stops at an EOS meanwhile has computed
+        one position in vain; its row of the step in flight is dropped."""
+        while True:
+            if self._flight is None:
+                out = self._start_step()
+                if self._flight is None:
+                    return out
+            flight, self._flight = self._flight, None
+            ahead = self._launch_ahead(flight) if self.config.launch_ahead else None
+            out = self._take(flight)
+            self._flight = ahead
+            if out or not self.scheduler.has_work():
+                return out
+            # every request of that step had gone already: on to the next one
+
+    def _start_step(self) -> List[Tuple[int, Optional[int], bool]]:
+        """Schedule a batch and run it.  A step of single tokens that the device samples is
+        only launched (``self._flight`` holds it then); any other is finished here."""
         sched = self.scheduler.schedule()
         self.stats_.preemptions = self.scheduler.num_preemptions
         if not sched.seqs:
@@ -167,8 +200,8 @@ class Engine:
                 raise RuntimeError("scheduler made no progress")
             return []
         # A step in which every request brings one token and the device kernel can sample for
-        # all of them runs as one captured graph, sampling included; the book-keeping below goes
-        # on while it runs, and only then are the tokens waited for.
+        # all of them runs as one captured graph, sampling included; the book-keeping goes on
+        # while it runs, and only then are the tokens waited for.
         wait = None
         singles = self._single_tokens(sched)
         try:
@@ -184,15 +217,19 @@ class Engine:
                                              [end - start - 1] if last else []))
                     final.append(last)
                 logits = self.runner.step(entries)
-            else:
-                final = [True] * len(sched.seqs)
         except Exception as exc:
             # engine.rs:523-528: a failed step fails its own requests and no others; their
             # pages are free again and the engine goes on with the rest.
-            for seq_id, _, _ in sched.seqs:
-                self._finish(self._seqs[seq_id], "error", error=f"{type(exc).__name__}: {exc}")
+            self._fail([seq_id for seq_id, _, _ in sched.seqs], exc)
             raise
         self.stats_.steps += 1
+        if wait is not None:
+            for seq_id, start, end in sched.seqs:
+                self.scheduler.advance(seq_id, end)
+                # (a prompt's last token, or a recomputed one, may come alone)
+                self.stats_.prefill_tokens += max(0, min(end, self._seqs[seq_id].prompt_len) - start)
+            self._flight = _Flight(singles[0], wait, side=0)
+            return []
         # Rows that yield a token, split between the device kernel and the host sampler.
         device_rows, device_modes, host_rows = [], [], []
         row = 0
@@ -201,7 +238,7 @@ class Engine:
             seq = self._seqs[seq_id]
             # prompt tokens of this portion (recomputed ones after a preemption count again)
             self.stats_.prefill_tokens += max(0, min(end, seq.prompt_len) - start)
-            if not last or wait is not None:
+            if not last:
                 continue
             mode = seq.sampler.device_mode(len(seq.tokens))
             if mode is not None:
@@ -211,13 +248,6 @@ class Engine:
                 host_rows.append((row, seq_id))
             row += 1
         picked: Dict[int, int] = {}
-        if wait is not None:
-            try:
-                picked = dict(zip(singles[0], wait()))
-            except Exception as exc:
-                for seq_id, _, _ in sched.seqs:
-                    self._finish(self._seqs[seq_id], "error", error=f"{type(exc).__name__}: {exc}")
-                raise
         if device_rows:
             idx = [r for r, _ in device_rows]
             sub = logits if len(idx) == logits.shape[0] else logits[
@@ -236,10 +266,76 @@ class Engine:
             if last:
                 out.append(self._accept(self._seqs[seq_id], picked[seq_id], now, grown))
         self.scheduler.append_tokens(grown)
+        self._note_stats()
+        return out
+
+    def _launch_ahead(self, flight: _Flight) -> Optional[_Flight]:
+        """Launch the step that follows ``flight`` before its tokens are known, if that step
+        is the same requests with one more token each whatever the tokens are; else None, and
+        nothing has changed."""
+        ids, seqs = flight.ids, self._seqs
+        sch = self.scheduler
+        if sch.num_waiting or sch.num_running != len(ids):
+            return None
+        modes = []
+        for seq_id in ids:
+            seq = seqs.get(seq_id)
+            # gone (stopped or cancelled while in flight), or the token in flight is its last
+            if seq is None or seq.output_len + 1 >= seq.params.max_tokens:
+                return None
+            mode = seq.sampler.device_mode(len(seq.tokens) + 1)
+            if mode is None:
+                return None
+            modes.append(mode)
+        cache = self.runner.cache
+        if any(cache.num_free_pages(g) < len(ids) for g in range(cache.num_groups)):
+            return None                      # the scheduler might have to preempt
+        sch.append_tokens(ids)
+        flight.appended = True
+        sched = sch.schedule()
+        if sched.copies or sched.preempted or [s for s, _, _ in sched.seqs] != ids \
+                or any(end - start != 1 for _, start, end in sched.seqs):
+            raise RuntimeError("the schedule of a step launched ahead is not the step before "
+                               "it with one more token each")
+        try:
+            wait = self.runner.step_chained(ids, modes, 1 - flight.side)
+        except Exception as exc:
+            self._fail(ids, exc)
+            raise
+        self.stats_.steps += 1
+        for seq_id, _, end in sched.seqs:
+            sch.advance(seq_id, end)
+        return _Flight(ids, wait, side=1 - flight.side)
+
+    def _take(self, flight: _Flight) -> List[Tuple[int, Optional[int], bool]]:
+        """Wait for a launched step and take its tokens; rows of requests that have gone
+        meanwhile are dropped."""
+        try:
+            tokens = flight.wait()
+        except Exception as exc:
+            self._fail(flight.ids, exc)
+            raise
+        out, grown = [], []
+        now = time.perf_counter()
+        for seq_id, token in zip(flight.ids, tokens):
+            seq = self._seqs.get(seq_id)
+            if seq is not None:
+                out.append(self._accept(seq, token, now, grown))
+        if not flight.appended:
+            self.scheduler.append_tokens(grown)
+        self._note_stats()
+        return out
+
+    def _fail(self, seq_ids: Sequence[int], exc: Exception) -> None:
+        for seq_id in seq_ids:
+            seq = self._seqs.get(seq_id)
+            if seq is not None:
+                self._finish(seq, "error", error=f"{type(exc).__name__}: {exc}")
+
+    def _note_stats(self) -> None:
         self.stats_.running = self.scheduler.num_running
         self.stats_.waiting = self.scheduler.num_waiting
         self.stats_.pages_used = self.stats_.pages_total - self.runner.cache.num_free_pages(0)
-        return out
 
     def _single_tokens(self, sched) -> Optional[Tuple[List[int], List[int], List[Tuple[int, float]]]]:
         """(request ids, their tokens, their (key, 1/T)) when every request of the schedule brings

@@ -6,8 +6,12 @@ per batch-size bucket into a HIP graph and replayed: the step's metadata lives i
 int32 buffer (filled on the host by the native page manager; the graph begins with its copy to
 the device), the kernels read it through fixed views, and the logits land in a static tensor.
 A second kind of graph goes on where the first ends: the sampling kernel on those logits (keys
-and temperatures travel with the metadata) and the copy of the tokens to pinned host memory,
-so that between two decode steps the host launches one graph and waits for one event.
+and temperatures travel with the metadata), which leaves the tokens where the next step's ids
+are.  Its launch copies the metadata to the device in front of it and the tokens to pinned
+host memory behind it, so that between two decode steps the host waits for one event; and a
+step of the same requests can be launched while the one before it still runs, on the tokens
+as they lie on the device: it brings everything but the ids from the host.  The host side of
+the metadata exists twice for that, the two taking turns.
 
 Unused rows of a bucket are padding requests of context 1 that read and write a scratch page
 beyond the manager's pages and a scratch state slot beyond its slots, so they touch nothing a
@@ -66,6 +70,32 @@ def context_bucket(context: int, limit: int) -> int:
     return min(b, limit)
 
 
+LOGITS, SAMPLED = "logits", "sampled"
+
+
+class _HostSide:
+    """One host copy of a bucket's metadata, pinned, with its views and the addresses that the
+    native page manager fills; where a sampling step leaves its tokens for the host, and the
+    event after the last step that was prepared here."""
+
+    def __init__(self, meta: MetadataBuffer, B: int, num_groups: int):
+        self.host = torch.zeros(meta.size, dtype=torch.int32).pin_memory()
+        self.np = self.host.numpy()
+        self.h = {name: meta.view(self.np, name) for name in meta.offsets}
+        self.h["seq_of_token"][:] = np.arange(B)
+        self.h["cu"][:] = np.arange(B + 1)
+        self.h["logit_rows"][:] = np.arange(B)
+        base = self.host.data_ptr()
+        ptr = lambda name: base + 4 * meta.offsets[name][0]
+        self.ptr_positions, self.ptr_slots = ptr("positions"), ptr("state_slots")
+        self.ptr_tables = (ctypes.c_void_p * num_groups)(
+            *[ptr(f"tables{g}") for g in range(num_groups)])
+        self.ptr_wslots = (ctypes.c_void_p * num_groups)(
+            *[ptr(f"slots{g}") for g in range(num_groups)])
+        self.tokens_host = torch.zeros(B, dtype=torch.int32).pin_memory()
+        self.done: Optional[torch.cuda.Event] = None
+
+
 class DecodeGraph:
     """The captured decode steps of one batch-size bucket: one static metadata buffer, and one
     HIP graph per context bucket."""
@@ -92,19 +122,12 @@ class DecodeGraph:
         # that sample inside the graph
         meta.reserve("sample_keys", B)
         meta.reserve("sample_inv_t", B)
-        self.host = torch.zeros(meta.size, dtype=torch.int32).pin_memory()
-        self.np = self.host.numpy()
+        # Two host sides take turns: a step is prepared in one while the step before it, which
+        # was prepared in the other, may not have read its metadata yet.
+        self.sides = [_HostSide(meta, B, ng), _HostSide(meta, B, ng)]
+        self.h = self.sides[0].h
         self.dev = torch.zeros(meta.size, dtype=torch.int32, device=dev)
         self.seq_ids = np.zeros(B, dtype=np.int64)
-        self.h = {name: meta.view(self.np, name) for name in meta.offsets}
-        self.h["seq_of_token"][:] = np.arange(B)
-        self.h["cu"][:] = np.arange(B + 1)
-        self.h["logit_rows"][:] = np.arange(B)
-        base = self.host.data_ptr()
-        ptr = lambda name: base + 4 * meta.offsets[name][0]
-        self.ptr_positions, self.ptr_slots = ptr("positions"), ptr("state_slots")
-        self.ptr_tables = (ctypes.c_void_p * ng)(*[ptr(f"tables{g}") for g in range(ng)])
-        self.ptr_wslots = (ctypes.c_void_p * ng)(*[ptr(f"slots{g}") for g in range(ng)])
         self.scratch_page = runner.pools.scratch_page
         self.scratch_state_slot = runner.pools.scratch_state_slot
         dview = lambda name: meta.view(self.dev, name)
@@ -112,11 +135,10 @@ class DecodeGraph:
                                  block_tables=dview(f"tables{g}").reshape(B, W),
                                  slots=dview(f"slots{g}")) for g in range(ng)]
         self.views = {name: dview(name) for name in meta.offsets}
-        # (context bucket, sampled) -> (graph, its static logits or sampled tokens)
-        self.graphs: Dict[Tuple[int, bool], Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
-        # where a sampling graph leaves its tokens for the host
-        self.tokens_host = torch.zeros(B, dtype=torch.int32).pin_memory()
-        self._done: Optional[torch.cuda.Event] = None
+        # (context bucket, LOGITS or SAMPLED) -> (graph, its static logits or sampled tokens)
+        self.graphs: Dict[Tuple[int, str], Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
+        # what of the metadata a chained step brings from the host: everything behind the ids
+        self.behind_ids = meta.offsets["positions"][0]
 
     def step_for(self, context_limit: int) -> StepContext:
         """The step as the kernels of a captured run see it: static views, and each planner's
@@ -147,72 +169,94 @@ class DecodeGraph:
             h["ids"][S:] = 0
             h["positions"][S:] = 0
             h["state_slots"][S:] = self.scratch_state_slot
-            for g in range(len(self.ptr_tables)):
+            for g in range(len(self.groups)):
                 h[f"tables{g}"].reshape(B, W)[S:, 0] = self.scratch_page
                 h[f"slots{g}"][S:] = self.scratch_page * self.runner.cache.page_size
         h["start_pos"][:] = h["positions"]
         h["ctx_lens"][:] = h["positions"] + 1
 
-    def prepare(self, seq_ids: Sequence[int], tokens: Sequence[int],
-                modes: Optional[Sequence[Tuple[int, float]]] = None) -> np.ndarray:
-        """Fill the host side of the metadata for one token per request (``modes``: each row's
-        (key, 1/T) for a step that samples inside the graph); returns the new tokens'
-        positions.  Nothing is launched yet."""
-        if self._done is not None:
-            self._done.synchronize()         # the last replay has read the host buffer
+    def prepare(self, seq_ids: Sequence[int], tokens: Optional[Sequence[int]],
+                modes: Optional[Sequence[Tuple[int, float]]] = None, side: int = 0) -> np.ndarray:
+        """Fill host side ``side`` of the metadata for one token per request (``modes``: each
+        row's (key, 1/T) for a step that samples inside the graph; ``tokens`` None: a chained
+        step, whose ids are on the device already); returns the new tokens' positions.  Nothing
+        is launched yet."""
+        hs = self.sides[side]
+        if hs.done is not None:
+            hs.done.synchronize()            # the last step prepared here has read this side
+        h = hs.h
         S = len(seq_ids)
         self.seq_ids[:S] = seq_ids
-        self.h["ids"][:S] = tokens
+        if tokens is not None:
+            h["ids"][:S] = tokens
         if modes is not None:
-            self.h["sample_keys"][:S] = np.asarray([k for k, _ in modes], dtype=np.uint32).view(np.int32)
-            self.h["sample_inv_t"][:S] = np.asarray([t for _, t in modes],
-                                                    dtype=np.float32).view(np.int32)
-            self.h["sample_keys"][S:] = 0
-            self.h["sample_inv_t"][S:] = 0
+            h["sample_keys"][:S] = np.asarray([k for k, _ in modes], dtype=np.uint32).view(np.int32)
+            h["sample_inv_t"][:S] = np.asarray([t for _, t in modes],
+                                               dtype=np.float32).view(np.int32)
+            h["sample_keys"][S:] = 0
+            h["sample_inv_t"][S:] = 0
         self.runner.cache.decode_batch(self.seq_ids.ctypes.data, S, self.width,
-                                       self.ptr_positions, self.ptr_slots, self.ptr_tables,
-                                       self.ptr_wslots)
-        self._pad_from(S)
-        return self.h["positions"][:S]
+                                       hs.ptr_positions, hs.ptr_slots, hs.ptr_tables,
+                                       hs.ptr_wslots)
+        self._pad_from(S, h)
+        return h["positions"][:S]
 
     def launch(self, num_seqs: int, context_limit: int) -> torch.Tensor:
-        """Run the prepared step.  Logits ``(num_seqs, vocab)``: a view of a static tensor that
-        the next call for the same context bucket overwrites."""
-        return self._replay(context_limit, False)[:num_seqs]
+        """Run the step prepared in side 0.  Logits ``(num_seqs, vocab)``: a view of a static
+        tensor that the next call for the same context bucket overwrites."""
+        graph, result = self._graph(context_limit, LOGITS)
+        graph.replay()          # begins with the copy of side 0 of the metadata to the device
+        hs = self.sides[0]
+        if hs.done is None:
+            hs.done = torch.cuda.Event()
+        hs.done.record()
+        return result[:num_seqs]
 
-    def launch_sampled(self, num_seqs: int, context_limit: int):
-        """Run the prepared step with the sampling inside.  Returns a function that waits for
-        the step and returns the requests' tokens."""
-        self._replay(context_limit, True)
-        done, tokens = self._done, self.tokens_host
+    def launch_sampled(self, num_seqs: int, context_limit: int, side: int = 0,
+                       chained: bool = False):
+        """Run the step prepared in ``side`` with the sampling inside; returns a function that
+        waits for the step and returns the requests' tokens.  ``chained``: the step's ids are
+        the tokens that the sampling of the step before it (the same requests in the same
+        rows) left on the device; that step may still be running."""
+        graph, _ = self._graph(context_limit, SAMPLED)        # (a capture runs a step of padding)
+        hs = self.sides[side]
+        lo = self.behind_ids if chained else 0
+        self.dev[lo:].copy_(hs.host[lo:], non_blocking=True)
+        graph.replay()
+        hs.tokens_host.copy_(self.views["ids"], non_blocking=True)
+        if hs.done is None:
+            hs.done = torch.cuda.Event()
+        hs.done.record()
+        done, tokens = hs.done, hs.tokens_host
 
         def wait() -> list:
             done.synchronize()
             return tokens[:num_seqs].tolist()
         return wait
 
-    def _replay(self, context_limit: int, sampled: bool) -> torch.Tensor:
-        key = (context_limit, sampled)
+    def _graph(self, context_limit: int, kind: str):
+        key = (context_limit, kind)
         if key not in self.graphs:
-            self._capture(context_limit, sampled)
-        graph, result = self.graphs[key]
-        graph.replay()          # begins with the copy of the metadata to the device
-        if self._done is None:
-            self._done = torch.cuda.Event()
-        self._done.record()
-        return result
+            self._capture(context_limit, kind)
+        return self.graphs[key]
 
-    def _capture(self, context_limit: int, sampled: bool) -> None:
-        """Capture the step: the copy of the host's metadata to the device, the model, and with
-        ``sampled`` the sampling kernel and the copy of its tokens to the host.  The warm-up
-        run works on metadata that is all padding: what it computes lands on the scratch page
-        and the scratch state slot, so that no request's cache or state moves before the first
-        replay (the capture itself runs nothing)."""
+    def _capture(self, context_limit: int, kind: str) -> None:
+        """Capture the step.  LOGITS: the copy of side 0 of the host's metadata to the device
+        and the model.  SAMPLED: the model and the sampling kernel, which leaves its tokens
+        where the next step's ids are; its launch copies the metadata to the device and the
+        tokens to the host, from and to whichever side it names.  The warm-up run works on
+        metadata that is all padding: what it computes lands on the scratch page and the
+        scratch state slot, so that no request's cache or state moves before the first replay
+        (the capture itself runs nothing); the ids on the device, which a chained step is
+        about to read, are put back after it."""
         from .. import ops
         runner = self.runner
-        padding = self.host.clone()
+        host = self.sides[0].host
+        padding = host.clone()
         flat = padding.numpy()
         self._pad_from(0, {name: self.meta.view(flat, name) for name in self.meta.offsets})
+        ids = self.views["ids"]
+        kept = ids.clone()
         self.dev.copy_(padding)
         step = self.step_for(context_limit)
         keys = self.views["sample_keys"]
@@ -220,7 +264,7 @@ class DecodeGraph:
 
         def run():
             logits = runner.model.forward(step, runner.pools)
-            return ops.sample_rows(logits, keys, inv_t) if sampled else logits
+            return logits if kind == LOGITS else ops.sample_rows(logits, keys, inv_t, out=ids)
 
         # One eager run first: it settles lazy initialisation (library loading, workspace
         # allocations) that must not happen under capture.
@@ -232,8 +276,8 @@ class DecodeGraph:
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with no_collection(), torch.cuda.graph(graph):
-            self.dev.copy_(self.host, non_blocking=True)
+            if kind == LOGITS:
+                self.dev.copy_(host, non_blocking=True)
             result = run()
-            if sampled:
-                self.tokens_host.copy_(result, non_blocking=True)
-        self.graphs[(context_limit, sampled)] = (graph, result)
+        ids.copy_(kept)
+        self.graphs[(context_limit, kind)] = (graph, result)

@@ -173,6 +173,18 @@ class ModelRunner:
             return None
         return self._decode_lists(seq_ids, tokens, modes)
 
+    def step_chained(self, seq_ids: Sequence[int], modes: Sequence[Tuple[int, float]],
+                     side: int) -> Callable[[], List[int]]:
+        """The step that follows a ``step_sampled`` or ``step_chained`` of the same requests in
+        the same order, launched while that step may still be running: every request brings
+        the token that step samples for it, which is on the device and nowhere else yet.
+        ``side`` (0 or 1) names the host buffers that the step uses; a step takes the side that
+        the step before it did not (``step_sampled`` takes side 0).  Positions must be reserved
+        as for any step.  Returns the function that waits for this step's tokens."""
+        if not self.use_graphs:
+            raise ValueError("chained steps need captured steps")
+        return self._decode_lists(seq_ids, None, modes, side)
+
     def _decode_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """A step of one token per request, replayed from the HIP graph of its batch-size
         bucket (captured at first use).  Same kernels, same results as the eager step."""
@@ -191,21 +203,25 @@ class ModelRunner:
             return logits[:0]
         return logits[torch.tensor(rows, device=logits.device)]
 
-    def _decode_lists(self, seq_ids: Sequence[int], tokens: Sequence[int],
-                      modes: Optional[Sequence[Tuple[int, float]]]):
+    def _decode_lists(self, seq_ids: Sequence[int], tokens: Optional[Sequence[int]],
+                      modes: Optional[Sequence[Tuple[int, float]]], side: int = 0):
         """The captured step for requests ``seq_ids`` bringing ``tokens``: the logits of all of
-        them, or with ``modes`` (the graph samples too) the function that waits for the tokens."""
+        them, or with ``modes`` (the graph samples too) the function that waits for the tokens.
+        ``tokens`` None: the chained step, on the tokens that the step before left on the
+        device."""
         from .graph import DecodeGraph, bucket_for, context_bucket
         S = len(seq_ids)
         if len(set(seq_ids)) != S:
             raise ValueError("a request appears twice in one step")
-        if min(tokens) < 0 or max(tokens) >= self.vocab_size:
+        if tokens is not None and (min(tokens) < 0 or max(tokens) >= self.vocab_size):
             raise ValueError(f"a token id is outside the vocabulary of {self.vocab_size}")
         bucket = bucket_for(S, self.max_num_seqs)
         graph = self._graphs.get(bucket)
         if graph is None:
+            if tokens is None:
+                raise ValueError("a chained step follows a captured step of the same requests")
             graph = self._graphs[bucket] = DecodeGraph(self, bucket)
-        positions = graph.prepare(seq_ids, tokens, modes)
+        positions = graph.prepare(seq_ids, tokens, modes, side)
         # Everything that can refuse the step is checked before anything is launched.
         longest = int(positions.max()) + 1
         if longest > self.model.max_positions:
@@ -213,11 +229,14 @@ class ModelRunner:
                              f"{self.model.max_positions}")
         if self.pools.state is not None:
             # a request whose first token this is starts from cleared state
-            self.pools.zero_states([int(graph.h["state_slots"][i]) for i in range(S)
-                                    if positions[i] == 0])
+            slots = graph.sides[side].h["state_slots"]
+            self.pools.zero_states([int(slots[i]) for i in range(S) if positions[i] == 0])
         ends = (positions + 1).tolist()
         limit = context_bucket(longest, self.model.max_positions)
-        result = graph.launch_sampled(S, limit) if modes is not None else graph.launch(S, limit)
+        if modes is not None:
+            result = graph.launch_sampled(S, limit, side, chained=tokens is None)
+        else:
+            result = graph.launch(S, limit)
         for seq, end in zip(seq_ids, ends):
             self.cache.advance(seq, end)
         return result

@@ -633,15 +633,19 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
 
 
 # ------------------------------------------------------------------------ sampling
-def sample_rows(logits: torch.Tensor, keys: torch.Tensor, inv_temps: torch.Tensor
-                ) -> torch.Tensor:
+def sample_rows(logits: torch.Tensor, keys: torch.Tensor, inv_temps: torch.Tensor,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One token per row of float32 ``logits (R, V)``: argmax where ``inv_temps`` is 0, else
-    Gumbel-max with noise keyed by ``keys`` (int32 bit patterns of the 32-bit row keys)."""
+    Gumbel-max with noise keyed by ``keys`` (int32 bit patterns of the 32-bit row keys).  The
+    tokens go to ``out`` (int32, ``R`` elements) when it is given."""
     stride = _rows_contig(logits, "logits")
     _check(logits, "logits", torch.float32)
     R, V = logits.shape
     _check(inv_temps, "inv_temps", torch.float32)
-    out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    if out is None:
+        out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    else:
+        _i32(out, "sampled tokens", R)
     # A large vocabulary is scanned in chunks by many workgroups and a second small kernel
     # picks among the chunks' winners; the result is the same token.
     chunks = min(64, max(1, V // 1024))

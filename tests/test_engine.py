@@ -166,8 +166,9 @@ def test_steps_that_sample_inside_the_graph_pick_the_eager_steps_tokens(backend,
         assert engine.runner.use_graphs == graphs
         sampled_steps = []
         if graphs:
-            real = engine.runner.step_sampled
+            real, chained = engine.runner.step_sampled, engine.runner.step_chained
             engine.runner.step_sampled = lambda i, t, m: sampled_steps.append(len(i)) or real(i, t, m)
+            engine.runner.step_chained = lambda i, m, s: sampled_steps.append(len(i)) or chained(i, m, s)
         runs[graphs] = [o.token_ids for o in engine.generate(prompts, params)]
         if graphs:
             assert len(sampled_steps) >= 10 and max(sampled_steps) == 5
@@ -179,6 +180,63 @@ def test_steps_that_sample_inside_the_graph_pick_the_eager_steps_tokens(backend,
         with_host[graphs] = [o.token_ids for o in engine.generate(prompts, mixed)]
     assert with_host[True] == with_host[False]
     assert with_host[True][:4] == runs[True][:4]
+
+
+def test_decode_steps_launched_ahead_give_the_same_completions(backend, dtype, folders):
+    """A decode step is launched on the tokens of the step before as they lie on the device,
+    before the host has seen them, wherever the next step does not depend on them.  The
+    completions are those of an engine that waits for every step: with requests that end at
+    different steps by their limit, requests that stop at an EOS (one position computed in
+    vain, its row dropped), a request added and one cancelled while steps are in flight, greedy
+    and with seeded temperature; and everything is given back at the end."""
+    if backend.type != "cuda":
+        pytest.skip("captured steps exist on the GPU only")
+    from rust_llm_inference_server_amd.engine import Engine
+    model = load(folders["b"], backend, dtype)
+    prompts = prompts_for(384, [3, 17, 40, 9, 1, 22], seed=18)
+    params = [SamplingParams.greedy(30), SamplingParams(temperature=0.7, seed=5, max_tokens=19),
+              SamplingParams(temperature=1.1, seed=6, max_tokens=30), SamplingParams.greedy(2),
+              SamplingParams(temperature=0.9, seed=7, max_tokens=25), SamplingParams.greedy(12)]
+
+    def run(ahead, eos=()):
+        cfg = EngineConfig(max_num_seqs=8, max_batched_tokens=32, num_pages=64, block_size=8,
+                           max_seq_len=256, watermark_pages=1, launch_ahead=ahead)
+        engine = Engine(model, cfg, eos_token_ids=eos)
+        chained = []
+        real = engine.runner.step_chained
+        engine.runner.step_chained = lambda i, m, s: chained.append(len(i)) or real(i, m, s)
+        ids = [engine.add_request(p, sp) for p, sp in zip(prompts[:4], params[:4])]
+        streamed = {}
+        calls = 0
+        while engine.has_work():
+            for seq_id, token, finished in engine.step():
+                if token is not None:
+                    streamed.setdefault(seq_id, []).append(token)
+            calls += 1
+            if calls == 6:                 # decoding is under way: one more request, one fewer
+                ids.append(engine.add_request(prompts[4], params[4]))
+                engine.cancel(ids[2])
+            if calls == 9:
+                ids.append(engine.add_request(prompts[5], params[5]))
+        done = {i: engine.pop_finished(i) for i in ids if i != ids[2]}
+        assert all(c is not None for c in done.values())
+        for i, c in done.items():
+            assert streamed.get(i, []) == c.token_ids
+        assert engine.runner.cache.num_free_pages() == 64
+        engine.runner.cache.check_invariants()
+        engine.scheduler.check()
+        return [(c.token_ids, c.finish_reason) for c in done.values()], chained
+
+    waited, none = run(False)
+    ahead, chained = run(True)
+    assert not none and len(chained) >= 12 and max(chained) >= 3
+    assert ahead == waited
+    # tokens that the runs above produced in the middle of a completion now end their requests
+    eos = {waited[0][0][7], waited[1][0][4], waited[3][0][9]}
+    stopped, _ = run(False, eos)
+    assert [r for _, r in stopped].count("stop") >= 3
+    ahead_stopped, chained = run(True, eos)
+    assert ahead_stopped == stopped and len(chained) >= 5
 
 
 def test_host_sampler_modes_run_and_are_reproducible(backend, tiny_folders):
