@@ -169,8 +169,8 @@ class Engine:
         and the exception goes on to the caller; requests outside the batch are untouched.
 
         Decoding runs one step ahead where it can: when every request of a step brings one
-        token and will bring one more whatever it samples (no request waits for admission,
-        none reaches its ``max_tokens``, pages are at hand), the next step is launched on the
+        token and will bring one more whatever it samples (no request can be admitted, none
+        reaches its ``max_tokens``, pages are at hand), the next step is launched on the
         tokens as they lie on the device before the host has seen them, and this call returns
         the tokens of the step before.  A request that stops at an EOS meanwhile has computed
         one position in vain; its row of the step in flight is dropped."""
@@ -275,8 +275,11 @@ class Engine:
         nothing has changed."""
         ids, seqs = flight.ids, self._seqs
         sch = self.scheduler
-        if sch.num_waiting or sch.num_running != len(ids):
+        if sch.num_running != len(ids):
             return None
+        if sch.num_waiting and len(ids) < self.config.max_num_seqs \
+                and self.config.scheduler != "static":
+            return None                      # the next step may admit a request
         modes = []
         for seq_id in ids:
             seq = seqs.get(seq_id)
