@@ -161,6 +161,13 @@ class Engine:
     def has_work(self) -> bool:
         return self.scheduler.has_work()
 
+    def warm_up(self) -> int:
+        """Capture the decode steps of every batch size and context that this engine can see
+        (they are captured at first use otherwise, some tens of milliseconds each, inside the
+        step that needs them); returns how many were captured.  The reference has no such
+        call: it has no captured steps."""
+        return self.runner.capture_decode_steps(self.max_seq_len)
+
     # --------------------------------------------------------------------- step
     def step(self) -> List[Tuple[int, Optional[int], bool]]:
         """One scheduled batch.  Returns ``(request id, token or None, finished)`` for every

@@ -185,6 +185,46 @@ class ModelRunner:
             raise ValueError("chained steps need captured steps")
         return self._decode_lists(seq_ids, None, modes, side)
 
+    def capture_decode_steps(self, longest: Optional[int] = None, sampled: bool = True,
+                             max_batch: Optional[int] = None) -> int:
+        """Capture now what decode steps would capture at first use: the step of every batch
+        bucket up to ``max_batch`` requests (``max_num_seqs`` by default) for every context
+        bucket up to ``longest`` positions (the model's limit by default); with ``sampled`` the
+        steps that sample inside, else those that return logits.  The captures run on padding
+        and move no request's cache or state.  Returns how many graphs were captured (0
+        without captured steps)."""
+        if not self.use_graphs:
+            return 0
+        from .graph import LOGITS, SAMPLED, DecodeGraph, bucket_for, context_bucket
+        limit = self.model.max_positions
+        longest = limit if longest is None else max(1, min(longest, limit))
+        top = self.max_num_seqs if max_batch is None else max(1, min(max_batch, self.max_num_seqs))
+        buckets, n = [], 1
+        while True:
+            b = bucket_for(n, self.max_num_seqs)
+            buckets.append(b)
+            if b >= top:
+                break
+            n = b + 1
+        contexts, c = [], 1
+        while True:
+            cb = context_bucket(c, limit)
+            contexts.append(cb)
+            if cb >= longest:
+                break
+            c = cb + 1
+        made = 0
+        kind = SAMPLED if sampled else LOGITS
+        for b in buckets:
+            graph = self._graphs.get(b)
+            if graph is None:
+                graph = self._graphs[b] = DecodeGraph(self, b)
+            for cb in contexts:
+                if (cb, kind) not in graph.graphs:
+                    graph._capture(cb, kind)
+                    made += 1
+        return made
+
     def _decode_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """A step of one token per request, replayed from the HIP graph of its batch-size
         bucket (captured at first use).  Same kernels, same results as the eager step."""

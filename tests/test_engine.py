@@ -252,6 +252,45 @@ def test_decode_steps_launched_ahead_give_the_same_completions(backend, dtype, f
     assert ahead_stopped == stopped and len(chained) >= 5
 
 
+def test_warm_up_captures_the_decode_steps_and_moves_nothing(backend, dtype, folders):
+    """``Engine.warm_up`` captures the decode steps of every batch and context bucket on
+    padding: afterwards no step captures any more, and a warm-up in the middle of a generation
+    (with a step in flight) leaves every request's cache, state and tokens as they were."""
+    if backend.type != "cuda":
+        pytest.skip("captured steps exist on the GPU only")
+    from rust_llm_inference_server_amd.engine.graph import DecodeGraph
+    model = load(folders["a"], backend, dtype, max_positions=128)
+    prompts = prompts_for(256, [5, 17, 33], seed=21)
+    params = [SamplingParams.greedy(20), SamplingParams(temperature=0.8, seed=3, max_tokens=16),
+              SamplingParams.greedy(9)]
+    want = [o.token_ids for o in engine_for(model, max_seq_len=128).generate(prompts, params)]
+    captures = []
+    real = DecodeGraph._capture
+
+    def counted(self, context_limit, kind):
+        captures.append((self.bucket, context_limit, kind))
+        return real(self, context_limit, kind)
+    DecodeGraph._capture = counted
+    try:
+        engine = engine_for(model, max_seq_len=128)
+        made = engine.warm_up()
+        assert made == len(captures) == 4              # batches of 1, 2, 4, 8; one context bucket
+        assert engine.warm_up() == 0
+        got = [o.token_ids for o in engine.generate(prompts, params)]
+        assert len(captures) == 4
+        late = engine_for(model, max_seq_len=128)
+        ids = [late.add_request(p, sp) for p, sp in zip(prompts, params)]
+        for _ in range(5):
+            late.step()
+        assert late.warm_up() > 0                      # a step is in flight meanwhile
+        while late.has_work():
+            late.step()
+        mid = [late.pop_finished(i).token_ids for i in ids]
+    finally:
+        DecodeGraph._capture = real
+    assert got == want and mid == want
+
+
 def test_host_sampler_modes_run_and_are_reproducible(backend, tiny_folders):
     model = load(tiny_folders["b"], backend)
     prompts = prompts_for(384, [7, 21], seed=5)
