@@ -139,6 +139,10 @@ class DecodeGraph:
         self.graphs: Dict[Tuple[int, str], Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
         # what of the metadata a chained step brings from the host: everything behind the ids
         self.behind_ids = meta.offsets["positions"][0]
+        # the requests of the step prepared last, and those whose sampled tokens are where the
+        # ids are (None: something else is there)
+        self._prepared: Optional[Tuple[int, ...]] = None
+        self._sampled_for: Optional[Tuple[int, ...]] = None
 
     def step_for(self, context_limit: int) -> StepContext:
         """The step as the kernels of a captured run see it: static views, and each planner's
@@ -187,6 +191,7 @@ class DecodeGraph:
         h = hs.h
         S = len(seq_ids)
         self.seq_ids[:S] = seq_ids
+        self._prepared = tuple(seq_ids)
         if tokens is not None:
             h["ids"][:S] = tokens
         if modes is not None:
@@ -205,6 +210,7 @@ class DecodeGraph:
         """Run the step prepared in side 0.  Logits ``(num_seqs, vocab)``: a view of a static
         tensor that the next call for the same context bucket overwrites."""
         graph, result = self._graph(context_limit, LOGITS)
+        self._sampled_for = None
         graph.replay()          # begins with the copy of side 0 of the metadata to the device
         hs = self.sides[0]
         if hs.done is None:
@@ -218,7 +224,11 @@ class DecodeGraph:
         waits for the step and returns the requests' tokens.  ``chained``: the step's ids are
         the tokens that the sampling of the step before it (the same requests in the same
         rows) left on the device; that step may still be running."""
+        if chained and self._sampled_for != self._prepared:
+            raise ValueError("a chained step follows a sampling step of the same requests in "
+                             "the same order")
         graph, _ = self._graph(context_limit, SAMPLED)        # (a capture runs a step of padding)
+        self._sampled_for = self._prepared
         hs = self.sides[side]
         lo = self.behind_ids if chained else 0
         self.dev[lo:].copy_(hs.host[lo:], non_blocking=True)

@@ -179,8 +179,10 @@ class ModelRunner:
         the same order, launched while that step may still be running: every request brings
         the token that step samples for it, which is on the device and nowhere else yet.
         ``side`` (0 or 1) names the host buffers that the step uses; a step takes the side that
-        the step before it did not (``step_sampled`` takes side 0).  Positions must be reserved
-        as for any step.  Returns the function that waits for this step's tokens."""
+        the step before it did not (``step_sampled`` takes side 0), and the tokens of the step
+        that had this side last must have been taken: at most two steps are under way.
+        Positions must be reserved as for any step.  Returns the function that waits for this
+        step's tokens."""
         if not self.use_graphs:
             raise ValueError("chained steps need captured steps")
         return self._decode_lists(seq_ids, None, modes, side)

@@ -113,6 +113,64 @@ def test_captured_decode_steps_match_eager_ones(case, dtype):
             assert torch.equal(out_g[k], out_e[k]), f"step {k}"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_chained_steps_sample_what_fed_steps_sample(case, dtype):
+    """``step_chained`` runs the same requests once more on the tokens that the sampling kernel
+    of the step before left on the device, launched before the host has seen them.  Step after
+    step it yields the tokens of a runner whose every step is fed from the host, greedy and
+    with temperature, with other graphs captured in the middle of the chain; and it refuses
+    to run when something else has been through the bucket's buffers since."""
+    from rust_llm_inference_server_amd.engine import StepEntry
+    from rust_llm_inference_server_amd.sampling import SamplingParams
+    from rust_llm_inference_server_amd.sampling.sampler import Sampler
+    name, cfg, per_dtype = case
+    folder, reqs, _ = per_dtype[dtype]
+    prompts = [list(t)[:n] for t, n in zip(reqs.values(), (9, 4, 13))]
+    samplers = [Sampler(SamplingParams.greedy(64)),
+                Sampler(SamplingParams(temperature=0.9, seed=4, max_tokens=64)),
+                Sampler(SamplingParams(temperature=1.3, seed=9, max_tokens=64))]
+    steps = 24
+
+    def start():
+        runner = make_runner(folder, dtype, 3 * 64, 8 if name == "b" else 16)
+        for i, p in enumerate(prompts):
+            runner.reserve(i, len(p) + steps + 1)
+        runner.step([StepEntry(i, p[:-1], []) for i, p in enumerate(prompts)])
+        return runner, [len(p) for p in prompts]
+
+    ids = [0, 1, 2]
+    fed, lens = start()
+    tokens, want = [p[-1] for p in prompts], []
+    for n in range(steps):
+        modes = [s.device_mode(l + n) for s, l in zip(samplers, lens)]
+        tokens = fed.step_sampled(ids, tokens, modes)()
+        want.append(tokens)
+
+    chained, lens = start()
+    modes = [s.device_mode(l) for s, l in zip(samplers, lens)]
+    wait = chained.step_sampled(ids, [p[-1] for p in prompts], modes)
+    got = []
+    for n in range(1, steps):
+        modes = [s.device_mode(l + n) for s, l in zip(samplers, lens)]
+        ahead = chained.step_chained(ids, modes, n % 2)     # launched before step n - 1 is taken
+        if n == steps // 2:
+            # (the capture of another kind of step for this very bucket runs a step of
+            # padding through the buffers that hold the tokens in flight, and puts them back)
+            assert chained.capture_decode_steps(sampled=False, max_batch=4) > 0
+        got.append(wait())
+        wait = ahead
+    got.append(wait())
+    assert got == want
+    modes = [s.device_mode(l + steps) for s, l in zip(samplers, lens)]
+    with pytest.raises(ValueError, match="same requests in the same order"):
+        chained.step_chained([1, 0, 2], modes, 0)
+    chained.step([StepEntry(i, [want[-1][i]], [0]) for i in ids])   # logits, through the bucket
+    for i in ids:
+        chained.reserve(i, lens[i] + steps + 2)
+    with pytest.raises(ValueError, match="same requests in the same order"):
+        chained.step_chained(ids, modes, 0)
+
+
 def test_capture_beside_the_garbage_of_an_earlier_runner(case):
     """A runner that has captured graphs is dropped while it sits in a reference cycle, so that
     only the cyclic collector can free it, and the collector is off: real garbage with HIP
