@@ -670,6 +670,18 @@ struct StreamNorm {
   float eps;
   const int* rows;           // null, or the row of resid/delta that token t reads
   float* resid_out;          // null, or where resid + delta goes (not resid itself)
+  // Without NORM, the two halves of a norm that sits between two products, neither of which
+  // needs a prologue over whole rows.  The product in front of the norm (ss_out given; one k
+  // slice, no gate) adds its result to resid (N wide, in place when resid_out is resid: every
+  // element is read and written by one thread), and stores the sum, the sum times the norm's
+  // weight in bfloat16, and per token and tile of output columns the sum of the squares.  The
+  // product behind the norm (scale_parts given) takes those rows as its x and scales its
+  // results by rsqrt(sum of the scale_count partial sums / K + eps) of their row.
+  bf16_t* xw_out;            // (T, N) bfloat16
+  float* ss_out;             // (16, ss_stride) float32: token-major, one entry per tile
+  const float* scale_parts;  // (16, ss_stride) float32, scale_count entries a token
+  int scale_count;
+  int ss_stride;             // a multiple of 4
 };
 
 __device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
@@ -686,13 +698,20 @@ __device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
   }
 }
 
-template <typename TC, bool GATED, int TR /* weight rows per tile: 16 or 8 */, bool NORM>
+// What a kernel does beside the product: nothing, the fused norm (x made from the residual in
+// the prologue), the scale from partial sums of squares, or joining the residual at the end.
+enum { kStreamPlain = 0, kStreamNorm = 1, kStreamScaled = 2, kStreamJoin = 3 };
+
+template <typename TC, bool GATED, int TR /* weight rows per tile: 16 or 8 */, int MODE>
 __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __restrict__ X,
                                                                 const bf16_t* __restrict__ W,
                                                                 TC* __restrict__ Y,
                                                                 const StreamShape sh,
                                                                 const StreamNorm nm) {
   extern __shared__ __attribute__((aligned(16))) unsigned char stream_smem[];
+  constexpr bool NORM = MODE == kStreamNorm, SCALED = MODE == kStreamScaled;
+  constexpr bool JOIN = MODE == kStreamJoin;
+  static_assert(!(JOIN && GATED), "a product that joins the residual has no gate");
   constexpr int kTileBytes = NORM ? kStreamTileBytes : TR * kStreamItem * 2;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, nwaves = blockDim.x / 64;
   unsigned char* tile_s = stream_smem + wave * kTileBytes;
@@ -743,6 +762,15 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
   // The rows of x in operand layout: token oi, k = kb + (4 j + og) * 8 .. + 8 for step j.
   Frag8 b[8];
   float inv_rms = 1.f;                   // NORM: of token tid / 16, in the threads that store
+  // SCALED: the scale comes as partial sums of squares, scale_count a token.  Thread (token
+  // tid / 16, i = tid % 16) of the 256 storing threads takes parts 4 i .. 4 i + 3, + 64, ...
+  // The first 64 * kScaleAhead of them are asked for here, without a condition (so that the
+  // loads in flight can be counted and nobody waits for these before the weights; the other
+  // waves ask for one address), and added up only when the first tile is stored.  The order of
+  // the sum depends on scale_count alone.
+  constexpr int kScaleAhead = 4;
+  float4 scale_ahead[SCALED ? kScaleAhead : 1];
+  bool scale_due = SCALED;
   if (!NORM) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -750,6 +778,18 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
       const bool ok = has_item && oi < T && k < K;
       const uint4 v = *(const uint4*)(X + (ok ? (long long)oi * sh.ldx + k : 0));
       b[j].u = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+    }
+    if constexpr (SCALED) {
+#pragma unroll
+      for (int j = 0; j < kScaleAhead; ++j) {
+        const int part = 4 * (tid % 16) + 64 * j;
+        const bool mine = tid < 256 && part < nm.scale_count;
+        const float4 v = *(const float4*)(nm.scale_parts +
+                                          (mine ? (long long)(tid / 16) * nm.ss_stride + part : 0));
+        scale_ahead[j] = make_float4(mine ? v.x : 0.f, mine && part + 1 < nm.scale_count ? v.y : 0.f,
+                                     mine && part + 2 < nm.scale_count ? v.z : 0.f,
+                                     mine && part + 3 < nm.scale_count ? v.w : 0.f);
+      }
     }
   } else {
     // Each wave makes its own 16 x 256 item of x: (resid + delta) * norm_weight, rounded to
@@ -874,6 +914,21 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
         *(uint4*)(tile_s + r * (kStreamItem * 2) + ((l32 ^ r) * 16)) = a[p];
       }
     }
+    // JOIN: this thread's element of the residual and of the norm's weight, asked for ahead of
+    // the next tile's weights (loads come back in order: who waits for these must not wait
+    // for those).
+    float join_resid = 0.f, join_weight = 0.f;
+    if constexpr (JOIN) {
+      const int t = (tid / 16) % 16, i = tid % 16;
+      const long long n = (long long)tile * TR + i;
+      const bool ok = tid < 256 && i < TR && t < T && n < N;
+      const long long at = ok ? (long long)t * N + n : 0;
+      const float r = nm.resid[at];
+      const float wn = nm.weight_f32 ? ((const float*)nm.weight)[ok ? n : 0]
+                                     : bf16_to_f32(((const bf16_t*)nm.weight)[ok ? n : 0]);
+      join_resid = ok ? r : 0.f;
+      join_weight = ok ? wn : 0.f;
+    }
     RLIS_STREAM_LOAD_TILE(a, tile + tile_step);  // on its way during the arithmetic
     if (has_item) {
       wave_lds_fence();
@@ -894,6 +949,19 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
     __syncthreads();
     if (tid < 256) {
       const int t = tid / 16, i = tid % 16;
+      if (SCALED && scale_due) {
+        float tot = 0.f;
+#pragma unroll
+        for (int j = 0; j < kScaleAhead; ++j)
+          tot += ((scale_ahead[j].x + scale_ahead[j].y) + scale_ahead[j].z) + scale_ahead[j].w;
+        for (int part = 4 * i + 64 * kScaleAhead; part < nm.scale_count; part += 64)
+          for (int e = 0; e < 4 && part + e < nm.scale_count; ++e)
+            tot += nm.scale_parts[(long long)t * nm.ss_stride + part + e];
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) tot += __shfl_xor(tot, o, kWave);
+        inv_rms = 1.0f / sqrtf(tot / (float)K + nm.eps);
+        scale_due = false;
+      }
       TC* y = Y + (long long)slice * sh.part_stride + (long long)t * sh.ldy;
       if (GATED) {
         constexpr int h = TR / 2;
@@ -908,6 +976,22 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
           up *= inv_rms;
           st(y + c, gate / (1.0f + expf(-gate)) * up);
         }
+      } else if (JOIN) {
+        const long long n = (long long)tile * TR + i;
+        float sq = 0.f;
+        if (i < TR && t < T && n < N) {
+          float sum = 0.f;
+          for (int w = 0; w < nwaves; ++w) sum += red_p[w * 256 + t * 16 + i];
+          sum *= inv_rms;
+          if (nm.round_parts) sum = bf16_to_f32(f32_to_bf16(sum));
+          const float total = join_resid + sum;
+          nm.resid_out[(long long)t * N + n] = total;
+          nm.xw_out[(long long)t * N + n] = f32_to_bf16(total * join_weight);
+          sq = total * total;
+        }
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) sq += __shfl_xor(sq, o, kWave);
+        if (i == 0) nm.ss_out[(long long)t * nm.ss_stride + tile] = sq;
       } else {
         const long long n = (long long)tile * TR + i;
         if (i < TR && t < T && n < N) {
@@ -928,15 +1012,15 @@ static int stream_slices(int K) { return ceil_div(ceil_div(K, kStreamItem), kStr
 // The fused norm needs whole rows in one workgroup.
 constexpr int kStreamNormMaxK = kStreamMaxWaves * kStreamItem;
 
-template <typename TC, bool GATED, int TR, bool NORM>
+template <typename TC, bool GATED, int TR, int MODE>
 static int launch_stream_tiles(const void* X, const void* W, void* Y, StreamShape sh,
                                const StreamNorm& nm, int nwaves, int num_cus,
                                hipStream_t stream) {
-  constexpr int kTileBytes = NORM ? kStreamTileBytes : TR * kStreamItem * 2;
+  constexpr int kTileBytes = MODE == kStreamNorm ? kStreamTileBytes : TR * kStreamItem * 2;
   static bool lds_raised = false;
   if (!lds_raised) {
     hipError_t e = hipFuncSetAttribute(
-        (const void*)gemm_bf16_stream_kernel<TC, GATED, TR, NORM>,
+        (const void*)gemm_bf16_stream_kernel<TC, GATED, TR, MODE>,
         hipFuncAttributeMaxDynamicSharedMemorySize, kStreamMaxWaves * (kTileBytes + 2048));
     RLIS_REQUIRE(e == hipSuccess, "gemm_bf16_stream: cannot raise the LDS limit: %s",
                  hipGetErrorString(e));
@@ -950,56 +1034,71 @@ static int launch_stream_tiles(const void* X, const void* W, void* Y, StreamShap
   long long groups = tiles;                                // workgroups per slice
   const long long cap = max(1, num_cus * per_cu / sh.num_slices);
   if (groups > cap) groups = cap;
-  gemm_bf16_stream_kernel<TC, GATED, TR, NORM>
+  gemm_bf16_stream_kernel<TC, GATED, TR, MODE>
       <<<(int)(groups * sh.num_slices), nwaves * 64, smem, stream>>>(
           (const bf16_t*)X, (const bf16_t*)W, (TC*)Y, sh, nm);
   return 0;
 }
 
-template <typename TC, bool GATED, bool NORM>
+// The compute units of the current device (0: unknown).
+static int stream_compute_units() {
+  static int num_cus = 0;
+  if (num_cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      num_cus = prop.multiProcessorCount;
+  }
+  return num_cus;
+}
+
+// Weight rows per tile: 8 when 16-row tiles would leave compute units without work (a unit draws
+// only its share of the memory bandwidth, however much it has in flight); with the fused norm
+// every workgroup reads all of x, so fewer, larger tiles win earlier.
+static int stream_tile_rows(int N, int slices, bool gated, bool norm, int num_cus) {
+  const long long tiles16 = (long long)ceil_div(N, gated ? 8 : 16) * slices;
+  return tiles16 < (norm ? num_cus / 2 : num_cus) ? 8 : 16;
+}
+
+template <typename TC, bool GATED, int MODE>
 static int launch_stream(const void* X, const void* W, void* Y, int T, int N, int K, long long ldx,
                          long long ldw, long long ldy, long long part_stride,
                          const StreamNorm& nm, hipStream_t stream) {
   const int nitems = ceil_div(K, kStreamItem);
   const int slices = stream_slices(K);
   const int nwaves = max(4, ceil_div(nitems, slices));
-  static int num_cus = 0;
-  if (num_cus == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    RLIS_REQUIRE(hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess,
-                 "gemm_bf16_stream: cannot read the device properties");
-    num_cus = prop.multiProcessorCount;
-  }
+  const int num_cus = stream_compute_units();
+  RLIS_REQUIRE(num_cus > 0, "gemm_bf16_stream: cannot read the device properties");
   StreamShape sh;
   sh.T = T; sh.N = N; sh.K = K; sh.ldx = ldx; sh.ldw = ldw; sh.ldy = ldy;
   sh.part_stride = part_stride;
   sh.num_slices = slices;
   sh.num_tiles = 0;
-  // Tiles of 8 rows when 16-row tiles would leave compute units without work: a unit draws
-  // only its share of the memory bandwidth, however much it has in flight.  With the fused
-  // norm every workgroup reads all of x, so fewer, larger tiles win earlier.
-  const long long tiles16 = (long long)ceil_div(N, GATED ? 8 : 16) * slices;
-  if (tiles16 < (NORM ? num_cus / 2 : num_cus))
-    return launch_stream_tiles<TC, GATED, 8, NORM>(X, W, Y, sh, nm, nwaves, num_cus, stream);
-  return launch_stream_tiles<TC, GATED, 16, NORM>(X, W, Y, sh, nm, nwaves, num_cus, stream);
+  if (stream_tile_rows(N, slices, GATED, MODE == kStreamNorm, num_cus) == 8)
+    return launch_stream_tiles<TC, GATED, 8, MODE>(X, W, Y, sh, nm, nwaves, num_cus, stream);
+  return launch_stream_tiles<TC, GATED, 16, MODE>(X, W, Y, sh, nm, nwaves, num_cus, stream);
 }
 
-template <bool NORM>
+template <int MODE>
 static int dispatch_stream(const char* name, const void* X, const void* W, void* Y, int y_dtype,
                            int T, int N, int K, long long ldx, long long ldw, long long ldy,
                            long long part_stride, int gated, const StreamNorm& nm,
                            hipStream_t stream) {
   RLIS_REQUIRE(!gated || y_dtype == RLIS_BF16, "%s: the gated form stores bfloat16", name);
   int rc;
-  if (gated)
-    rc = launch_stream<bf16_t, true, NORM>(X, W, Y, T, N, K, ldx, ldw, ldy, part_stride, nm, stream);
-  else if (y_dtype == RLIS_F32)
-    rc = launch_stream<float, false, NORM>(X, W, Y, T, N, K, ldx, ldw, ldy, part_stride, nm, stream);
-  else if (y_dtype == RLIS_BF16)
-    rc = launch_stream<bf16_t, false, NORM>(X, W, Y, T, N, K, ldx, ldw, ldy, part_stride, nm, stream);
-  else
-    RLIS_REQUIRE(false, "%s: unknown output dtype %d", name, y_dtype);
+  if constexpr (MODE == kStreamJoin) {
+    RLIS_REQUIRE(!gated, "%s: a product that joins the residual has no gate", name);
+    rc = launch_stream<bf16_t, false, MODE>(X, W, Y, T, N, K, ldx, ldw, ldy, part_stride, nm, stream);
+  } else {
+    if (gated)
+      rc = launch_stream<bf16_t, true, MODE>(X, W, Y, T, N, K, ldx, ldw, ldy, part_stride, nm, stream);
+    else if (y_dtype == RLIS_F32)
+      rc = launch_stream<float, false, MODE>(X, W, Y, T, N, K, ldx, ldw, ldy, part_stride, nm, stream);
+    else if (y_dtype == RLIS_BF16)
+      rc = launch_stream<bf16_t, false, MODE>(X, W, Y, T, N, K, ldx, ldw, ldy, part_stride, nm, stream);
+    else
+      RLIS_REQUIRE(false, "%s: unknown output dtype %d", name, y_dtype);
+  }
   if (rc) return rc;
   RLIS_LAUNCH_CHECK(name);
   return 0;
@@ -1025,8 +1124,75 @@ RLIS_API int rlis_gemm_bf16_stream(const void* X, const void* W, void* Y, int y_
                "no gate", K, slices);
   if (T == 0) return 0;
   StreamNorm nm = {};
-  return dispatch_stream<false>("gemm_bf16_stream", X, W, Y, y_dtype, T, N, K, ldx, ldw, ldy,
+  return dispatch_stream<kStreamPlain>("gemm_bf16_stream", X, W, Y, y_dtype, T, N, K, ldx, ldw, ldy,
                                 part_stride, gated, nm, stream);
+}
+
+// A norm between two products without a pass over whole rows, in two calls (T <= 16, bfloat16
+// operands, one k slice each).  rlis_gemm_bf16_stream_join: s = resid + x W^T (the product
+// rounded to bfloat16 first with round_sum), stored to resid_out (resid itself is fine);
+// xw_out (T, N) bfloat16 = s * norm_weight; ss_out (16, ss_stride) float32 = per token the sums
+// of s^2 over each of the rlis_gemm_bf16_stream_join_tiles(N, K) tiles of columns (ss_stride a
+// multiple of 4, at least that many; what lies behind them in a row is not written).  resid and
+// resid_out are (T, N) float32 contiguous.  rlis_gemm_bf16_stream_scaled: y = (x W^T) *
+// rsqrt(sum of the row's scale_count partial sums / K + eps), gated as rlis_gemm_bf16_stream:
+// with x = xw_out and the partial sums of the first call, the RMSNorm of s in front of this
+// product.
+RLIS_API int rlis_gemm_bf16_stream_join_tiles(int N, int K) {
+  const int cus = stream_compute_units();
+  return cus > 0 ? ceil_div(N, stream_tile_rows(N, stream_slices(K), false, false, cus)) : 0;
+}
+
+RLIS_API int rlis_gemm_bf16_stream_join(const void* X, const void* W, int T, int N, int K,
+                                        long long ldx, long long ldw, const float* resid,
+                                        float* resid_out, const void* norm_weight,
+                                        int norm_weight_dtype, int round_sum, void* xw_out,
+                                        float* ss_out, int ss_stride, hipStream_t stream) {
+  if (check_skinny("gemm_bf16_stream_join", X, W, T, N, K, ldx, ldw, N)) return 1;
+  RLIS_REQUIRE(T <= 16, "gemm_bf16_stream_join: T=%d rows, at most 16", T);
+  RLIS_REQUIRE(stream_slices(K) == 1, "gemm_bf16_stream_join: K=%d takes more than one slice", K);
+  RLIS_REQUIRE(resid && resid_out && norm_weight && xw_out && ss_out,
+               "gemm_bf16_stream_join: an operand is missing");
+  RLIS_REQUIRE(norm_weight_dtype == RLIS_F32 || norm_weight_dtype == RLIS_BF16,
+               "gemm_bf16_stream_join: unknown norm weight dtype %d", norm_weight_dtype);
+  RLIS_REQUIRE(ss_stride % 4 == 0 && ss_stride >= rlis_gemm_bf16_stream_join_tiles(N, K) &&
+                   ((uintptr_t)ss_out % 16) == 0,
+               "gemm_bf16_stream_join: the sums of squares need rows of %d entries or more, a "
+               "multiple of 4, 16-byte aligned", rlis_gemm_bf16_stream_join_tiles(N, K));
+  if (T == 0) return 0;
+  StreamNorm nm = {};
+  nm.resid = resid;
+  nm.resid_out = resid_out;
+  nm.weight = norm_weight;
+  nm.weight_f32 = norm_weight_dtype == RLIS_F32;
+  nm.round_parts = round_sum;
+  nm.xw_out = (bf16_t*)xw_out;
+  nm.ss_out = ss_out;
+  nm.ss_stride = ss_stride;
+  return dispatch_stream<kStreamJoin>("gemm_bf16_stream_join", X, W, xw_out, RLIS_BF16, T, N, K, ldx,
+                                ldw, N, 0, 0, nm, stream);
+}
+
+RLIS_API int rlis_gemm_bf16_stream_scaled(const void* X, const void* W, void* Y, int y_dtype,
+                                          int T, int N, int K, long long ldx, long long ldw,
+                                          long long ldy, int gated, const float* scale_parts,
+                                          int scale_count, int ss_stride, float eps,
+                                          hipStream_t stream) {
+  if (check_skinny("gemm_bf16_stream_scaled", X, W, T, N, K, ldx, ldw, ldy)) return 1;
+  RLIS_REQUIRE(T <= 16, "gemm_bf16_stream_scaled: T=%d rows, at most 16", T);
+  RLIS_REQUIRE(stream_slices(K) == 1, "gemm_bf16_stream_scaled: K=%d takes more than one slice",
+               K);
+  RLIS_REQUIRE(scale_parts && scale_count > 0 && ss_stride % 4 == 0 && ss_stride >= scale_count &&
+                   ((uintptr_t)scale_parts % 16) == 0,
+               "gemm_bf16_stream_scaled: %d partial sums in rows of %d", scale_count, ss_stride);
+  if (T == 0) return 0;
+  StreamNorm nm = {};
+  nm.scale_parts = scale_parts;
+  nm.scale_count = scale_count;
+  nm.ss_stride = ss_stride;
+  nm.eps = eps;
+  return dispatch_stream<kStreamScaled>("gemm_bf16_stream_scaled", X, W, Y, y_dtype, T, N, K, ldx, ldw,
+                                ldy, 0, gated, nm, stream);
 }
 
 // RMSNorm and projection in one pass, for T <= 16 tokens and K <= 4096:
@@ -1061,7 +1227,7 @@ RLIS_API int rlis_norm_linear_bf16(const float* resid, const void* delta, int de
                    (norm_weight_dtype == RLIS_F32 || norm_weight_dtype == RLIS_BF16),
                "norm_linear: unknown dtypes %d %d", delta_dtype, norm_weight_dtype);
   if (T == 0) return 0;
-  StreamNorm nm;
+  StreamNorm nm = {};
   nm.resid = resid;
   nm.delta = delta;
   nm.delta_f32 = delta_dtype == RLIS_F32;
@@ -1073,6 +1239,6 @@ RLIS_API int rlis_norm_linear_bf16(const float* resid, const void* delta, int de
   nm.eps = eps;
   nm.rows = rows;
   nm.resid_out = delta ? resid_out : nullptr;
-  return dispatch_stream<true>("norm_linear", nullptr, W, Y, y_dtype, T, N, K, K, ldw, ldy, 0,
+  return dispatch_stream<kStreamNorm>("norm_linear", nullptr, W, Y, y_dtype, T, N, K, K, ldw, ldy, 0,
                                gated, nm, stream);
 }

@@ -30,6 +30,10 @@ SPLITK_MAX_ROWS = 64
 SPLIT_MIXED_ATTENTION = True
 # The norm in front of a projection goes into the streaming kernel where that applies.
 FUSE_NORM_LINEAR = True
+# A projection whose result joins the residual stream in front of such a norm adds it there
+# itself and hands the norm's sums over, so that the product behind the norm needs no pass over
+# whole rows (up to 16 rows, one k slice on both sides).
+JOIN_NORM_LINEAR = True
 # The matrix-core decode attention rotates q and k and stores the new k, v itself where it can.
 FUSE_ROPE_DECODE = True
 # "library": bf16 products with more rows than the streaming kernel takes go to torch
@@ -296,6 +300,97 @@ def norm_linear(resid: torch.Tensor, delta: Optional[torch.Tensor], norm_weight:
                  w.data_ptr(), y.data_ptr(), _DT[out_dtype], R, N, K, ldw, N, int(bool(gated)),
                  lib.stream_ptr())
     return y, resid_sum
+
+
+class PendingProduct:
+    """``x @ w.T`` on its way into the residual stream, not run yet: the norm that follows can
+    then run it with the residual add and its own multiplies inside (``linear_join_norm``);
+    ``run()`` is the plain product, as ``linear(..., partials=True)`` gives it."""
+
+    __slots__ = ("x", "w", "out_dtype")
+
+    def __init__(self, x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype]):
+        self.x, self.w, self.out_dtype = x, w, out_dtype
+
+    @property
+    def shape(self) -> Tuple[int, int]:
+        return (self.x.shape[0], self.w.shape[0])
+
+    def run(self) -> torch.Tensor:
+        return linear(self.x, self.w, self.out_dtype, partials=True)
+
+
+def _streams_in_one_slice(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return (x.dim() == 2 and w.dim() == 2 and x.dtype == torch.bfloat16
+            and w.dtype == torch.bfloat16 and 0 < x.shape[0] <= STREAM_MAX_ROWS
+            and x.shape[1] == w.shape[1] and x.shape[1] % 8 == 0 and stream_slices(x.shape[1]) == 1
+            and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0
+            and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def pending_linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None):
+    """The projection whose result joins the residual stream: ``linear(x, w, out_dtype,
+    partials=True)``, or where the norm behind it may take it in (``JOIN_NORM_LINEAR``; up to 16
+    rows of bfloat16, one k slice, an output width that the next product can read as its rows)
+    a ``PendingProduct`` that has not run."""
+    if JOIN_NORM_LINEAR and _streams_in_one_slice(x, w) and w.shape[0] % 8 == 0:
+        return PendingProduct(x, w, out_dtype)
+    return linear(x, w, out_dtype, partials=True)
+
+
+def can_join_norm_linear(product: PendingProduct, resid: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether ``linear_join_norm`` and ``linear_scaled`` take this product, residual and the
+    weight of the product behind the norm."""
+    T, H = resid.shape
+    return (JOIN_NORM_LINEAR and resid.dtype == torch.float32 and resid.is_contiguous()
+            and product.shape == (T, H) and w.dim() == 2 and w.shape[1] == H
+            and w.dtype == torch.bfloat16 and w.stride(1) == 1 and w.stride(0) % 8 == 0
+            and w.data_ptr() % 16 == 0 and stream_slices(H) == 1)
+
+
+def linear_join_norm(product: PendingProduct, resid: torch.Tensor, norm_weight: torch.Tensor,
+                     round_sum: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Runs the product with what follows it inside: ``resid += x @ w.T`` (the product rounded
+    to bfloat16 first with ``round_sum``, as a bfloat16 model's block output is), in place.
+    Returns ``(xw, ss)``: ``resid * norm_weight`` in bfloat16 and, ``(16, tiles)`` float32, per
+    row and tile of columns the sum of ``resid ** 2`` (rows from ``T`` on are not meant), for
+    ``linear_scaled``."""
+    x, w = product.x, product.w
+    T, K = x.shape
+    N = w.shape[0]
+    _check(norm_weight, "norm weight", ndim=1)
+    if norm_weight.numel() != N or not norm_weight.is_contiguous():
+        raise KernelError(f"linear_join_norm: norm weight has {norm_weight.numel()} entries, "
+                          f"rows have {N}")
+    tiles = lib.load().rlis_gemm_bf16_stream_join_tiles(N, K)
+    if tiles <= 0:
+        raise KernelError("linear_join_norm: cannot read the device properties")
+    xw = torch.empty((T, N), dtype=torch.bfloat16, device=x.device)
+    stride = -(-tiles // 4) * 4
+    ss = torch.empty((16, stride), dtype=torch.float32, device=x.device)[:, :tiles]
+    lib.call("rlis_gemm_bf16_stream_join", x.data_ptr(), w.data_ptr(), T, N, K, x.stride(0),
+             w.stride(0), resid.data_ptr(), resid.data_ptr(), norm_weight.data_ptr(),
+             _dt(norm_weight), int(bool(round_sum)), xw.data_ptr(), ss.data_ptr(), stride,
+             lib.stream_ptr())
+    return xw, ss
+
+
+def linear_scaled(xw: torch.Tensor, ss: torch.Tensor, eps: float, w: torch.Tensor,
+                  out_dtype: torch.dtype, gated: bool = False) -> torch.Tensor:
+    """``(xw * rsqrt(mean of the rows' squares + eps)) @ w.T`` (``gated`` as ``linear_swiglu``),
+    the rows' sums of squares given as ``linear_join_norm`` leaves them: the RMSNorm of the
+    residual and the product behind it."""
+    T, K = xw.shape
+    N = w.shape[0]
+    if gated:
+        if N % 2:
+            raise KernelError("linear_scaled: a gated weight needs an even number of rows")
+        N //= 2
+    y = torch.empty((T, N), dtype=out_dtype, device=xw.device)
+    lib.call("rlis_gemm_bf16_stream_scaled", xw.data_ptr(), w.data_ptr(), y.data_ptr(),
+             _DT[out_dtype], T, N, K, xw.stride(0), w.stride(0), N, int(bool(gated)),
+             ss.data_ptr(), ss.shape[1], ss.stride(0), float(eps), lib.stream_ptr())
+    return y
 
 
 def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:

@@ -27,6 +27,8 @@ _SIGNATURES = {
     "rlis_gemm_bf16_skinny_swiglu": [P, P, P, I, I, I, L, L, L, P],
     "rlis_gemm_bf16_stream": [P, P, P, I, I, I, I, L, L, L, L, I, P],
     "rlis_gemm_bf16_splitk": [P, P, P, I, I, I, L, L, L, P],
+    "rlis_gemm_bf16_stream_join": [P, P, I, I, I, L, L, P, P, P, I, I, P, P, I, P],
+    "rlis_gemm_bf16_stream_scaled": [P, P, P, I, I, I, I, L, L, L, I, P, I, I, F, P],
     "rlis_norm_linear_bf16": [P, P, I, I, L, I, P, I, F, P, P, P, P, I, I, I, I, L, L, I, P],
     "rlis_attn_generic": [P, I, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P, P],
     "rlis_attn_decode": [P, I, L, P, L, P, P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, I, I, P, P],
@@ -71,6 +73,8 @@ def load() -> ctypes.CDLL:
     lib.rlis_gemm_bf16_stream_slices.argtypes = [I]
     lib.rlis_gemm_bf16_splitk_slices.restype = c_int
     lib.rlis_gemm_bf16_splitk_slices.argtypes = [I, I]
+    lib.rlis_gemm_bf16_stream_join_tiles.restype = c_int
+    lib.rlis_gemm_bf16_stream_join_tiles.argtypes = [I, I]
     lib.rlis_attn_register_unit.restype = c_int
     lib.rlis_attn_register_unit.argtypes = [I, P, P]
     lib.rlis_norm_linear_max_k.restype = c_int

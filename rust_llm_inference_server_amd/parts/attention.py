@@ -87,4 +87,4 @@ class PagedAttention(Mixer):
                                  write_kv=binding.writes, plan=step.plans.get(self.planner.key()),
                                  interleaved=bool(getattr(self.position, "interleaved", False)),
                                  bias_slopes=getattr(self.position, "bias_slopes", None))
-        return ops.linear(out, self.w_o, self.act_dtype, partials=True)
+        return ops.pending_linear(out, self.w_o, self.act_dtype)

@@ -271,7 +271,9 @@ class PositionEncoding(Part):
 class Mixer(Part):
     """``forward(x, step, binding)`` maps activations ``(T, H)`` to ``(T, H)``.  The result goes
     to the residual stream, so it may also be a stack ``(S, T, H)`` of float32 partial sums
-    (what ``ops.linear(..., partials=True)`` returns), which the stream adds in order.
+    (what ``ops.linear(..., partials=True)`` returns), which the stream adds in order, or the
+    last projection not run yet (what ``ops.pending_linear`` returns), which the norm behind
+    it may run with the add inside; ``as_tensor`` gives the tensor either way.
 
     ``cache_request()`` says what the mixer keeps in pages (None: nothing);
     ``state_bytes()`` how many bytes of fixed-size state it keeps per request (0: none).  A
@@ -297,7 +299,8 @@ class Mixer(Part):
 
 class FeedForward(Part):
     """``forward(x, step)`` maps activations ``(T, H)`` to ``(T, H)``, row by row (or to a
-    stack of float32 partial sums of that, as a mixer may)."""
+    stack of float32 partial sums of that, or to a projection that has not run yet, as a mixer
+    may)."""
 
     takes_normed_input = False       # as for a mixer
 
@@ -328,6 +331,14 @@ class Head(Part):
         raise NotImplementedError
 
 
+def as_tensor(delta: Any) -> torch.Tensor:
+    """What a mixer or a feed-forward returned, as one ``(T, H)`` tensor: a projection that has
+    not run yet runs now, a stack of partial sums is added up."""
+    if not isinstance(delta, torch.Tensor):
+        delta = delta.run()
+    return delta.sum(0) if delta.dim() == 3 else delta
+
+
 class ResidualStream:
     """The residual sum, kept in 32-bit, plus a delta that has not been added yet.
 
@@ -343,18 +354,26 @@ class ResidualStream:
     def __init__(self, x: torch.Tensor, act_dtype: torch.dtype = torch.float32):
         assert x.dtype == torch.float32
         self.x = x
-        self.pending: Optional[torch.Tensor] = None
+        # a tensor, or a product that has not run yet (``ops.pending_linear``), which a norm
+        # may run with the add and its own multiplies inside
+        self.pending: Any = None
         self.round_parts = act_dtype == torch.bfloat16
 
-    def add(self, delta: torch.Tensor) -> None:
+    def add(self, delta: Any) -> None:
         if self.pending is not None:
             self.flush()
         self.pending = delta
+
+    def delta(self) -> Optional[torch.Tensor]:
+        """The pending delta as a tensor (a product that has not run yet runs now)."""
+        if self.pending is not None and not isinstance(self.pending, torch.Tensor):
+            self.pending = self.pending.run()
+        return self.pending
 
     def flush(self) -> torch.Tensor:
         """Fold a pending delta into the residual and return the residual."""
         if self.pending is not None:
             from .. import ops
-            ops.add_residual(self.x, self.pending, round_parts=self.round_parts)
+            ops.add_residual(self.x, self.delta(), round_parts=self.round_parts)
             self.pending = None
         return self.x

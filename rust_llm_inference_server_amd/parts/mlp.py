@@ -39,4 +39,4 @@ class SwiGLU(FeedForward):
 
     def forward(self, x: Any, step: Any) -> torch.Tensor:
         hidden = project(x, self.w_gate_up, self.act_dtype, gated=True)
-        return ops.linear(hidden, self.w_down, self.act_dtype, partials=True)
+        return ops.pending_linear(hidden, self.w_down, self.act_dtype)

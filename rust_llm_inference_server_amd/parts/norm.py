@@ -28,12 +28,12 @@ class RMSNorm(Norm):
         self.out_dtype = ctx.act_dtype
 
     def forward(self, stream: ResidualStream) -> torch.Tensor:
-        delta, stream.pending = stream.pending, None
+        delta, stream.pending = stream.delta(), None
         return ops.add_rmsnorm(stream.x, delta, self.weight, self.eps, self.out_dtype,
                                round_parts=stream.round_parts)
 
     def forward_rows(self, stream: ResidualStream, rows: torch.Tensor) -> torch.Tensor:
-        return ops.add_rmsnorm(stream.x, stream.pending, self.weight, self.eps, self.out_dtype,
+        return ops.add_rmsnorm(stream.x, stream.delta(), self.weight, self.eps, self.out_dtype,
                                rows=rows, round_parts=stream.round_parts)
 
     def fused_linear(self, stream: ResidualStream, w: torch.Tensor, out_dtype: torch.dtype,
@@ -41,7 +41,15 @@ class RMSNorm(Norm):
         count = stream.x.shape[0] if rows is None else rows.numel()
         if self.out_dtype != torch.bfloat16 or not ops.can_fuse_norm_linear(stream.x, w, count):
             return None
-        y, total = ops.norm_linear(stream.x, stream.pending, self.weight, self.eps, w, out_dtype,
+        product = stream.pending
+        if isinstance(product, ops.PendingProduct) and rows is None \
+                and ops.can_join_norm_linear(product, stream.x, w):
+            # The product in front adds itself to the residual and leaves the rows times this
+            # norm's weight and their sums of squares; the product behind scales by them.
+            xw, ss = ops.linear_join_norm(product, stream.x, self.weight, stream.round_parts)
+            stream.pending = None
+            return ops.linear_scaled(xw, ss, self.eps, w, out_dtype, gated=gated)
+        y, total = ops.norm_linear(stream.x, stream.delta(), self.weight, self.eps, w, out_dtype,
                                    gated=gated, rows=rows, round_parts=stream.round_parts)
         if rows is None:
             stream.x, stream.pending = total, None

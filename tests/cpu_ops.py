@@ -41,6 +41,10 @@ def linear(x, w, out_dtype=None, partials=False):
     return (x.float() @ w.float().t()).to(out_dtype or x.dtype)
 
 
+def pending_linear(x, w, out_dtype=None):
+    return linear(x, w, out_dtype, partials=True)
+
+
 def linear_swiglu(x, w_gate_up):
     return swiglu(linear(x, w_gate_up, x.dtype))
 
@@ -149,7 +153,7 @@ def install(monkeypatch) -> None:
     import rust_llm_inference_server_amd.ops as ops
     import rust_llm_inference_server_amd.engine.runner as runner
     for name in ("embed", "add_residual", "add_rmsnorm", "swiglu", "linear", "linear_swiglu",
-                 "can_fuse_norm_linear", "rope_kv_write", "rope_attention",
+                 "pending_linear", "can_fuse_norm_linear", "rope_kv_write", "rope_attention",
                  "copy_pages", "attention_planner", "paged_attention", "sample_rows"):
         monkeypatch.setattr(ops, name, globals()[name])
     monkeypatch.setattr(runner, "default_device", lambda: torch.device("cpu"))

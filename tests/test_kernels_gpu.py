@@ -332,6 +332,64 @@ def test_norm_linear(ops, T, N, K, parts, rows, norm_dtype):
                                    rtol=3e-2)
 
 
+@pytest.mark.parametrize("T,H,K,N", [(1, 2048, 2048, 4096), (8, 2048, 2048, 16384), (16, 104, 344, 72),
+                                     (5, 4096, 1000, 1002), (7, 776, 4096, 64), (13, 3072, 3072, 512)])
+@pytest.mark.parametrize("norm_dtype", DTYPES, ids=["normw32", "normw16"])
+@pytest.mark.parametrize("round_sum", [True, False])
+def test_linear_join_norm_and_linear_scaled(ops, T, H, K, N, norm_dtype, round_sum):
+    """A norm between two streaming products in two kernels with no pass over whole rows: the
+    first adds x @ w1.T to the residual (rounded to bfloat16 first, or not), in place, and
+    leaves the rows times the norm's weight and their sums of squares per tile of columns; the
+    second multiplies those rows by w2 and scales by the rsqrt of the mean square, plain and
+    gated.  Against float64 formulas, and against the one-kernel norm in front of the second
+    product fed with the first product's result (the same roundings, another order of the sums
+    of squares)."""
+    x = rnd(T, K, dtype=torch.bfloat16, seed=1)
+    w1 = rnd(H, K, dtype=torch.bfloat16, seed=2, scale=0.05)
+    w2 = rnd(N, H, dtype=torch.bfloat16, seed=3, scale=0.05)
+    resid = rnd(T, H, seed=4, scale=3.0)
+    nw = (rnd(H, seed=5).abs() + 0.5).to(norm_dtype)
+    eps = 1e-5
+    product = ops.pending_linear(x, w1, torch.bfloat16)
+    assert isinstance(product, ops.PendingProduct) and product.shape == (T, H)
+    assert ops.can_join_norm_linear(product, resid, w2)
+    delta = x.double() @ w1.double().t()
+    if round_sum:
+        delta = delta.float().to(torch.bfloat16).double()
+    s = resid.double() + delta
+    normed = s / torch.sqrt((s * s).mean(-1, keepdim=True) + eps) * nw.double()
+    want = normed @ w2.double().t()
+    # the one-kernel norm on the plain product's result
+    ref_y, ref_total = ops.norm_linear(resid, product.run() if round_sum else
+                                       ops.linear(x, w1, torch.float32).unsqueeze(0),
+                                       nw, eps, w2, torch.float32, round_parts=round_sum)
+    mine = resid.clone()
+    xw, ss = ops.linear_join_norm(product, mine, nw, round_sum)
+    torch.testing.assert_close(mine.double(), s, atol=2e-2 if round_sum else 1e-3, rtol=1e-2)
+    torch.testing.assert_close(mine, ref_total, atol=1e-6 if round_sum else 1e-4, rtol=1e-6)
+    assert xw.dtype == torch.bfloat16 and xw.shape == (T, H) and ss.shape[0] == 16
+    torch.testing.assert_close(ss[:T].sum(1).double(), (mine.double() ** 2).sum(-1), rtol=1e-5, atol=1e-5)
+    assert torch.equal(xw, (mine * nw.float()).to(torch.bfloat16))
+    for out_dtype in (torch.float32, torch.bfloat16):
+        got = ops.linear_scaled(xw, ss, eps, w2, out_dtype)
+        assert got.dtype == out_dtype and got.shape == (T, N)
+        scale = max(1.0, want.abs().max().item())
+        torch.testing.assert_close(got.double(), want, atol=scale / 64, rtol=2e-2)
+    got = ops.linear_scaled(xw, ss, eps, w2, torch.float32)
+    torch.testing.assert_close(got, ref_y, atol=max(1.0, want.abs().max().item()) * 1e-4, rtol=1e-4)
+    if N % 2 == 0:
+        got = ops.linear_scaled(xw, ss, eps, w2, torch.bfloat16, gated=True)
+        g, u = want[:, :N // 2], want[:, N // 2:]
+        want_g = torch.nn.functional.silu(g) * u
+        torch.testing.assert_close(got.double(), want_g, atol=max(1.0, want_g.abs().max().item()) / 32,
+                                   rtol=3e-2)
+    # more than one k slice, more than 16 rows, or float32: the plain product comes back
+    assert isinstance(ops.pending_linear(rnd(T, 8192, dtype=torch.bfloat16), rnd(64, 8192, dtype=torch.bfloat16)),
+                      torch.Tensor)
+    assert isinstance(ops.pending_linear(rnd(17, K, dtype=torch.bfloat16), w1), torch.Tensor)
+    assert isinstance(ops.pending_linear(rnd(T, K), rnd(H, K)), torch.Tensor)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,I,K", [(1, 8192, 2048), (8, 172, 104), (16, 320, 192), (33, 1000, 256),
                                    (8, 8192, 2048), (3, 1001, 4608), (8, 77, 14336),

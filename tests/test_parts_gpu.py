@@ -71,7 +71,8 @@ def test_feed_forward_embedding_and_head_parts(dtype):
     x = torch.randn(9, H).to(dtype)
     wf = {k: v.float() for k, v in w.items()}
     tol = 2e-5 if dtype == torch.float32 else 3e-2
-    torch.testing.assert_close(mlp.forward(x.to(DEV), None).float().cpu(),
+    from rust_llm_inference_server_amd.parts.base import as_tensor
+    torch.testing.assert_close(as_tensor(mlp.forward(x.to(DEV), None)).float().cpu(),
                                plain.swiglu_mlp(x.float(), wf, "m"), atol=tol, rtol=tol)
     emb = create("embedding", PartSpec("token", {"vocab_size": V, "hidden_size": H}), "e", ctx)
     ids = [5, 130, 0, 5]
