@@ -58,6 +58,60 @@ def test_position_part_tables():
                                              "scaling": {"rope_type": "yarn"}}), "", ctx_for({}))
 
 
+def test_a_pending_projection_meets_the_norm_behind_it():
+    """A mixer's or feed-forward's last projection may reach the residual stream not yet run
+    (``ops.pending_linear``).  A norm whose consumer takes the norm into its own kernel then
+    runs the projection with the residual add inside and hands rows and sums of squares to the
+    consumer's product; any other taker (a plain norm, a norm over selected rows, a flush) gets
+    the tensor.  Every way ends with the same residual and, within the bfloat16 tolerance, the
+    same normalised product."""
+    from rust_llm_inference_server_amd import ops
+    from rust_llm_inference_server_amd.parts import PartSpec, ResidualStream, create
+    from rust_llm_inference_server_amd.parts.base import NormedInput, as_tensor
+    dtype = torch.bfloat16
+    H, K, N, T = 192, 320, 400, 9
+    w = {"n.weight": 1 + 0.1 * torch.randn(H)}
+    norm = create("norm", PartSpec("rmsnorm", {"size": H, "eps": 1e-6}), "n", ctx_for(w, dtype))
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(T, K, generator=g) * 0.5).to(dtype).to(DEV)
+    w1 = (torch.randn(H, K, generator=g) * 0.05).to(dtype).to(DEV)
+    w2 = (torch.randn(N, H, generator=g) * 0.05).to(dtype).to(DEV)
+    resid = torch.randn(T, H, generator=g).to(DEV)
+    delta = (x.float() @ w1.float().t()).to(dtype).float()
+    want_resid = resid + delta
+    want = plain.rms_norm(want_resid.cpu(), w["n.weight"], 1e-6) @ w2.float().cpu().t()
+
+    def stream_with_pending():
+        stream = ResidualStream(resid.clone(), dtype)
+        pending = ops.pending_linear(x, w1, dtype)
+        assert isinstance(pending, ops.PendingProduct)
+        stream.add(pending)
+        return stream
+
+    calls = []
+    real = ops.linear_join_norm
+    ops.linear_join_norm = lambda *a: calls.append(1) or real(*a)
+    try:
+        stream = stream_with_pending()
+        joined = NormedInput(norm, stream).linear(w2, dtype)
+    finally:
+        ops.linear_join_norm = real
+    assert calls and stream.pending is None
+    torch.testing.assert_close(stream.x, want_resid, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(joined.float().cpu(), want, atol=3e-2, rtol=3e-2)
+    stream = stream_with_pending()
+    plainly = ops.linear(norm.forward(stream), w2, dtype)           # a norm that stands alone
+    torch.testing.assert_close(stream.x, want_resid, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(plainly.float(), joined.float(), atol=3e-2, rtol=3e-2)
+    stream = stream_with_pending()
+    rows = torch.tensor([4, 1], dtype=torch.int32, device=DEV)
+    some = norm.forward_rows(stream, rows)                          # leaves the residual alone
+    assert isinstance(stream.pending, torch.Tensor)
+    torch.testing.assert_close(ops.linear(some, w2, dtype).float(), joined.float()[[4, 1]], atol=3e-2, rtol=3e-2)
+    torch.testing.assert_close(stream.flush(), want_resid, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(as_tensor(ops.pending_linear(x, w1, dtype)).float(), delta, atol=0, rtol=0)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_feed_forward_embedding_and_head_parts(dtype):
     from rust_llm_inference_server_amd.parts import PartSpec, create
