@@ -469,12 +469,9 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_splitk_kernel(const bf16_t* 
   constexpr int XIT = NT * 16 * PIECES / 256;
   Frag8 a[STEPS], ahead[WALK ? STEPS : 1];
   uint4 xv[XIT];
+  // (x first: loads come back in order, and the rows of x, which the L2 holds, are on their way
+  // to LDS while the weights still arrive)
   auto load = [&](int k0, Frag8 (&w)[STEPS]) __attribute__((always_inline)) {
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      const int k = k0 + s * 32 + lq * 8;
-      w[s].u = *(const uint4*)(wrow + (k < K ? k : 0));
-    }
 #pragma unroll
     for (int j = 0; j < XIT; ++j) {
       const int i = tid + j * 256;
@@ -482,6 +479,11 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_splitk_kernel(const bf16_t* 
       const bool ok = tok < T && k < K;
       const uint4 v = *(const uint4*)(X + (ok ? (long long)tok * ldx + k : 0));
       xv[j] = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+    }
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      const int k = k0 + s * 32 + lq * 8;
+      w[s].u = *(const uint4*)(wrow + (k < K ? k : 0));
     }
   };
 
