@@ -14,7 +14,8 @@ typedef int (*DecodeUnit)(const void* q, long long q_stride, void* out, long lon
                           const void* v_pages, const int* block_tables, int max_pages,
                           const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift,
                           int window, float scale, int splits, int part_keys, int max_parts,
-                          int merge_inside, const DecodeRope* rope, hipStream_t stream);
+                          int merge_inside, int walk, const DecodeRope* rope,
+                          hipStream_t stream);
 
 // The units (attention_mfma.hip compiled for a padded head size of 32, 64, ... 256) are
 // libraries of their own, built and loaded when a model needs them and registered here.
@@ -44,6 +45,9 @@ static int unit_result(const char* name, int rc, int d) {
     rlis_set_error("%s: partitions must be a multiple of 256 keys", name);
   else if (rc == 4)
     rlis_set_error("%s: too many sequences and KV heads to merge inside the kernel", name);
+  else if (rc == 5)
+    rlis_set_error("%s: a workgroup walks several partitions only when it merges inside, with "
+                   "partitions of a multiple of 512 keys whose results fit 64 KB of LDS", name);
   else if (rc >= 1000)
     rlis_set_error("%s: launch failed: %s", name, hipGetErrorString((hipError_t)(rc - 1000)));
   else rlis_set_error("%s: unit error %d", name, rc);
@@ -115,13 +119,18 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
 // finish, counted in device memory that the library owns, instead of by a second kernel (which
 // still runs for more than 65,536 sequences times KV heads).  Same sums in the same order
 // either way.  Launches that overlap in time on one device must pass 0.
+//
+// walk: partitions that one workgroup takes in a row (1: a workgroup each), when merging
+// inside.  The partitions, their sums and the order in which they are merged stay what
+// part_keys makes them, so every walk gives the same floats; fewer workgroups pay fewer
+// start-ups and hand-overs, which a batch that fills the chip anyway does not need.
 RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
                                    long long out_stride, float* part_ml, float* part_acc,
                                    void* k_pages, void* v_pages,
                                    const int* block_tables, int max_pages, const int* ctx_lens,
                                    int S, int nh, int nkv, int d, int page_size, int window,
                                    float scale, int splits, int part_keys, int max_parts,
-                                   int merge_inside, const float* cos, const float* sin,
+                                   int merge_inside, int walk, const float* cos, const float* sin,
                                    int rot, const int* positions, const int* slots,
                                    long long k_off, long long v_off, hipStream_t stream) {
   DecodeRope rope;
@@ -163,11 +172,14 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
   const DecodeUnit unit = decode_units[unit_index(d)];
   RLIS_REQUIRE(unit != nullptr, "attn_decode_mfma: the unit for head size %d is not loaded", d);
   const int inside = merge_inside && splits > 1 && (long long)S * nkv <= 65536;
+  RLIS_REQUIRE(walk >= 1, "attn_decode_mfma: %d partitions per workgroup", walk);
+  if (!inside) walk = 1;          // same floats either way
+  if (walk > splits) walk = splits;
   const int rc = unit_result(
       "attn_decode_mfma",
       unit(q, q_stride, out, out_stride, part_ml, part_acc, k_pages, v_pages, block_tables,
            max_pages, ctx_lens, S, nh, nkv, d, page_shift, window, scale, splits, part_keys,
-           max_parts, inside, &rope, stream),
+           max_parts, inside, walk, &rope, stream),
       d);
   if (rc) return rc;
   if (splits > 1 && S > 0 && !inside)

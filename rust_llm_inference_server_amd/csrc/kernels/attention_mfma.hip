@@ -52,6 +52,7 @@ constexpr int kUnitTooManyTiles = 1;
 constexpr int kUnitBadRotation = 2;
 constexpr int kUnitBadPartition = 3;
 constexpr int kUnitTooManyArrivals = 4;
+constexpr int kUnitBadWalk = 5;
 constexpr int kUnitLaunchFailed = 1000;       // + the hipError_t
 #define RLIS_UNIT_LAUNCH_CHECK()                                 \
   do {                                                           \
@@ -502,6 +503,16 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
 // empty result.  Page ids of a chunk are fetched one chunk ahead of its keys and values, which
 // are fetched one chunk ahead of use.
 //
+// How the keys are cut into partitions fixes the arithmetic (which sums are formed and in which
+// order they meet); how many workgroups share them does not.  With walk > 1 a workgroup takes
+// `walk` partitions in a row (merging inside only): at the end of each its waves park their
+// sums in LDS, each by itself, and start the next from nothing; after the last key the
+// workgroup merges the waves of every partition as a workgroup of its own would have, and
+// treats the results as it would treat those of other workgroups.
+// Every float is the one that walk = 1 gives; the caller picks walk by how many workgroups fill
+// the chip (a full batch needs no help from partitions, and every workgroup costs three round
+// trips to memory before its first key and a hand-over after its last).
+//
 // With rope.positions the kernel also does what rope_kv_write does for the step's own tokens
 // (crates/model/src/llama.rs:205-222): every workgroup rotates its queries in registers
 // (rotate-half over the whole head, which must be as wide as this unit: the partner of a dim
@@ -533,6 +544,13 @@ static __device__ unsigned decode_arrivals[kArrivalSlots];
 // barrier in front of the arrival count waits for); such a load does not take a stale line.
 // That keeps the whole-cache write-backs and invalidations of device-scope fences out of the
 // kernel: 256 workgroups fencing cost more than the second kernel they were to save.
+// a * b rounded to float32 by itself: the empty statement hides the product from the compiler,
+// which would otherwise fuse it with an addition behind it.
+__device__ __forceinline__ float rounded_product(float a, float b) {
+  float p = a * b;
+  asm volatile("" : "+v"(p));
+  return p;
+}
 __device__ __forceinline__ void store_shared_result(float* p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -540,14 +558,21 @@ __device__ __forceinline__ float load_shared_result(const float* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-__global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
+// Up to head size 64 two workgroups share a compute unit (four waves per SIMD, 128 registers
+// each): the bound keeps the compiler from taking the few registers more that would halve that.
+// WALKS: the form in which a workgroup may take several partitions (walk > 1); the other form
+// is spared what that costs in registers.
+template <bool WALKS>
+__global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNEL_NAME(
     const bf16_t* __restrict__ q, long long q_stride, bf16_t* __restrict__ out,
     long long out_stride, float* __restrict__ part_ml, float* __restrict__ part_acc,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ ctx_lens,
     int nh, int nkv, int d, int page_shift, float scale, int window, int splits, int part_keys,
-    int max_parts, int merge_inside, const DecodeRope rope) {
-  extern __shared__ float dsm[];           // ml: waves * g * 2 ; acc: waves * g * d
+    int max_parts, int merge_inside, int walk_arg, const DecodeRope rope) {
+  const int walk = WALKS ? walk_arg : 1;
+  // per partition that the workgroup walks: ml waves * g * 2, then acc waves * g * d
+  extern __shared__ float dsm[];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int l16 = lane % 16, lq = lane / 16;
   const int kvh = blockIdx.x, seq = blockIdx.y, split = blockIdx.z;
@@ -588,12 +613,14 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
   const int lo32 = lo & ~31;
   constexpr int kStride = 32 * kDecodeWaves;       // keys between two chunks of one wave
   const int part = decode_part_len(ctx - lo32, part_keys, max_parts);   // a multiple of kStride
-  const int kbeg = lo32 + split * part;
-  const int kend = min(ctx, kbeg + part);
   // Merging inside: only the partitions that hold keys of this sequence run, and the last of
   // them to finish merges them all; a sequence with one such partition stores its result itself.
   const int own = merge_inside ? max(1, min(splits, (ctx - lo32 + part - 1) / part)) : splits;
-  if (split >= own) return;
+  const int first = split * walk;            // this workgroup's partitions: first .. first + mine
+  if (first >= own) return;
+  const int mine = min(walk, own - first);
+  const int kbeg = lo32 + first * part;
+  const int kend = min(ctx, kbeg + mine * part);
 
   // A wave takes its chunks two at a time: the page ids of both, then all their keys and
   // values, are on their way before the first product, and the page ids of the next two follow
@@ -750,50 +777,40 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
     }
   };
 
-  if (one_by_one) {
-    // One chunk at a time: at most one for every wave of the workgroup, or a wide head.
-    for (; c0 < kend; c0 += kStride) {
-      RLIS_DEC_CHUNK(c0, pk_a, pv_a, k_a, v_a);
-      RLIS_DEC_PAGES(c0 + kStride, pk_a, pv_a);
-      compute(c0, k_a, v_a);
-    }
-  } else if constexpr (kPairs) {
-    for (; c0 < kend; c0 += 2 * kStride) {
-      RLIS_DEC_CHUNK(c0, pk_a, pv_a, k_a, v_a);
-      RLIS_DEC_CHUNK(c0 + kStride, pk_b, pv_b, k_b, v_b);
-      RLIS_DEC_PAGES(c0 + 2 * kStride, pk_a, pv_a);
-      RLIS_DEC_PAGES(c0 + 3 * kStride, pk_b, pv_b);
-      compute(c0, k_a, v_a);
-      if (c0 + kStride < kend) compute(c0 + kStride, k_b, v_b);
-    }
-  }
-#undef RLIS_DEC_CHUNK
-#undef RLIS_DEC_PAGES
-
-  // ---- merge the waves (in wave order), then store the partition ------------------
-  l_run = xor32_sum(xor16_sum(l_run));
-  float* ml_s = dsm;                       // [wave][head][2]
-  float* acc_s = dsm + kDecodeWaves * g * 2;   // [wave][head][d]
-  if (l16 < g) {
-    if (lq == 0) {
-      ml_s[(wave * g + l16) * 2] = m_run;
-      ml_s[(wave * g + l16) * 2 + 1] = l_run;
-    }
-#pragma unroll
-    for (int db = 0; db < D / 16; ++db)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int dim = db * 16 + lq * 4 + r;
-        if (dim < d) acc_s[(wave * g + l16) * d + dim] = o_acc[db][r];
+  // ---- the end of a partition: every wave parks its sums in LDS ----------------------
+  // One region per partition that the workgroup walks: [wave][head][2] maxima and
+  // denominators, then [wave][head][d] sums.  A wave parks and goes on by itself: nothing is
+  // merged, and no wave waits for another, before the workgroup's last key.
+  const int region_floats = kDecodeWaves * g * (2 + d);
+  constexpr float kLn2 = 0.6931471805599453f;       // attn_reduce works with natural-log maxima
+  auto park = [&](int n) __attribute__((always_inline)) {
+    float* ml_s = dsm + n * region_floats;
+    float* acc_s = ml_s + kDecodeWaves * g * 2;
+    const float l_all = xor32_sum(xor16_sum(l_run));
+    if (l16 < g) {
+      if (lq == 0) {
+        ml_s[(wave * g + l16) * 2] = m_run;
+        ml_s[(wave * g + l16) * 2 + 1] = l_all;
       }
-  }
-  __syncthreads();
-  for (int i = tid; i < g * d; i += 64 * kDecodeWaves) {
-    const int hh = i / d, j = i % d;
+#pragma unroll
+      for (int db = 0; db < D / 16; ++db)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int dim = db * 16 + lq * 4 + r;
+          if (dim < d) acc_s[(wave * g + l16) * d + dim] = o_acc[db][r];
+        }
+    }
+  };
+  // Partition n, dim j of head hh, over the parked waves in wave order: the sum, the base-2
+  // maximum and the denominator.
+  auto merged = [&](int n, int hh, int j, float& a, float& big, float& lsum)
+                    __attribute__((always_inline)) {
+    const float* ml_s = dsm + n * region_floats;
+    const float* acc_s = ml_s + kDecodeWaves * g * 2;
     // Without branches, so that all the reads are issued together: a wave that saw no key has
     // maximum -inf, weight 0 (selected, since -inf - -inf is no number) and sums of zeros.
     float mw[kDecodeWaves], lw[kDecodeWaves], aw[kDecodeWaves];
-    float big = -INFINITY;
+    big = -INFINITY;
 #pragma unroll
     for (int w = 0; w < kDecodeWaves; ++w) {
       mw[w] = ml_s[(w * g + hh) * 2];
@@ -801,27 +818,95 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
       aw[w] = acc_s[(w * g + hh) * d + j];
       big = fmaxf(big, mw[w]);
     }
-    float lsum = 0.f, a = 0.f;
+    lsum = 0.f;
+    a = 0.f;
 #pragma unroll
     for (int w = 0; w < kDecodeWaves; ++w) {
       const float e = (mw[w] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw[w] - big);
       lsum += lw[w] * e;
       a += aw[w] * e;
     }
+  };
+
+  // The chunks of one partition after the other (a walked partition is a multiple of two
+  // chunks per wave: the caller sees to it).  The page ids asked for in a partition's last
+  // round are those of the next one's first chunks, so nothing starts anew at the seam: the
+  // wave parks what it has and goes on from nothing.
+  int kept = 0;
+  int stop = (WALKS && mine > 1) ? kbeg + part : kend;      // where the partition at hand ends
+  for (;;) {
+    if (one_by_one) {
+      // One chunk at a time: at most one for every wave of the workgroup, or a wide head.
+      for (; c0 < stop; c0 += kStride) {
+        RLIS_DEC_CHUNK(c0, pk_a, pv_a, k_a, v_a);
+        RLIS_DEC_PAGES(c0 + kStride, pk_a, pv_a);
+        compute(c0, k_a, v_a);
+      }
+    } else if constexpr (kPairs) {
+      for (; c0 < stop; c0 += 2 * kStride) {
+        RLIS_DEC_CHUNK(c0, pk_a, pv_a, k_a, v_a);
+        RLIS_DEC_CHUNK(c0 + kStride, pk_b, pv_b, k_b, v_b);
+        RLIS_DEC_PAGES(c0 + 2 * kStride, pk_a, pv_a);
+        RLIS_DEC_PAGES(c0 + 3 * kStride, pk_b, pv_b);
+        compute(c0, k_a, v_a);
+        if (c0 + kStride < kend) compute(c0 + kStride, k_b, v_b);
+      }
+    }
+    if (!WALKS || stop >= kend) break;
+    park(kept);
+    ++kept;
+    stop = min(stop + part, kend);
+    m_run = -INFINITY;
+    l_run = 0.f;
+#pragma unroll
+    for (int db = 0; db < D / 16; ++db) o_acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+#undef RLIS_DEC_CHUNK
+#undef RLIS_DEC_PAGES
+
+  // ---- the workgroup's last key: merge the waves of every partition, then store ---------
+  park(kept);                    // kept = mine - 1
+  __syncthreads();
+  for (int i = tid; i < g * d; i += 64 * kDecodeWaves) {
+    const int hh = i / d, j = i % d;
     const int h = kvh * g + hh;
+    float a, big, lsum;
     if (own == 1) {
+      merged(0, hh, j, a, big, lsum);
       out[(long long)seq * out_stride + h * d + j] = f32_to_bf16(a / lsum);
+    } else if (WALKS && mine == own) {
+      // All partitions of the sequence were this workgroup's: it merges them as the last to
+      // arrive merges those of other workgroups (below), the same sums in the same order.
+      // (the maximum times ln 2 is rounded by itself, as on its way through memory: no fused
+      // multiply-add with the subtraction behind it)
+      float top = -INFINITY;
+      for (int n = 0; n < mine; ++n) {
+        merged(n, hh, j, a, big, lsum);
+        if (lsum > 0.f) top = fmaxf(top, rounded_product(big, kLn2));
+      }
+      float l_all = 0.f, a_all = 0.f;
+      for (int n = 0; n < mine; ++n) {
+        merged(n, hh, j, a, big, lsum);
+        const float e = lsum > 0.f ? expf(rounded_product(big, kLn2) - top) : 0.f;
+        if (e > 0.f) {
+          l_all += lsum * e;
+          a_all += a * e;
+        }
+      }
+      out[(long long)seq * out_stride + h * d + j] = f32_to_bf16(a_all / l_all);
     } else {
-      const long long idx = ((long long)seq * nh + h) * splits + split;
-      store_shared_result(part_acc + idx * d + j, a);
-      if (j == 0) {
-        // attn_reduce works with natural-log maxima: m * ln 2
-        store_shared_result(part_ml + idx * 2, big * 0.6931471805599453f);
-        store_shared_result(part_ml + idx * 2 + 1, lsum);
+      const long long idx = ((long long)seq * nh + h) * splits + first;
+      for (int n = 0; n < mine; ++n) {
+        merged(n, hh, j, a, big, lsum);
+        store_shared_result(part_acc + (idx + n) * d + j, a);
+        if (j == 0) {
+          store_shared_result(part_ml + (idx + n) * 2, rounded_product(big, kLn2));
+          store_shared_result(part_ml + (idx + n) * 2 + 1, lsum);
+        }
       }
     }
   }
-  if (!merge_inside || own == 1) return;
+  if (!merge_inside || own == 1 || mine == own) return;
 
   // ---- the last partition of (sequence, KV head) to arrive merges them all -------------
   // Every thread's stores have arrived before it passes the barrier; thread 0 then counts this
@@ -833,7 +918,7 @@ __global__ __launch_bounds__(512) void DECODE_KERNEL_NAME(
   if (tid == 0) {
     unsigned* slot = decode_arrivals + (seq * nkv + kvh);
     const bool last = __hip_atomic_fetch_add(slot, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
-                      (unsigned)(own - 1);
+                      (unsigned)((own + walk - 1) / walk - 1);
     if (last) __hip_atomic_store(slot, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     merges = last;
   }
@@ -891,21 +976,29 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
     const void* q, long long q_stride, void* out, long long out_stride, float* part_ml,
     float* part_acc, const void* k_pages, const void* v_pages, const int* block_tables,
     int max_pages, const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift, int window,
-    float scale, int splits, int part_keys, int max_parts, int merge_inside,
+    float scale, int splits, int part_keys, int max_parts, int merge_inside, int walk,
     const DecodeRope* rope, hipStream_t stream) {
   if (S == 0) return 0;
   if (part_keys % (32 * kDecodeWaves) != 0 || part_keys <= 0) return kUnitBadPartition;
   if (merge_inside && (long long)S * nkv > kArrivalSlots) return kUnitTooManyArrivals;
+  const int g = nh / nkv;
+  const size_t smem = (size_t)(walk < 1 ? 1 : walk) * kDecodeWaves * g * (2 + d) * sizeof(float);
+  // several partitions per workgroup: merging inside, whole pairs of chunks, results that fit
+  if (walk < 1 || (walk > 1 && (!merge_inside || part_keys % (64 * kDecodeWaves) != 0 ||
+                                smem > 64 * 1024)))
+    return kUnitBadWalk;
   // rotation inside the kernel needs head_dim = rotated width = 64, 128 or 256
   if (rope->positions && rope->cos && !(D % 64 == 0 && rope->rot == D && d == D))
     return kUnitBadRotation;
-  const int g = nh / nkv;
-  dim3 grid(nkv, S, splits);
-  const size_t smem = (size_t)kDecodeWaves * g * (2 + d) * sizeof(float);
-  DECODE_KERNEL_NAME<<<grid, 64 * kDecodeWaves, smem, stream>>>(
-      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, part_ml, part_acc,
-      (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, max_pages, ctx_lens, nh, nkv, d,
-      page_shift, scale, window, splits, part_keys, max_parts, merge_inside, *rope);
+  dim3 grid(nkv, S, (splits + walk - 1) / walk);
+#define RLIS_DEC_LAUNCH(WALKS)                                                                    \
+  DECODE_KERNEL_NAME<WALKS><<<grid, 64 * kDecodeWaves, smem, stream>>>(                          \
+      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, part_ml, part_acc,                   \
+      (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, max_pages, ctx_lens, nh, nkv, \
+      d, page_shift, scale, window, splits, part_keys, max_parts, merge_inside, walk, *rope)
+  if (walk > 1) RLIS_DEC_LAUNCH(true);
+  else RLIS_DEC_LAUNCH(false);
+#undef RLIS_DEC_LAUNCH
   RLIS_UNIT_LAUNCH_CHECK();
   return 0;
 }

@@ -6,6 +6,7 @@ the CPU; without the compiled library or without a GPU the first call raises.
 """
 from __future__ import annotations
 
+import functools
 import math
 from typing import Optional, Tuple
 
@@ -62,6 +63,20 @@ DECODE_ATTENTION = "matrix"
 # 1.125 GB, take the same time either way).
 MERGE_DECODE_INSIDE = True
 MERGE_DECODE_INSIDE_MAX_BYTES = 9 << 27        # 1.125 GB
+# Partitions that one workgroup of that kernel takes in a row: None = by how many workgroups
+# the batch makes (``attention_plan.decode_walk``), a number = that many (tests: every walk
+# gives the same floats).
+DECODE_WALK: Optional[int] = None
+
+
+@functools.lru_cache(maxsize=None)
+def _compute_units_of(index: int) -> int:
+    return int(torch.cuda.get_device_properties(index).multi_processor_count)
+
+
+def _compute_units(device: torch.device) -> int:
+    return _compute_units_of(device.index if device.index is not None
+                             else torch.cuda.current_device())
 
 
 def _dt(t: torch.Tensor) -> int:
@@ -657,13 +672,19 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                 slots_p = None if slots is None else _i32(slots, "slots", S)
                 if cos is not None:
                     cos_p, sin_p, rot = cos.data_ptr(), sin.data_ptr(), 2 * cos.shape[1]
-            inside = MERGE_DECODE_INSIDE and (S * nkv * depth * ap.DECODE_PART_KEYS * d * 4
+            walk = DECODE_WALK or ap.decode_walk(S, nkv, depth, nh // nkv, d,
+                                                 _compute_units(qkv.device))
+            # (a workgroup that walks all of a sequence's partitions hands nothing over)
+            inside = MERGE_DECODE_INSIDE and (walk >= depth or
+                                              S * nkv * depth * ap.DECODE_PART_KEYS * d * 4
                                               <= MERGE_DECODE_INSIDE_MAX_BYTES)
+            if not inside:
+                walk = 1
             lib.call("rlis_attn_decode_mfma", qkv.data_ptr(), q_stride, out.data_ptr(), nh * d,
                      ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
                      block_tables.data_ptr(), max_pages, _i32(step.ctx_lens, "ctx_lens", S), S,
                      nh, nkv, d, page_size, win, float(scale), depth, ap.DECODE_PART_KEYS,
-                     ap.DECODE_MAX_PARTS, int(inside), cos_p, sin_p, rot, pos_p,
+                     ap.DECODE_MAX_PARTS, int(inside), walk, cos_p, sin_p, rot, pos_p,
                      slots_p, nh * d, (nh + nkv) * d, stream)
         else:
             lib.call("rlis_attn_decode", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(),

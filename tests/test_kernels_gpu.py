@@ -824,6 +824,63 @@ def test_attention_decode_partitions_merged_inside_the_kernel(ops, nh, nkv, d, p
         ops.MERGE_DECODE_INSIDE, ops.MERGE_DECODE_INSIDE_MAX_BYTES = old
 
 
+@pytest.mark.parametrize("nh,nkv,d,ps,rotate", [(32, 8, 64, 16, True), (24, 8, 128, 16, True),
+                                                (8, 2, 256, 16, True), (5, 5, 48, 16, False),
+                                                (9, 3, 112, 16, False)])
+@pytest.mark.parametrize("window", [None, 700])
+def test_attention_decode_workgroups_that_walk_partitions(ops, nh, nkv, d, ps, rotate, window):
+    """A workgroup of the matrix-core decode kernel that takes several partitions in a row
+    (what a full batch gets instead of one workgroup per partition) against one workgroup per
+    partition: the same floats for every walk, in the output and in the pages, since the
+    partitions, their sums and the order of the merge stay what the sequence's own length makes
+    them.  The kernel rotates and stores the step's own key itself here; the walking form waits
+    for that store in front of its last round of chunks only.  Contexts end at, just before
+    and just behind the edges of partitions and of rounds; a walk whose parked sums do not fit
+    the LDS is refused."""
+    from rust_llm_inference_server_amd.ops import attention_plan
+    from rust_llm_inference_server_amd.ops.lib import KernelError
+    dtype = torch.bfloat16
+    lens = [1, 300, 512, 513, 1024, 1025, 1026, 1280, 1281, 1536, 1537, 2047, 2048, 2049, 2100,
+            3000, 4000, 5000]
+    cached, new = [l - 1 for l in lens], [1] * len(lens)
+    scale = 1.0 / math.sqrt(d)
+    qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=d + 7)
+    cos = sin = None
+    if rotate:
+        ang = rnd(max(lens) + 1, d // 2, seed=6, scale=3.0)
+        cos, sin = torch.cos(ang), torch.sin(ang)
+    tables = bt.cpu()
+    slots = torch.tensor([int(tables[s, (l - 1) // ps]) * ps + (l - 1) % ps for s, l in enumerate(lens)],
+                         dtype=torch.int32, device=DEV)
+    room = (64 * 1024) // (8 * (nh // nkv) * (d + 2) * 4)
+    old = ops.DECODE_WALK, ops.MERGE_DECODE_INSIDE_MAX_BYTES
+    try:
+        ops.MERGE_DECODE_INSIDE_MAX_BYTES = 1 << 50
+        for part_keys, max_parts in ((1024, 16), (512, 16), (512, 2)):
+            with attention_constants(DECODE_PART_KEYS=part_keys, DECODE_MAX_PARTS=max_parts):
+                results = {}
+                for walk in (1, 2, 3, 5, 16):
+                    ops.DECODE_WALK = walk
+                    q2, k2, v2 = qkv.clone(), kp.clone(), vp.clone()
+                    deep = min(walk, attention_plan.decode_depth(max(lens)))   # what is asked for
+                    if deep > 1 and deep > room:
+                        with pytest.raises(KernelError, match="walks several partitions"):
+                            ops.rope_attention(q2, nh, nkv, d, cos, sin, step.positions, slots, k2, v2,
+                                               ps, bt, step, scale, window)
+                        continue
+                    out = ops.rope_attention(q2, nh, nkv, d, cos, sin, step.positions, slots, k2, v2,
+                                             ps, bt, step, scale, window)
+                    results[walk] = (out.cpu(), k2.cpu(), v2.cpu())
+                o1, k1, v1 = results.pop(1)
+                assert not torch.equal(k1, kp.cpu())                  # the new keys were stored
+                for walk, (o, k, v) in results.items():
+                    where = f"cut {part_keys} x {max_parts}, walk {walk}"
+                    assert torch.equal(o, o1), where
+                    assert torch.equal(k, k1) and torch.equal(v, v1), where
+    finally:
+        ops.DECODE_WALK, ops.MERGE_DECODE_INSIDE_MAX_BYTES = old
+
+
 @pytest.mark.parametrize("kind,dtype", kinds_and_dtypes("generic", "prefill", "decode"))
 def test_attention_finds_a_far_key(ops, dtype, kind, decode_kind):
     """One key among hundreds is made to stand out (its key vector equals the scaled query
