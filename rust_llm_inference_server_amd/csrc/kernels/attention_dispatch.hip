@@ -47,7 +47,8 @@ static int unit_result(const char* name, int rc, int d) {
     rlis_set_error("%s: too many sequences and KV heads to merge inside the kernel", name);
   else if (rc == 5)
     rlis_set_error("%s: a workgroup walks several partitions only when it merges inside, with "
-                   "partitions of a multiple of 512 keys whose results fit 64 KB of LDS", name);
+                   "partitions of a multiple of 512 keys whose parked sums fit the LDS (64 KB up "
+                   "to head size 64, 159 KB beyond)", name);
   else if (rc >= 1000)
     rlis_set_error("%s: launch failed: %s", name, hipGetErrorString((hipError_t)(rc - 1000)));
   else rlis_set_error("%s: unit error %d", name, rc);

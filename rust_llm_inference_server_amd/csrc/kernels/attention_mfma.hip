@@ -983,10 +983,23 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
   if (merge_inside && (long long)S * nkv > kArrivalSlots) return kUnitTooManyArrivals;
   const int g = nh / nkv;
   const size_t smem = (size_t)(walk < 1 ? 1 : walk) * kDecodeWaves * g * (2 + d) * sizeof(float);
-  // several partitions per workgroup: merging inside, whole pairs of chunks, results that fit
+  // several partitions per workgroup: merging inside, whole pairs of chunks, and parked sums
+  // that fit the LDS (up to head size 64 two workgroups share a compute unit's 160 KB)
+  constexpr size_t kWalkBytes = D <= 64 ? 64 * 1024 : 159 * 1024;
   if (walk < 1 || (walk > 1 && (!merge_inside || part_keys % (64 * kDecodeWaves) != 0 ||
-                                smem > 64 * 1024)))
+                                smem > kWalkBytes)))
     return kUnitBadWalk;
+  if (smem > 64 * 1024) {
+    // more dynamic LDS than a kernel gets unasked
+    static size_t granted = 0;
+    if (smem > granted) {
+      const hipError_t e = hipFuncSetAttribute(
+          reinterpret_cast<const void*>(&DECODE_KERNEL_NAME<true>),
+          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWalkBytes);
+      if (e != hipSuccess) return kUnitLaunchFailed + (int)e;
+      granted = kWalkBytes;
+    }
+  }
   // rotation inside the kernel needs head_dim = rotated width = 64, 128 or 256
   if (rope->positions && rope->cos && !(D % 64 == 0 && rope->rot == D && d == D))
     return kUnitBadRotation;

@@ -60,6 +60,14 @@ def decode_depth(max_context: int) -> int:
     return max(1, min(DECODE_MAX_PARTS, -(-max_context // DECODE_PART_KEYS)))
 
 
+def decode_walk_room(group: int, head_dim: int) -> int:
+    """Partitions whose parked sums (eight waves, ``group`` heads, ``head_dim`` + 2 floats) a
+    decode workgroup has LDS for: 64 KB up to head size 64, where two workgroups share a compute
+    unit's 160 KB, 159 KB beyond, where a compute unit holds one."""
+    lds = 64 * 1024 if head_dim <= 64 else 159 * 1024
+    return lds // (8 * group * (head_dim + 2) * 4)
+
+
 def decode_walk(num_seqs: int, num_kv_heads: int, depth: int, group: int, head_dim: int,
                 compute_units: int) -> int:
     """Partitions that one workgroup of the matrix-core decode kernel takes in a row, for a
@@ -69,13 +77,13 @@ def decode_walk(num_seqs: int, num_kv_heads: int, depth: int, group: int, head_d
     every walk.  Sequences times KV heads that fill the compute units by themselves take one
     workgroup each; fewer keep as many workgroups each as bring them to about what the compute
     units hold at once (two workgroups each up to head size 64, one beyond).  The eight waves'
-    sums of every walked partition must fit 64 KB of LDS, and the kernel walks whole pairs of
-    chunks only (partitions of a multiple of 512 keys)."""
+    sums of every walked partition must fit the LDS (``decode_walk_room``), and the kernel walks
+    whole pairs of chunks only (partitions of a multiple of 512 keys)."""
     if depth <= 1 or DECODE_PART_KEYS % 512 != 0:
         return 1
     resident = 2 if head_dim <= 64 else 1
     each = max(1, compute_units * resident // max(1, num_seqs * num_kv_heads))
-    room = (64 * 1024) // (8 * group * (head_dim + 2) * 4)
+    room = decode_walk_room(group, head_dim)
     return max(1, min(depth // each, depth, room))
 
 

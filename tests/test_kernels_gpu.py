@@ -852,7 +852,7 @@ def test_attention_decode_workgroups_that_walk_partitions(ops, nh, nkv, d, ps, r
     tables = bt.cpu()
     slots = torch.tensor([int(tables[s, (l - 1) // ps]) * ps + (l - 1) % ps for s, l in enumerate(lens)],
                          dtype=torch.int32, device=DEV)
-    room = (64 * 1024) // (8 * (nh // nkv) * (d + 2) * 4)
+    room = attention_plan.decode_walk_room(nh // nkv, d)
     old = ops.DECODE_WALK, ops.MERGE_DECODE_INSIDE_MAX_BYTES
     try:
         ops.MERGE_DECODE_INSIDE_MAX_BYTES = 1 << 50
