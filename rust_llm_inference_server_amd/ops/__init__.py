@@ -60,7 +60,8 @@ DECODE_ATTENTION = "matrix"
 # upper bound, since a captured step's grid is as deep as its context bucket's longest context
 # needs and most sequences are shorter; 64 requests of the 3B shape with contexts up to 2,300,
 # 1.07 GB by this count, gain 3 % of their step inside; 32 requests of the 8B shape at 8,300,
-# 1.125 GB, take the same time either way).
+# 1.125 GB, take the same time either way).  Grids whose workgroups walk several partitions
+# merge inside whatever their size: their workgroups are few.
 MERGE_DECODE_INSIDE = True
 MERGE_DECODE_INSIDE_MAX_BYTES = 9 << 27        # 1.125 GB
 # Partitions that one workgroup of that kernel takes in a row: None = by how many workgroups
@@ -674,8 +675,8 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                     cos_p, sin_p, rot = cos.data_ptr(), sin.data_ptr(), 2 * cos.shape[1]
             walk = DECODE_WALK or ap.decode_walk(S, nkv, depth, nh // nkv, d,
                                                  _compute_units(qkv.device))
-            # (a workgroup that walks all of a sequence's partitions hands nothing over)
-            inside = MERGE_DECODE_INSIDE and (walk >= depth or
+            # (workgroups that walk partitions are few, and hand over little or nothing)
+            inside = MERGE_DECODE_INSIDE and (walk > 1 or
                                               S * nkv * depth * ap.DECODE_PART_KEYS * d * 4
                                               <= MERGE_DECODE_INSIDE_MAX_BYTES)
             if not inside:
