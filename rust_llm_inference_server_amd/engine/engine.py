@@ -216,8 +216,10 @@ class Engine:
             if singles is not None:
                 wait = self.runner.step_sampled(*singles)
             if wait is None:
+                # (single tokens lead the step, the longest contexts first, as above)
+                in_order = sorted(sched.seqs, key=lambda t: (t[2] - t[1] != 1, -t[2]))
                 entries, final = [], []
-                for seq_id, start, end in sched.seqs:
+                for seq_id, start, end in in_order:
                     seq = self._seqs[seq_id]
                     last = end == len(seq.tokens)
                     entries.append(StepEntry(seq_id, seq.tokens[start:end],
@@ -240,7 +242,7 @@ class Engine:
         # Rows that yield a token, split between the device kernel and the host sampler.
         device_rows, device_modes, host_rows = [], [], []
         row = 0
-        for (seq_id, start, end), last in zip(sched.seqs, final):
+        for (seq_id, start, end), last in zip(in_order, final):
             self.scheduler.advance(seq_id, end)
             seq = self._seqs[seq_id]
             # prompt tokens of this portion (recomputed ones after a preemption count again)
@@ -269,7 +271,7 @@ class Engine:
                 picked[seq_id] = seq.sampler.sample(lrow, seq.tokens, len(seq.tokens))
         out, grown = [], []
         now = time.perf_counter()
-        for (seq_id, _, _), last in zip(sched.seqs, final):
+        for (seq_id, _, _), last in zip(in_order, final):
             if last:
                 out.append(self._accept(self._seqs[seq_id], picked[seq_id], now, grown))
         self.scheduler.append_tokens(grown)
@@ -303,7 +305,7 @@ class Engine:
         sch.append_tokens(ids)
         flight.appended = True
         sched = sch.schedule()
-        if sched.copies or sched.preempted or [s for s, _, _ in sched.seqs] != ids \
+        if sched.copies or sched.preempted or sorted(s for s, _, _ in sched.seqs) != sorted(ids) \
                 or any(end - start != 1 for _, start, end in sched.seqs):
             raise RuntimeError("the schedule of a step launched ahead is not the step before "
                                "it with one more token each")
@@ -349,8 +351,11 @@ class Engine:
 
     def _single_tokens(self, sched) -> Optional[Tuple[List[int], List[int], List[Tuple[int, float]]]]:
         """(request ids, their tokens, their (key, 1/T)) when every request of the schedule brings
-        its last known token alone and the device kernel can sample for it; else None."""
-        ids, tokens, modes = [], [], []
+        its last known token alone and the device kernel can sample for it; else None.  The
+        longest contexts come first: the attention kernel's workgroups start in the batch's
+        order, and the long walks should not be the last to start.  (A row does not depend on
+        its place in the batch, and the order holds while the same requests go on decoding.)"""
+        rows = []
         seqs = self._seqs
         for seq_id, start, end in sched.seqs:
             seq = seqs[seq_id]
@@ -359,10 +364,9 @@ class Engine:
             mode = seq.sampler.device_mode(end)
             if mode is None:
                 return None
-            ids.append(seq_id)
-            tokens.append(seq.tokens[start])
-            modes.append(mode)
-        return ids, tokens, modes
+            rows.append((-end, len(rows), seq_id, seq.tokens[start], mode))
+        rows.sort()
+        return [r[2] for r in rows], [r[3] for r in rows], [r[4] for r in rows]
 
     def _accept(self, seq: _Sequence, token: int, now: float, grown: List[int]
                 ) -> Tuple[int, Optional[int], bool]:

@@ -337,6 +337,41 @@ def test_cancel_returns_the_pages(backend, tiny_folders):
     assert engine.runner.cache.num_free_pages() == 16
 
 
+def test_decoding_requests_go_to_the_step_longest_context_first(backend, tiny_folders, monkeypatch):
+    """The attention kernel's workgroups start in the batch's order, so the engine hands the
+    requests of a step over with single tokens first and the longest contexts in front; what
+    each request generates does not depend on that (the other tests), and steps launched
+    ahead keep the order of the step before them."""
+    model = load(tiny_folders["a"], backend, max_positions=128)
+    engine = engine_for(model, launch_ahead=True)
+    lengths = [5, 31, 12, 40, 7]
+    ids = [engine.add_request(p, SamplingParams.greedy(6)) for p in prompts_for(256, lengths, seed=3)]
+    runner, seen = engine.runner, []
+    real_step, real_sampled, real_chained = runner.step, runner.step_sampled, runner.step_chained
+
+    def note(order):
+        held = [len(engine._seqs[i].tokens) for i in order]
+        seen.append((list(order), held))
+
+    monkeypatch.setattr(runner, "step", lambda entries: (
+        note([e.seq_id for e in entries if len(e.tokens) == 1]), real_step(entries))[1])
+    monkeypatch.setattr(runner, "step_sampled", lambda i, t, m: (note(i), real_sampled(i, t, m))[1])
+    monkeypatch.setattr(runner, "step_chained", lambda i, m, side: (
+        seen.append((list(i), None)), real_chained(i, m, side))[1])
+    while engine.has_work():
+        engine.step()
+    assert all(engine.pop_finished(i).finish_reason == "length" for i in ids)
+    decoding = [order for order, held in seen if held is not None and len(order) > 1]
+    assert decoding, "no step with several decoding requests"
+    for order, held in seen:
+        if held is not None:
+            assert held == sorted(held, reverse=True), (order, held)
+    # a step launched ahead lists the requests as the step before it did
+    for before, after in zip(seen, seen[1:]):
+        if after[1] is None:
+            assert after[0] == before[0]
+
+
 def test_a_failed_step_fails_only_its_own_requests(backend, tiny_folders):
     """crates/engine/src/engine.rs:523-528.  The first step holds a portion of the long request
     alone (it uses the whole budget); the model step is made to raise once."""
