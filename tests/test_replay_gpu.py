@@ -289,7 +289,9 @@ def test_decode_logits_do_not_depend_on_the_neighbours(tmp_path, use_graphs):
     of a decoding request are bit for bit the same alone in its steps as beside two others, and
     the same from captured steps as from eager ones.  A request's context is cut by its own
     length, the products run the same kernel for 1 and for 3 rows, and a block's output is
-    rounded once whichever kernel made it."""
+    rounded once whichever kernel made it.  Nor do they depend on how many workgroups share a
+    context's partitions (what the attention picks by the size of the batch): with one
+    workgroup for both partitions of the long context, the same bits."""
     folder = make_model_folder(tmp_path / "long", LONG, seed=6, dtype=torch.bfloat16)
     reqs = traces.random_requests(LONG["vocab_size"], [1500 + 8, 40 + 8, 1020 + 8], seed=5)
     keys = sorted(reqs)
@@ -311,12 +313,20 @@ def test_decode_logits_do_not_depend_on_the_neighbours(tmp_path, use_graphs):
                     out[(i, t)] = logits[row].clone()
         return out
 
+    from rust_llm_inference_server_amd import ops
     together = run([[0, 1, 2]], use_graphs)
     alone = run([[0], [1], [2]], use_graphs)
     other = run([[2, 0], [1]], not use_graphs)
+    old = ops.DECODE_WALK
+    try:
+        ops.DECODE_WALK = 2
+        walked = run([[0, 1, 2]], use_graphs)
+    finally:
+        ops.DECODE_WALK = old
     for key in together:
         assert torch.equal(together[key], alone[key]), f"request {key[0]} step {key[1]}: alone"
         assert torch.equal(together[key], other[key]), f"request {key[0]} step {key[1]}: other mode"
+        assert torch.equal(together[key], walked[key]), f"request {key[0]} step {key[1]}: walked"
     w, c = plain.read_weights(folder), plain.read_config(folder)
     for i, k in enumerate(keys):
         ref = plain.forward(w, c, reqs[k])
