@@ -14,7 +14,7 @@ typedef int (*DecodeUnit)(const void* q, long long q_stride, void* out, long lon
                           const void* v_pages, const int* block_tables, int max_pages,
                           const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift,
                           int window, float scale, int splits, int part_keys, int max_parts,
-                          int merge_inside, int walk, const DecodeRope* rope,
+                          int merge_inside, int groups, int cap, const DecodeRope* rope,
                           hipStream_t stream);
 
 // The units (attention_mfma.hip compiled for a padded head size of 32, 64, ... 256) are
@@ -121,17 +121,20 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
 // still runs for more than 65,536 sequences times KV heads).  Same sums in the same order
 // either way.  Launches that overlap in time on one device must pass 0.
 //
-// walk: partitions that one workgroup takes in a row (1: a workgroup each), when merging
-// inside.  The partitions, their sums and the order in which they are merged stay what
-// part_keys makes them, so every walk gives the same floats; fewer workgroups pay fewer
-// start-ups and hand-overs, which a batch that fills the chip anyway does not need.
+// groups, cap: when merging inside, a sequence's partitions are dealt out evenly to `groups`
+// workgroups (to more where a share would pass `cap` partitions, which is what the LDS holds
+// of parked sums; cap = 1: a workgroup per partition).  The partitions, their sums and the
+// order in which they are merged stay what part_keys makes them, so the floats are the same
+// whoever computes them; fewer workgroups pay fewer start-ups and hand-overs, which a batch
+// that fills the chip anyway does not need.
 RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
                                    long long out_stride, float* part_ml, float* part_acc,
                                    void* k_pages, void* v_pages,
                                    const int* block_tables, int max_pages, const int* ctx_lens,
                                    int S, int nh, int nkv, int d, int page_size, int window,
                                    float scale, int splits, int part_keys, int max_parts,
-                                   int merge_inside, int walk, const float* cos, const float* sin,
+                                   int merge_inside, int groups, int cap, const float* cos,
+                                   const float* sin,
                                    int rot, const int* positions, const int* slots,
                                    long long k_off, long long v_off, hipStream_t stream) {
   DecodeRope rope;
@@ -173,14 +176,15 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
   const DecodeUnit unit = decode_units[unit_index(d)];
   RLIS_REQUIRE(unit != nullptr, "attn_decode_mfma: the unit for head size %d is not loaded", d);
   const int inside = merge_inside && splits > 1 && (long long)S * nkv <= 65536;
-  RLIS_REQUIRE(walk >= 1, "attn_decode_mfma: %d partitions per workgroup", walk);
-  if (!inside) walk = 1;          // same floats either way
-  if (walk > splits) walk = splits;
+  RLIS_REQUIRE(groups >= 1 && cap >= 1, "attn_decode_mfma: %d workgroups of up to %d partitions",
+               groups, cap);
+  if (!inside) cap = 1;           // same floats either way
+  if (cap > splits) cap = splits;
   const int rc = unit_result(
       "attn_decode_mfma",
       unit(q, q_stride, out, out_stride, part_ml, part_acc, k_pages, v_pages, block_tables,
            max_pages, ctx_lens, S, nh, nkv, d, page_shift, window, scale, splits, part_keys,
-           max_parts, inside, walk, &rope, stream),
+           max_parts, inside, groups, cap, &rope, stream),
       d);
   if (rc) return rc;
   if (splits > 1 && S > 0 && !inside)

@@ -504,14 +504,16 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
 // are fetched one chunk ahead of use.
 //
 // How the keys are cut into partitions fixes the arithmetic (which sums are formed and in which
-// order they meet); how many workgroups share them does not.  With walk > 1 a workgroup takes
-// `walk` partitions in a row (merging inside only): at the end of each its waves park their
-// sums in LDS, each by itself, and start the next from nothing; after the last key the
-// workgroup merges the waves of every partition as a workgroup of its own would have, and
-// treats the results as it would treat those of other workgroups.
-// Every float is the one that walk = 1 gives; the caller picks walk by how many workgroups fill
-// the chip (a full batch needs no help from partitions, and every workgroup costs three round
-// trips to memory before its first key and a hand-over after its last).
+// order they meet); how many workgroups share them does not.  With cap > 1 (merging inside
+// only) a sequence's partitions are dealt out evenly to `groups` workgroups, or to as many more
+// as it takes for none to get more than `cap`, each taking its share in a row: at the end of a
+// partition its waves park their sums in LDS, each by itself, and start the next from nothing;
+// after the last key the workgroup merges the waves of every partition as a workgroup of its
+// own would have, and treats the results as it would treat those of other workgroups.
+// Every float is the one that a workgroup per partition gives; the caller picks `groups` by how
+// many workgroups fill the chip (a full batch needs no help from partitions, and every
+// workgroup costs three round trips to memory before its first key and a hand-over after its
+// last) and `cap` by what the LDS holds.
 //
 // With rope.positions the kernel also does what rope_kv_write does for the step's own tokens
 // (crates/model/src/llama.rs:205-222): every workgroup rotates its queries in registers
@@ -560,7 +562,7 @@ __device__ __forceinline__ float load_shared_result(const float* p) {
 
 // Up to head size 64 two workgroups share a compute unit (four waves per SIMD, 128 registers
 // each): the bound keeps the compiler from taking the few registers more that would halve that.
-// WALKS: the form in which a workgroup may take several partitions (walk > 1); the other form
+// WALKS: the form in which a workgroup may take several partitions (cap > 1); the other form
 // is spared what that costs in registers.
 template <bool WALKS>
 __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNEL_NAME(
@@ -569,8 +571,7 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ ctx_lens,
     int nh, int nkv, int d, int page_shift, float scale, int window, int splits, int part_keys,
-    int max_parts, int merge_inside, int walk_arg, const DecodeRope rope) {
-  const int walk = WALKS ? walk_arg : 1;
+    int max_parts, int merge_inside, int groups, int cap, const DecodeRope rope) {
   // per partition that the workgroup walks: ml waves * g * 2, then acc waves * g * d
   extern __shared__ float dsm[];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
@@ -616,9 +617,14 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
   // Merging inside: only the partitions that hold keys of this sequence run, and the last of
   // them to finish merges them all; a sequence with one such partition stores its result itself.
   const int own = merge_inside ? max(1, min(splits, (ctx - lo32 + part - 1) / part)) : splits;
-  const int first = split * walk;            // this workgroup's partitions: first .. first + mine
-  if (first >= own) return;
-  const int mine = min(walk, own - first);
+  // This workgroup's partitions: first .. first + mine, one of `sharers` even shares.
+  int sharers = own, first = split, mine = 1;
+  if constexpr (WALKS) {
+    sharers = min(own, max(groups, (own + cap - 1) / cap));
+    first = split * own / sharers;
+    mine = (split + 1) * own / sharers - first;
+  }
+  if (split >= sharers) return;
   const int kbeg = lo32 + first * part;
   const int kend = min(ctx, kbeg + mine * part);
 
@@ -918,7 +924,7 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
   if (tid == 0) {
     unsigned* slot = decode_arrivals + (seq * nkv + kvh);
     const bool last = __hip_atomic_fetch_add(slot, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
-                      (unsigned)((own + walk - 1) / walk - 1);
+                      (unsigned)(sharers - 1);
     if (last) __hip_atomic_store(slot, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     merges = last;
   }
@@ -976,18 +982,18 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
     const void* q, long long q_stride, void* out, long long out_stride, float* part_ml,
     float* part_acc, const void* k_pages, const void* v_pages, const int* block_tables,
     int max_pages, const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift, int window,
-    float scale, int splits, int part_keys, int max_parts, int merge_inside, int walk,
+    float scale, int splits, int part_keys, int max_parts, int merge_inside, int groups, int cap,
     const DecodeRope* rope, hipStream_t stream) {
   if (S == 0) return 0;
   if (part_keys % (32 * kDecodeWaves) != 0 || part_keys <= 0) return kUnitBadPartition;
   if (merge_inside && (long long)S * nkv > kArrivalSlots) return kUnitTooManyArrivals;
   const int g = nh / nkv;
-  const size_t smem = (size_t)(walk < 1 ? 1 : walk) * kDecodeWaves * g * (2 + d) * sizeof(float);
+  const size_t smem = (size_t)(cap < 1 ? 1 : cap) * kDecodeWaves * g * (2 + d) * sizeof(float);
   // several partitions per workgroup: merging inside, whole pairs of chunks, and parked sums
   // that fit the LDS (up to head size 64 two workgroups share a compute unit's 160 KB)
   constexpr size_t kWalkBytes = D <= 64 ? 64 * 1024 : 159 * 1024;
-  if (walk < 1 || (walk > 1 && (!merge_inside || part_keys % (64 * kDecodeWaves) != 0 ||
-                                smem > kWalkBytes)))
+  if (cap < 1 || groups < 1 || (cap > 1 && (!merge_inside || part_keys % (64 * kDecodeWaves) != 0 ||
+                                            smem > kWalkBytes)))
     return kUnitBadWalk;
   if (smem > 64 * 1024) {
     // more dynamic LDS than a kernel gets unasked
@@ -1003,13 +1009,17 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
   // rotation inside the kernel needs head_dim = rotated width = 64, 128 or 256
   if (rope->positions && rope->cos && !(D % 64 == 0 && rope->rot == D && d == D))
     return kUnitBadRotation;
-  dim3 grid(nkv, S, (splits + walk - 1) / walk);
+  // deep enough for the sequence with the most partitions, whichever rule binds for it
+  const int by_cap = (splits + cap - 1) / cap;
+  dim3 grid(nkv, S, cap > 1 ? (groups > by_cap ? (groups < splits ? groups : splits) : by_cap)
+                            : splits);
 #define RLIS_DEC_LAUNCH(WALKS)                                                                    \
   DECODE_KERNEL_NAME<WALKS><<<grid, 64 * kDecodeWaves, smem, stream>>>(                          \
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, part_ml, part_acc,                   \
       (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, max_pages, ctx_lens, nh, nkv, \
-      d, page_shift, scale, window, splits, part_keys, max_parts, merge_inside, walk, *rope)
-  if (walk > 1) RLIS_DEC_LAUNCH(true);
+      d, page_shift, scale, window, splits, part_keys, max_parts, merge_inside, groups, cap,   \
+      *rope)
+  if (cap > 1) RLIS_DEC_LAUNCH(true);
   else RLIS_DEC_LAUNCH(false);
 #undef RLIS_DEC_LAUNCH
   RLIS_UNIT_LAUNCH_CHECK();

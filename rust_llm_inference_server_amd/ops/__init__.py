@@ -64,9 +64,10 @@ DECODE_ATTENTION = "matrix"
 # merge inside whatever their size: their workgroups are few.
 MERGE_DECODE_INSIDE = True
 MERGE_DECODE_INSIDE_MAX_BYTES = 9 << 27        # 1.125 GB
-# Partitions that one workgroup of that kernel takes in a row: None = by how many workgroups
-# the batch makes (``attention_plan.decode_walk``), a number = that many (tests: every walk
-# gives the same floats).
+# The most partitions that one workgroup of that kernel takes in a row: None = by how many
+# workgroups the batch makes (``attention_plan.decode_shares``), a number = that many, dealt
+# out to as few workgroups as that allows (tests: the floats are the same however a sequence's
+# partitions are dealt out).
 DECODE_WALK: Optional[int] = None
 
 
@@ -673,19 +674,20 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                 slots_p = None if slots is None else _i32(slots, "slots", S)
                 if cos is not None:
                     cos_p, sin_p, rot = cos.data_ptr(), sin.data_ptr(), 2 * cos.shape[1]
-            walk = DECODE_WALK or ap.decode_walk(S, nkv, depth, nh // nkv, d,
-                                                 _compute_units(qkv.device))
-            # (workgroups that walk partitions are few, and hand over little or nothing)
-            inside = MERGE_DECODE_INSIDE and (walk > 1 or
+            if DECODE_WALK:
+                groups, cap = -(-depth // DECODE_WALK), DECODE_WALK
+            else:
+                groups, cap = ap.decode_shares(S, nkv, depth, nh // nkv, d,
+                                               _compute_units(qkv.device))
+            # (workgroups that take several partitions are few, and hand over little or nothing)
+            inside = MERGE_DECODE_INSIDE and (cap > 1 or
                                               S * nkv * depth * ap.DECODE_PART_KEYS * d * 4
                                               <= MERGE_DECODE_INSIDE_MAX_BYTES)
-            if not inside:
-                walk = 1
             lib.call("rlis_attn_decode_mfma", qkv.data_ptr(), q_stride, out.data_ptr(), nh * d,
                      ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
                      block_tables.data_ptr(), max_pages, _i32(step.ctx_lens, "ctx_lens", S), S,
                      nh, nkv, d, page_size, win, float(scale), depth, ap.DECODE_PART_KEYS,
-                     ap.DECODE_MAX_PARTS, int(inside), walk, cos_p, sin_p, rot, pos_p,
+                     ap.DECODE_MAX_PARTS, int(inside), groups, cap, cos_p, sin_p, rot, pos_p,
                      slots_p, nh * d, (nh + nkv) * d, stream)
         else:
             lib.call("rlis_attn_decode", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(),

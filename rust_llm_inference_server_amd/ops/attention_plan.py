@@ -68,23 +68,27 @@ def decode_walk_room(group: int, head_dim: int) -> int:
     return lds // (8 * group * (head_dim + 2) * 4)
 
 
-def decode_walk(num_seqs: int, num_kv_heads: int, depth: int, group: int, head_dim: int,
-                compute_units: int) -> int:
-    """Partitions that one workgroup of the matrix-core decode kernel takes in a row, for a
-    grid ``depth`` partitions deep.  This is the one choice here that looks at the batch, and
-    it may: the partitions and the order of their sums stay what a sequence's own length makes
-    them, only the workgroups that share them change, and the kernel gives the same floats for
-    every walk.  Sequences times KV heads that fill the compute units by themselves take one
-    workgroup each; fewer keep as many workgroups each as bring them to about what the compute
-    units hold at once (two workgroups each up to head size 64, one beyond).  The eight waves'
-    sums of every walked partition must fit the LDS (``decode_walk_room``), and the kernel walks
-    whole pairs of chunks only (partitions of a multiple of 512 keys)."""
+def decode_shares(num_seqs: int, num_kv_heads: int, depth: int, group: int, head_dim: int,
+                  compute_units: int) -> Tuple[int, int]:
+    """(groups, cap) for the matrix-core decode kernel under a grid ``depth`` partitions deep:
+    a sequence's partitions are dealt out evenly to ``groups`` workgroups, none of which takes
+    more than ``cap`` (a sequence with more partitions than that gets more workgroups); cap 1:
+    a workgroup per partition.  This is the one choice here that looks at the batch, and it
+    may: the partitions and the order of their sums stay what a sequence's own length makes
+    them, only the workgroups that share them change, and the kernel gives the same floats
+    however they are dealt out.  Sequences times KV heads that fill the compute units by
+    themselves take one workgroup each; fewer take as many each as bring them to about what the
+    compute units hold at once (two workgroups each up to head size 64, one beyond).  The
+    eight waves' sums of every partition in a share must fit the LDS (``decode_walk_room``),
+    and the kernel takes shares of whole pairs of chunks only (partitions of a multiple of 512
+    keys)."""
     if depth <= 1 or DECODE_PART_KEYS % 512 != 0:
-        return 1
+        return depth, 1
     resident = 2 if head_dim <= 64 else 1
     each = max(1, compute_units * resident // max(1, num_seqs * num_kv_heads))
-    room = decode_walk_room(group, head_dim)
-    return max(1, min(depth // each, depth, room))
+    groups = min(depth, each)
+    cap = min(decode_walk_room(group, head_dim), -(-depth // groups))
+    return (groups, cap) if cap > 1 else (depth, 1)
 
 
 class AttentionPlanner(StepPlanner):

@@ -87,35 +87,37 @@ def test_decode_partitions_follow_the_sequence_alone():
     assert not fixed.arrays and fixed.values["decode_depth"] == 2 and fixed.values["num_decode"] == 8
 
 
-def test_workgroups_walk_partitions_where_the_batch_fills_the_chip():
-    """How many partitions a decode workgroup takes in a row: one where sequences times KV heads
-    leave compute units idle, all of them where the batch fills the chip by itself; never more
-    than the LDS holds parked sums for, and none unless partitions are whole pairs of chunks."""
+def test_partitions_are_dealt_out_by_how_far_the_batch_fills_the_chip():
+    """(workgroups per sequence and KV head, most partitions in one): a workgroup per partition
+    where sequences times KV heads leave compute units idle, one workgroup for all of them
+    where the batch fills the chip by itself; never more in one than the LDS holds parked sums
+    for, and one each unless partitions are whole pairs of chunks."""
     units = 256
-    # 8 sequences x 8 KV heads: 64 workgroups want 4 partitions each at head size 128, 8 at 64
-    assert ap.decode_walk(8, 8, 4, 4, 128, units) == 1
-    assert ap.decode_walk(8, 8, 8, 4, 128, units) == 2
-    assert ap.decode_walk(8, 8, 8, 4, 64, units) == 1
-    assert ap.decode_walk(8, 8, 5, 4, 128, units) == 1        # never fewer workgroups than asked
-    # 64 x 8 fill the chip: one workgroup walks a sequence's partitions, as far as the LDS goes
-    assert ap.decode_walk(64, 8, 2, 3, 128, units) == 2
-    assert ap.decode_walk(64, 8, 4, 4, 64, units) == 4
-    assert ap.decode_walk(32, 8, 16, 4, 128, units) == 9      # 16.6 KB of parked sums a partition
-    assert ap.decode_walk(32, 8, 16, 3, 128, units) == 13
-    assert ap.decode_walk(64, 8, 16, 4, 64, units) == 7       # 8.4 KB each, in 64 KB
-    assert ap.decode_walk(64, 8, 16, 16, 256, units) == 1     # 132 KB a partition: none to spare
-    assert ap.decode_walk(1, 8, 16, 4, 64, units) == 1
-    assert ap.decode_walk(64, 8, 1, 4, 64, units) == 1
+    # 8 sequences x 8 KV heads: 64 of them want 4 workgroups each at head size 128, 8 at 64
+    assert ap.decode_shares(8, 8, 4, 4, 128, units) == (4, 1)
+    assert ap.decode_shares(8, 8, 8, 4, 128, units) == (4, 2)
+    assert ap.decode_shares(8, 8, 5, 4, 128, units) == (4, 2)     # 5 partitions: 1, 1, 1, 2
+    assert ap.decode_shares(8, 8, 8, 4, 64, units) == (8, 1)
+    # 64 x 8 fill the chip: one workgroup takes a sequence's partitions, as far as the LDS goes
+    assert ap.decode_shares(64, 8, 2, 3, 128, units) == (1, 2)
+    assert ap.decode_shares(64, 8, 4, 4, 64, units) == (1, 4)
+    assert ap.decode_shares(32, 8, 16, 4, 128, units) == (1, 9)   # 16.6 KB of parked sums each
+    assert ap.decode_shares(32, 8, 16, 3, 128, units) == (1, 13)
+    assert ap.decode_shares(64, 8, 16, 4, 64, units) == (1, 7)    # 8.4 KB each, in 64 KB
+    assert ap.decode_shares(64, 8, 16, 16, 256, units) == (16, 1)  # 132 KB each: none to spare
+    assert ap.decode_shares(1, 8, 16, 4, 64, units) == (16, 1)
+    assert ap.decode_shares(64, 8, 1, 4, 64, units) == (1, 1)
     for seqs in (1, 3, 8, 24, 64, 300):
         for depth in range(1, 17):
             for group, d in ((1, 48), (4, 64), (3, 128), (4, 128), (8, 128), (4, 256)):
-                walk = ap.decode_walk(seqs, 8, depth, group, d, units)
-                assert 1 <= walk <= depth
-                assert walk == 1 or walk * 8 * group * (d + 2) * 4 <= (64 if d <= 64 else 159) * 1024
+                groups, cap = ap.decode_shares(seqs, 8, depth, group, d, units)
+                assert 1 <= groups <= depth and 1 <= cap <= depth
+                assert cap == 1 or cap * 8 * group * (d + 2) * 4 <= (64 if d <= 64 else 159) * 1024
+                assert groups == depth if cap == 1 else groups * cap >= depth or cap < depth
     old = ap.DECODE_PART_KEYS
     try:
         ap.DECODE_PART_KEYS = 768                             # a chunk and a half per wave
-        assert ap.decode_walk(64, 8, 4, 4, 64, units) == 1
+        assert ap.decode_shares(64, 8, 4, 4, 64, units) == (4, 1)
     finally:
         ap.DECODE_PART_KEYS = old
 
