@@ -996,14 +996,17 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
                                             smem > kWalkBytes)))
     return kUnitBadWalk;
   if (smem > 64 * 1024) {
-    // more dynamic LDS than a kernel gets unasked
-    static size_t granted = 0;
-    if (smem > granted) {
-      const hipError_t e = hipFuncSetAttribute(
-          reinterpret_cast<const void*>(&DECODE_KERNEL_NAME<true>),
-          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWalkBytes);
+    // more dynamic LDS than a kernel gets unasked: asked for once on every device
+    constexpr int kDevices = 64;
+    static bool granted[kDevices];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return kUnitLaunchFailed + (int)e;
+    if (dev < 0 || dev >= kDevices || !granted[dev]) {
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(&DECODE_KERNEL_NAME<true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWalkBytes);
       if (e != hipSuccess) return kUnitLaunchFailed + (int)e;
-      granted = kWalkBytes;
+      if (dev >= 0 && dev < kDevices) granted[dev] = true;
     }
   }
   // rotation inside the kernel needs head_dim = rotated width = 64, 128 or 256
