@@ -790,28 +790,27 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
   const int region_floats = kDecodeWaves * g * (2 + d);
   constexpr float kLn2 = 0.6931471805599453f;       // attn_reduce works with natural-log maxima
   auto park = [&](int n) __attribute__((always_inline)) {
-    float* ml_s = dsm + n * region_floats;
-    float* acc_s = ml_s + kDecodeWaves * g * 2;
+    float* ml_s = dsm + (WALKS ? n * region_floats : 0);
     const float l_all = xor32_sum(xor16_sum(l_run));
     if (l16 < g) {
       if (lq == 0) {
         ml_s[(wave * g + l16) * 2] = m_run;
         ml_s[(wave * g + l16) * 2 + 1] = l_all;
       }
+      // this lane's dims lq * 4 + r of every block of 16, of its head's row
+      float* row = ml_s + kDecodeWaves * g * 2 + (wave * g + l16) * d + lq * 4;
 #pragma unroll
       for (int db = 0; db < D / 16; ++db)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int dim = db * 16 + lq * 4 + r;
-          if (dim < d) acc_s[(wave * g + l16) * d + dim] = o_acc[db][r];
-        }
+        for (int r = 0; r < 4; ++r)
+          if (db * 16 + lq * 4 + r < d) row[db * 16 + r] = o_acc[db][r];
     }
   };
   // Partition n, dim j of head hh, over the parked waves in wave order: the sum, the base-2
   // maximum and the denominator.
   auto merged = [&](int n, int hh, int j, float& a, float& big, float& lsum)
                     __attribute__((always_inline)) {
-    const float* ml_s = dsm + n * region_floats;
+    const float* ml_s = dsm + (WALKS ? n * region_floats : 0);
     const float* acc_s = ml_s + kDecodeWaves * g * 2;
     // Without branches, so that all the reads are issued together: a wave that saw no key has
     // maximum -inf, weight 0 (selected, since -inf - -inf is no number) and sums of zeros.
@@ -877,10 +876,20 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
     const int hh = i / d, j = i % d;
     const int h = kvh * g + hh;
     float a, big, lsum;
-    if (own == 1) {
+    if (!WALKS || mine == 1) {
+      // one partition: the sequence's only one, or one to hand over
       merged(0, hh, j, a, big, lsum);
-      out[(long long)seq * out_stride + h * d + j] = f32_to_bf16(a / lsum);
-    } else if (WALKS && mine == own) {
+      if (own == 1) {
+        out[(long long)seq * out_stride + h * d + j] = f32_to_bf16(a / lsum);
+      } else {
+        const long long idx = ((long long)seq * nh + h) * splits + first;
+        store_shared_result(part_acc + idx * d + j, a);
+        if (j == 0) {
+          store_shared_result(part_ml + idx * 2, rounded_product(big, kLn2));
+          store_shared_result(part_ml + idx * 2 + 1, lsum);
+        }
+      }
+    } else if (mine == own) {
       // All partitions of the sequence were this workgroup's: it merges them as the last to
       // arrive merges those of other workgroups (below), the same sums in the same order.
       // (the maximum times ln 2 is rounded by itself, as on its way through memory: no fused
