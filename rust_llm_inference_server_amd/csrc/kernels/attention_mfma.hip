@@ -563,10 +563,11 @@ __device__ __forceinline__ float load_shared_result(const float* p) {
 // Up to head size 64 two workgroups share a compute unit (four waves per SIMD, 128 registers
 // each): the bound keeps the compiler from taking the few registers more that would halve that.
 // WALKS: the form in which a workgroup may take several partitions (cap > 1); the other form
-// is spared what that costs in registers.  EXACT: the head is as wide as the unit and a page
-// holds 16 positions, the usual case: with both known to the compiler the offsets of a lane's
-// loads within a key's row and a value's page become constants of the instructions (30 fewer
-// registers at head size 128, a tenth fewer instructions in the chunk loop).
+// is spared what that costs in registers.  EXACT: the head is as wide as the unit, a page holds
+// 16 positions and there is no window, the usual case: with that known to the compiler the
+// offsets of a lane's loads within a key's row and a value's page become constants of the
+// instructions (30 fewer registers at head size 128, a tenth fewer instructions in the chunk
+// loop), and no key is masked for lying in front of a window.
 constexpr int kExactPageShift = 4;
 template <bool WALKS, bool EXACT>
 __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNEL_NAME(
@@ -579,6 +580,7 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
   if constexpr (EXACT) {
     d = D;
     page_shift = kExactPageShift;
+    window = 0;
   }
   // per partition that the workgroup walks: ml waves * g * 2, then acc waves * g * d
   extern __shared__ float dsm[];
@@ -1042,7 +1044,7 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
       (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, max_pages, ctx_lens, nh, nkv, \
       d, page_shift, scale, window, splits, part_keys, max_parts, merge_inside, groups, cap,   \
       *rope)
-  const bool exact = d == D && page_shift == kExactPageShift;
+  const bool exact = d == D && page_shift == kExactPageShift && window <= 0;
   if (cap > 1 && exact) RLIS_DEC_LAUNCH(true, true);
   else if (cap > 1) RLIS_DEC_LAUNCH(true, false);
   else if (exact) RLIS_DEC_LAUNCH(false, true);
