@@ -29,6 +29,7 @@ struct LtApi {
   decltype(&hipblasLtMatmulDescCreate) desc_create = nullptr;
   decltype(&hipblasLtMatmulDescSetAttribute) desc_set = nullptr;
   decltype(&hipblasLtMatrixLayoutCreate) layout_create = nullptr;
+  decltype(&hipblasLtMatrixLayoutSetAttribute) layout_set = nullptr;
   decltype(&hipblasLtMatmulPreferenceCreate) pref_create = nullptr;
   decltype(&hipblasLtMatmulPreferenceSetAttribute) pref_set = nullptr;
   decltype(&hipblasLtMatmulPreferenceDestroy) pref_destroy = nullptr;
@@ -43,8 +44,8 @@ struct LtPlan {
   size_t workspace = 0;
 };
 
-// (device, T, N, K, ldx, ldw, ldy, float32 result, workspace limit)
-using LtKey = std::tuple<int, int, int, int, long long, long long, long long, int, size_t>;
+// (device, T, N, K, ldx, ldw, ldy, float32 result, workspace limit, k slices)
+using LtKey = std::tuple<int, int, int, int, long long, long long, long long, int, size_t, int>;
 
 std::mutex lt_mutex;
 LtApi lt;
@@ -73,6 +74,7 @@ RLIS_API int rlis_lt_open(const char* path) {
                   lookup(lt.desc_create, "hipblasLtMatmulDescCreate") &&
                   lookup(lt.desc_set, "hipblasLtMatmulDescSetAttribute") &&
                   lookup(lt.layout_create, "hipblasLtMatrixLayoutCreate") &&
+                  lookup(lt.layout_set, "hipblasLtMatrixLayoutSetAttribute") &&
                   lookup(lt.pref_create, "hipblasLtMatmulPreferenceCreate") &&
                   lookup(lt.pref_set, "hipblasLtMatmulPreferenceSetAttribute") &&
                   lookup(lt.pref_destroy, "hipblasLtMatmulPreferenceDestroy") &&
@@ -94,14 +96,20 @@ RLIS_API int rlis_lt_is_open() {
 // y (T, N) = x (T, K) W^T for W (N, K), all row-major with rows ldx, ldw, ldy elements apart;
 // x and W bfloat16, y bfloat16 or float32 (out_f32), float32 accumulation.  `workspace` is
 // device memory of workspace_bytes that the caller keeps for these calls (none: 0).
-RLIS_API int rlis_lt_gemm_bf16(const void* X, const void* W, void* Y, int out_f32, int T, int N,
-                               int K, long long ldx, long long ldw, long long ldy,
-                               void* workspace, size_t workspace_bytes, hipStream_t stream) {
+// slices > 1: k is cut into that many equal slices, one batched call, and slice s leaves its
+// float32 partial sums at Y + s * y_stride (a stack for a consumer that adds them in order).
+static int lt_gemm(const void* X, const void* W, void* Y, int out_f32, int T, int N, int K,
+                   long long ldx, long long ldw, long long ldy, int slices, long long y_stride,
+                   void* workspace, size_t workspace_bytes, hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && N > 0 && K > 0 && ldx >= K && ldw >= K && ldy >= N,
                "lt_gemm: bad sizes T=%d N=%d K=%d ldx=%lld ldw=%lld ldy=%lld", T, N, K, ldx, ldw,
                ldy);
+  RLIS_REQUIRE(slices >= 1 && K % slices == 0 && (slices == 1 || (out_f32 && y_stride >= (long long)T * ldy)),
+               "lt_gemm: %d slices of k=%d with results %lld apart", slices, K, y_stride);
   RLIS_REQUIRE(workspace || workspace_bytes == 0, "lt_gemm: a workspace size without a workspace");
   if (T == 0) return 0;
+  const int full_k = K;
+  K /= slices;
   int device = 0;
   hipError_t he = hipGetDevice(&device);
   RLIS_REQUIRE(he == hipSuccess, "lt_gemm: %s", hipGetErrorString(he));
@@ -117,7 +125,7 @@ RLIS_API int rlis_lt_gemm_bf16(const void* X, const void* W, void* Y, int out_f3
       h = lt_handles.emplace(device, made).first;
     }
     handle = h->second;
-    const LtKey key(device, T, N, K, ldx, ldw, ldy, out_f32 ? 1 : 0, workspace_bytes);
+    const LtKey key(device, T, N, full_k, ldx, ldw, ldy, out_f32 ? 1 : 0, workspace_bytes, slices);
     auto p = lt_plans.find(key);
     if (p == lt_plans.end()) {
       // Column-major view: y^T (N, T) = W^T-as-stored transposed (N, K) times x-as-stored (K, T).
@@ -130,6 +138,18 @@ RLIS_API int rlis_lt_gemm_bf16(const void* X, const void* W, void* Y, int out_f3
       ok = ok && lt.layout_create(&made.a, HIP_R_16BF, K, N, ldw) == HIPBLAS_STATUS_SUCCESS;
       ok = ok && lt.layout_create(&made.b, HIP_R_16BF, K, T, ldx) == HIPBLAS_STATUS_SUCCESS;
       ok = ok && lt.layout_create(&made.c, out_type, N, T, ldy) == HIPBLAS_STATUS_SUCCESS;
+      if (slices > 1) {
+        // slice s: k from s * K on in both operands, its result y_stride further on
+        const int32_t count = slices;
+        const int64_t k_step = K, y_step = y_stride;
+        for (hipblasLtMatrixLayout_t m : {made.a, made.b, made.c}) {
+          ok = ok && lt.layout_set(m, HIPBLASLT_MATRIX_LAYOUT_BATCH_COUNT, &count, sizeof(count)) ==
+                         HIPBLAS_STATUS_SUCCESS;
+          ok = ok && lt.layout_set(m, HIPBLASLT_MATRIX_LAYOUT_STRIDED_BATCH_OFFSET,
+                                   m == made.c ? &y_step : &k_step, sizeof(int64_t)) ==
+                         HIPBLAS_STATUS_SUCCESS;
+        }
+      }
       RLIS_REQUIRE(ok, "lt_gemm: cannot describe the product T=%d N=%d K=%d", T, N, K);
       hipblasLtMatmulPreference_t pref = nullptr;
       ok = lt.pref_create(&pref) == HIPBLAS_STATUS_SUCCESS;
@@ -159,4 +179,20 @@ RLIS_API int rlis_lt_gemm_bf16(const void* X, const void* W, void* Y, int out_f3
   RLIS_REQUIRE(st == HIPBLAS_STATUS_SUCCESS, "lt_gemm: the product T=%d N=%d K=%d failed (%d)", T,
                N, K, (int)st);
   return 0;
+}
+
+RLIS_API int rlis_lt_gemm_bf16(const void* X, const void* W, void* Y, int out_f32, int T, int N,
+                               int K, long long ldx, long long ldw, long long ldy,
+                               void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  return lt_gemm(X, W, Y, out_f32, T, N, K, ldx, ldw, ldy, 1, 0, workspace, workspace_bytes, stream);
+}
+
+// The same product as a stack of `slices` float32 partial sums (slices, T, N), y_stride
+// elements apart: one batched call over equal slices of k.
+RLIS_API int rlis_lt_gemm_bf16_slices(const void* X, const void* W, float* Y, int T, int N, int K,
+                                      long long ldx, long long ldw, long long ldy, int slices,
+                                      long long y_stride, void* workspace, size_t workspace_bytes,
+                                      hipStream_t stream) {
+  return lt_gemm(X, W, Y, 1, T, N, K, ldx, ldw, ldy, slices, y_stride, workspace, workspace_bytes,
+                 stream);
 }

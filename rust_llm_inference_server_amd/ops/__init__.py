@@ -81,6 +81,27 @@ def _compute_units(device: torch.device) -> int:
                              else torch.cuda.current_device())
 
 
+# A product over a long k whose result joins the residual stream (the consumer takes a stack of
+# partial sums) at the row counts of a budgeted step: the library's kernels for one such
+# product are few workgroups with long loops over k; as one batched call over slices of k they
+# are more and shorter (3B shape, down projection at 512 rows: 51 -> 36 us, against which the
+# consumer reads 25 MB more).  Rows and k from which on, rows up to which, and the slices' k
+# (the shorter up to LIBRARY_SLICES_FINE_ROWS rows).
+LIBRARY_SLICES_MIN_ROWS = 65
+LIBRARY_SLICES_MAX_ROWS = 1024
+LIBRARY_SLICES_MIN_K = 8192
+LIBRARY_SLICES_FINE_ROWS = 256
+
+
+def library_slices(T: int, K: int) -> int:
+    """k slices of the library's product at ``T`` rows over ``K`` when its consumer takes
+    partial sums (1: one product).  It follows from the row count and k alone."""
+    if not (LIBRARY_SLICES_MIN_ROWS <= T <= LIBRARY_SLICES_MAX_ROWS) or K < LIBRARY_SLICES_MIN_K:
+        return 1
+    step = 1024 if T <= LIBRARY_SLICES_FINE_ROWS else 2048
+    return K // step if K % step == 0 else 1
+
+
 def _dt(t: torch.Tensor) -> int:
     try:
         return _DT[t.dtype]
@@ -233,6 +254,12 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         return y
     if bf16 and aligned and T > STREAM_MAX_ROWS and BF16_GEMM == "library":
         ws = lib.library_workspace(x.device) if LIBRARY_GEMM_DIRECT else None
+        slices = library_slices(T, K) if partials and ws is not None else 1
+        if slices > 1:
+            y = torch.empty((slices, T, N), dtype=torch.float32, device=x.device)
+            lib.call("rlis_lt_gemm_bf16_slices", x.data_ptr(), w.data_ptr(), y.data_ptr(), T, N, K,
+                     ldx, ldw, N, slices, T * N, ws.data_ptr(), ws.numel(), stream)
+            return y
         if ws is not None and out_dtype in (torch.bfloat16, torch.float32):
             y = torch.empty((T, N), dtype=out_dtype, device=x.device)
             lib.call("rlis_lt_gemm_bf16", x.data_ptr(), w.data_ptr(), y.data_ptr(),

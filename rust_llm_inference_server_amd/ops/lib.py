@@ -42,6 +42,7 @@ _SIGNATURES = {
                                 ctypes.c_double, P],
     "rlis_lt_open": [c_char_p],
     "rlis_lt_gemm_bf16": [P, P, P, I, I, I, I, L, L, L, P, ctypes.c_size_t, P],
+    "rlis_lt_gemm_bf16_slices": [P, P, P, I, I, I, L, L, L, I, L, P, ctypes.c_size_t, P],
 }
 
 

@@ -282,6 +282,36 @@ def test_library_product_called_directly(ops, out_dtype, T, N, K):
         ops.LIBRARY_GEMM_DIRECT = old
 
 
+@pytest.mark.parametrize("T,N,K", [(100, 2048, 8192), (512, 3072, 8192), (300, 136, 14336), (1024, 264, 8192),
+                                   (65, 8, 8192)])
+def test_library_product_in_slices_of_k(ops, T, N, K):
+    """A product over a long k whose consumer takes partial sums goes to the library as one
+    batched call over slices of k, at the row counts of a budgeted step: the stack's slices
+    against float64 products over the same slice, their sum against the whole product, rows of
+    the operands inside wider arrays, twice (the kept plan); and the rule for the slices."""
+    from rust_llm_inference_server_amd.ops import lib
+    assert lib.library_workspace(torch.device(DEV)) is not None, "hipBLASLt's entry points were not found"
+    assert ops.library_slices(64, 8192) == 1 and ops.library_slices(2048, 8192) == 1
+    assert ops.library_slices(512, 4096) == 1 and ops.library_slices(512, 8192 + 8) == 1
+    assert ops.library_slices(512, 8192) == 4 and ops.library_slices(256, 8192) == 8
+    assert ops.library_slices(300, 14336) == 7 and ops.library_slices(100, 14336) == 14
+    slices = ops.library_slices(T, K)
+    assert slices > 1
+    wide_x = rnd(T, K + 24, dtype=torch.bfloat16, seed=5)
+    wide_w = rnd(N, K + 8, dtype=torch.bfloat16, seed=6, scale=0.05)
+    for x, w in ((wide_x[:, :K].contiguous(), wide_w[:, :K].contiguous()), (wide_x[:, 8:8 + K], wide_w[:, :K])):
+        for _ in range(2):
+            got = ops.linear(x, w, torch.bfloat16, partials=True)
+            assert got.dtype == torch.float32 and got.shape == (slices, T, N)
+            step = K // slices
+            for s in range(slices):
+                want = (x[:, s * step:(s + 1) * step].double() @ w[:, s * step:(s + 1) * step].double().t()).float()
+                scale = max(1.0, want.abs().max().item())
+                torch.testing.assert_close(got[s], want, atol=2e-5 * scale * math.sqrt(step / 64), rtol=1e-2)
+            whole = ops.linear(x, w, torch.float32)
+            torch.testing.assert_close(got.sum(0), whole, atol=1e-3, rtol=1e-3)
+
+
 @pytest.mark.parametrize("T,N,K,parts,rows", [(1, 2048, 2048, 0, False), (8, 3072, 2048, 1, False),
                                               (16, 344, 104, 2, False), (5, 1001, 4096, 1, False),
                                               (3, 128256, 256, 1, True), (7, 64, 776, 3, True),
