@@ -444,7 +444,13 @@ __global__ void swiglu_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __r
     for (int j = 0; j < 4; ++j) {
       const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
       const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
-      const float r0 = g0 / (1.0f + expf(-g0)) * u0, r1 = g1 / (1.0f + expf(-g1)) * u1;
+      // silu(g) * u with the hardware's exponential and reciprocal (an ulp each, far inside
+      // what the rounding to bfloat16 leaves): the library functions made this kernel spend as
+      // long on arithmetic as on its bytes.
+      const float e0 = __builtin_amdgcn_exp2f(g0 * -1.4426950408889634f);
+      const float e1 = __builtin_amdgcn_exp2f(g1 * -1.4426950408889634f);
+      const float r0 = g0 * __builtin_amdgcn_rcpf(1.0f + e0) * u0;
+      const float r1 = g1 * __builtin_amdgcn_rcpf(1.0f + e1) * u1;
       ow[j] = (uint32_t)f32_to_bf16(r0) | ((uint32_t)f32_to_bf16(r1) << 16);
     }
     *(uint4*)(out + i * 8) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
