@@ -60,7 +60,9 @@ def test_random_configuration_mixed_trace(seed, tmp_path):
 
 # Layer sizes of the larger shapes the engine is meant for (Llama-3.2-3B and Llama-3.1-8B), with
 # one layer and a small vocabulary so that the plain implementation stays quick: widths of 12
-# and 16 k items, a feed-forward width that takes two k slices, head size 128.
+# and 16 k items, a feed-forward width that takes two k slices, head size 128.  The whole
+# prompts bring more than 64 rows to the down projection, whose k of 8,192 and 14,336 then goes
+# to the library in slices.
 LARGE_LAYERS = {
     "3b-layer": dict(hidden_size=3072, intermediate_size=8192, num_attention_heads=24,
                      num_key_value_heads=8, head_dim=128, factor=32.0, tie=True),
@@ -84,14 +86,16 @@ def test_layer_sizes_of_larger_models(name, tmp_path):
     }
     folder = make_model_folder(tmp_path / "m", cfg, seed=11, dtype=torch.bfloat16)
     w, c = plain.read_weights(folder), plain.read_config(folder)
-    reqs = traces.random_requests(cfg["vocab_size"], [70, 9, 40], seed=5)
+    reqs = traces.random_requests(cfg["vocab_size"], [100, 9, 40], seed=5)
     ref = {k: plain.forward(w, c, t) for k, t in reqs.items()}
     spread = max(r.abs().max().item() for r in ref.values())
+    from rust_llm_inference_server_amd import ops
+    assert ops.library_slices(100, p["intermediate_size"]) > 1
     for dtype in ("float32", "bfloat16"):
         # The gates of the tiny models are absolute, for logits of about +-1; these logits are
         # larger, so the gates go with their size.
         tol = TOL[dtype] * max(1.0, spread)
-        for build in (traces.trace_tail, traces.trace_mixed):
+        for build in (traces.trace_whole, traces.trace_tail, traces.trace_mixed):
             steps, max_tokens = build(reqs)
             runner = make_runner(folder, dtype, max_tokens, page_size=16)
             outputs = traces.replay_in_process(runner, steps)
