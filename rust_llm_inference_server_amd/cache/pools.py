@@ -9,8 +9,12 @@ own arrays and gets them the same way.  One page id addresses the same page in e
 slot of its group, as one block id addresses every layer in the reference
 (crates/model/src/paged.rs:1-7, 41-60).  Pools are allocated once, zeroed.
 
-One page beyond the manager's is scratch, and one state slot beyond the manager's: padding
-rows of a captured decode step read and write them, so they touch nothing a request owns."""
+One page beyond the manager's is scratch in every group, and one state slot beyond the
+manager's: padding rows of a captured decode step read and write them, so they touch nothing a
+request owns.
+
+``pool_pages`` is the sizing rule: how many pages each group gets out of one budget of bytes,
+from each group's own bytes per page and window."""
 from __future__ import annotations
 
 from typing import Dict, List, Optional, Sequence
@@ -18,6 +22,42 @@ from typing import Dict, List, Optional, Sequence
 import torch
 
 from ..parts.base import CacheBinding
+
+
+def pool_pages(cache_groups: Sequence, act_dtype: torch.dtype, page_size: int, budget_bytes: int,
+               max_num_seqs: int, max_batched_tokens: int, max_seq_len: int) -> List[int]:
+    """Pages for every group's pool out of ``budget_bytes``.
+
+    A model whose groups all keep every position gets the reference's rule (crates/engine/src/
+    engine.rs:252-262): budget / bytes of one page across all groups, the same count for each.
+    A group that keeps a window only never holds more per request than the window plus the
+    positions of one step that are reserved before the window has moved on (and one page for
+    where in a page the window begins), except at admission, when a request's whole known
+    length is reserved in every group: so its pool is capped at what ``max_num_seqs`` requests
+    hold that way, but never below one request of ``max_seq_len`` (what admission needs), and
+    what the cap leaves of the budget goes to the groups that keep everything."""
+    per_page = [max(1, len(g.writer_runs)) * g.request.bytes_per_token(act_dtype) * page_size
+                for g in cache_groups]
+    if not per_page:
+        return []
+    even = budget_bytes // sum(per_page)
+    pages = [even] * len(per_page)
+    for_one = -(-max_seq_len // page_size) + 1
+    left = budget_bytes
+    full = []
+    for i, g in enumerate(cache_groups):
+        w = g.request.window
+        if w:
+            held = -(-(w + max_batched_tokens) // page_size) + 1
+            pages[i] = min(even, max(for_one, max_num_seqs * held))
+            left -= pages[i] * per_page[i]
+        else:
+            full.append(i)
+    if full and len(full) < len(per_page):
+        share = left // sum(per_page[i] for i in full)
+        for i in full:
+            pages[i] = max(even, share)
+    return pages
 
 
 class CachePools:
@@ -29,13 +69,13 @@ class CachePools:
         self.device = device
         # Per group: array name -> (layer slots, pages + 1, *page shape).
         self.arrays: List[Dict[str, torch.Tensor]] = []
-        self.scratch_page = max(num_pages) if len(num_pages) else 0
+        # Per group: the page beyond the manager's, which padding rows read and write.
+        self.scratch_pages: List[int] = [int(n) for n in num_pages]
         for layout, pages in zip(cache_groups, num_pages):
             n = max(1, len(layout.writer_runs))
-            total = self.scratch_page + 1
             self.arrays.append({
-                a.name: torch.zeros((n, total) + a.page_shape(page_size), dtype=dtype,
-                                    device=device)
+                a.name: torch.zeros((n, int(pages) + 1) + a.page_shape(page_size),
+                                    dtype=a.dtype or dtype, device=device)
                 for a in layout.request.arrays})
         self.state: Optional[torch.Tensor] = None
         self.scratch_state_slot = num_state_slots

@@ -4,7 +4,9 @@ import os
 from typing import List
 
 from .engine import EngineConfig
-from .llama import ConfigError, LlamaConfig, RopeScaling
+from .errors import ConfigError
+from .generation import read_eos_token_ids
+from .llama import LlamaConfig, RopeScaling
 
 _PRESET_DIR = os.path.join(os.path.dirname(__file__), "presets")
 
@@ -23,4 +25,5 @@ def preset_dict(name: str) -> dict:
 
 
 __all__ = ["ConfigError", "EngineConfig", "LlamaConfig", "RopeScaling", "preset_dict",
+           "read_eos_token_ids",
            "preset_names"]

@@ -20,8 +20,7 @@ from dataclasses import dataclass, field
 from typing import Any, Dict, Optional, Tuple
 
 
-class ConfigError(ValueError):
-    """A configuration key is missing, has the wrong type or an unsupported value."""
+from .errors import ConfigError  # noqa: E402  (also found here by its older importers)
 
 
 def _need(d: Dict[str, Any], key: str, typ, where: str = "config.json"):

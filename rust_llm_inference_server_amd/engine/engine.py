@@ -19,6 +19,7 @@ from typing import Callable, Dict, Iterable, List, Optional, Sequence, Tuple, Un
 
 import torch
 
+from ..cache.pools import pool_pages
 from ..config.engine import EngineConfig
 from ..models.spec import Model
 from ..sampling.params import SamplingParams
@@ -100,20 +101,22 @@ class Engine:
         if isinstance(model, str):
             model = load_model(model, dtype, max_positions=cfg.max_seq_len)
         self.model = model
-        elem = 2 if model.act_dtype == torch.bfloat16 else 4
+        budget = max(cfg.max_batched_tokens, cfg.max_num_seqs)
         if cfg.num_pages is not None:
-            num_pages = cfg.num_pages
+            pools = [cfg.num_pages] * max(1, len(model.cache_groups))
         else:
-            # engine.rs:252-262: pool bytes / (bytes of K and V per token * block size)
-            per_token = sum(len(g.writer_runs) * g.request.elements_per_token()
-                            for g in model.cache_groups) * elem
-            num_pages = int(cfg.kv_cache_gb * (1 << 30)) // max(1, per_token * cfg.block_size)
+            # engine.rs:252-262: pool bytes / (bytes of K and V per token * block size), here
+            # per group from its own arrays, dtypes and window
+            pools = pool_pages(model.cache_groups, model.act_dtype, cfg.block_size,
+                               int(cfg.kv_cache_gb * (1 << 30)), cfg.max_num_seqs, budget,
+                               min(cfg.max_seq_len, model.max_positions)) or [2]
+        num_pages = min(pools)
         if num_pages < 2:
             raise ValueError(f"the cache pool holds {num_pages} pages; at least 2 are needed")
         watermark = cfg.watermark_pages
         if watermark is None:
             watermark = max(1, num_pages // 100)            # engine.rs:263-271
-        self.runner = ModelRunner(model, num_pages=num_pages, page_size=cfg.block_size,
+        self.runner = ModelRunner(model, num_pages=pools, page_size=cfg.block_size,
                                   max_num_seqs=cfg.max_num_seqs,
                                   max_batched_tokens=max(cfg.max_batched_tokens, cfg.max_num_seqs),
                                   use_graphs=cfg.use_graphs)
@@ -123,13 +126,17 @@ class Engine:
         # engine.rs:280: the longest request is bounded by the rope table and by the pool
         self.max_seq_len = min(model.max_positions, self.scheduler.max_seq_tokens)
         if eos_token_ids is None:
-            eos_token_ids = getattr(getattr(model, "config", None), "eos_token_ids", ())
+            # what the folder's generation_config.json or config.json named (load_model), else
+            # what the typed configuration carries (a model built in memory)
+            eos_token_ids = getattr(model, "eos_token_ids", None)
+            if eos_token_ids is None:
+                eos_token_ids = getattr(getattr(model, "config", None), "eos_token_ids", ())
         self.eos_token_ids = set(int(t) for t in eos_token_ids)
         self._seqs: Dict[int, _Sequence] = {}
         self._finished: Dict[int, Completion] = {}
         self._flight: Optional[_Flight] = None
         self._next_id = 0
-        self.stats_ = EngineStats(pages_total=num_pages)
+        self.stats_ = EngineStats(pages_total=pools[0])
 
     # ----------------------------------------------------------------- requests
     def add_request(self, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None
@@ -225,7 +232,7 @@ class Engine:
                     entries.append(StepEntry(seq_id, seq.tokens[start:end],
                                              [end - start - 1] if last else []))
                     final.append(last)
-                logits = self.runner.step(entries)
+                logits = self.runner.step(entries, keep=False)    # sampled from at once
         except Exception as exc:
             # engine.rs:523-528: a failed step fails its own requests and no others; their
             # pages are free again and the engine goes on with the rest.

@@ -128,7 +128,7 @@ class DecodeGraph:
         self.h = self.sides[0].h
         self.dev = torch.zeros(meta.size, dtype=torch.int32, device=dev)
         self.seq_ids = np.zeros(B, dtype=np.int64)
-        self.scratch_page = runner.pools.scratch_page
+        self.scratch_pages = list(runner.pools.scratch_pages) or [0] * ng
         self.scratch_state_slot = runner.pools.scratch_state_slot
         dview = lambda name: meta.view(self.dev, name)
         self.groups = [GroupStep(page_size=ps, window=cache.groups[g].window,
@@ -174,8 +174,8 @@ class DecodeGraph:
             h["positions"][S:] = 0
             h["state_slots"][S:] = self.scratch_state_slot
             for g in range(len(self.groups)):
-                h[f"tables{g}"].reshape(B, W)[S:, 0] = self.scratch_page
-                h[f"slots{g}"][S:] = self.scratch_page * self.runner.cache.page_size
+                h[f"tables{g}"].reshape(B, W)[S:, 0] = self.scratch_pages[g]
+                h[f"slots{g}"][S:] = self.scratch_pages[g] * self.runner.cache.page_size
         h["start_pos"][:] = h["positions"]
         h["ctx_lens"][:] = h["positions"] + 1
 

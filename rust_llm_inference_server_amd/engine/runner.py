@@ -9,12 +9,14 @@ program, the perplexity tool and the benchmark all call it.  Its contract is the
 crates/model/src/paged.rs:154-161, 255-296)."""
 from __future__ import annotations
 
+import os
 from typing import Callable, Dict, List, Optional, Sequence, Tuple, Union
 
 import torch
 
 from ..cache.manager import CacheManager, GroupSpec
 from ..cache.pools import CachePools
+from ..config.generation import read_eos_token_ids
 from ..models.spec import Model
 from ..registry import architecture_of, read_config_dict
 from ..weights.loader import load_weights
@@ -56,21 +58,28 @@ def load_model(folder: str, dtype: Union[str, torch.dtype], max_positions: int,
     limit = getattr(cfg, "max_position_embeddings", max_positions)
     model = Model(spec, weights, act, device, min(max_positions, limit))
     model.config = cfg
+    # generation_config.json first, config.json second (crates/engine/src/tokenizer.rs:64-85)
+    model.eos_token_ids = read_eos_token_ids(folder) if os.path.isdir(folder) else ()
     return model
 
 
 def random_model(config: Union[dict, object], seed: int, dtype: Union[str, torch.dtype],
                  max_positions: int, device: Optional[torch.device] = None,
-                 architecture: str = "LlamaForCausalLM") -> Model:
-    """A model with seeded random weights, built in memory from a configuration."""
+                 architecture: Optional[str] = None) -> Model:
+    """A model with seeded random weights, built in memory from a configuration: a config.json
+    dict (its ``architectures`` names the model) or a typed configuration (its ``architecture``
+    does); ``architecture`` names it for a configuration that does not."""
     from ..registry import architecture as lookup
     device = device or default_device()
     act = parse_dtype(dtype)
     if isinstance(config, dict):
-        arch = architecture_of(config) if "architectures" in config else lookup(architecture)
+        arch = lookup(architecture) if architecture else architecture_of(config)
         cfg = arch.parse_config(config)
     else:
-        arch, cfg = lookup(getattr(config, "architecture", architecture)), config
+        name = architecture or getattr(config, "architecture", None)
+        if not name:
+            raise ValueError("random_model: the configuration names no architecture")
+        arch, cfg = lookup(name), config
     spec = arch.build_spec(cfg)
     weights = random_weights(spec.tensor_specs(), seed, act, device)
     limit = getattr(cfg, "max_position_embeddings", max_positions)
@@ -80,9 +89,10 @@ def random_model(config: Union[dict, object], seed: int, dtype: Union[str, torch
 
 
 class ModelRunner:
-    """A model with its cache.  ``num_pages`` sizes every page group's pool."""
+    """A model with its cache.  ``num_pages`` sizes every page group's pool: one number for
+    all of them, or one per group (``cache.pools.pool_pages`` makes those from a budget)."""
 
-    def __init__(self, model: Model, num_pages: int, page_size: int = 16,
+    def __init__(self, model: Model, num_pages: Union[int, Sequence[int]], page_size: int = 16,
                  max_num_seqs: int = 64, max_batched_tokens: Optional[int] = None,
                  use_graphs: bool = True):
         self.model = model
@@ -92,12 +102,19 @@ class ModelRunner:
         self.page_size = page_size
         self.max_num_seqs = max_num_seqs
         self.max_batched_tokens = max_batched_tokens
-        groups = [GroupSpec(num_pages, g.request.window) for g in model.cache_groups]
+        if isinstance(num_pages, int):
+            per_group = [num_pages] * max(1, len(model.cache_groups))
+        else:
+            per_group = [int(n) for n in num_pages]
+            if len(per_group) != max(1, len(model.cache_groups)):
+                raise ValueError(f"{len(per_group)} pool sizes for "
+                                 f"{len(model.cache_groups)} page groups")
+        groups = [GroupSpec(n, g.request.window) for n, g in zip(per_group, model.cache_groups)]
         if not groups:
-            groups = [GroupSpec(num_pages, None)]      # the manager always has one group
+            groups = [GroupSpec(per_group[0], None)]   # the manager always has one group
         self.cache = CacheManager(page_size, groups,
                                   max_num_seqs if model.state_bytes else 0)
-        self.pools = CachePools(model.cache_groups, [num_pages] * len(model.cache_groups),
+        self.pools = CachePools(model.cache_groups, per_group[:len(model.cache_groups)],
                                 page_size, model.act_dtype, model.device,
                                 max_num_seqs if model.state_bytes else 0, model.state_bytes)
         self.vocab_size = model.spec.vocab_size
@@ -134,15 +151,17 @@ class ModelRunner:
         return self.cache.num_computed(seq_id)
 
     # -------------------------------------------------------------------- step
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], keep: bool = True) -> torch.Tensor:
         """Run one batch; returns float32 logits ``(wanted rows, vocab)`` in the order of the
-        entries and of their ``want`` lists."""
+        entries and of their ``want`` lists.  The tensor is the caller's to keep; with
+        ``keep=False`` it may be a view of a captured step's static output, which the next
+        step overwrites (for callers that are done with the logits before they step again)."""
         if len(entries) > self.max_num_seqs:
             raise ValueError(f"{len(entries)} requests in one step, max_num_seqs is "
                              f"{self.max_num_seqs}")
         total = sum(len(e.tokens) for e in entries)
         if self.use_graphs and total == len(entries) and total > 0:
-            return self._decode_step(entries)
+            return self._decode_step(entries, keep)
         if self.max_batched_tokens is not None and total > self.max_batched_tokens:
             raise ValueError(f"{total} tokens in one step, max_batched_tokens is "
                              f"{self.max_batched_tokens}")
@@ -227,9 +246,10 @@ class ModelRunner:
                     made += 1
         return made
 
-    def _decode_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def _decode_step(self, entries: Sequence[StepEntry], keep: bool = True) -> torch.Tensor:
         """A step of one token per request, replayed from the HIP graph of its batch-size
-        bucket (captured at first use).  Same kernels, same results as the eager step."""
+        bucket (captured at first use).  Same kernels, same results as the eager step.  The
+        graph's output is static; ``keep`` copies what is returned out of it."""
         S = len(entries)
         rows: List[int] = []
         for i, e in enumerate(entries):
@@ -240,10 +260,10 @@ class ModelRunner:
         logits = self._decode_lists([e.seq_id for e in entries],
                                     [int(e.tokens[0]) for e in entries], None)
         if rows == list(range(S)):
-            return logits
+            return logits.clone() if keep else logits
         if not rows:
-            return logits[:0]
-        return logits[torch.tensor(rows, device=logits.device)]
+            return logits[:0].clone()
+        return logits[torch.tensor(rows, device=logits.device)]      # (indexing copies)
 
     def _decode_lists(self, seq_ids: Sequence[int], tokens: Optional[Sequence[int]],
                       modes: Optional[Sequence[Tuple[int, float]]], side: int = 0):

@@ -10,6 +10,7 @@ import math
 
 from ..config.llama import LlamaConfig
 from ..parts.base import PartSpec
+from ..registry import Architecture, register_architecture
 from .spec import LayerSpec, ModelSpec
 
 
@@ -48,3 +49,11 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
         head_prefix="lm_head",
         optional_tensors=("lm_head.weight",) if tied else (),
     )
+
+
+register_architecture(Architecture(
+    name="LlamaForCausalLM",
+    parse_config=LlamaConfig.from_dict,
+    build_spec=llama_spec,
+    config_to_dict=lambda cfg: cfg.to_dict(),
+))

@@ -50,15 +50,29 @@ PAGE = -1     # in a PageArray's shape: the axis that is as long as a page has p
 class PageArray:
     """One array a mixer keeps per page: its name and the shape of one page, in which ``PAGE``
     marks the axis of positions.  Keys of 8 heads of 64 are ``("k", (8, PAGE, 64))``; one latent
-    vector of 96 numbers per position is ``("latent", (PAGE, 96))``."""
+    vector of 96 numbers per position is ``("latent", (PAGE, 96))``.  ``dtype`` None: the
+    model's activation dtype; a mixer that caches something in a precision of its own (float32
+    sums in a bfloat16 model, 8-bit codes) names the torch dtype here, and the pools allocate
+    and size that array by it."""
 
     name: str
     shape: Tuple[int, ...]
+    dtype: Optional[torch.dtype] = None
 
     def __post_init__(self):
         if self.shape.count(PAGE) != 1 or any(n <= 0 for n in self.shape if n != PAGE):
             raise ValueError(f"page array '{self.name}': shape {self.shape} needs positive sizes "
                              "and the position axis exactly once")
+        if self.dtype is not None and not isinstance(self.dtype, torch.dtype):
+            raise ValueError(f"page array '{self.name}': dtype must be a torch dtype or None, "
+                             f"got {self.dtype!r}")
+
+    def element_size(self, act_dtype: torch.dtype) -> int:
+        """Bytes of one element, in a model whose activations are ``act_dtype``."""
+        return torch.empty((), dtype=self.dtype or act_dtype).element_size()
+
+    def bytes_per_token(self, act_dtype: torch.dtype) -> int:
+        return self.elements_per_token() * self.element_size(act_dtype)
 
     def page_shape(self, page_size: int) -> Tuple[int, ...]:
         return tuple(page_size if n == PAGE else n for n in self.shape)
@@ -73,7 +87,7 @@ class PageArray:
 @dataclass(frozen=True)
 class CacheRequest:
     """What a mixer keeps in pages for every cached position: a kind of its own, given as the
-    arrays of one page (each in the activation dtype), for every earlier position (``window``
+    arrays of one page (each in the activation dtype unless it names its own), for every earlier position (``window``
     None) or for the last ``window`` positions only.  Mixers with equal requests share a page
     group; the pools are allocated from the request, so a mixer that caches something else than
     keys and values names its own arrays.  ``CacheRequest.kv`` is the kind attention uses."""
@@ -98,6 +112,10 @@ class CacheRequest:
 
     def elements_per_token(self) -> int:
         return sum(a.elements_per_token() for a in self.arrays)
+
+    def bytes_per_token(self, act_dtype: torch.dtype) -> int:
+        """Bytes that one cached position takes in one layer slot of the group."""
+        return sum(a.bytes_per_token(act_dtype) for a in self.arrays)
 
 
 @dataclass

@@ -1,35 +1,50 @@
 """One registry from an architecture's name (``architectures[0]`` of config.json) to its typed
 configuration and its model specification.  The reference dispatches on the file kind only
 (crates/model/src/lib.rs:21-32) and matches names just for GGUF (gguf.rs:64-76); here the name
-in config.json chooses the model everywhere: loader, engine, replay."""
+in config.json chooses the model everywhere: loader, engine, replay.
+
+The registry names no architecture itself.  Each architecture registers from its own module
+(``models/llama.py`` does for ``LlamaForCausalLM``); the modules that ship with the package are
+imported, once, at the first lookup."""
 from __future__ import annotations
 
 import json
 import os
 from dataclasses import dataclass
-from typing import Any, Callable, Dict
+from typing import TYPE_CHECKING, Any, Callable, Dict
 
-from .config.llama import ConfigError, LlamaConfig
-from .models.llama import llama_spec
-from .models.spec import ModelSpec
+from .config.errors import ConfigError
+
+if TYPE_CHECKING:
+    from .models.spec import ModelSpec
 
 
 @dataclass
 class Architecture:
     name: str
     parse_config: Callable[[Dict[str, Any]], Any]      # config.json dict -> typed config
-    build_spec: Callable[[Any], ModelSpec]             # typed config -> model specification
+    build_spec: Callable[[Any], "ModelSpec"]           # typed config -> model specification
     config_to_dict: Callable[[Any], Dict[str, Any]]    # typed config -> config.json dict
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
+_shipped_loaded = False
 
 
 def register_architecture(arch: Architecture) -> None:
     _ARCHITECTURES[arch.name] = arch
 
 
+def _load_shipped() -> None:
+    """Import the package's own model modules, which register their architectures."""
+    global _shipped_loaded
+    if not _shipped_loaded:
+        _shipped_loaded = True
+        from . import models  # noqa: F401
+
+
 def architecture(name: str) -> Architecture:
+    _load_shipped()
     if name not in _ARCHITECTURES:
         raise ConfigError(f"architecture '{name}' is not supported "
                           f"(known: {', '.join(sorted(_ARCHITECTURES))})")
@@ -37,6 +52,7 @@ def architecture(name: str) -> Architecture:
 
 
 def architecture_names():
+    _load_shipped()
     return sorted(_ARCHITECTURES)
 
 
@@ -60,11 +76,3 @@ def read_config_dict(path: str) -> Dict[str, Any]:
     if not isinstance(d, dict):
         raise ConfigError(f"{path}: top level must be an object")
     return d
-
-
-register_architecture(Architecture(
-    name="LlamaForCausalLM",
-    parse_config=LlamaConfig.from_dict,
-    build_spec=llama_spec,
-    config_to_dict=lambda cfg: cfg.to_dict(),
-))

@@ -205,3 +205,55 @@ def test_random_operations_keep_the_invariants(ops, page, window, slots):
     assert m.num_free_pages(0) == 12 and m.num_free_pages(1) == 12
     assert m.num_free_slots() == slots
     m.check_invariants()
+
+
+# ------------------------------------------------------------------ the pools' sizing rule
+class _Layout:
+    """What the pools look at of a model's page group: its cache request and its layer slots."""
+
+    def __init__(self, request, slots):
+        self.request, self.writer_runs = request, list(range(slots))
+
+
+def test_pools_are_sized_per_group_from_their_own_bytes_and_window():
+    """All groups keep everything: the reference's rule, budget / bytes of one page across all
+    groups (crates/engine/src/engine.rs:252-262).  A windowed group is capped at what
+    ``max_num_seqs`` requests can hold of it (window + one step + a page each) but holds one
+    request of the longest length, and the groups that keep everything get what that leaves."""
+    import torch
+    from rust_llm_inference_server_amd.cache.pools import CachePools, pool_pages
+    from rust_llm_inference_server_amd.parts.base import PAGE, CacheRequest, PageArray
+    full = _Layout(CacheRequest.kv(2, 16), slots=3)                  # 3 layers of K and V
+    bf16, f32 = torch.bfloat16, torch.float32
+    per_token = 3 * 2 * 2 * 16
+    budget = 1 << 20
+    assert pool_pages([full], bf16, 16, budget, 8, 64, 512) == [budget // (per_token * 2 * 16)]
+    assert pool_pages([full], f32, 16, budget, 8, 64, 512) == [budget // (per_token * 4 * 16)]
+    assert pool_pages([], bf16, 16, budget, 8, 64, 512) == []
+    # a page array with a dtype of its own is counted by it
+    latent = _Layout(CacheRequest((PageArray("latent", (PAGE, 20), dtype=f32),)), slots=2)
+    assert latent.request.bytes_per_token(bf16) == latent.request.bytes_per_token(f32) == 80
+    both = pool_pages([full, latent], bf16, 16, budget, 8, 64, 512)
+    assert both == [budget // ((per_token * 2 + 2 * 80) * 16)] * 2
+    # a window of 32 in one layer: 8 requests x (ceil((32 + 64) / 16) + 1) = 56 pages, but one
+    # request of 2,048 positions needs 129; the full group gets what is left of the budget
+    win = _Layout(CacheRequest.kv(2, 16, window=32), slots=1)
+    budget = 4 << 20
+    pages = pool_pages([full, win], bf16, 16, budget, 8, 64, 2048)
+    even = budget // ((per_token + 2 * 2 * 16) * 2 * 16)
+    assert even > 129 and pages[1] == 129
+    assert pages[0] == (budget - 129 * (2 * 2 * 16) * 2 * 16) // (per_token * 2 * 16) > even
+    assert pool_pages([full, win], bf16, 16, budget, 8, 64, 128)[1] == 56
+    # never more than an even split would give the windowed group
+    assert pool_pages([full, win], bf16, 16, 1 << 16, 8, 64, 2048)[1] == (1 << 16) // (
+        (per_token + 2 * 2 * 16) * 2 * 16)
+    # the pools follow: each group its own count (+ one scratch page), each array its own dtype
+    pools = CachePools([full, latent, win], [7, 5, 3], 16, bf16, torch.device("cpu"))
+    assert pools.arrays[0]["k"].shape == (3, 8, 2, 16, 16) and pools.arrays[0]["k"].dtype == bf16
+    assert pools.arrays[0]["v"].shape == (3, 8, 2, 16, 16)
+    assert pools.arrays[1]["latent"].shape == (2, 6, 16, 20) and pools.arrays[1]["latent"].dtype == f32
+    assert pools.arrays[2]["k"].shape == (1, 4, 2, 16, 16)
+    assert pools.scratch_pages == [7, 5, 3]
+    assert pools.bytes_per_page(1) == 2 * 16 * 20 * 4 and pools.bytes_per_page(0) == per_token * 2 * 16
+    with pytest.raises(ValueError, match="dtype"):
+        PageArray("x", (PAGE, 4), dtype="float32")

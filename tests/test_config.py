@@ -93,6 +93,30 @@ def test_eos_ids_number_or_list():
     assert LlamaConfig.from_dict(d).eos_token_ids == (7, 9)
 
 
+def test_eos_ids_come_from_generation_config_first(tmp_path):
+    """crates/engine/src/tokenizer.rs:64-85: ``generation_config.json`` decides when it holds
+    ``eos_token_id`` as a number or a list, else ``config.json`` does; a file without the key
+    (or with something else there) is passed over.  ``load_model`` hands the ids to the engine."""
+    import json
+    from rust_llm_inference_server_amd.config import read_eos_token_ids
+    folder = tmp_path / "m"
+    folder.mkdir()
+    assert read_eos_token_ids(str(folder)) == ()
+    (folder / "config.json").write_text(json.dumps(dict(TINY_A, eos_token_id=7)))
+    assert read_eos_token_ids(str(folder)) == (7,)
+    (folder / "generation_config.json").write_text(json.dumps({"temperature": 0.6}))
+    assert read_eos_token_ids(str(folder)) == (7,)                   # no key there: passed over
+    (folder / "generation_config.json").write_text(json.dumps({"eos_token_id": "</s>"}))
+    assert read_eos_token_ids(str(folder)) == (7,)                   # not a number or a list
+    (folder / "generation_config.json").write_text(json.dumps({"eos_token_id": [9, 11, 13]}))
+    assert read_eos_token_ids(str(folder)) == (9, 11, 13)            # the instruct models' case
+    (folder / "generation_config.json").write_text(json.dumps({"eos_token_id": 5}))
+    assert read_eos_token_ids(str(folder)) == (5,)
+    (folder / "generation_config.json").write_text("{broken")
+    with pytest.raises(ConfigError, match="generation_config.json: not valid JSON"):
+        read_eos_token_ids(str(folder))
+
+
 def test_registry_names_the_model_by_its_architecture():
     assert architecture_names() == ["LlamaForCausalLM"]
     arch = architecture_of(TINY_A)

@@ -324,6 +324,36 @@ def test_eos_and_limits(backend, tiny_folders):
         stops.add_request([256], SamplingParams())
 
 
+def test_the_folders_generation_config_names_the_stop_tokens(backend, tiny_folders, tmp_path):
+    """An engine built from a folder stops at the ids of its ``generation_config.json``, which
+    come before those of ``config.json`` (crates/engine/src/tokenizer.rs:64-85)."""
+    import json
+    import shutil
+    from rust_llm_inference_server_amd.engine import Engine
+    prompt = prompts_for(256, [6], seed=6)[0]
+    sp = SamplingParams(temperature=2.0, seed=3, max_tokens=4)       # (greedy repeats itself here)
+    greedy = engine_for(load(tiny_folders["a"], backend, max_positions=128)).generate(
+        [prompt], sp)[0].token_ids
+    assert len(set(greedy[:3])) == 3
+    folder = tmp_path / "with_generation_config"
+    shutil.copytree(tiny_folders["a"], folder)
+    config = json.loads((folder / "config.json").read_text())
+    config["eos_token_id"] = greedy[2]
+    (folder / "config.json").write_text(json.dumps(config))
+    cfg = EngineConfig(max_num_seqs=2, max_batched_tokens=64, num_pages=16, block_size=8, max_seq_len=128)
+
+    def run():
+        engine = Engine(load(str(folder), backend, max_positions=128), cfg)
+        out = engine.generate([prompt], sp)[0]
+        return engine.eos_token_ids, out.finish_reason, out.token_ids
+
+    assert run() == ({greedy[2]}, "stop", greedy[:2])               # config.json alone
+    (folder / "generation_config.json").write_text(json.dumps({"eos_token_id": [greedy[1], 300]}))
+    assert run() == ({greedy[1], 300}, "stop", greedy[:1])          # generation_config.json first
+    (folder / "generation_config.json").write_text(json.dumps({"do_sample": True}))
+    assert run()[1:] == ("stop", greedy[:2])                        # no ids there: config.json
+
+
 def test_cancel_returns_the_pages(backend, tiny_folders):
     model = load(tiny_folders["a"], backend, max_positions=128)
     engine = engine_for(model, num_pages=16)
@@ -353,8 +383,8 @@ def test_decoding_requests_go_to_the_step_longest_context_first(backend, tiny_fo
         held = [len(engine._seqs[i].tokens) for i in order]
         seen.append((list(order), held))
 
-    monkeypatch.setattr(runner, "step", lambda entries: (
-        note([e.seq_id for e in entries if len(e.tokens) == 1]), real_step(entries))[1])
+    monkeypatch.setattr(runner, "step", lambda entries, **kw: (
+        note([e.seq_id for e in entries if len(e.tokens) == 1]), real_step(entries, **kw))[1])
     monkeypatch.setattr(runner, "step_sampled", lambda i, t, m: (note(i), real_sampled(i, t, m))[1])
     monkeypatch.setattr(runner, "step_chained", lambda i, m, side: (
         seen.append((list(i), None)), real_chained(i, m, side))[1])
@@ -381,11 +411,11 @@ def test_a_failed_step_fails_only_its_own_requests(backend, tiny_folders):
     b = engine.add_request(prompts_for(256, [5], seed=1)[0], SamplingParams.greedy(4))
     real, calls = engine.runner.step, []
 
-    def failing(entries):
+    def failing(entries, **kw):
         calls.append([e.seq_id for e in entries])
         if len(calls) == 1:
             raise RuntimeError("the device said no")
-        return real(entries)
+        return real(entries, **kw)
 
     engine.runner.step = failing
     with pytest.raises(RuntimeError, match="the device said no"):

@@ -453,7 +453,8 @@ def register_latent_toy():
     """Defined and registered here, in the test: a mixer whose memory of the past grows with
     the length but is no pair of keys and values.  It keeps one latent vector of ``rank``
     numbers per position in pages of its own kind and gives every token the mean of the latents
-    up to and including its own, projected back up."""
+    up to and including its own, projected back up.  The latents are cached in float32 whatever
+    the model's activation dtype is: the page array names its own dtype."""
     from rust_llm_inference_server_amd.parts import Mixer, TensorSpec, register
     from rust_llm_inference_server_amd.parts.base import PAGE, CacheRequest, PageArray, join
 
@@ -473,7 +474,7 @@ def register_latent_toy():
             self.act_dtype = ctx.act_dtype
 
         def cache_request(self):
-            return CacheRequest((PageArray("latent", (PAGE, self.rank)),))
+            return CacheRequest((PageArray("latent", (PAGE, self.rank), dtype=torch.float32),))
 
         def forward(self, x, step, binding):
             group = step.groups[binding.group]
@@ -556,6 +557,10 @@ def test_toy_mixer_with_a_cache_kind_of_its_own(tmp_path, dtype, tol):
         g = model.cache_groups.index(latent_group)
         assert set(runner.pools.arrays[g]) == {"latent"}
         assert runner.pools.arrays[g]["latent"].shape[2:] == (16, rank)
+        # its pages are float32 in the bfloat16 model too, and are counted as such
+        assert runner.pools.arrays[g]["latent"].dtype == torch.float32
+        assert latent_group.request.bytes_per_token(model.act_dtype) == 4 * rank
+        assert runner.pools.bytes_per_page(g) == 2 * 16 * rank * 4
         got = traces.collect(steps, traces.replay_in_process(runner, steps), 97)
         for k, tokens in reqs.items():
             mine = torch.stack([got[k][p] for p in range(len(tokens))])

@@ -324,3 +324,95 @@ def test_the_two_plain_implementations_agree(tiny_folders, name):
         assert (a - b).abs().max().item() < 1e-4
     # the llama3 bands of the two agree too (tiny b and d scale their frequencies)
     assert abs(b).max().item() > 0.05
+
+
+# ------------------------------------------------- the whole model from library routines
+def library_forward(w, c, ids, mistake=None):
+    """The decoder of crates/model/src/llama.rs:264-286 put together from torch's own routines
+    and nothing of plain_llama's but the inverse frequencies (pinned above by the reference's
+    vector): ``F.embedding``, ``F.rms_norm``, ``F.linear``, ``F.silu``, the rotation as a
+    multiplication of complex numbers (dims j and j + d/2 are the real and imaginary part,
+    rope.rs:5-8) and ``F.scaled_dot_product_attention`` with its own causal mask and its own
+    grouping of query heads (``enable_gqa``: query head h reads KV head h // group,
+    attention.rs:240-245).  ``mistake`` builds a plausible misreading instead."""
+    H, eps = c["hidden_size"], c["rms_norm_eps"]
+    nh, nkv, d = c["num_attention_heads"], c["num_key_value_heads"], c["head_dim"]
+    n = len(ids)
+    angles = torch.outer(torch.arange(n, dtype=torch.float32),
+                         plain.inv_freqs(d, c["rope_theta"], c.get("rope_scaling")))
+    turn = torch.polar(torch.ones_like(angles), angles)[:, None, :]           # e^(i p f_j)
+
+    def rotate(t):                                                             # (n, heads, d)
+        z = torch.complex(t[..., :d // 2].contiguous(), t[..., d // 2:].contiguous()) * turn
+        return torch.cat([z.real, z.imag], dim=-1)
+
+    def norm(x, name):
+        return F.rms_norm(x, (H,), w[name], eps)
+
+    x = F.embedding(torch.tensor(ids), w["model.embed_tokens.weight"])
+    for layer in range(c["num_hidden_layers"]):
+        p = f"model.layers.{layer}"
+
+        def mixer(h):
+            q = rotate(F.linear(h, w[f"{p}.self_attn.q_proj.weight"]).view(n, nh, d))
+            k = rotate(F.linear(h, w[f"{p}.self_attn.k_proj.weight"]).view(n, nkv, d))
+            v = F.linear(h, w[f"{p}.self_attn.v_proj.weight"]).view(n, nkv, d)
+            a = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None],
+                                               v.transpose(0, 1)[None], is_causal=True,
+                                               enable_gqa=True)[0]
+            return F.linear(a.transpose(0, 1).reshape(n, nh * d), w[f"{p}.self_attn.o_proj.weight"])
+
+        def feed_forward(h):
+            return F.linear(F.silu(F.linear(h, w[f"{p}.mlp.gate_proj.weight"]))
+                            * F.linear(h, w[f"{p}.mlp.up_proj.weight"]), w[f"{p}.mlp.down_proj.weight"])
+
+        first, second = f"{p}.input_layernorm.weight", f"{p}.post_attention_layernorm.weight"
+        if mistake == "post-norm":                      # norm after the residual add
+            x = norm(x + mixer(x), first)
+            x = norm(x + feed_forward(x), second)
+        elif mistake == "parallel":                     # both parts read the same stream
+            x = x + mixer(norm(x, first)) + feed_forward(norm(x, second))
+        elif mistake == "one residual":                 # the feed-forward's input is not added back
+            x = x + mixer(norm(x, first))
+            x = feed_forward(norm(x, second))
+        elif mistake == "norms swapped":
+            x = x + mixer(norm(x, second))
+            x = x + feed_forward(norm(x, first))
+        else:                                           # llama.rs:264-279
+            x = x + mixer(norm(x, first))
+            x = x + feed_forward(norm(x, second))
+    if mistake != "no final norm":
+        x = norm(x, "model.norm.weight")                # llama.rs:280-283
+    head = "model.embed_tokens.weight" if c.get("tie_word_embeddings") else "lm_head.weight"
+    return F.linear(x, w[head])
+
+
+@pytest.mark.parametrize("name", ["a", "b", "c", "d"])
+def test_the_whole_model_reduces_to_library_routines(tiny_folders, name):
+    """Block order, the two residual adds, the final norm in front of the head, the rotation's
+    pairing and sign, the grouping of heads and the causal mask, all at once, against a model
+    assembled from the library's routines (each of which is documented on its own): every logit
+    of a 40-token sequence within 1e-5 for the four tiny configurations (tied and untied heads,
+    scaled and unscaled frequencies, head_dim * heads != hidden, one KV head for several
+    queries).  The norm weights are 1 + N(0, 0.02) and are spread further here, so that a norm
+    in the wrong place or a missing one shows; each plausible misreading moves the logits by
+    more than a hundred times the gate.  (The reference holds its model against the
+    ``transformers`` package, scripts/parity/dump_reference.py:99-154; that package's model
+    code is not imported here, so the pin is to the library routines the formulas reduce to.)"""
+    w, c = plain.read_weights(tiny_folders[name]), plain.read_config(tiny_folders[name])
+    g = torch.Generator().manual_seed(5)
+    w = dict(w)
+    for k in w:
+        if k.endswith("norm.weight"):
+            w[k] = w[k] + 0.5 * torch.rand(w[k].shape, generator=g)
+    ids = torch.randint(0, c["vocab_size"], (40,), generator=g).tolist()
+    mine, want = plain.forward(w, c, ids), library_forward(w, c, ids)
+    assert mine.shape == want.shape == (40, c["vocab_size"])
+    assert (mine - want).abs().max().item() < 1e-5
+    assert want.abs().max().item() > 0.05
+    for mistake in ("post-norm", "parallel", "one residual", "norms swapped", "no final norm"):
+        wrong = library_forward(w, c, ids, mistake)
+        assert (mine - wrong).abs().max().item() > 1e-3, mistake
+    # one token at position 0 sees itself only: the attention returns its value, rotation or not
+    one = plain.forward(w, c, ids[:1])
+    assert (one - want[:1]).abs().max().item() < 1e-5
