@@ -9,24 +9,29 @@ the engine (schedule, forward from the paged cache, on-device greedy sampling, t
 back), bracketed by device synchronisation.  On the same line: a 2,048-token prefill with its
 fraction of the bf16 matrix peak, the decode step's achieved fraction of the HBM roofline
 (bytes that must be read: every weight once plus the live requests' cache), and under
-``points`` decode throughput at batch 1, 8 and 64 after 512-token prompts (each with its
-fraction of the HBM roofline, ``..._frac``) and, while the time budget lasts (``--extra-seconds``;
-``--skip-extra`` leaves them out), two more workloads, each in a fresh model:
+``points`` decode throughput at batch 1, 8 and 64 over 256 new tokens after 512-token prompts,
+whatever ``--steps`` says (each with its fraction of the HBM roofline, ``..._frac``, and the mean
+context of its timed steps, ``..._ctx``) and, while the time budget lasts (``--extra-seconds``;
+``--skip-extra`` leaves them out), three more workloads, each in a fresh model:
 
 * ``serve_3b_...``: 64 requests with prompts of 128 to 2,048 tokens through the engine under
   continuous batching with a token budget of 512 (chunked prefill), 256 new tokens each, at the
   Llama-3.2-3B shape: generated tokens per second from the first arrival to the last end;
 * ``long_8b_...``: 32 requests of 8,192 prompt tokens and 128 new tokens each at the
   Llama-3.1-8B shape: the same, plus tokens per second and HBM fraction of the steps that only
-  decode (context about 8,256), and the prompt tokens per second of the steps before them.
+  decode (context about 8,256), and the prompt tokens per second of the steps before them;
+* ``deep_8b_...``: the whole Llama-3.1-8B shape decoding at batch 4 with 32,768 positions each,
+  and one prompt of 8,192 tokens in one step.
 
-Each of the two runs as a child process (the second command below, and the third): a failure
-there is reported on stderr and leaves the headline as it is.
+Each of them runs as a child process (the commands below): a failure there is reported on
+stderr and leaves the headline as it is.
 Weights are random (N(0, 0.02)), prompts are uniform random token ids.
 
     python bench.py --serve --model llama-3.2-3b --max-batched-tokens 512
     python bench.py --serve --model llama-3.1-8b --requests 32 --min-prompt 8192 \\
         --max-prompt 8192 --new-tokens 128 --max-batched-tokens 8192
+    python bench.py --model llama-3.1-8b --batch 4 --context 32768 --prefill-tokens 8192 \
+        --steps 32 --warmup 4 --skip-points
 
 run one of those workloads alone and print its own JSON line."""
 import argparse
@@ -60,14 +65,18 @@ class Shape:
         self.V = cfg["vocab_size"]
         self.layer_params = ((self.nh + 2 * self.nkv) * self.d * self.H + self.H * self.nh * self.d
                              + 3 * self.H * self.I + 2 * self.H)
-        tied = cfg["tie_word_embeddings"]
-        self.weight_bytes = (self.L * self.layer_params + self.V * self.H + self.H
-                             + (0 if tied else self.V * self.H)) * elem
+        # What a decode step reads of the weights: the layers, the final norm and the output
+        # head once (tied or not, it is one (V, H) matrix), and one row of the embedding table
+        # per request; an untied model's embedding table is otherwise not touched.
+        self.step_weight_bytes = (self.L * self.layer_params + self.V * self.H + self.H) * elem
+        self.elem = elem
         self.kv_bytes_per_token = 2 * self.L * self.nkv * self.d * elem
 
     def decode_step_bytes(self, batch: int, mean_context: float) -> float:
-        """What a decode step has to read: every weight once and the live requests' cache."""
-        return self.weight_bytes + batch * mean_context * self.kv_bytes_per_token
+        """What a decode step has to read: every weight it uses once and the live requests'
+        cache."""
+        return (self.step_weight_bytes + batch * self.H * self.elem
+                + batch * mean_context * self.kv_bytes_per_token)
 
     def prefill_flops(self, T: int) -> float:
         linear = 2.0 * T * self.L * (self.layer_params - 2 * self.H)
@@ -172,7 +181,10 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
-    ap.add_argument("--points-context", type=int, default=512)
+    ap.add_argument("--points-context", type=int, default=512,
+                    help="prompt length of the decode points at batch 1, 8 and 64")
+    ap.add_argument("--points-new-tokens", type=int, default=256,
+                    help="timed decode steps of each of those points")
     ap.add_argument("--skip-points", action="store_true")
     ap.add_argument("--skip-prefill", action="store_true")
     ap.add_argument("--skip-extra", action="store_true",
@@ -246,16 +258,23 @@ def main() -> int:
     model, cfg, full_layers = build_model(args.model, args.dtype, args.layers, longest)
     shape = Shape(cfg, elem)
 
-    def decode_run(batch, context, steps, warmup):
+    def decode_run(batch, context, steps, warmup, prompt_len=None):
         """tokens/s, ms/step and mean context of `steps` decode steps of `batch` requests, none
-        of which goes beyond `context`.  Prompts are prefilled in portions under the engine's
+        of which goes beyond `context` (or, with `prompt_len`, after prompts of that length).
+        Prompts are prefilled in portions under the engine's
         token budget while earlier requests already decode, so every request is given room for
         the steps that the prefill of the others takes; the timed steps are pure decode steps."""
         budget = max(args.max_batched_tokens, batch)
+        if prompt_len is not None:
+            budget = max(budget, batch * prompt_len)      # all prompts in one step
+            context = prompt_len
         prefill_steps = -(-batch * context // budget) + 1
         new_tokens = steps + warmup + prefill_steps + 1
-        context = max(context, new_tokens + 16)           # more steps than the context holds
-        prompt_len = context - new_tokens
+        if prompt_len is not None:
+            context = prompt_len + new_tokens
+        else:
+            context = max(context, new_tokens + 16)       # more steps than the context holds
+            prompt_len = context - new_tokens
         pages = batch * (-(-context // PAGE) + 1) + 8
         engine = Engine(model, EngineConfig(max_num_seqs=max(batch, 1), max_batched_tokens=budget,
                                             num_pages=pages, block_size=PAGE,
@@ -311,26 +330,50 @@ def main() -> int:
 
     points = {}
     if not args.skip_points:
-        # the metric's own workload: 512-token prompts, then decode at batch 1, 8 and 64
+        # the metric's own workload: 512-token prompts, then 256 new tokens at batch 1, 8 and 64
+        # (after W untimed decode steps, so the timed steps' mean context is 640 + W)
         for b in (1, 8, 64):
-            steps = min(K, 128)
-            ctx = args.points_context + steps + W
-            v, ms, mean = decode_run(b, ctx, steps, W)
+            v, ms, mean = decode_run(b, 0, args.points_new_tokens, W, prompt_len=args.points_context)
             frac = shape.decode_step_bytes(b, mean) / (ms * 1e-3) / 1e9 / HBM_GBPS
-            name = f"decode_b{b}" if b != args.batch else f"decode_b{b}_ctx{args.points_context}"
+            name = f"decode_b{b}" if b != args.batch else f"decode_b{b}_p{args.points_context}"
             points[name] = round(v, 1)
             points[name + "_frac"] = round(frac, 4)
-            say(f"decode b{b} after {args.points_context}-token prompts: {v:.0f} tok/s, "
-                f"{ms:.3f} ms/step, {frac:.3f} of HBM")
+            points[name + "_ctx"] = round(mean, 1)
+            say(f"decode b{b}, {args.points_new_tokens} new tokens after {args.points_context}-token "
+                f"prompts: {v:.0f} tok/s, {ms:.3f} ms/step, {frac:.3f} of HBM at mean context {mean:.0f}")
 
     # ---- the larger workloads, each in a model of its own ------------------------------------
     extras = [] if args.skip_extra or args.skip_points or args.layers else [
         ("serve_3b", "llama-3.2-3b", dict(n=64, lo=128, hi=2048, new=256, budget=512)),
         ("long_8b", "llama-3.1-8b", dict(n=32, lo=8192, hi=8192, new=128, budget=8192)),
     ]
+    if extras:
+        extras.append(("deep_8b", "llama-3.1-8b", None))
     for key, name, wl in extras:
         if time.time() - started > args.extra_seconds:
             say(f"{key}: left out, the run is older than {args.extra_seconds:.0f}s")
+            continue
+        if wl is None:
+            # the whole 8B shape: decode at batch 4 with 32,768 positions, a prompt of 8,192
+            cmd = [sys.executable, os.path.abspath(__file__), "--model", name, "--dtype", args.dtype,
+                   "--batch", "4", "--context", "32768", "--prefill-tokens", "8192", "--steps", "32",
+                   "--warmup", "4", "--skip-points"]
+            try:
+                child = subprocess.run(cmd, stdout=subprocess.PIPE, text=True, timeout=240)
+                line = (child.stdout.strip().splitlines() or [""])[-1]
+                if child.returncode != 0 or not line.startswith("{"):
+                    raise RuntimeError(f"exit code {child.returncode}")
+                r = json.loads(line)
+                points[f"{key}_b4_ctx32k_tok_s"] = r["value"]
+                points[f"{key}_b4_ctx32k_ms"] = r["ms_per_step"]
+                points[f"{key}_b4_ctx32k_frac"] = r["roofline"]["frac"]
+                points[f"{key}_prefill8192_tok_s"] = r["prefill"]["value"]
+                points[f"{key}_prefill8192_frac"] = r["prefill"]["frac"]
+                say(f"{key}: batch 4 at 32,768 positions {r['ms_per_step']:.2f} ms/step, "
+                    f"{r['roofline']['frac']:.3f} of HBM; prefill of 8,192 tokens "
+                    f"{r['prefill']['value']:.0f} tok/s, {r['prefill']['frac']:.3f} of the matrix peak")
+            except Exception as exc:
+                say(f"{key} failed: {type(exc).__name__}: {exc}")
             continue
         # A process of its own: whatever happens there, the headline below is printed.
         cmd = [sys.executable, os.path.abspath(__file__), "--serve", "--model", name, "--dtype",
@@ -366,7 +409,8 @@ def main() -> int:
                    "hidden": shape.H, "heads": shape.nh, "kv_heads": shape.nkv, "head_dim": shape.d,
                    "intermediate": shape.I, "vocab": shape.V, "global_batch": args.batch,
                    "seq_len": args.context, "page_size": PAGE, "prefill_tokens": T,
-                   "points_context": args.points_context, "parallelism": "single GPU"},
+                   "points_prompt": args.points_context, "points_new_tokens": args.points_new_tokens,
+                   "parallelism": "single GPU"},
         "prefill": prefill, "roofline": roofline, "points": points,
     }))
     return 0
