@@ -60,6 +60,9 @@ def pool_pages(cache_groups: Sequence, act_dtype: torch.dtype, page_size: int, b
     return pages
 
 
+COUNTERS = 1 << 16
+
+
 class CachePools:
     def __init__(self, cache_groups: Sequence, num_pages: Sequence[int], page_size: int,
                  dtype: torch.dtype, device: torch.device, num_state_slots: int = 0,
@@ -77,6 +80,8 @@ class CachePools:
                 a.name: torch.zeros((n, int(pages) + 1) + a.page_shape(page_size),
                                     dtype=a.dtype or dtype, device=device)
                 for a in layout.request.arrays})
+        # Zeros that the kernels of one launch may count in and leave zero again (CacheBinding).
+        self.counters = torch.zeros(COUNTERS, dtype=torch.int32, device=device)
         self.state: Optional[torch.Tensor] = None
         self.scratch_state_slot = num_state_slots
         if state_bytes > 0 and num_state_slots > 0:
@@ -84,7 +89,7 @@ class CachePools:
                                      device=device)
 
     def binding(self, rb) -> CacheBinding:
-        b = CacheBinding(group=rb.group, writes=rb.writes)
+        b = CacheBinding(group=rb.group, writes=rb.writes, counters=self.counters)
         if rb.group >= 0:
             b.pages = {name: t[rb.slot] for name, t in self.arrays[rb.group].items()}
         if rb.state_bytes and self.state is not None:

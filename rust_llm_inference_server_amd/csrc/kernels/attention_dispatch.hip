@@ -15,7 +15,7 @@ typedef int (*DecodeUnit)(const void* q, long long q_stride, void* out, long lon
                           const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift,
                           int window, float scale, int splits, int part_keys, int max_parts,
                           int merge_inside, int groups, int cap, const DecodeRope* rope,
-                          hipStream_t stream);
+                          const DecodeMerge* merge, hipStream_t stream);
 
 // The units (attention_mfma.hip compiled for a padded head size of 32, 64, ... 256) are
 // libraries of their own, built and loaded when a model needs them and registered here.
@@ -116,10 +116,12 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
 // and the new k are rotated by positions[s], without them nothing is; with slots the new k and
 // v go to the pages at slots[s] (page * page_size + offset).
 //
-// merge_inside != 0: the partitions of a sequence are merged by the last of their workgroups to
-// finish, counted in device memory that the library owns, instead of by a second kernel (which
-// still runs for more than 65,536 sequences times KV heads).  Same sums in the same order
-// either way.  Launches that overlap in time on one device must pass 0.
+// arrivals != null: the partitions of a sequence are merged by the last of their workgroups to
+// finish instead of by a second kernel (which still runs for more than arrival_slots sequences
+// times KV heads).  The workgroups count themselves in at arrivals[sequence * nkv + KV head]:
+// arrival_slots counters of the caller's, all zero before the launch and all zero again after
+// it.  Same sums in the same order either way.  Launches that overlap in time (several streams)
+// must not share counters: each stream, or each owner of a stream, brings its own.
 //
 // groups, cap: when merging inside, a sequence's partitions are dealt out evenly to `groups`
 // workgroups (to more where a share would pass `cap` partitions, which is what the LDS holds
@@ -133,8 +135,8 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
                                    const int* block_tables, int max_pages, const int* ctx_lens,
                                    int S, int nh, int nkv, int d, int page_size, int window,
                                    float scale, int splits, int part_keys, int max_parts,
-                                   int merge_inside, int groups, int cap, const float* cos,
-                                   const float* sin,
+                                   unsigned* arrivals, int arrival_slots, int groups, int cap,
+                                   const float* cos, const float* sin,
                                    int rot, const int* positions, const int* slots,
                                    long long k_off, long long v_off, hipStream_t stream) {
   DecodeRope rope;
@@ -175,7 +177,12 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
   while ((1 << page_shift) < page_size) ++page_shift;
   const DecodeUnit unit = decode_units[unit_index(d)];
   RLIS_REQUIRE(unit != nullptr, "attn_decode_mfma: the unit for head size %d is not loaded", d);
-  const int inside = merge_inside && splits > 1 && (long long)S * nkv <= 65536;
+  RLIS_REQUIRE(!arrivals || (arrival_slots > 0 && ((uintptr_t)arrivals % 4) == 0),
+               "attn_decode_mfma: %d arrival counters", arrival_slots);
+  const int inside = arrivals && splits > 1 && (long long)S * nkv <= arrival_slots;
+  DecodeMerge merge;
+  merge.arrivals = inside ? arrivals : nullptr;
+  merge.slots = inside ? arrival_slots : 0;
   RLIS_REQUIRE(groups >= 1 && cap >= 1, "attn_decode_mfma: %d workgroups of up to %d partitions",
                groups, cap);
   if (!inside) cap = 1;           // same floats either way
@@ -184,7 +191,7 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
       "attn_decode_mfma",
       unit(q, q_stride, out, out_stride, part_ml, part_acc, k_pages, v_pages, block_tables,
            max_pages, ctx_lens, S, nh, nkv, d, page_shift, window, scale, splits, part_keys,
-           max_parts, inside, groups, cap, &rope, stream),
+           max_parts, inside, groups, cap, &rope, &merge, stream),
       d);
   if (rc) return rc;
   if (splits > 1 && S > 0 && !inside)

@@ -531,13 +531,10 @@ __device__ __forceinline__ void load8f(const float* p, float (&v)[8]) {
 
 constexpr int kDecodeWaves = 8;
 
-// Arrival counts of the partitions of one (sequence, KV head), for merging inside the kernel:
-// zero when the library is loaded, and set back to zero by the workgroup that merges, so every
-// launch finds zeros.  Each device holds its own copy.  Launches that overlap on one device
-// (two streams) would count into each other's slots: such callers merge outside.
-constexpr int kArrivalSlots = 65536;
+// Arrival counts of the partitions of one (sequence, KV head), for merging inside the kernel,
+// live in the caller's memory (DecodeMerge): zero before a launch, and set back to zero by the
+// workgroup that merges, so the next launch finds zeros.
 constexpr int kMergeAhead = 8;           // partitions whose results the merge loads at once
-static __device__ unsigned decode_arrivals[kArrivalSlots];
 
 // Partial results pass between workgroups of one launch, which may run on different compute
 // dies, each with a cache of its own between it and memory.  They are therefore stored and
@@ -576,7 +573,8 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ ctx_lens,
     int nh, int nkv, int d, int page_shift, float scale, int window, int splits, int part_keys,
-    int max_parts, int merge_inside, int groups, int cap, const DecodeRope rope) {
+    int max_parts, int merge_inside, int groups, int cap, const DecodeRope rope,
+    const DecodeMerge merge) {
   if constexpr (EXACT) {
     d = D;
     page_shift = kExactPageShift;
@@ -941,7 +939,7 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
   __builtin_amdgcn_s_waitcnt(0);         // all counters at zero: this wave's stores have arrived
   __syncthreads();
   if (tid == 0) {
-    unsigned* slot = decode_arrivals + (seq * nkv + kvh);
+    unsigned* slot = merge.arrivals + (seq * nkv + kvh);
     const bool last = __hip_atomic_fetch_add(slot, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
                       (unsigned)(sharers - 1);
     if (last) __hip_atomic_store(slot, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1002,10 +1000,11 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
     float* part_acc, const void* k_pages, const void* v_pages, const int* block_tables,
     int max_pages, const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift, int window,
     float scale, int splits, int part_keys, int max_parts, int merge_inside, int groups, int cap,
-    const DecodeRope* rope, hipStream_t stream) {
+    const DecodeRope* rope, const DecodeMerge* merge, hipStream_t stream) {
   if (S == 0) return 0;
   if (part_keys % (32 * kDecodeWaves) != 0 || part_keys <= 0) return kUnitBadPartition;
-  if (merge_inside && (long long)S * nkv > kArrivalSlots) return kUnitTooManyArrivals;
+  if (merge_inside && (!merge->arrivals || (long long)S * nkv > merge->slots))
+    return kUnitTooManyArrivals;
   const int g = nh / nkv;
   const size_t smem = (size_t)(cap < 1 ? 1 : cap) * kDecodeWaves * g * (2 + d) * sizeof(float);
   // several partitions per workgroup: merging inside, whole pairs of chunks, and parked sums
@@ -1043,7 +1042,7 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, part_ml, part_acc,                   \
       (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, max_pages, ctx_lens, nh, nkv, \
       d, page_shift, scale, window, splits, part_keys, max_parts, merge_inside, groups, cap,   \
-      *rope)
+      *rope, *merge)
   const bool exact = d == D && page_shift == kExactPageShift && window <= 0;
   if (cap > 1 && exact) RLIS_DEC_LAUNCH(true, true);
   else if (cap > 1) RLIS_DEC_LAUNCH(true, false);

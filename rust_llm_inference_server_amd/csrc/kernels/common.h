@@ -131,6 +131,16 @@ struct DecodeRope {
   int rot;                // rotated width of a head
 };
 
+// Where the workgroups of one decode attention launch count themselves in when they merge a
+// sequence's partitions inside the kernel: `slots` counters in device memory, one per (sequence,
+// KV head), that the caller owns.  They are zero before the launch and the workgroup that
+// merges sets its counter back to zero, so they are zero again after it.  Launches that share
+// the counters must not overlap in time: a caller with several streams brings one set each.
+struct DecodeMerge {
+  unsigned* arrivals;     // null: the partitions are merged by a second kernel
+  int slots;
+};
+
 // Keys per partition of a decode context of n visible keys: part_keys up to max_parts
 // partitions, then the multiple of part_keys that keeps them at max_parts.  It depends on the
 // sequence's own length and on constants only, so a sequence is cut (and its partitions are

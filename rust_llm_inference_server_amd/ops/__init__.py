@@ -52,8 +52,10 @@ FORCE_ATTENTION: Optional[str] = None
 DECODE_ATTENTION = "matrix"
 # The matrix-core decode attention merges a sequence's partitions in the workgroup that finishes
 # last instead of in a second kernel (the same sums either way; tests compare the two).  The
-# arrival counts are the library's, one set per device: a caller whose launches overlap on one
-# device (several streams) switches this off.  It pays while the kernel is short: every
+# workgroups count themselves in in ``counters``, int32 zeros that the caller owns (a model's
+# runner brings its own, so two runners on two streams do not count into each other's; a call
+# without them gets a set that all such calls on the device share, one stream at a time).
+# It pays while the kernel is short: every
 # workgroup ends with a round trip to memory in which it streams nothing, about 3 % of a long
 # kernel's time, against the 5 us of the second kernel; so it is used up to this many bytes of
 # keys and values under the grid (partitions x partition length x 2 x head size x 2 bytes: an
@@ -69,6 +71,21 @@ MERGE_DECODE_INSIDE_MAX_BYTES = 9 << 27        # 1.125 GB
 # out to as few workgroups as that allows (tests: the floats are the same however a sequence's
 # partitions are dealt out).
 DECODE_WALK: Optional[int] = None
+
+
+_shared_counters: dict = {}
+
+
+def _counters_for(device: torch.device) -> torch.Tensor:
+    """The arrival counters of callers that bring none: one set per device, made at first use
+    (not under stream capture: a captured step brings its runner's)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    c = _shared_counters.get(index)
+    if c is None:
+        if torch.cuda.is_current_stream_capturing():
+            raise KernelError("attention: a captured step must bring its own counters")
+        c = _shared_counters[index] = torch.zeros(1 << 16, dtype=torch.int32, device=device)
+    return c
 
 
 @functools.lru_cache(maxsize=None)
@@ -583,7 +600,8 @@ def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
                    block_tables: torch.Tensor, step, scale: float,
                    window: Optional[int] = None, write_kv: bool = True,
                    plan: Optional[StepPlan] = None, interleaved: bool = False,
-                   bias_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   bias_slopes: Optional[torch.Tensor] = None,
+                   counters: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``rope_kv_write`` followed by ``paged_attention``.  A decode batch that takes the
     matrix-core decode kernel does both in that kernel when the whole head is rotated
     (rotate-half) and is 64, 128 or 256 wide (or nothing is rotated); ``qkv`` is then left
@@ -602,12 +620,12 @@ def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
         if write_kv and slots is None:
             raise KernelError("rope_attention: a cache write needs slots")
         return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
-                               scale, window, plan=plan,
+                               scale, window, plan=plan, counters=counters,
                                rope=(cos, sin, positions, slots if write_kv else None))
     rope_kv_write(qkv, nh, nkv, d, cos, sin, positions, slots, k_pages, v_pages, page_size,
                   write_kv=write_kv, interleaved=interleaved)
     return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
-                           scale, window, plan=plan, bias_slopes=bias_slopes)
+                           scale, window, plan=plan, bias_slopes=bias_slopes, counters=counters)
 
 
 def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
@@ -615,7 +633,8 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                     block_tables: torch.Tensor, step, scale: float,
                     window: Optional[int] = None, force: Optional[str] = None,
                     rope: Optional[tuple] = None, plan: Optional[StepPlan] = None,
-                    bias_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    bias_slopes: Optional[torch.Tensor] = None,
+                    counters: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of the step's new tokens over the paged cache -> ``(T, nh * d)``.
 
     ``qkv`` holds the rotated queries in its first ``nh * d`` columns; K and V of the new
@@ -631,7 +650,10 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     softmax; the vector-unit kernels take it, so such a batch goes to them.
     ``force`` names one of 'generic', 'decode', 'prefill' for tests.  ``rope`` (from
     ``rope_attention`` only): ``(cos, sin, positions, slots)`` for the matrix-core decode kernel
-    to rotate and store the step's tokens itself."""
+    to rotate and store the step's tokens itself.  ``counters``: int32 zeros on the device, the
+    caller's, in which the matrix-core decode kernel's workgroups count themselves in when they
+    merge partitions inside the kernel (they leave zeros); launches that may overlap in time
+    must not share them."""
     q_stride = _rows_contig(qkv, "qkv")
     T = qkv.shape[0]
     nh, nkv, d = num_heads, num_kv_heads, head_dim
@@ -707,15 +729,19 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                 groups, cap = ap.decode_shares(S, nkv, depth, nh // nkv, d,
                                                _compute_units(qkv.device))
             # (workgroups that take several partitions are few, and hand over little or nothing)
-            inside = MERGE_DECODE_INSIDE and (cap > 1 or
-                                              S * nkv * depth * ap.DECODE_PART_KEYS * d * 4
-                                              <= MERGE_DECODE_INSIDE_MAX_BYTES)
+            inside = depth > 1 and MERGE_DECODE_INSIDE and (
+                cap > 1 or S * nkv * depth * ap.DECODE_PART_KEYS * d * 4
+                <= MERGE_DECODE_INSIDE_MAX_BYTES)
+            arrivals_p, arrival_slots = None, 0
+            if inside:
+                arrivals = counters if counters is not None else _counters_for(qkv.device)
+                arrivals_p, arrival_slots = _i32(arrivals, "counters", 1), arrivals.numel()
             lib.call("rlis_attn_decode_mfma", qkv.data_ptr(), q_stride, out.data_ptr(), nh * d,
                      ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
                      block_tables.data_ptr(), max_pages, _i32(step.ctx_lens, "ctx_lens", S), S,
                      nh, nkv, d, page_size, win, float(scale), depth, ap.DECODE_PART_KEYS,
-                     ap.DECODE_MAX_PARTS, int(inside), groups, cap, cos_p, sin_p, rot, pos_p,
-                     slots_p, nh * d, (nh + nkv) * d, stream)
+                     ap.DECODE_MAX_PARTS, arrivals_p, arrival_slots, groups, cap, cos_p, sin_p,
+                     rot, pos_p, slots_p, nh * d, (nh + nkv) * d, stream)
         else:
             lib.call("rlis_attn_decode", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(),
                      nh * d, ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),

@@ -32,7 +32,7 @@ _SIGNATURES = {
     "rlis_norm_linear_bf16": [P, P, I, I, L, I, P, I, F, P, P, P, P, I, I, I, I, L, L, I, P],
     "rlis_attn_generic": [P, I, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P, P],
     "rlis_attn_decode": [P, I, L, P, L, P, P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, I, I, P, P],
-    "rlis_attn_decode_mfma": [P, L, P, L, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, I, I, I, I, I,
+    "rlis_attn_decode_mfma": [P, L, P, L, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, I, I, P, I, I, I,
                               P, P, I, P, P, L, L, P],
     "rlis_attn_prefill_mfma": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, I, P, P,
                                P],

@@ -86,5 +86,6 @@ class PagedAttention(Mixer):
                                  group.block_tables, step, self.scale, self.window,
                                  write_kv=binding.writes, plan=step.plans.get(self.planner.key()),
                                  interleaved=bool(getattr(self.position, "interleaved", False)),
-                                 bias_slopes=getattr(self.position, "bias_slopes", None))
+                                 bias_slopes=getattr(self.position, "bias_slopes", None),
+                                 counters=binding.counters)
         return ops.pending_linear(out, self.w_o, self.act_dtype)

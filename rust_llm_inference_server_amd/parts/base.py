@@ -127,12 +127,15 @@ class CacheBinding:
     tables and slots of that group).  ``writes`` is false when the run reads the cache another
     run has written in the same step.  ``state`` is the run's slice of the fixed-size
     per-request state buffer, ``(num_slots, state_bytes)`` uint8, or None when the mixer asked
-    for none."""
+    for none.  ``counters`` is a run of int32 zeros on the device that belongs to the runner
+    (and so to its stream): a mixer's kernels may count in it within one launch, the
+    workgroups of the decode attention do when they merge partitions, if they leave zeros."""
 
     group: int = -1
     pages: Dict[str, torch.Tensor] = field(default_factory=dict)
     writes: bool = True
     state: Optional[torch.Tensor] = None
+    counters: Optional[torch.Tensor] = None
 
     @property
     def k_pages(self) -> Optional[torch.Tensor]:

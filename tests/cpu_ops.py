@@ -90,7 +90,7 @@ def attention_planner(num_heads, num_kv_heads, head_dim, dtype, biased=False):
 
 def paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, page_size,
                     block_tables, step, scale, window=None, force=None, plan=None,
-                    bias_slopes=None):
+                    bias_slopes=None, counters=None):
     assert bias_slopes is None, "the test double adds no bias"
     T = qkv.shape[0]
     nh, nkv, d = num_heads, num_kv_heads, head_dim
@@ -114,7 +114,7 @@ def paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, pa
 
 def rope_attention(qkv, num_heads, num_kv_heads, head_dim, cos, sin, positions, slots, k_pages,
                    v_pages, page_size, block_tables, step, scale, window=None, write_kv=True,
-                   plan=None, interleaved=False, bias_slopes=None):
+                   plan=None, interleaved=False, bias_slopes=None, counters=None):
     rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, cos, sin, positions, slots, k_pages,
                   v_pages, page_size, write_kv=write_kv)
     return paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, page_size,

@@ -829,7 +829,9 @@ def test_attention_decode_partitions_merged_inside_the_kernel(ops, nh, nkv, d, p
     to finish does it) against the same kernel followed by the merge kernel: bit for bit the
     same, whichever workgroup comes last, and again on every further call (the arrival counts
     go back to zero by themselves).  Sequences with one partition beside ones with many, and a
-    grid deeper than most sequences need."""
+    grid deeper than most sequences need.  The counts live in the caller's memory: a call with
+    counters of its own gives the same floats and leaves them zero, and a second caller's
+    counters are not touched by it."""
     dtype = torch.bfloat16
     lens = [1, 5, 300, 1024, 1025, 2100, 4000, 9000, 255, 256, 257, 3, 2048, 2049]
     cached, new = [l - 1 for l in lens], [1] * len(lens)
@@ -850,6 +852,18 @@ def test_attention_decode_partitions_merged_inside_the_kernel(ops, nh, nkv, d, p
                     inside = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale,
                                                  window, force="decode")
                     assert torch.equal(inside, outside), f"cut {part_keys} x {max_parts}, call {call}"
+                mine = torch.zeros(len(lens) * nkv, dtype=torch.int32, device=DEV)
+                other = torch.full((64,), 7, dtype=torch.int32, device=DEV)
+                for call in range(2):
+                    inside = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale,
+                                                 window, force="decode", counters=mine)
+                    assert torch.equal(inside, outside)
+                    assert int(mine.abs().sum()) == 0 and int((other - 7).abs().sum()) == 0
+                # fewer counters than (sequence, KV head) pairs: the second kernel merges
+                few = torch.zeros(len(lens) * nkv - 1, dtype=torch.int32, device=DEV)
+                inside = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window,
+                                             force="decode", counters=few)
+                assert torch.equal(inside, outside) and int(few.abs().sum()) == 0
     finally:
         ops.MERGE_DECODE_INSIDE, ops.MERGE_DECODE_INSIDE_MAX_BYTES = old
 

@@ -70,8 +70,9 @@ def test_replay_families(case, dtype, family):
     outputs = traces.replay_in_process(runner, steps)
     worst = check(steps, outputs, reqs, ref, cfg["vocab_size"], TOL[dtype])
     print(f"{name} {dtype} {family}: worst |diff| {worst:.3e}")
-    # every page came back
+    # every page came back, and the kernels left the runner's counters at zero
     assert runner.cache.num_free_pages(0) == runner.cache.num_pages(0)
+    assert int(runner.pools.counters.abs().sum()) == 0
 
 
 def test_engine_matches_the_second_plain_implementation(case):
