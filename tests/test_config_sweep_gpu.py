@@ -92,9 +92,11 @@ def test_layer_sizes_of_larger_models(name, tmp_path):
     from rust_llm_inference_server_amd import ops
     assert ops.library_slices(100, p["intermediate_size"]) > 1
     for dtype in ("float32", "bfloat16"):
-        # The gates of the tiny models are absolute, for logits of about +-1; these logits are
-        # larger, so the gates go with their size.
-        tol = TOL[dtype] * max(1.0, spread)
+        # float32: the reference's absolute gate of 1e-4 as it is (measured 2.1e-5 and 2.9e-5 on
+        # logits of up to 5.1 and 6.0).  bfloat16: the tiny models' gate of 2e-2 is for logits of
+        # about +-1 and goes with the size of these (measured 0.047 and 0.060, 0.009 and 0.010
+        # of the largest logit).
+        tol = TOL[dtype] if dtype == "float32" else TOL[dtype] * max(1.0, spread)
         for build in (traces.trace_whole, traces.trace_tail, traces.trace_mixed):
             steps, max_tokens = build(reqs)
             runner = make_runner(folder, dtype, max_tokens, page_size=16)
