@@ -110,10 +110,25 @@ def plan_name(index: int, array: str) -> str:
     return f"plan{index}.{array}"
 
 
-# Names of the arrays that every step carries, in the order of the host runtime's layout
-# (csrc/runtime/step_builder.h); each page group adds its write slots and block tables.
-_FIXED_ARRAYS = ("ids", "positions", "seq_of_token", "cu", "start_pos", "ctx_lens", "logit_rows",
-                 "state_slots")
+# The arrays that every step carries and how long each is (T tokens, S sequences, R wanted rows),
+# in the order of the host runtime's layout (csrc/runtime/step_builder.h); each page group adds
+# its write slots and its block tables, W pages wide.  This one table lays out the eager step
+# (the runtime's and its Python twin's) and the static buffer of a captured step: an array is
+# declared here once, and filled by the runtime's builder and by the twin.
+COMMON_ARRAYS = (("ids", "T"), ("positions", "T"), ("seq_of_token", "T"), ("cu", "S+1"),
+                 ("start_pos", "S"), ("ctx_lens", "S"), ("logit_rows", "R"), ("state_slots", "S"))
+GROUP_ARRAYS = (("slots{g}", "T"), ("tables{g}", "S*W"))
+
+
+def common_layout(T: int, S: int, R: int, widths: Sequence[int]) -> List[Tuple[str, int]]:
+    """(name, length) of every common array of a step with ``T`` tokens, ``S`` sequences and
+    ``R`` wanted rows whose page groups have block tables ``widths`` pages wide, in order."""
+    def length(kind: str, W: int = 0) -> int:
+        return {"T": T, "S": S, "S+1": S + 1, "R": R, "S*W": S * W}[kind]
+    out = [(name, length(kind)) for name, kind in COMMON_ARRAYS]
+    for g, W in enumerate(widths):
+        out += [(name.format(g=g), length(kind, W)) for name, kind in GROUP_ARRAYS]
+    return out
 
 
 def _common_native(entries: Sequence[StepEntry], cache, vocab_size: int, spare: int):
@@ -135,7 +150,7 @@ def _common_native(entries: Sequence[StepEntry], cache, vocab_size: int, spare: 
         raise ValueError("a request's tokens and wanted indices must be flat lists of integers") \
             from None
     info = np.zeros(6 + ng, dtype=np.int32)
-    offsets = np.zeros(len(_FIXED_ARRAYS) + 2 * ng, dtype=np.int64)
+    offsets = np.zeros(len(COMMON_ARRAYS) + len(GROUP_ARRAYS) * ng, dtype=np.int64)
     order = np.zeros(n, dtype=np.int32)
     args = (n, seqs.ctypes.data, counts.ctypes.data, tokens.ctypes.data, want_counts.ctypes.data,
             wants.ctypes.data)
@@ -144,12 +159,8 @@ def _common_native(entries: Sequence[StepEntry], cache, vocab_size: int, spare: 
     cache.step_fill(*args, vocab_size, host.data_ptr(), total)
     T, S, R = int(info[0]), int(info[1]), int(info[2])
     widths = [int(w) for w in info[6:]]
-    sizes = [T, T, T, S + 1, S, S, R, S]
-    names = list(_FIXED_ARRAYS)
-    for g in range(ng):
-        names += [f"slots{g}", f"tables{g}"]
-        sizes += [T, S * widths[g]]
-    layout = {name: (int(o), int(c)) for name, o, c in zip(names, offsets, sizes)}
+    layout = {name: (int(o), int(c))
+              for (name, c), o in zip(common_layout(T, S, R, widths), offsets)}
     return host, total, layout, (T, S, R, int(info[3]), int(info[4]), int(info[5]), widths,
                                  order.tolist())
 
@@ -296,21 +307,22 @@ def build_step_in_python(entries: Sequence[StepEntry], cache, device: torch.devi
     lengths = StepLengths(np.asarray(start_pos, dtype=np.int64), np.asarray(new, dtype=np.int64),
                           num_single, ps)
 
-    meta = MetadataBuffer()
-    meta.put("ids", np.concatenate(ids))
-    meta.put("positions", np.concatenate(positions))
-    meta.put("seq_of_token", np.repeat(np.arange(S, dtype=np.int32), new))
-    meta.put("cu", cu)
-    meta.put("start_pos", start_pos)
-    meta.put("ctx_lens", ctx_lens)
-    meta.put("logit_rows", logit_rows)
-    meta.put("state_slots", state_slots)
+    made = {"ids": np.concatenate(ids), "positions": np.concatenate(positions),
+            "seq_of_token": np.repeat(np.arange(S, dtype=np.int32), new), "cu": cu,
+            "start_pos": start_pos, "ctx_lens": ctx_lens, "logit_rows": logit_rows,
+            "state_slots": state_slots}
     for g in range(ng):
-        meta.put(f"slots{g}", np.concatenate(slots[g]))
+        made[f"slots{g}"] = np.concatenate(slots[g])
         rows = np.zeros((S, widths[g]), dtype=np.int32)
         for r, t in enumerate(tables[g]):
             rows[r, :len(t)] = np.maximum(np.asarray(t, dtype=np.int32), 0)
-        meta.put(f"tables{g}", rows)
+        made[f"tables{g}"] = rows
+    meta = MetadataBuffer()
+    for name, count in common_layout(T, S, len(logit_rows), widths):
+        meta.put(name, made[name])
+        if meta.offsets[name][1] != count:
+            raise AssertionError(f"step array '{name}' has {meta.offsets[name][1]} entries, "
+                                 f"the layout says {count}")
     host_plans: List[Tuple[Any, HostPlan]] = []
     for k, planner in enumerate(planners):
         plan = planner.plan(lengths)

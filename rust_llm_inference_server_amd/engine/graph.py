@@ -32,7 +32,7 @@ import numpy as np
 import torch
 
 from ..stepplan import StepPlan
-from .batch import GroupStep, MetadataBuffer, StepContext
+from .batch import GroupStep, MetadataBuffer, StepContext, common_layout
 
 
 def bucket_for(n: int, limit: int) -> int:
@@ -108,16 +108,11 @@ class DecodeGraph:
         ps = cache.page_size
         self.width = W = max(8, -(-(-(-model.max_positions // ps)) // 8) * 8)
         ng = cache.num_groups
-        # ---- static layout: the step builder's arrays, at their largest --------------------
+        # ---- static layout: the step builder's arrays for B single tokens, all wanted, with
+        # block tables at their widest --------------------------------------------------------
         self.meta = meta = MetadataBuffer()
-        for name in ("ids", "positions", "seq_of_token"):
-            meta.reserve(name, B)
-        meta.reserve("cu", B + 1)
-        for name in ("start_pos", "ctx_lens", "logit_rows", "state_slots"):
-            meta.reserve(name, B)
-        for g in range(ng):
-            meta.reserve(f"slots{g}", B)
-            meta.reserve(f"tables{g}", B * W)
+        for name, count in common_layout(B, B, B, [W] * ng):
+            meta.reserve(name, count)
         # what the sampling kernel needs per row (bit patterns; 1/T = 0: greedy), for the steps
         # that sample inside the graph
         meta.reserve("sample_keys", B)

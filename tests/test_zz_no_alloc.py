@@ -69,6 +69,14 @@ def test_static_sampling_matches_the_allocating_entry_point_twice_in_a_row():
     # one chunk: no scratch at all
     got, want = _both(lib, *_case(7, 257, seed=3), chunks=1)
     assert got == want
+    # and against the plain implementation itself (argmax and Gumbel-max keyed by the row's
+    # key, crates/model/src/sampling.rs:45-110), not only against the other entry point
+    import plain_llama as plain
+    logits, keys, inv_t = _case(6, 1500, seed=5)
+    got, _ = _both(lib, logits, keys, inv_t, chunks=4)
+    for r in range(6):
+        key = int(keys[r]) & 0xFFFFFFFF
+        assert got[r] == plain.sample_row(logits[r].cpu(), key, float(inv_t[r])), r
 
 
 def test_static_sampling_refuses_more_than_its_scratch_holds():
