@@ -280,6 +280,9 @@ def main() -> int:
                                             num_pages=pages, block_size=PAGE,
                                             max_seq_len=context + 8, watermark_pages=0))
         sp = SamplingParams(max_tokens=new_tokens, ignore_eos=True)
+        # the decode steps' graphs are captured before the first request arrives, as a server
+        # does when it starts (Engine.warm_up): the warm-up steps below are then replays
+        engine.runner.capture_decode_steps(longest=context + 8, max_batch=batch)
         for p in prompts(batch, prompt_len, shape.V):
             engine.add_request(p, sp)
         while engine.stats().prefill_tokens < batch * prompt_len or engine.stats().waiting:
