@@ -249,6 +249,58 @@ def test_window_layers_beside_full_layers(dtype, tol):
     runner.cache.check_invariants()
 
 
+def test_engine_sizes_the_pools_of_windowed_layers_by_their_windows():
+    """An engine over full and windowed layers, its pools cut from one budget of bytes: the
+    windowed groups get what ``max_num_seqs`` requests can hold of them (but room for one
+    request of the longest length, which admission reserves whole), the group that keeps
+    everything gets the rest.  Requests longer than the windows, prompts in portions, more
+    requests than seats: every greedy token is the plain implementation's, the windowed pools
+    never run dry, and every page comes back."""
+    from rust_llm_inference_server_amd.config import EngineConfig
+    from rust_llm_inference_server_amd.engine import Engine
+    from rust_llm_inference_server_amd.models import Model
+    from rust_llm_inference_server_amd.sampling import SamplingParams
+    from rust_llm_inference_server_amd.weights import random_weights
+    layers = [dict(nh=4, nkv=2, d=16, window=None), dict(nh=4, nkv=2, d=16, window=24),
+              dict(nh=2, nkv=1, d=32, window=5)]
+    spec = toy_spec([layer_spec(64, L["nh"], L["nkv"], L["d"], 96, 1e-5, 1e4, L["window"]) for L in layers])
+    w = random_weights(spec.tensor_specs(), 3, torch.float32)
+    model = Model(spec, {k: v.to(DEV) for k, v in w.items()}, torch.float32, DEV, 256)
+    per_page = 64 * 4 * 8                                  # K and V of one layer, a page of 8
+    engine = Engine(model, EngineConfig(kv_cache_gb=100 * 3 * per_page / (1 << 30), block_size=8,
+                                        max_num_seqs=4, max_batched_tokens=32, max_seq_len=256))
+    cache = engine.runner.cache
+    pools = [cache.num_pages(g) for g in range(3)]
+    # window 24: 4 x (ceil((24 + 32) / 8) + 1) = 32 pages, window 5: 4 x 6 = 24; one request of
+    # 256 positions needs 33 either way; the rest of 300 pages' worth of bytes goes to group 0
+    assert pools == [300 - 2 * 33, 33, 33]
+    assert [t.shape[1] for g in engine.runner.pools.arrays for t in g.values()] == \
+        [pools[0] + 1] * 2 + [34] * 4
+    assert engine.max_seq_len == (33 - 1) * 8
+    g = torch.Generator().manual_seed(9)
+    lengths, new = [70, 9, 130, 33, 200, 2, 51], 14
+    prompts = [torch.randint(0, 97, (n,), generator=g).tolist() for n in lengths]
+    low = [cache.num_pages(i) for i in range(3)]
+    ids = [engine.add_request(p, SamplingParams.greedy(new)) for p in prompts]
+    while engine.has_work():
+        engine.step()
+        low = [min(a, cache.num_free_pages(i)) for i, a in enumerate(low)]
+        cache.check_invariants()
+    runs = [(0, None), (1, None), (2, None)]
+    for p, i in zip(prompts, ids):
+        got = engine.pop_finished(i)
+        assert got.finish_reason == "length"
+        tokens = list(p)
+        for t in got.token_ids:
+            logits = plain_toy_forward(w, tokens, layers, runs)[-1]
+            assert int(torch.argmax(logits)) == t, (len(p), len(tokens))
+            tokens.append(t)
+    assert [cache.num_free_pages(i) for i in range(3)] == pools
+    # the windowed pools were used hard (admission reserves whole prompts there) but held
+    assert low[1] < 16 and low[2] < 16 and low[0] > 100, low
+    assert engine.stats().preemptions == 0
+
+
 @pytest.mark.parametrize("dtype,tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
 def test_run_order_names_a_layer_twice_and_shares_a_cache(dtype, tol):
     """Run order: layer 0, layer 1, layer 0 again (a second cache of its own), then layer 1
