@@ -88,7 +88,10 @@ def load() -> ctypes.CDLL:
 # ---------------------------------------------------------------- the library's products
 # Workspace that hipBLASLt may use for a product, per device (what the tensor library grants it
 # on this family of chips).  Allocated when the kernels are loaded and at the first product on
-# any other device, never while a stream is capturing.
+# any other device, never while a stream is capturing.  One per device, not per stream: library
+# products whose algorithm uses the workspace must not overlap in time on one device (an engine
+# runs its steps on one stream; the algorithms that the heuristics have picked for the shapes
+# met so far ask for none).
 LT_WORKSPACE_BYTES = 76 << 20
 _LT_OPEN: Optional[bool] = None
 _LT_WORKSPACES: dict = {}

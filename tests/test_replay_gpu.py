@@ -335,6 +335,56 @@ def test_decode_logits_do_not_depend_on_the_neighbours(tmp_path, use_graphs):
             assert (together[(i, t)].cpu() - ref[len(reqs[k]) - 8 + t]).abs().max().item() < TOL["bfloat16"]
 
 
+def test_two_runners_decode_on_two_streams_at_once(tmp_path):
+    """Two runners over one model, each on a stream and a thread of its own, decode contexts of
+    several partitions at the same time.  The decode attention merges a sequence's partitions
+    inside the kernel and counts the workgroups' arrivals in memory that each runner owns, so
+    neither counts into the other's: both give, step for step and bit for bit, what they give
+    one after the other, and both leave their counters at zero."""
+    import threading
+    from rust_llm_inference_server_amd.engine import ModelRunner, StepEntry, load_model
+    folder = make_model_folder(tmp_path / "long", LONG, seed=6, dtype=torch.bfloat16)
+    model = load_model(folder, "bfloat16", max_positions=4096)
+    reqs = [traces.random_requests(LONG["vocab_size"], [2100 + 24, 3000 + 24, 1030 + 24], seed=s)
+            for s in (5, 6)]
+    steps = 24
+
+    def decode(which, stream, out, barrier=None):
+        with torch.cuda.stream(stream):
+            runner = ModelRunner(model, num_pages=3 * 200, page_size=16, max_num_seqs=4,
+                                 use_graphs=False)
+            keys = sorted(reqs[which])
+            for i, k in enumerate(keys):
+                runner.reserve(i, len(reqs[which][k]))
+                runner.step([StepEntry(i, reqs[which][k][:-steps], [])])
+            stream.synchronize()
+            if barrier is not None:
+                barrier.wait()
+            rows = []
+            for t in range(steps):
+                logits = runner.step([StepEntry(i, [reqs[which][k][len(reqs[which][k]) - steps + t]], [0])
+                                      for i, k in enumerate(keys)])
+                rows.append(logits)
+            stream.synchronize()
+            out[which] = (torch.stack(rows).cpu(), int(runner.pools.counters.abs().sum()))
+
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    apart, together = {}, {}
+    for which in (0, 1):
+        decode(which, streams[which], apart)
+    barrier = threading.Barrier(2)
+    threads = [threading.Thread(target=decode, args=(w, streams[w], together, barrier)) for w in (0, 1)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=120)
+    assert all(not th.is_alive() for th in threads) and set(together) == {0, 1}
+    for which in (0, 1):
+        assert apart[which][1] == 0 and together[which][1] == 0
+        assert torch.equal(together[which][0], apart[which][0]), f"runner {which}"
+    assert not torch.equal(apart[0][0], apart[1][0])
+
+
 @pytest.mark.parametrize("wide", [False, True], ids=["tiles64", "tiles128"])
 def test_long_prompt_whole_and_in_portions(tmp_path, wide):
     """A prompt of 2,600 tokens in one step and in portions of 512 and 200 beside a decoding
