@@ -8,7 +8,8 @@ typedef int (*PrefillUnit)(const void* q, long long q_stride, void* out, long lo
                            int max_pages, const int* cu_seqlens, const int* start_pos,
                            const int* tile_map, int num_tiles, int nh, int nkv, int d,
                            int page_shift, int window, float scale, int tile_queries, int splits,
-                           int row0, float* part_ml, float* part_acc, hipStream_t stream);
+                           int row0, float* part_ml, float* part_acc, const float* cos,
+                           const float* sin, int rot, hipStream_t stream);
 typedef int (*DecodeUnit)(const void* q, long long q_stride, void* out, long long out_stride,
                           float* part_ml, float* part_acc, const void* k_pages,
                           const void* v_pages, const int* block_tables, int max_pages,
@@ -65,6 +66,10 @@ int rlis_launch_attn_reduce_bf16(void* out, long long out_stride, const float* p
 // and part_acc (rows, nh, part_stride, d) float32, indexed by the row relative to row0, and are
 // merged afterwards by rlis_attn_reduce_rows.  part_stride is at least the largest run count
 // (1: no sequence has runs, nothing is stored there).
+//
+// cos == null: q is rotated already.  Otherwise cos/sin are float32 (max positions, rot / 2)
+// with rot = d = 64, 128 or 256, and the kernel turns each query by its position (start_pos of
+// its sequence plus its index among the new tokens) as it loads it; q itself stays as it is.
 RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out,
                                     long long out_stride, const void* k_pages,
                                     const void* v_pages, const int* block_tables, int max_pages,
@@ -72,7 +77,8 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
                                     const int* unit_map, int num_tiles, int nh, int nkv, int d,
                                     int page_size, int window, float scale, int tile_queries,
                                     int splits, int row0, float* part_ml,
-                                    float* part_acc, hipStream_t stream) {
+                                    float* part_acc, const float* cos, const float* sin,
+                                    int rot, hipStream_t stream) {
   // unit_map lists tiles of tile_queries new tokens: 64 (0 means that too) or 128.
   if (tile_queries == 0) tile_queries = 64;
   RLIS_REQUIRE(tile_queries == 64 || tile_queries == 128,
@@ -94,13 +100,15 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
   RLIS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)k_pages % 16) == 0 &&
                    ((uintptr_t)v_pages % 16) == 0,
                "attn_prefill_mfma: operands must be 16-byte aligned with row strides in steps of 8");
+  RLIS_REQUIRE(!cos || (sin && ((uintptr_t)cos % 16) == 0 && ((uintptr_t)sin % 16) == 0),
+               "attn_prefill_mfma: a rotation needs cos and sin, 16-byte aligned");
   const PrefillUnit unit = prefill_units[unit_index(d)];
   RLIS_REQUIRE(unit != nullptr, "attn_prefill_mfma: the unit for head size %d is not loaded", d);
   return unit_result(
       "attn_prefill_mfma",
       unit(q, q_stride, out, out_stride, k_pages, v_pages, block_tables, max_pages, cu_seqlens,
            start_pos, unit_map, num_tiles, nh, nkv, d, page_shift, window, scale, tile_queries,
-           splits, row0, part_ml, part_acc, stream),
+           splits, row0, part_ml, part_acc, cos, sin, rot, stream),
       d);
 }
 

@@ -98,7 +98,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_seqlens,
     const int* __restrict__ start_pos, const int* __restrict__ unit_map, int nh, int nkv, int d,
     int page_shift, float scale, int window, int num_tiles, int tiles_per_round, int part_stride,
-    int row0, float* __restrict__ part_ml, float* __restrict__ part_acc) {
+    int row0, float* __restrict__ part_ml, float* __restrict__ part_acc,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t) {
   constexpr int BN = tile_keys(QB);
   // V^T tile rows: 64 keys padded to a stride of 32 bytes mod 64; 32 keys unpadded, with the
   // 16-byte piece index XORed with (-(row / 4)) & 3, which frees reads and stores of conflicts.
@@ -151,6 +152,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
         qf[b][ks].u = *(const uint4*)(q + (long long)(tok_begin + my_qi[b]) * q_stride + h * d + dim);
       else
         qf[b][ks].u = make_uint4(0, 0, 0, 0);
+    }
+  }
+  // With cos_t the queries arrive unrotated, and the kernel turns them by their positions as
+  // rope_kv_write would have turned them in place (the dispatcher: rot == d == D, a multiple
+  // of 64).  The angles are asked for here, with the queries (a query past the end takes the
+  // last one's: it is zero anyway), and used once the first tiles' loads are on their way.
+  constexpr int QHS = D % 64 == 0 ? D / 64 : 1;
+  float q_cos[QB][QHS][8], q_sin[QB][QHS][8];
+  if constexpr (D % 64 == 0) {
+    if (cos_t != nullptr) {
+#pragma unroll
+      for (int b = 0; b < QB; ++b) {
+        const long long row = (long long)(P + min(my_qi[b], n_new - 1)) * (D / 2);
+#pragma unroll
+        for (int ks = 0; ks < QHS; ++ks) {
+          const float* cs = cos_t + row + ks * 32 + lq * 8;
+          const float* sn = sin_t + row + ks * 32 + lq * 8;
+          *(float4*)&q_cos[b][ks][0] = *(const float4*)cs;
+          *(float4*)&q_cos[b][ks][4] = *(const float4*)(cs + 4);
+          *(float4*)&q_sin[b][ks][0] = *(const float4*)sn;
+          *(float4*)&q_sin[b][ks][4] = *(const float4*)(sn + 4);
+        }
+      }
     }
   }
 
@@ -272,6 +296,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
   RLIS_STORE_TILE(tile_ka, tile_va, 0);
   RLIS_LOAD_TILE(kt0 + 2 * BN, page_ka, page_va, tile_ka, tile_va);
   RLIS_LOAD_PAGES(kt0 + 4 * BN, page_ka, page_va);
+  // The unrotated queries are turned by the angles asked for above (rotate-half over the
+  // whole head): dim j of a lane's fragment ks meets dim j + D / 2 in its fragment ks + D / 64.
+  // Here, behind the first tiles' loads, nothing is waited for that has not arrived anyway.
+  if constexpr (D % 64 == 0) {
+    if (cos_t != nullptr) {
+#pragma unroll
+      for (int b = 0; b < QB; ++b) {
+#pragma unroll
+        for (int ks = 0; ks < QHS; ++ks) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float x1 = (float)qf[b][ks].v[e], x2 = (float)qf[b][ks + QHS].v[e];
+            qf[b][ks].v[e] = (__bf16)(x1 * q_cos[b][ks][e] - x2 * q_sin[b][ks][e]);
+            qf[b][ks + QHS].v[e] = (__bf16)(x2 * q_cos[b][ks][e] + x1 * q_sin[b][ks][e]);
+          }
+        }
+      }
+    }
+  }
   __syncthreads();
   // The arithmetic of one tile, which LDS holds.
   auto compute = [&](int k0, int buf) __attribute__((always_inline)) {
@@ -464,8 +507,11 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
     const void* v_pages, const int* block_tables, int max_pages, const int* cu_seqlens,
     const int* start_pos, const int* tile_map, int num_tiles, int nh, int nkv, int d,
     int page_shift, int window, float scale, int tile_queries, int splits, int row0,
-    float* part_ml, float* part_acc, hipStream_t stream) {
+    float* part_ml, float* part_acc, const float* cos, const float* sin, int rot,
+    hipStream_t stream) {
   if (num_tiles == 0) return 0;
+  // rotation inside the kernel needs head_dim = rotated width = 64, 128 or 256
+  if (cos && !(sin && D % 64 == 0 && rot == D && d == D)) return kUnitBadRotation;
   const long long blocks = (long long)num_tiles * nh;
   if (blocks >= (1ll << 31)) return kUnitTooManyTiles;
   // 256 compute units: a round is the units whose blocks fill them once.
@@ -474,12 +520,14 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
     KERNEL_NAME<2><<<(int)blocks, 256, 0, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,
         (const bf16_t*)v_pages, block_tables, max_pages, cu_seqlens, start_pos, tile_map, nh, nkv,
-        d, page_shift, scale, window, num_tiles, tiles_per_round, splits, row0, part_ml, part_acc);
+        d, page_shift, scale, window, num_tiles, tiles_per_round, splits, row0, part_ml, part_acc, cos,
+        sin);
   else
     KERNEL_NAME<1><<<(int)blocks, 256, 0, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,
         (const bf16_t*)v_pages, block_tables, max_pages, cu_seqlens, start_pos, tile_map, nh, nkv,
-        d, page_shift, scale, window, num_tiles, tiles_per_round, splits, row0, part_ml, part_acc);
+        d, page_shift, scale, window, num_tiles, tiles_per_round, splits, row0, part_ml, part_acc, cos,
+        sin);
   RLIS_UNIT_LAUNCH_CHECK();
   return 0;
 }

@@ -484,7 +484,8 @@ RLIS_API int rlis_swiglu(void* out, const void* gu, int dtype, int T, int I, hip
 // at [v_off, v_off + nkv*d).  The first rot_dim dims of every q and k head are rotated
 // (rotate-half: dim j pairs with j + rot_dim/2; or, `interleaved`, dim 2j pairs with 2j + 1;
 // either way with the j-th angle of the position's row), the rest pass through.  q is rotated in
-// place.  When write_kv is set, rotated k goes to k_pages[page][kv head][offset][d] and v to
+// place (not at all without rotate_q: the consumer turns it as it loads it).  When write_kv is
+// set, rotated k goes to k_pages[page][kv head][offset][d] and v to
 // v_pages[page][kv head][d][offset] (v is stored transposed inside a page), with
 // page = slot / page_size, offset = slot % page_size; rotated k is not stored back to qkv.
 template <typename TX>
@@ -495,7 +496,7 @@ __global__ void rope_kv_write_kernel(TX* __restrict__ qkv, long long row_stride,
                                      const int* __restrict__ positions,
                                      const int* __restrict__ slots, TX* __restrict__ k_pages,
                                      TX* __restrict__ v_pages, int page_size, int write_kv,
-                                     int interleaved) {
+                                     int interleaved, int rotate_q) {
   const int t = blockIdx.x;
   TX* row = qkv + (long long)t * row_stride;
   const int pos = positions[t];
@@ -503,7 +504,7 @@ __global__ void rope_kv_write_kernel(TX* __restrict__ qkv, long long row_stride,
   const float* c = cos_t + (long long)pos * half;
   const float* s = sin_t + (long long)pos * half;
   // q heads: rotate in place.
-  for (int i = threadIdx.x; i < nh * half; i += blockDim.x) {
+  for (int i = threadIdx.x; i < (rotate_q ? nh * half : 0); i += blockDim.x) {
     const int h = i / half, j = i - h * half;
     TX* p = row + h * d;
     const int a = interleaved ? 2 * j : j, b = interleaved ? 2 * j + 1 : j + half;
@@ -542,11 +543,10 @@ __global__ void rope_kv_write_kernel(TX* __restrict__ qkv, long long row_stride,
 }
 
 // bfloat16 with every head segment a multiple of 8 wide: 16-byte accesses.  The first
-// `qk_blocks` workgroups rotate q in place and k into its page, kRopeTokQK tokens each; the
-// others take kRopeTokV tokens times kRopeVCols value columns each and turn them through LDS, so
+// `qk_blocks` workgroups rotate q in place and k into its page, tok_qk tokens each (heads from
+// first_head on: nh when q is left alone); the others take kRopeTokV tokens times kRopeVCols value columns each and turn them through LDS, so
 // that lanes which are neighbours in a page's (d, offset) layout store neighbouring offsets
 // (tokens with adjacent slots fill whole 32-byte runs, whatever their alignment).
-constexpr int kRopeTokQK = 2;
 constexpr int kRopeTokV = 16;
 constexpr int kRopeVCols = 256;                // v columns per workgroup
 constexpr int kRopeVRow = kRopeVCols + 8;      // padded: rows stay 16-byte aligned, banks spread
@@ -572,18 +572,18 @@ __global__ __launch_bounds__(256) void rope_kv_write_bf16x8_kernel(
     int d, int rot_dim, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int* __restrict__ positions, const int* __restrict__ slots,
     bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages, int page_size, int write_kv,
-    int qk_blocks) {
+    int qk_blocks, int tok_qk, int first_head) {
   const int tid = threadIdx.x;
   const int half = rot_dim / 2;
   if ((int)blockIdx.x < qk_blocks) {
-    const int t0 = blockIdx.x * kRopeTokQK;
+    const int t0 = blockIdx.x * tok_qk;
     const int hc = half / 8;                             // chunks of 8 pairs per head
-    const int heads = nh + (write_kv ? nkv : 0);
+    const int heads = nh + (write_kv ? nkv : 0) - first_head;
     const int per_tok = heads * hc;
-    for (int i = tid; i < kRopeTokQK * per_tok; i += blockDim.x) {
+    for (int i = tid; i < tok_qk * per_tok; i += blockDim.x) {
       const int tt = i / per_tok, r = i - tt * per_tok, t = t0 + tt;
       if (t >= T) break;
-      const int h = r / hc, j = (r - h * hc) * 8;
+      const int h = first_head + r / hc, j = (r - (h - first_head) * hc) * 8;
       const bool is_k = h >= nh;
       const int slot = is_k ? slots[t] : 0;
       if (slot < 0) continue;
@@ -612,7 +612,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_bf16x8_kernel(
     }
     if (write_kv && d > rot_dim) {                       // the dims of k that are not rotated
       const int tc = (d - rot_dim) / 8, per = nkv * tc;
-      for (int i = tid; i < kRopeTokQK * per; i += blockDim.x) {
+      for (int i = tid; i < tok_qk * per; i += blockDim.x) {
         const int tt = i / per, r = i - tt * per, t = t0 + tt;
         if (t >= T) break;
         const int h = r / tc, j = rot_dim + (r - h * tc) * 8;
@@ -661,34 +661,41 @@ RLIS_API int rlis_rope_kv_write(void* qkv, int dtype, long long row_stride, int 
                                 int T, int nh, int nkv, int d, int rot_dim, const float* cos_t,
                                 const float* sin_t, const int* positions, const int* slots,
                                 void* k_pages, void* v_pages, int page_size, int write_kv,
-                                int interleaved, hipStream_t stream) {
+                                int interleaved, int rotate_q, hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && d > 0, "rope_kv_write: bad sizes");
   RLIS_REQUIRE(rot_dim >= 0 && rot_dim <= d && rot_dim % 2 == 0,
                "rope_kv_write: rot_dim %d must be even and at most head_dim %d", rot_dim, d);
   RLIS_REQUIRE(!write_kv || (page_size > 0 && k_pages && v_pages && slots),
                "rope_kv_write: cache write asked for without pages");
-  if (T == 0) return 0;
+  if (T == 0 || (!rotate_q && !write_kv)) return 0;
   const bool by8 = !interleaved && dtype == RLIS_BF16 && d % 8 == 0 && rot_dim % 16 == 0 && row_stride % 8 == 0 &&
                    k_off % 8 == 0 && v_off % 8 == 0 && ((uintptr_t)qkv % 16) == 0 &&
                    ((uintptr_t)cos_t % 16) == 0 && ((uintptr_t)sin_t % 16) == 0 &&
                    (!write_kv || (((uintptr_t)k_pages % 16) == 0 && T <= (1 << 30)));
   if (by8) {
-    const int qk_blocks = ceil_div(T, kRopeTokQK);
+    // about 64 chunks of 8 pairs or more to a workgroup of the first kind
+    const int first_head = rotate_q ? 0 : nh;
+    const int per_tok = (nh + (write_kv ? nkv : 0) - first_head) * (rot_dim / 16);
+    int tok_qk = 2;
+    while (tok_qk < 16 && tok_qk * per_tok < 256) tok_qk *= 2;
+    const int qk_blocks = (per_tok > 0 || (write_kv && d > rot_dim)) ? ceil_div(T, tok_qk) : 0;
     const int v_blocks = write_kv ? ceil_div(T, kRopeTokV) * ceil_div(nkv * d, kRopeVCols) : 0;
+    if (qk_blocks + v_blocks == 0) return 0;             // nothing is rotated, nothing stored
     rope_kv_write_bf16x8_kernel<<<qk_blocks + v_blocks, 256, 0, stream>>>(
         (bf16_t*)qkv, row_stride, k_off, v_off, T, nh, nkv, d, rot_dim, cos_t, sin_t, positions,
-        slots, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, write_kv, qk_blocks);
+        slots, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, write_kv, qk_blocks, tok_qk,
+        first_head);
     RLIS_LAUNCH_CHECK("rope_kv_write");
     return 0;
   }
   if (dtype == RLIS_F32)
     rope_kv_write_kernel<float><<<T, 256, 0, stream>>>(
         (float*)qkv, row_stride, k_off, v_off, nh, nkv, d, rot_dim, cos_t, sin_t, positions,
-        slots, (float*)k_pages, (float*)v_pages, page_size, write_kv, interleaved);
+        slots, (float*)k_pages, (float*)v_pages, page_size, write_kv, interleaved, rotate_q);
   else if (dtype == RLIS_BF16)
     rope_kv_write_kernel<bf16_t><<<T, 256, 0, stream>>>(
         (bf16_t*)qkv, row_stride, k_off, v_off, nh, nkv, d, rot_dim, cos_t, sin_t, positions,
-        slots, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, write_kv, interleaved);
+        slots, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, write_kv, interleaved, rotate_q);
   else
     RLIS_REQUIRE(false, "rope_kv_write: unknown dtype %d", dtype);
   RLIS_LAUNCH_CHECK("rope_kv_write");

@@ -37,6 +37,9 @@ FUSE_NORM_LINEAR = True
 JOIN_NORM_LINEAR = True
 # The matrix-core decode attention rotates q and k and stores the new k, v itself where it can.
 FUSE_ROPE_DECODE = True
+# The matrix-core prefill attention rotates its queries as it loads them where it can (the
+# rotation kernel then turns and stores the keys and values only).
+FUSE_ROPE_PREFILL = True
 # "library": bf16 products with more rows than the streaming kernel takes go to torch
 # (hipBLASLt); "own": they take the hand-written skinny and matrix-core kernels.
 BF16_GEMM = "library"
@@ -490,9 +493,11 @@ def rope_kv_write(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
                   cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
                   positions: torch.Tensor, slots: Optional[torch.Tensor],
                   k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor],
-                  page_size: int, write_kv: bool = True, interleaved: bool = False) -> None:
+                  page_size: int, write_kv: bool = True, interleaved: bool = False,
+                  rotate_q: bool = True) -> None:
     """Rotate the q and k heads of ``qkv (T, (nh + 2 nkv) d)`` by their positions (q in
-    place) and, when ``write_kv``, store rotated k and v into the pages at ``slots``.
+    place; not at all without ``rotate_q``, for a consumer that turns q as it loads it) and,
+    when ``write_kv``, store rotated k and v into the pages at ``slots``.
     The rotation pairs dim ``j`` with ``j + rot/2`` (rotate-half, the reference's), or with
     ``interleaved`` dim ``2j`` with ``2j + 1``.
 
@@ -527,7 +532,8 @@ def rope_kv_write(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
         kp, vp, sp = k_pages.data_ptr(), v_pages.data_ptr(), _i32(slots, "slots", T)
     lib.call("rlis_rope_kv_write", qkv.data_ptr(), _dt(qkv), stride, nh * d, (nh + nkv) * d, T,
              nh, nkv, d, rot, cos_ptr, sin_ptr, _i32(positions, "positions", T), sp, kp, vp,
-             page_size, int(bool(write_kv)), int(bool(interleaved)), lib.stream_ptr())
+             page_size, int(bool(write_kv)), int(bool(interleaved)), int(bool(rotate_q)),
+             lib.stream_ptr())
 
 
 def copy_pages(pages: torch.Tensor, src: torch.Tensor, dst: torch.Tensor) -> None:
@@ -605,23 +611,35 @@ def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
     """``rope_kv_write`` followed by ``paged_attention``.  A decode batch that takes the
     matrix-core decode kernel does both in that kernel when the whole head is rotated
     (rotate-half) and is 64, 128 or 256 wide (or nothing is rotated); ``qkv`` is then left
-    unrotated.  ``interleaved`` and ``bias_slopes`` as in ``rope_kv_write`` and
-    ``paged_attention``."""
+    unrotated.  Under the same conditions a batch with portions of prompts leaves the queries
+    unrotated too: ``rope_kv_write`` turns and stores the keys and values alone, and the
+    matrix-core kernels (prefill for the portions, decode for single tokens beside them) turn
+    each query as they load it.  ``interleaved`` and ``bias_slopes`` as in ``rope_kv_write``
+    and ``paged_attention``."""
     nh, nkv, d = num_heads, num_kv_heads, head_dim
     _rows_contig(qkv, "qkv")
     kind, mfma = _attention_kernel(qkv, nh, nkv, d, page_size, step, None, bias_slopes is not None)
     fusable = cos is None or (2 * cos.shape[1] == d and d in (64, 128, 256) and not interleaved)
-    if mfma and fusable and FUSE_ROPE_DECODE and qkv.shape[1] == (nh + 2 * nkv) * d:
-        if cos is not None:
-            _check(cos, "cos", torch.float32, 2)
-            _check(sin, "sin", torch.float32, 2)
-            if cos.shape != sin.shape or not (cos.is_contiguous() and sin.is_contiguous()):
-                raise KernelError("rope_attention: cos and sin must match and be contiguous")
+    whole_rows = qkv.shape[1] == (nh + 2 * nkv) * d
+    if cos is not None and fusable and whole_rows and (mfma or kind == "prefill"):
+        _check(cos, "cos", torch.float32, 2)
+        _check(sin, "sin", torch.float32, 2)
+        if cos.shape != sin.shape or not (cos.is_contiguous() and sin.is_contiguous()):
+            raise KernelError("rope_attention: cos and sin must match and be contiguous")
+    if mfma and fusable and FUSE_ROPE_DECODE and whole_rows:
         if write_kv and slots is None:
             raise KernelError("rope_attention: a cache write needs slots")
         return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
                                scale, window, plan=plan, counters=counters,
                                rope=(cos, sin, positions, slots if write_kv else None))
+    if (kind == "prefill" and cos is not None and fusable and FUSE_ROPE_PREFILL and whole_rows
+            and (_decode_mfma_ok(qkv, nh, nkv, d, page_size)
+                 or (plan is not None and not plan.value("num_decode")))):
+        rope_kv_write(qkv, nh, nkv, d, cos, sin, positions, slots, k_pages, v_pages, page_size,
+                      write_kv=write_kv, rotate_q=False)
+        return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
+                               scale, window, plan=plan, counters=counters,
+                               rope=(cos, sin, positions, None))
     rope_kv_write(qkv, nh, nkv, d, cos, sin, positions, slots, k_pages, v_pages, page_size,
                   write_kv=write_kv, interleaved=interleaved)
     return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
@@ -650,7 +668,9 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     softmax; the vector-unit kernels take it, so such a batch goes to them.
     ``force`` names one of 'generic', 'decode', 'prefill' for tests.  ``rope`` (from
     ``rope_attention`` only): ``(cos, sin, positions, slots)`` for the matrix-core decode kernel
-    to rotate and store the step's tokens itself.  ``counters``: int32 zeros on the device, the
+    to rotate and store the step's tokens itself; with portions of prompts in the batch
+    ``slots`` is None (the pages hold the step's keys and values already) and both matrix-core
+    kernels turn the unrotated queries as they load them.  ``counters``: int32 zeros on the device, the
     caller's, in which the matrix-core decode kernel's workgroups count themselves in when they
     merge partitions inside the kernel (they leave zeros); launches that may overlap in time
     must not share them."""
@@ -685,8 +705,10 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
             raise KernelError(f"attention: {bias_slopes.numel()} bias slopes for {nh} heads")
         slopes_ptr = bias_slopes.data_ptr()
     kind, mfma = _attention_kernel(qkv, nh, nkv, d, page_size, step, force, slopes_ptr is not None)
-    if rope is not None and not mfma:
-        raise KernelError("attention: only the matrix-core decode kernel rotates and stores")
+    if rope is not None and not (mfma or (kind == "prefill" and rope[3] is None
+                                          and rope[0] is not None)):
+        raise KernelError("attention: only the matrix-core kernels rotate, and only the decode "
+                          "kernel stores")
     if slopes_ptr is not None and kind == "prefill":
         raise KernelError("attention: the matrix-core prefill kernel takes no bias on the scores")
     if kind == "generic":
@@ -779,6 +801,10 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     ml_ptr = None if part_ml is None else part_ml.data_ptr()
     acc_ptr = None if part_acc is None else part_acc.data_ptr()
     launched = False
+    cos_p = sin_p = None
+    rot = 0
+    if rope is not None:
+        cos_p, sin_p, rot = rope[0].data_ptr(), rope[1].data_ptr(), 2 * rope[0].shape[1]
     # Tiles of 64 queries, and tiles of 128 (two query blocks per wave, half the LDS traffic per
     # flop) for the sequences whose own lengths ask for them.
     for tile, name in ((64, "units64"), (128, "units128")):
@@ -792,7 +818,7 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                  _i32(step.cu_seqlens, "cu_seqlens", step.num_seqs + 1),
                  _i32(step.start_pos, "start_pos", step.num_seqs),
                  _i32(plan[name], name, 4 * n), n, nh, nkv, d, page_size, win, float(scale), tile,
-                 max_runs, row0, ml_ptr, acc_ptr, stream)
+                 max_runs, row0, ml_ptr, acc_ptr, cos_p, sin_p, rot, stream)
     if not launched and T > row0:
         raise KernelError("attention: the plan holds no tiles for the step's portions")
     if launched and max_runs > 1:

@@ -19,7 +19,7 @@ _SIGNATURES = {
     "rlis_add_residual": [P, P, I, L, I, I, P],
     "rlis_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, I, L, I, P],
     "rlis_swiglu": [P, P, I, I, I, P],
-    "rlis_rope_kv_write": [P, I, L, I, I, I, I, I, I, I, P, P, P, P, P, P, I, I, I, P],
+    "rlis_rope_kv_write": [P, I, L, I, I, I, I, I, I, I, P, P, P, P, P, P, I, I, I, I, P],
     "rlis_copy_pages": [P, I, I, L, L, P, P, I, P],
     "rlis_gemm_plain": [P, I, P, I, P, I, I, I, I, L, L, L, P],
     "rlis_gemm_bf16_mfma": [P, P, P, I, I, I, I, L, L, L, P],
@@ -35,7 +35,7 @@ _SIGNATURES = {
     "rlis_attn_decode_mfma": [P, L, P, L, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, I, I, P, I, I, I,
                               P, P, I, P, P, L, L, P],
     "rlis_attn_prefill_mfma": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, I, P, P,
-                               P],
+                               P, P, I, P],
     "rlis_attn_reduce_rows": [P, L, P, P, P, P, I, I, I, I, I, P],
     "rlis_sample_rows": [P, L, I, I, P, P, P, I, P, P, P],
     "rlis_fill_normal_device": [P, I, L, ctypes.c_ulonglong, ctypes.c_ulonglong, ctypes.c_double,

@@ -805,6 +805,55 @@ def test_rope_attention_decode_in_one_kernel(ops, nh, nkv, d, ps, rotate, window
                 assert torch.equal(k1, kp.float().cpu()) and torch.equal(v1, vp.cpu())
 
 
+@pytest.mark.parametrize("nh,nkv,d,ps", [(32, 8, 64, 16), (24, 8, 128, 16), (8, 2, 256, 16), (8, 8, 64, 32),
+                                         (5, 5, 48, 16), (34, 2, 64, 16), (16, 2, 256, 16)])
+@pytest.mark.parametrize("window", [None, 70])
+def test_rope_attention_turns_queries_inside_the_prefill_kernel(ops, nh, nkv, d, ps, window):
+    """A batch with portions of prompts: rope_kv_write leaves q alone and the matrix-core
+    kernels (prefill for the portions in tiles of 64 and of 128 queries and with their keys cut
+    into runs, decode for the single tokens that lead the batch) turn each query as they load
+    it, against rope_kv_write on all heads followed by attention: same output within a
+    rounding, the very same pages, q left unrotated.  Head size 48, and groups of query heads
+    that the decode kernel does not take (17 heads per KV head; 8 heads of 256 dims) with
+    single tokens in the batch, take the two-kernel path inside rope_attention."""
+    dtype = torch.bfloat16
+    cached = [5, 63, 300, 0, 40, 0, 130, 17, 2100, 700]
+    new = [1, 1, 1, 33, 70, 2, 129, 64, 150, 300]
+    scale = 1.0 / math.sqrt(d)
+    qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=d + 3)
+    ang = rnd(max(c + n for c, n in zip(cached, new)) + 1, d // 2, seed=7, scale=3.0)
+    cos, sin = torch.cos(ang), torch.sin(ang)
+    tables = bt.cpu()
+    slots = torch.tensor([int(tables[s, p // ps]) * ps + p % ps
+                          for s, (c, n) in enumerate(zip(cached, new)) for p in range(c, c + n)],
+                         dtype=torch.int32, device=DEV)
+    results = []
+    for fused in (False, True):
+        q2, k2, v2 = qkv.clone(), kp.clone(), vp.clone()
+        old = ops.FUSE_ROPE_PREFILL
+        try:
+            ops.FUSE_ROPE_PREFILL = fused
+            out = ops.rope_attention(q2, nh, nkv, d, cos, sin, step.positions, slots, k2, v2, ps,
+                                     bt, step, scale, window)
+        finally:
+            ops.FUSE_ROPE_PREFILL = old
+        results.append((out.float().cpu(), q2.cpu(), k2.cpu(), v2.cpu()))
+    (o0, q0, k0, v0), (o1, q1, k1, v1) = results
+    torch.testing.assert_close(o1, o0, atol=2e-2, rtol=2e-2)
+    assert torch.equal(k1, k0) and torch.equal(v1, v0)
+    g = nh // nkv
+    takes_it = d in (64, 128, 256) and g <= 16 and g * (d + 2) * 32 <= 65536
+    assert torch.equal(q1[:, :nh * d], qkv.cpu()[:, :nh * d]) == takes_it
+    assert not torch.equal(q0[:, :nh * d], qkv.cpu()[:, :nh * d])
+    # and the rotated queries' result is the plain one over the keys that the pages now hold
+    for s, (c, n) in enumerate(zip(cached, new)):
+        for p in range(c, c + n):
+            ks[s][p] = k0[int(tables[s, p // ps]), :, p % ps, :].float()
+            vs[s][p] = v0[int(tables[s, p // ps]), :, :, p % ps].float()
+    want = reference_attention(q0, ks, vs, cu, cached, new, nh, nkv, d, scale, window)
+    torch.testing.assert_close(o1, want, atol=2e-2, rtol=2e-2)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_decode_long_split(ops, dtype, decode_kind):
     """Long contexts beside short ones with many partitions, some of them empty
