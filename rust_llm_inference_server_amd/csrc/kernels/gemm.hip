@@ -626,7 +626,7 @@ RLIS_API int rlis_gemm_bf16_splitk(const void* X, const void* W, void* Y, int T,
 // ============================================================ streaming skinny product
 // y (T <= 16, N) = x W^T at the speed of the weight stream.
 //
-// Work is cut into tiles of 16 (or 8) weight rows times a k slice of up to 16 items of 256; a
+// Work is cut into tiles of 16 (or 12, or 8) weight rows times a k slice of up to 16 items of 256; a
 // workgroup has one wave per item and walks over tiles (persistent, its slice fixed), so the
 // rows of x that a wave needs are loaded once, straight into operand layout, and stay in
 // registers.  An item's weights are loaded row by row, 512 contiguous bytes per half wave,
@@ -634,9 +634,13 @@ RLIS_API int rlis_gemm_bf16_splitk(const void* X, const void* W, void* Y, int T,
 // matrix-core operand wants lane l to hold row l % 16 instead, so the item goes through an
 // LDS tile private to the wave (chunks XOR-swizzled by row, so both directions are free of
 // bank conflicts).  One v_mfma_f32_16x16x32_bf16 accumulator per wave; the waves of a
-// workgroup are summed in LDS in wave order.  With more than one slice (K > 4096) every slice
-// stores its own float32 partial result, which the consumer adds in slice order: the order
-// of a sum depends on K alone.  The gated form pairs gate rows with their up rows in one
+// workgroup are summed in LDS in wave order.  Rows of 4096 < K <= 8192 in whole fours of items
+// stay in one slice (plain and joining products only, tiles of 8 weight rows): a wave then
+// takes four neighbouring items (IPW = 4; at most eight waves, which leaves each the registers
+// for four items of x), each through an LDS tile of its own into the same accumulator, so that
+// a projection over a feed-forward's width can still add itself to the residual.  With more than
+// one slice (K > 8192) every slice stores its own float32 partial result, which the consumer
+// adds in slice order: the order of a sum depends on K alone.  The gated form pairs gate rows with their up rows in one
 // tile and applies the SwiGLU before the store.
 constexpr int kStreamItem = 256;                        // k per item
 constexpr int kStreamTileBytes = 16 * kStreamItem * 2;  // one wave's tile in LDS
@@ -704,8 +708,9 @@ __device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
 // the prologue), the scale from partial sums of squares, or joining the residual at the end.
 enum { kStreamPlain = 0, kStreamNorm = 1, kStreamScaled = 2, kStreamJoin = 3 };
 
-template <typename TC, bool GATED, int TR /* weight rows per tile: 16 or 8 */, int MODE>
-__global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __restrict__ X,
+template <typename TC, bool GATED, int TR /* weight rows per tile: 16, 12 or 8 */, int MODE,
+          int IPW /* k items per wave: 1 or 4 */>
+__global__ __launch_bounds__(IPW == 1 ? 1024 : 512) void gemm_bf16_stream_kernel(const bf16_t* __restrict__ X,
                                                                 const bf16_t* __restrict__ W,
                                                                 TC* __restrict__ Y,
                                                                 const StreamShape sh,
@@ -714,25 +719,41 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
   constexpr bool NORM = MODE == kStreamNorm, SCALED = MODE == kStreamScaled;
   constexpr bool JOIN = MODE == kStreamJoin;
   static_assert(!(JOIN && GATED), "a product that joins the residual has no gate");
+  static_assert(IPW == 1 || (IPW == 4 && TR == 8 && !GATED && (MODE == kStreamPlain || JOIN)),
+                "four items per wave: tiles of 8 rows of a plain or joining product");
   constexpr int kTileBytes = NORM ? kStreamTileBytes : TR * kStreamItem * 2;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, nwaves = blockDim.x / 64;
-  unsigned char* tile_s = stream_smem + wave * kTileBytes;
-  float* red = (float*)(stream_smem + nwaves * kTileBytes);            // [2][nwaves][256]
+  unsigned char* tile_s = stream_smem + wave * (IPW * kTileBytes);     // a tile per item
+  float* red = (float*)(stream_smem + nwaves * (IPW * kTileBytes));    // [2][nwaves][256]
   const int half = lane / 32, l32 = lane % 32;          // loading: row parity, 16-byte chunk
   const int oi = lane % 16, og = lane / 16;             // operand: row (or token), k group
   const int T = sh.T, N = sh.N, K = sh.K;
   const int slice = blockIdx.x % sh.num_slices;
   const int tile_step = gridDim.x / sh.num_slices;
   const int nitems = (K + kStreamItem - 1) / kStreamItem;
-  const int item = slice * nwaves + wave;               // this wave's k item
+  const int item = (slice * nwaves + wave) * IPW;       // this wave's (first) k item
   const bool has_item = item < nitems;
   const int kb = item * kStreamItem;
-  const int ka = kb + l32 * 8;                          // this lane's k when loading weights
-  const bool a_ok = has_item && ka < K;
   // Loads are never predicated off (that would cost registers for the zeros): a row past the
   // end reads row 0 instead and is not stored; a k past the end reads k = 0 instead and meets
   // a zero in the rows of x (weights are finite).
-  const bf16_t* w_lane = W + (a_ok ? ka : 0);
+  // With several items per wave the order of the first loads matters (below): the two
+  // pointers then pass through an empty statement, after which the compiler knows nothing
+  // about what they point to and keeps their loads on their side of a memory barrier.
+  // (They are declared as pointers to global memory, which the compiler could no longer tell
+  // by itself.)
+  typedef const __attribute__((address_space(1))) bf16_t* GlobalBf16;
+  typedef uint32_t Bits4 __attribute__((ext_vector_type(4)));
+  typedef const __attribute__((address_space(1))) Bits4* GlobalU4;
+  GlobalBf16 w_base = (GlobalBf16)W;
+  GlobalBf16 x_base = (GlobalBf16)X;
+  if constexpr (IPW > 1) asm volatile("" : "+s"(w_base), "+s"(x_base));
+  GlobalBf16 w_lane[IPW];
+#pragma unroll
+  for (int it = 0; it < IPW; ++it) {
+    const int ka = kb + it * kStreamItem + l32 * 8;     // this lane's k when loading weights
+    w_lane[it] = w_base + ((item + it < nitems && ka < K) ? ka : 0);
+  }
 
   // Tile row r = 2 p + half of tile `tile` is weight row tile * rows + r; gated, the first
   // half of a tile's rows are the gate rows of consecutive columns and the second half their
@@ -743,26 +764,33 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
     const int tl_ = (tile_);                                                                    \
     if (tl_ < sh.num_tiles) {                                                                   \
       const int col0 = tl_ * cols_per_tile + half;                                              \
-      const bf16_t* w_tile = w_lane + (long long)col0 * sh.ldw;                                 \
-      _Pragma("unroll") for (int p = 0; p < TR / 2; ++p) {                                      \
-        const int c = GATED ? (2 * p) % cols_per_tile : 2 * p; /* column within the tile */     \
-        const long long up = (GATED && 2 * p >= cols_per_tile) ? (long long)N * sh.ldw : 0;     \
-        const bf16_t* ptr = col0 + c < N ? w_tile + (long long)c * sh.ldw + up : w_lane;        \
-        const uint4 v_ = *(const uint4*)ptr;   /* a k past the end meets a zero of x */         \
-        a[p].x = v_.x;          /* member by member: a struct copy would go through scratch */  \
-        a[p].y = v_.y;                                                                          \
-        a[p].z = v_.z;                                                                          \
-        a[p].w = v_.w;                                                                          \
+      _Pragma("unroll") for (int it_ = 0; it_ < IPW; ++it_) {                                   \
+        GlobalBf16 w_tile = w_lane[it_] + (long long)col0 * sh.ldw;                             \
+        _Pragma("unroll") for (int p = 0; p < TR / 2; ++p) {                                    \
+          const int c = GATED ? (2 * p) % cols_per_tile : 2 * p; /* column within the tile */   \
+          const long long up = (GATED && 2 * p >= cols_per_tile) ? (long long)N * sh.ldw : 0;   \
+          GlobalBf16 ptr = col0 + c < N ? w_tile + (long long)c * sh.ldw + up : w_lane[it_];    \
+          const Bits4 v_ = *(GlobalU4)ptr;       /* a k past the end meets a zero of x */       \
+          a[it_][p].x = v_.x;   /* member by member: a struct copy would go through scratch */  \
+          a[it_][p].y = v_.y;                                                                   \
+          a[it_][p].z = v_.z;                                                                   \
+          a[it_][p].w = v_.w;                                                                   \
+        }                                                                                       \
       }                                                                                         \
     }                                                                                           \
   }
 
-  uint4 a[TR / 2];
+  uint4 a[IPW][TR / 2];
   int tile = blockIdx.x / sh.num_slices;
   RLIS_STREAM_LOAD_TILE(a, tile);        // the first tile is on its way during the prologue
+  // The weights are asked for first: loads are served in order, and behind four items of x
+  // (one address for eight loads: the compiler would gladly issue them first) the first weight
+  // would leave two microseconds late.
+  if constexpr (IPW > 1) asm volatile("" ::: "memory");
 
-  // The rows of x in operand layout: token oi, k = kb + (4 j + og) * 8 .. + 8 for step j.
-  Frag8 b[8];
+  // The rows of x in operand layout: token oi, k = kb + (4 j + og) * 8 .. + 8 for step j (of
+  // item `it`, kStreamItem further on).
+  Frag8 b[IPW][8];
   float inv_rms = 1.f;                   // NORM: of token tid / 16, in the threads that store
   // SCALED: the scale comes as partial sums of squares, scale_count a token.  Thread (token
   // tid / 16, i = tid % 16) of the 256 storing threads takes parts 4 i .. 4 i + 3, + 64, ...
@@ -775,11 +803,22 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
   bool scale_due = SCALED;
   if (!NORM) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int k = kb + (4 * j + og) * 8;
-      const bool ok = has_item && oi < T && k < K;
-      const uint4 v = *(const uint4*)(X + (ok ? (long long)oi * sh.ldx + k : 0));
-      b[j].u = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+    for (int it = 0; it < IPW; ++it) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int k = kb + it * kStreamItem + (4 * j + og) * 8;
+        const bool ok = item + it < nitems && oi < T && k < K;
+        if constexpr (IPW == 1) {
+          const uint4 v = *(const uint4*)(X + (ok ? (long long)oi * sh.ldx + k : 0));
+          b[it][j].u = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+        } else {
+          // Every wave has whole items (the launch sees to that), and a token past the end
+          // takes the last one's row: its products are not stored.  So nothing is zeroed, no
+          // load is waited for here, and the eight loads of an item share one address.
+          GlobalBf16 xb = x_base + (long long)min(oi, T - 1) * sh.ldx + kb + it * kStreamItem + og * 8;
+          b[it][j].v = __builtin_bit_cast(bf16x8, *(GlobalU4)(xb + j * 32));
+        }
+      }
     }
     if constexpr (SCALED) {
 #pragma unroll
@@ -894,7 +933,7 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
       for (int j = 0; j < 8; ++j) {
         const uint4 v = *(const uint4*)(tile_s + oi * (kStreamItem * 2) + (((4 * j + og) ^ oi) * 16));
         const bool tok = oi < T;
-        b[j].u = make_uint4(tok ? v.x : 0u, tok ? v.y : 0u, tok ? v.z : 0u, tok ? v.w : 0u);
+        b[0][j].u = make_uint4(tok ? v.x : 0u, tok ? v.y : 0u, tok ? v.z : 0u, tok ? v.w : 0u);
       }
       wave_lds_fence();
     }
@@ -911,38 +950,64 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     if (has_item) {
 #pragma unroll
-      for (int p = 0; p < TR / 2; ++p) {
-        const int r = 2 * p + half;
-        *(uint4*)(tile_s + r * (kStreamItem * 2) + ((l32 ^ r) * 16)) = a[p];
+      for (int it = 0; it < IPW; ++it) {
+#pragma unroll
+        for (int p = 0; p < TR / 2; ++p) {
+          const int r = 2 * p + half;
+          *(uint4*)(tile_s + it * kTileBytes + r * (kStreamItem * 2) + ((l32 ^ r) * 16)) = a[it][p];
+        }
       }
     }
     // JOIN: this thread's element of the residual and of the norm's weight, asked for ahead of
     // the next tile's weights (loads come back in order: who waits for these must not wait
     // for those).
-    float join_resid = 0.f, join_weight = 0.f;
+    // Both are kept as loaded and looked at only after the products (a conversion or a select
+    // here would wait for them, and with them for every load issued before).
+    float join_resid = 0.f;
+    uint32_t join_weight_bits = 0;
     if constexpr (JOIN) {
       const int t = (tid / 16) % 16, i = tid % 16;
       const long long n = (long long)tile * TR + i;
       const bool ok = tid < 256 && i < TR && t < T && n < N;
-      const long long at = ok ? (long long)t * N + n : 0;
-      const float r = nm.resid[at];
-      const float wn = nm.weight_f32 ? ((const float*)nm.weight)[ok ? n : 0]
-                                     : bf16_to_f32(((const bf16_t*)nm.weight)[ok ? n : 0]);
-      join_resid = ok ? r : 0.f;
-      join_weight = ok ? wn : 0.f;
+      join_resid = nm.resid[ok ? (long long)t * N + n : 0];
+      if (nm.weight_f32)
+        join_weight_bits = ((const uint32_t*)nm.weight)[ok ? n : 0];
+      else
+        join_weight_bits = ((const bf16_t*)nm.weight)[ok ? n : 0];
     }
-    RLIS_STREAM_LOAD_TILE(a, tile + tile_step);  // on its way during the arithmetic
+    // The next tile is on its way during the arithmetic; with several items per wave only
+    // after it, so that the weights' registers are free for the reads from LDS to run ahead
+    // of the products (such workgroups seldom have a second tile).
+    if constexpr (IPW == 1) RLIS_STREAM_LOAD_TILE(a, tile + tile_step);
     if (has_item) {
       wave_lds_fence();
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        Frag8 af;
-        // tile rows beyond TR repeat the first ones: their products are not stored
-        af.u = *(const uint4*)(tile_s + (oi % TR) * (kStreamItem * 2) + (((4 * j + og) ^ (oi % TR)) * 16));
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af.v, b[j].v, acc, 0, 0, 0);
+      for (int it = 0; it < IPW; ++it) {
+#pragma unroll
+        for (int j0 = 0; j0 < 8; j0 += 4) {
+          Bits4 af[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            // tile rows beyond TR repeat the first ones: their products are not stored
+            af[j] = *(const Bits4*)(tile_s + it * kTileBytes + (oi % TR) * (kStreamItem * 2) +
+                                    (((4 * (j0 + j) + og) ^ (oi % TR)) * 16));
+          }
+          // With two waves per SIMD nobody else fills the time a read from LDS takes: four are
+          // asked for before the first of their products (the statement, which every read
+          // feeds and every product depends on, keeps the compiler from pairing each read
+          // with its product again).
+          if constexpr (IPW > 1)
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(af[0]), "+v"(af[1]), "+v"(af[2]), "+v"(af[3]));
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af[j]),
+                                                          b[it][j0 + j].v, acc, 0, 0, 0);
+        }
       }
       wave_lds_fence();
     }
+    if constexpr (IPW > 1) RLIS_STREAM_LOAD_TILE(a, tile + tile_step);
     // acc: token oi, tile rows og * 4 + r.  red[par][wave][token][row]; the buffer of the
     // tile before is still being read by slower waves, the one before that is free again
     // after this tile's barrier.
@@ -987,6 +1052,8 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
           sum *= inv_rms;
           if (nm.round_parts) sum = bf16_to_f32(f32_to_bf16(sum));
           const float total = join_resid + sum;
+          const float join_weight = __uint_as_float(nm.weight_f32 ? join_weight_bits
+                                                                  : join_weight_bits << 16);
           nm.resid_out[(long long)t * N + n] = total;
           nm.xw_out[(long long)t * N + n] = f32_to_bf16(total * join_weight);
           sq = total * total;
@@ -1008,22 +1075,34 @@ __global__ __launch_bounds__(1024) void gemm_bf16_stream_kernel(const bf16_t* __
 #undef RLIS_STREAM_LOAD_TILE
 }
 
-// A workgroup takes up to 16 k items, one per wave; longer rows are cut into slices.  Both
-// are functions of K alone.
-static int stream_slices(int K) { return ceil_div(ceil_div(K, kStreamItem), kStreamMaxWaves); }
-// The fused norm needs whole rows in one workgroup.
+// A workgroup takes up to 16 k items, one per wave, or up to 32 in whole fours, four per wave
+// (plain and joining products); other rows are cut into slices of up to 16 items.  All of it
+// follows from K alone.
+constexpr int kStreamFour = 4;
+static int stream_items_per_wave(int K) {
+  const int nitems = ceil_div(K, kStreamItem);
+  return K % (kStreamFour * kStreamItem) == 0 && nitems > kStreamMaxWaves &&
+                 nitems <= 2 * kStreamMaxWaves
+             ? kStreamFour : 1;
+}
+static int stream_slices(int K) {
+  return stream_items_per_wave(K) > 1 ? 1 : ceil_div(ceil_div(K, kStreamItem), kStreamMaxWaves);
+}
+// The fused norm needs whole rows in one workgroup, one item per wave; so do the gated and the
+// scaled form.
 constexpr int kStreamNormMaxK = kStreamMaxWaves * kStreamItem;
 
-template <typename TC, bool GATED, int TR, int MODE>
+template <typename TC, bool GATED, int TR, int MODE, int IPW = 1>
 static int launch_stream_tiles(const void* X, const void* W, void* Y, StreamShape sh,
                                const StreamNorm& nm, int nwaves, int num_cus,
                                hipStream_t stream) {
-  constexpr int kTileBytes = MODE == kStreamNorm ? kStreamTileBytes : TR * kStreamItem * 2;
+  constexpr int kTileBytes = IPW * (MODE == kStreamNorm ? kStreamTileBytes : TR * kStreamItem * 2);
   static bool lds_raised = false;
   if (!lds_raised) {
     hipError_t e = hipFuncSetAttribute(
-        (const void*)gemm_bf16_stream_kernel<TC, GATED, TR, MODE>,
-        hipFuncAttributeMaxDynamicSharedMemorySize, kStreamMaxWaves * (kTileBytes + 2048));
+        (const void*)gemm_bf16_stream_kernel<TC, GATED, TR, MODE, IPW>,
+        hipFuncAttributeMaxDynamicSharedMemorySize,
+        (IPW == 1 ? kStreamMaxWaves : 2 * kStreamMaxWaves / IPW) * (kTileBytes + 2048));
     RLIS_REQUIRE(e == hipSuccess, "gemm_bf16_stream: cannot raise the LDS limit: %s",
                  hipGetErrorString(e));
     lds_raised = true;
@@ -1036,7 +1115,7 @@ static int launch_stream_tiles(const void* X, const void* W, void* Y, StreamShap
   long long groups = tiles;                                // workgroups per slice
   const long long cap = max(1, num_cus * per_cu / sh.num_slices);
   if (groups > cap) groups = cap;
-  gemm_bf16_stream_kernel<TC, GATED, TR, MODE>
+  gemm_bf16_stream_kernel<TC, GATED, TR, MODE, IPW>
       <<<(int)(groups * sh.num_slices), nwaves * 64, smem, stream>>>(
           (const bf16_t*)X, (const bf16_t*)W, (TC*)Y, sh, nm);
   return 0;
@@ -1054,12 +1133,25 @@ static int stream_compute_units() {
   return num_cus;
 }
 
-// Weight rows per tile: 8 when 16-row tiles would leave compute units without work (a unit draws
-// only its share of the memory bandwidth, however much it has in flight); with the fused norm
-// every workgroup reads all of x, so fewer, larger tiles win earlier.
-static int stream_tile_rows(int N, int slices, bool gated, bool norm, int num_cus) {
-  const long long tiles16 = (long long)ceil_div(N, gated ? 8 : 16) * slices;
-  return tiles16 < (norm ? num_cus / 2 : num_cus) ? 8 : 16;
+// Weight rows per tile: 16, 12 or 8.  A compute unit draws only its share of the memory
+// bandwidth, however much it has in flight, so what counts is the most weight rows that any
+// unit streams: rounds of tiles over the units times the rows of a tile.  Ties go to the
+// larger tile (fewer workgroups, fewer prologues).
+static int stream_tile_rows(int N, int K, bool gated, bool norm, int num_cus) {
+  if (stream_items_per_wave(K) > 1) return 8;            // what the registers hold
+  const int slices = stream_slices(K);
+  int best = 16;
+  long long best_cost = 0;
+  for (int tr : {16, 12, 8}) {
+    const long long tiles = (long long)ceil_div(N, gated ? tr / 2 : tr) * slices;
+    const long long cost = ceil_div_ll(tiles, num_cus) * tr;
+    if (tr == 16 || cost < best_cost) {
+      best = tr;
+      best_cost = cost;
+    }
+  }
+  (void)norm;
+  return best;
 }
 
 template <typename TC, bool GATED, int MODE>
@@ -1067,8 +1159,8 @@ static int launch_stream(const void* X, const void* W, void* Y, int T, int N, in
                          long long ldw, long long ldy, long long part_stride,
                          const StreamNorm& nm, hipStream_t stream) {
   const int nitems = ceil_div(K, kStreamItem);
-  const int slices = stream_slices(K);
-  const int nwaves = max(4, ceil_div(nitems, slices));
+  const int slices = stream_slices(K), ipw = stream_items_per_wave(K);
+  const int nwaves = max(4, ceil_div(nitems, slices * ipw));
   const int num_cus = stream_compute_units();
   RLIS_REQUIRE(num_cus > 0, "gemm_bf16_stream: cannot read the device properties");
   StreamShape sh;
@@ -1076,9 +1168,21 @@ static int launch_stream(const void* X, const void* W, void* Y, int T, int N, in
   sh.part_stride = part_stride;
   sh.num_slices = slices;
   sh.num_tiles = 0;
-  if (stream_tile_rows(N, slices, GATED, MODE == kStreamNorm, num_cus) == 8)
-    return launch_stream_tiles<TC, GATED, 8, MODE>(X, W, Y, sh, nm, nwaves, num_cus, stream);
-  return launch_stream_tiles<TC, GATED, 16, MODE>(X, W, Y, sh, nm, nwaves, num_cus, stream);
+  if (ipw > 1) {
+    if constexpr (!GATED && (MODE == kStreamPlain || MODE == kStreamJoin))
+      return launch_stream_tiles<TC, false, 8, MODE, kStreamFour>(X, W, Y, sh, nm, nwaves, num_cus,
+                                                                  stream);
+    RLIS_REQUIRE(false, "gemm_bf16_stream: K=%d is too long for this form (at most %d)", K,
+                 kStreamNormMaxK);
+  }
+  switch (stream_tile_rows(N, K, GATED, MODE == kStreamNorm, num_cus)) {
+    case 8:
+      return launch_stream_tiles<TC, GATED, 8, MODE>(X, W, Y, sh, nm, nwaves, num_cus, stream);
+    case 12:
+      return launch_stream_tiles<TC, GATED, 12, MODE>(X, W, Y, sh, nm, nwaves, num_cus, stream);
+    default:
+      return launch_stream_tiles<TC, GATED, 16, MODE>(X, W, Y, sh, nm, nwaves, num_cus, stream);
+  }
 }
 
 template <int MODE>
@@ -1113,7 +1217,8 @@ RLIS_API int rlis_gemm_bf16_stream_slices(int K) { return stream_slices(K); }
 // The longest row that rlis_norm_linear_bf16 takes.
 RLIS_API int rlis_norm_linear_max_k() { return kStreamNormMaxK; }
 
-// gated == 0: y (T, N) = x W^T.  gated != 0: W is (2N, K) = [Wg; Wu] and
+// gated == 0: y (T, N) = x W^T (one result up to K = 8192, float32 partial results per slice
+// beyond).  gated != 0: W is (2N, K) = [Wg; Wu] and
 // y (T, N) = silu(x Wg^T) * (x Wu^T), K <= 4096.  T <= 16, bfloat16 operands, K a multiple of 8.
 RLIS_API int rlis_gemm_bf16_stream(const void* X, const void* W, void* Y, int y_dtype, int T,
                                    int N, int K, long long ldx, long long ldw, long long ldy,
@@ -1124,6 +1229,8 @@ RLIS_API int rlis_gemm_bf16_stream(const void* X, const void* W, void* Y, int y_
   RLIS_REQUIRE(slices == 1 || (!gated && y_dtype == RLIS_F32 && part_stride >= (long long)T * ldy),
                "gemm_bf16_stream: K=%d takes %d slices, which need float32 partial results and "
                "no gate", K, slices);
+  RLIS_REQUIRE(!gated || K <= kStreamNormMaxK, "gemm_bf16_stream: the gated form takes K up to "
+               "%d, not %d", kStreamNormMaxK, K);
   if (T == 0) return 0;
   StreamNorm nm = {};
   return dispatch_stream<kStreamPlain>("gemm_bf16_stream", X, W, Y, y_dtype, T, N, K, ldx, ldw, ldy,
@@ -1142,7 +1249,7 @@ RLIS_API int rlis_gemm_bf16_stream(const void* X, const void* W, void* Y, int y_
 // product.
 RLIS_API int rlis_gemm_bf16_stream_join_tiles(int N, int K) {
   const int cus = stream_compute_units();
-  return cus > 0 ? ceil_div(N, stream_tile_rows(N, stream_slices(K), false, false, cus)) : 0;
+  return cus > 0 ? ceil_div(N, stream_tile_rows(N, K, false, false, cus)) : 0;
 }
 
 RLIS_API int rlis_gemm_bf16_stream_join(const void* X, const void* W, int T, int N, int K,
@@ -1182,8 +1289,8 @@ RLIS_API int rlis_gemm_bf16_stream_scaled(const void* X, const void* W, void* Y,
                                           hipStream_t stream) {
   if (check_skinny("gemm_bf16_stream_scaled", X, W, T, N, K, ldx, ldw, ldy)) return 1;
   RLIS_REQUIRE(T <= 16, "gemm_bf16_stream_scaled: T=%d rows, at most 16", T);
-  RLIS_REQUIRE(stream_slices(K) == 1, "gemm_bf16_stream_scaled: K=%d takes more than one slice",
-               K);
+  RLIS_REQUIRE(K <= kStreamNormMaxK, "gemm_bf16_stream_scaled: K=%d, at most %d", K,
+               kStreamNormMaxK);
   RLIS_REQUIRE(scale_parts && scale_count > 0 && ss_stride % 4 == 0 && ss_stride >= scale_count &&
                    ((uintptr_t)scale_parts % 16) == 0,
                "gemm_bf16_stream_scaled: %d partial sums in rows of %d", scale_count, ss_stride);

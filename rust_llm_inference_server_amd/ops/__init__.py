@@ -238,8 +238,14 @@ def swiglu(gu: torch.Tensor) -> torch.Tensor:
 
 # ----------------------------------------------------------------------- products
 def stream_slices(K: int) -> int:
-    """Number of k slices the streaming kernel cuts a product over ``K`` into."""
+    """Number of k slices the streaming kernel cuts a plain product over ``K`` into."""
     return lib.load().rlis_gemm_bf16_stream_slices(K)
+
+
+def _one_item_per_wave(K: int) -> bool:
+    """Whether a row of ``K`` fits the streaming kernel's forms that take one k item per wave
+    (the fused norm, the gated and the scaled form)."""
+    return K <= lib.load().rlis_norm_linear_max_k()
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
@@ -409,7 +415,7 @@ def can_join_norm_linear(product: PendingProduct, resid: torch.Tensor, w: torch.
     return (JOIN_NORM_LINEAR and resid.dtype == torch.float32 and resid.is_contiguous()
             and product.shape == (T, H) and w.dim() == 2 and w.shape[1] == H
             and w.dtype == torch.bfloat16 and w.stride(1) == 1 and w.stride(0) % 8 == 0
-            and w.data_ptr() % 16 == 0 and stream_slices(H) == 1)
+            and w.data_ptr() % 16 == 0 and _one_item_per_wave(H))
 
 
 def linear_join_norm(product: PendingProduct, resid: torch.Tensor, norm_weight: torch.Tensor,
@@ -473,7 +479,7 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
                and 0 < T and K == w_gate_up.shape[1] and K % 8 == 0
                and ldx % 8 == 0 and ldw % 8 == 0 and x.data_ptr() % 16 == 0
                and w_gate_up.data_ptr() % 16 == 0)
-    streamed = fusable and T <= STREAM_MAX_ROWS and stream_slices(K) == 1
+    streamed = fusable and T <= STREAM_MAX_ROWS and _one_item_per_wave(K)
     skinny = fusable and not streamed and T <= SKINNY_MAX_ROWS and \
         (BF16_GEMM == "own" or T <= STREAM_MAX_ROWS)
     if not (streamed or skinny):

@@ -201,7 +201,7 @@ def test_linear_streaming_kernel(ops, out_dtype, T, N, K):
         else:
             got = ops.linear(x, w, out_dtype)
         gated = None
-        if N % 2 == 0 and out_dtype == torch.bfloat16 and ops.stream_slices(K) == 1:
+        if N % 2 == 0 and out_dtype == torch.bfloat16 and K <= 4096:
             gated = ops.linear_swiglu(x, w)
     finally:
         ops.STREAM_MAX_ROWS = old
@@ -363,7 +363,10 @@ def test_norm_linear(ops, T, N, K, parts, rows, norm_dtype):
 
 
 @pytest.mark.parametrize("T,H,K,N", [(1, 2048, 2048, 4096), (8, 2048, 2048, 16384), (16, 104, 344, 72),
-                                     (5, 4096, 1000, 1002), (7, 776, 4096, 64), (13, 3072, 3072, 512)])
+                                     (5, 4096, 1000, 1002), (7, 776, 4096, 64), (13, 3072, 3072, 512),
+                                     (8, 3072, 2048, 3072), (16, 2560, 3072, 520), (3, 4088, 4096, 72),
+                                     (8, 2048, 8192, 3072), (16, 3072, 8192, 520), (3, 1000, 5120, 72),
+                                     (1, 2048, 6144, 64)])
 @pytest.mark.parametrize("norm_dtype", DTYPES, ids=["normw32", "normw16"])
 @pytest.mark.parametrize("round_sum", [True, False])
 def test_linear_join_norm_and_linear_scaled(ops, T, H, K, N, norm_dtype, round_sum):
@@ -373,7 +376,8 @@ def test_linear_join_norm_and_linear_scaled(ops, T, H, K, N, norm_dtype, round_s
     second multiplies those rows by w2 and scales by the rsqrt of the mean square, plain and
     gated.  Against float64 formulas, and against the one-kernel norm in front of the second
     product fed with the first product's result (the same roundings, another order of the sums
-    of squares)."""
+    of squares).  Tiles of 8, 12 and 16 weight rows; first products over a feed-forward's width
+    (4096 < K <= 8192 in whole fours of k items) take four items per wave."""
     x = rnd(T, K, dtype=torch.bfloat16, seed=1)
     w1 = rnd(H, K, dtype=torch.bfloat16, seed=2, scale=0.05)
     w2 = rnd(N, H, dtype=torch.bfloat16, seed=3, scale=0.05)
@@ -414,7 +418,7 @@ def test_linear_join_norm_and_linear_scaled(ops, T, H, K, N, norm_dtype, round_s
         torch.testing.assert_close(got.double(), want_g, atol=max(1.0, want_g.abs().max().item()) / 32,
                                    rtol=3e-2)
     # more than one k slice, more than 16 rows, or float32: the plain product comes back
-    assert isinstance(ops.pending_linear(rnd(T, 8192, dtype=torch.bfloat16), rnd(64, 8192, dtype=torch.bfloat16)),
+    assert isinstance(ops.pending_linear(rnd(T, 8448, dtype=torch.bfloat16), rnd(64, 8448, dtype=torch.bfloat16)),
                       torch.Tensor)
     assert isinstance(ops.pending_linear(rnd(17, K, dtype=torch.bfloat16), w1), torch.Tensor)
     assert isinstance(ops.pending_linear(rnd(T, K), rnd(H, K)), torch.Tensor)
