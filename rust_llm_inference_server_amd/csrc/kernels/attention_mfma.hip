@@ -640,9 +640,14 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
   // workgroup has 512 threads) are all asked for before anything is waited for.
   const bool rotates = rope.positions != nullptr;
   const bool stores_kv = rotates && rope.slots != nullptr;
+  // None of these loads sits under a condition: a load in a branch makes the compiler wait,
+  // where the branches meet, for everything asked for so far.  What is not wanted is read from
+  // a place that is there anyway and dropped.
   const int ctx = ctx_lens[seq];
-  const int pos = rotates ? rope.positions[seq] : 0;
-  const int slot = stores_kv ? rope.slots[seq] : -1;
+  const int pos_read = (rotates ? rope.positions : ctx_lens)[seq];
+  const int slot_read = (stores_kv ? rope.slots : ctx_lens)[seq];
+  const int pos = rotates ? pos_read : 0;
+  const int slot = stores_kv ? slot_read : -1;
   Frag8 qf[D / 32];
 #pragma unroll
   for (int ks = 0; ks < D / 32; ++ks) {
@@ -654,14 +659,12 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
   const int half = rope.rot / 2;
   const bool kv_thread = stores_kv && tid < d;
   const bool k_turns = kv_thread && rope.cos && tid < rope.rot;
-  bf16_t new_k = 0, new_partner = 0, new_v = 0;
-  if (kv_thread) {
-    const bf16_t* krow = q + (long long)seq * q_stride + rope.k_off + kvh * d;
-    const bf16_t* vrow = q + (long long)seq * q_stride + rope.v_off + kvh * d;
-    new_k = krow[tid];
-    new_v = vrow[tid];
-    if (k_turns) new_partner = krow[tid < half ? tid + half : tid - half];
-  }
+  // (without a cache write the same elements of the q row stand in)
+  const int kv_i = min(tid, d - 1);
+  const int partner_i = kv_i < half ? kv_i + half : max(kv_i - half, 0);
+  const bf16_t* krow = q + (long long)seq * q_stride + (stores_kv ? rope.k_off : 0) + kvh * d;
+  const bf16_t* vrow = q + (long long)seq * q_stride + (stores_kv ? rope.v_off : 0) + kvh * d;
+  const bf16_t new_k = krow[kv_i], new_v = vrow[kv_i], new_partner = krow[min(partner_i, d - 1)];
 
   // ---- what follows from the context length ---------------------------------------------
   const int* table = block_tables + (long long)seq * max_pages;
@@ -736,26 +739,29 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
   const bool one_by_one = part <= kStride || !kPairs;
   RLIS_DEC_PAGES(c0, pk_a, pv_a);
   if constexpr (kPairs) {
-    if (!one_by_one) RLIS_DEC_PAGES(c0 + kStride, pk_b, pv_b);
+    // (clamped loads: harmless where a wave has one chunk only, and no branch around loads)
+    RLIS_DEC_PAGES(c0 + kStride, pk_b, pv_b);
   }
+  // The angles, again without a branch: where nothing is rotated the q row itself (D / 2
+  // floats are D bf16 elements of it) is read instead and dropped.
   constexpr int HS = D % 64 == 0 ? D / 64 : 1;     // fragments between a dim and its partner
   const bool q_turns = D % 64 == 0 && rotates && rope.cos;   // the dispatcher: rot == d == D
+  const float* no_angles = (const float*)(q + (long long)seq * q_stride);
   float q_cos[HS][8], q_sin[HS][8];
-  if (q_turns) {
-    const float* cs = rope.cos + (long long)pos * (D / 2);
-    const float* sn = rope.sin + (long long)pos * (D / 2);
+  if constexpr (D % 64 == 0) {
+    const float* cs = q_turns ? rope.cos + (long long)pos * (D / 2) : no_angles;
+    const float* sn = q_turns ? rope.sin + (long long)pos * (D / 2) : no_angles;
 #pragma unroll
     for (int ks = 0; ks < HS; ++ks) {
       load8f(cs + ks * 32 + lq * 8, q_cos[ks]);
       load8f(sn + ks * 32 + lq * 8, q_sin[ks]);
     }
   }
-  float k_cos = 1.f, k_sin = 0.f;
-  if (k_turns) {
-    const int j = tid < half ? tid : tid - half;
-    k_cos = rope.cos[(long long)pos * half + j];
-    k_sin = rope.sin[(long long)pos * half + j];
-  }
+  const bool k_angles = stores_kv && rope.cos && half > 0;
+  const int k_j = min(kv_i < half ? kv_i : kv_i - half, max(half - 1, 0));
+  const float k_cos_read = (k_angles ? rope.cos + (long long)pos * half + k_j : no_angles)[0];
+  const float k_sin_read = (k_angles ? rope.sin + (long long)pos * half + k_j : no_angles)[0];
+  const float k_cos = k_turns ? k_cos_read : 1.f, k_sin = k_turns ? k_sin_read : 0.f;
 
   // ---- the step's own key and value go to the pages before anyone reads them back --------
   if (stores_kv && kbeg < ctx && kend == ctx) {
