@@ -15,6 +15,7 @@
 // In every kernel an output element is a sum over k in an order that depends only on the
 // kernel and K, never on which other rows are in the batch.
 #include "common.h"
+#include "gemm_stream.h"
 
 // ============================================================== plain FMA product
 template <typename TA, typename TB, typename TC>
@@ -110,15 +111,6 @@ RLIS_API int rlis_gemm_plain(const void* A, int a_dtype, const void* B, int b_dt
 }
 
 // ================================================================ MFMA bf16 product
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
-union Frag8 {
-  uint4 u;
-  bf16x8 v;
-};
-
 // Tile 128 x 128 x 64, four waves in a 2 x 2 arrangement, each wave 64 x 64 as 2 x 2 blocks of
 // v_mfma_f32_32x32x16_bf16.  Operand fragments: lane l holds row (or column) l % 32 and the 8
 // consecutive k at (l / 32) * 8; the accumulator holds column l % 32 and rows
@@ -642,53 +634,7 @@ RLIS_API int rlis_gemm_bf16_splitk(const void* X, const void* W, void* Y, int T,
 // one slice (K > 8192) every slice stores its own float32 partial result, which the consumer
 // adds in slice order: the order of a sum depends on K alone.  The gated form pairs gate rows with their up rows in one
 // tile and applies the SwiGLU before the store.
-constexpr int kStreamItem = 256;                        // k per item
-constexpr int kStreamTileBytes = 16 * kStreamItem * 2;  // one wave's tile in LDS
 constexpr int kStreamMaxWaves = 16;
-
-__device__ __forceinline__ void wave_lds_fence() {
-  // LDS operations of one wave execute in order; this only stops the compiler from moving
-  // reads of other lanes' data above the writes.
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
-struct StreamShape {
-  int T, N, K;
-  long long ldx, ldw, ldy, part_stride;   // part_stride: elements between partial results
-  int num_tiles, num_slices;
-};
-
-// NORM: x is not given but made on the fly as (resid + delta) * norm_weight, and the products
-// are scaled by rsqrt(mean((resid + delta)^2) + eps) of their row at the end, which is the
-// RMSNorm of crates/model/src/layers.rs:103-122 in front of the projection (the scale is one
-// number per row and commutes with the product).  Needs all of K in one slice, so that the
-// workgroup sees whole rows.  Workgroup 0 also stores resid + delta to resid_out.
-struct StreamNorm {
-  const float* resid;        // (rows, K) float32
-  const void* delta;         // null, or `parts` arrays (rows, K), part_stride elements apart
-  int delta_f32, parts;
-  int round_parts;           // round the sum of the parts to bfloat16 before it is added
-  long long part_stride;
-  const void* weight;        // (K)
-  int weight_f32;
-  float eps;
-  const int* rows;           // null, or the row of resid/delta that token t reads
-  float* resid_out;          // null, or where resid + delta goes (not resid itself)
-  // Without NORM, the two halves of a norm that sits between two products, neither of which
-  // needs a prologue over whole rows.  The product in front of the norm (ss_out given; one k
-  // slice, no gate) adds its result to resid (N wide, in place when resid_out is resid: every
-  // element is read and written by one thread), and stores the sum, the sum times the norm's
-  // weight in bfloat16, and per token and tile of output columns the sum of the squares.  The
-  // product behind the norm (scale_parts given) takes those rows as its x and scales its
-  // results by rsqrt(sum of the scale_count partial sums / K + eps) of their row.
-  bf16_t* xw_out;            // (T, N) bfloat16
-  float* ss_out;             // (16, ss_stride) float32: token-major, one entry per tile
-  const float* scale_parts;  // (16, ss_stride) float32, scale_count entries a token
-  int scale_count;
-  int ss_stride;             // a multiple of 4
-};
 
 __device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
   const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
@@ -703,10 +649,6 @@ __device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
     v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
   }
 }
-
-// What a kernel does beside the product: nothing, the fused norm (x made from the residual in
-// the prologue), the scale from partial sums of squares, or joining the residual at the end.
-enum { kStreamPlain = 0, kStreamNorm = 1, kStreamScaled = 2, kStreamJoin = 3 };
 
 template <typename TC, bool GATED, int TR /* weight rows per tile: 16, 12 or 8 */, int MODE,
           int IPW /* k items per wave: 1 or 4 */>
@@ -1121,8 +1063,7 @@ static int launch_stream_tiles(const void* X, const void* W, void* Y, StreamShap
   return 0;
 }
 
-// The compute units of the current device (0: unknown).
-static int stream_compute_units() {
+int rlis_stream_compute_units() {
   static int num_cus = 0;
   if (num_cus == 0) {
     int dev = 0;
@@ -1133,13 +1074,7 @@ static int stream_compute_units() {
   return num_cus;
 }
 
-// Weight rows per tile: 16, 12 or 8.  A compute unit draws only its share of the memory
-// bandwidth, however much it has in flight, so what counts is the most weight rows that any
-// unit streams: rounds of tiles over the units times the rows of a tile.  Ties go to the
-// larger tile (fewer workgroups, fewer prologues).
-static int stream_tile_rows(int N, int K, bool gated, bool norm, int num_cus) {
-  if (stream_items_per_wave(K) > 1) return 8;            // what the registers hold
-  const int slices = stream_slices(K);
+int rlis_stream_balanced_rows(int N, int slices, bool gated, int num_cus) {
   int best = 16;
   long long best_cost = 0;
   for (int tr : {16, 12, 8}) {
@@ -1150,8 +1085,14 @@ static int stream_tile_rows(int N, int K, bool gated, bool norm, int num_cus) {
       best_cost = cost;
     }
   }
-  (void)norm;
   return best;
+}
+
+// Weight rows per tile of the kernel for up to 16 rows of x.
+static int stream_tile_rows(int N, int K, bool gated, bool norm, int num_cus) {
+  (void)norm;
+  if (stream_items_per_wave(K) > 1) return 8;            // what the registers hold
+  return rlis_stream_balanced_rows(N, stream_slices(K), gated, num_cus);
 }
 
 template <typename TC, bool GATED, int MODE>
@@ -1161,7 +1102,7 @@ static int launch_stream(const void* X, const void* W, void* Y, int T, int N, in
   const int nitems = ceil_div(K, kStreamItem);
   const int slices = stream_slices(K), ipw = stream_items_per_wave(K);
   const int nwaves = max(4, ceil_div(nitems, slices * ipw));
-  const int num_cus = stream_compute_units();
+  const int num_cus = rlis_stream_compute_units();
   RLIS_REQUIRE(num_cus > 0, "gemm_bf16_stream: cannot read the device properties");
   StreamShape sh;
   sh.T = T; sh.N = N; sh.K = K; sh.ldx = ldx; sh.ldw = ldw; sh.ldy = ldy;
@@ -1214,17 +1155,27 @@ static int dispatch_stream(const char* name, const void* X, const void* W, void*
 // float32 partial results, part_stride elements apart, to be added in order.
 RLIS_API int rlis_gemm_bf16_stream_slices(int K) { return stream_slices(K); }
 
+// The most rows of x that rlis_gemm_bf16_stream and its joining and scaled forms take for rows
+// of K: 16, or up to 64 where K is a whole number of items and short enough for the kernel that
+// keeps 32 or 64 rows in registers.
+RLIS_API int rlis_gemm_bf16_stream_max_rows(int K) { return rlis_stream_wide_rows(K); }
+
 // The longest row that rlis_norm_linear_bf16 takes.
 RLIS_API int rlis_norm_linear_max_k() { return kStreamNormMaxK; }
 
 // gated == 0: y (T, N) = x W^T (one result up to K = 8192, float32 partial results per slice
 // beyond).  gated != 0: W is (2N, K) = [Wg; Wu] and
-// y (T, N) = silu(x Wg^T) * (x Wu^T), K <= 4096.  T <= 16, bfloat16 operands, K a multiple of 8.
+// y (T, N) = silu(x Wg^T) * (x Wu^T), K <= 4096.  bfloat16 operands, K a multiple of 8, up to
+// rlis_gemm_bf16_stream_max_rows(K) rows (more than 16 go to the kernel of gemm_wide.hip).
 RLIS_API int rlis_gemm_bf16_stream(const void* X, const void* W, void* Y, int y_dtype, int T,
                                    int N, int K, long long ldx, long long ldw, long long ldy,
                                    long long part_stride, int gated, hipStream_t stream) {
   if (check_skinny("gemm_bf16_stream", X, W, T, N, K, ldx, ldw, ldy)) return 1;
-  RLIS_REQUIRE(T <= 16, "gemm_bf16_stream: T=%d rows, at most 16", T);
+  if (T > 16) {
+    StreamNorm none = {};
+    return rlis_launch_stream_wide("gemm_bf16_stream", kStreamPlain, X, W, Y, y_dtype, T, N, K, ldx,
+                                   ldw, ldy, gated, none, stream);
+  }
   const int slices = stream_slices(K);
   RLIS_REQUIRE(slices == 1 || (!gated && y_dtype == RLIS_F32 && part_stride >= (long long)T * ldy),
                "gemm_bf16_stream: K=%d takes %d slices, which need float32 partial results and "
@@ -1237,10 +1188,10 @@ RLIS_API int rlis_gemm_bf16_stream(const void* X, const void* W, void* Y, int y_
                                 part_stride, gated, nm, stream);
 }
 
-// A norm between two products without a pass over whole rows, in two calls (T <= 16, bfloat16
+// A norm between two products without a pass over whole rows, in two calls (rows as above, bfloat16
 // operands, one k slice each).  rlis_gemm_bf16_stream_join: s = resid + x W^T (the product
 // rounded to bfloat16 first with round_sum), stored to resid_out (resid itself is fine);
-// xw_out (T, N) bfloat16 = s * norm_weight; ss_out (16, ss_stride) float32 = per token the sums
+// xw_out (T, N) bfloat16 = s * norm_weight; ss_out (T up to a multiple of 16, ss_stride) float32 = per token the sums
 // of s^2 over each of the rlis_gemm_bf16_stream_join_tiles(N, K) tiles of columns (ss_stride a
 // multiple of 4, at least that many; what lies behind them in a row is not written).  resid and
 // resid_out are (T, N) float32 contiguous.  rlis_gemm_bf16_stream_scaled: y = (x W^T) *
@@ -1248,7 +1199,7 @@ RLIS_API int rlis_gemm_bf16_stream(const void* X, const void* W, void* Y, int y_
 // with x = xw_out and the partial sums of the first call, the RMSNorm of s in front of this
 // product.
 RLIS_API int rlis_gemm_bf16_stream_join_tiles(int N, int K) {
-  const int cus = stream_compute_units();
+  const int cus = rlis_stream_compute_units();
   return cus > 0 ? ceil_div(N, stream_tile_rows(N, K, false, false, cus)) : 0;
 }
 
@@ -1258,7 +1209,6 @@ RLIS_API int rlis_gemm_bf16_stream_join(const void* X, const void* W, int T, int
                                         int norm_weight_dtype, int round_sum, void* xw_out,
                                         float* ss_out, int ss_stride, hipStream_t stream) {
   if (check_skinny("gemm_bf16_stream_join", X, W, T, N, K, ldx, ldw, N)) return 1;
-  RLIS_REQUIRE(T <= 16, "gemm_bf16_stream_join: T=%d rows, at most 16", T);
   RLIS_REQUIRE(stream_slices(K) == 1, "gemm_bf16_stream_join: K=%d takes more than one slice", K);
   RLIS_REQUIRE(resid && resid_out && norm_weight && xw_out && ss_out,
                "gemm_bf16_stream_join: an operand is missing");
@@ -1278,6 +1228,9 @@ RLIS_API int rlis_gemm_bf16_stream_join(const void* X, const void* W, int T, int
   nm.xw_out = (bf16_t*)xw_out;
   nm.ss_out = ss_out;
   nm.ss_stride = ss_stride;
+  if (T > 16)
+    return rlis_launch_stream_wide("gemm_bf16_stream_join", kStreamJoin, X, W, xw_out, RLIS_BF16, T,
+                                   N, K, ldx, ldw, N, 0, nm, stream);
   return dispatch_stream<kStreamJoin>("gemm_bf16_stream_join", X, W, xw_out, RLIS_BF16, T, N, K, ldx,
                                 ldw, N, 0, 0, nm, stream);
 }
@@ -1288,7 +1241,6 @@ RLIS_API int rlis_gemm_bf16_stream_scaled(const void* X, const void* W, void* Y,
                                           int scale_count, int ss_stride, float eps,
                                           hipStream_t stream) {
   if (check_skinny("gemm_bf16_stream_scaled", X, W, T, N, K, ldx, ldw, ldy)) return 1;
-  RLIS_REQUIRE(T <= 16, "gemm_bf16_stream_scaled: T=%d rows, at most 16", T);
   RLIS_REQUIRE(K <= kStreamNormMaxK, "gemm_bf16_stream_scaled: K=%d, at most %d", K,
                kStreamNormMaxK);
   RLIS_REQUIRE(scale_parts && scale_count > 0 && ss_stride % 4 == 0 && ss_stride >= scale_count &&
@@ -1300,6 +1252,9 @@ RLIS_API int rlis_gemm_bf16_stream_scaled(const void* X, const void* W, void* Y,
   nm.scale_count = scale_count;
   nm.ss_stride = ss_stride;
   nm.eps = eps;
+  if (T > 16)
+    return rlis_launch_stream_wide("gemm_bf16_stream_scaled", kStreamScaled, X, W, Y, y_dtype, T, N, K,
+                                   ldx, ldw, ldy, gated, nm, stream);
   return dispatch_stream<kStreamScaled>("gemm_bf16_stream_scaled", X, W, Y, y_dtype, T, N, K, ldx, ldw,
                                 ldy, 0, gated, nm, stream);
 }

@@ -24,6 +24,10 @@ _DT = {torch.float32: 0, torch.bfloat16: 1}
 SKINNY_MAX_ROWS = 64
 # ... and with at most this many rows the streaming kernel (16 at most; 0 switches it off).
 STREAM_MAX_ROWS = 16
+# ... and, where the rows are short enough for a wave to keep 32 of them in registers (k up to
+# 3072), with up to this many rows its form for 17 to 32 rows (0 switches that off: such steps
+# then take the library's products, the split-k kernel and the norm and SwiGLU kernels).
+STREAM_WIDE_MAX_ROWS = 32
 # A product whose result joins the residual stream as partial sums (``partials=True``) takes the
 # split-k kernel from 17 rows up to this many (64 at most; 0 switches it off).
 SPLITK_MAX_ROWS = 64
@@ -242,6 +246,13 @@ def stream_slices(K: int) -> int:
     return lib.load().rlis_gemm_bf16_stream_slices(K)
 
 
+def stream_rows(K: int) -> int:
+    """The most rows of ``x`` that the streaming kernels take for rows of ``K``."""
+    if STREAM_MAX_ROWS < 16 or STREAM_WIDE_MAX_ROWS <= 16:
+        return STREAM_MAX_ROWS
+    return max(16, min(STREAM_WIDE_MAX_ROWS, lib.load().rlis_gemm_bf16_stream_max_rows(K)))
+
+
 def _one_item_per_wave(K: int) -> bool:
     """Whether a row of ``K`` fits the streaming kernel's forms that take one k item per wave
     (the fused norm, the gated and the scaled form)."""
@@ -272,6 +283,12 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     bf16 = x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
     aligned = (K % 8 == 0 and ldx % 8 == 0 and ldw % 8 == 0
                and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+    if bf16 and aligned and STREAM_MAX_ROWS < T <= stream_rows(K):
+        # 17 to 32 rows over a k that a wave holds in registers: one result, whoever asks
+        y = torch.empty((T, N), dtype=out_dtype, device=x.device)
+        lib.call("rlis_gemm_bf16_stream", x.data_ptr(), w.data_ptr(), y.data_ptr(),
+                 _DT[y.dtype], T, N, K, ldx, ldw, N, T * N, 0, stream)
+        return y
     if bf16 and aligned and partials and STREAM_MAX_ROWS < T <= SPLITK_MAX_ROWS:
         slices = lib.load().rlis_gemm_bf16_splitk_slices(N, K)
         y = torch.empty((slices, T, N), dtype=torch.float32, device=x.device)
@@ -392,7 +409,7 @@ class PendingProduct:
 
 def _streams_in_one_slice(x: torch.Tensor, w: torch.Tensor) -> bool:
     return (x.dim() == 2 and w.dim() == 2 and x.dtype == torch.bfloat16
-            and w.dtype == torch.bfloat16 and 0 < x.shape[0] <= STREAM_MAX_ROWS
+            and w.dtype == torch.bfloat16 and 0 < x.shape[0] <= stream_rows(x.shape[1])
             and x.shape[1] == w.shape[1] and x.shape[1] % 8 == 0 and stream_slices(x.shape[1]) == 1
             and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0
             and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
@@ -415,7 +432,9 @@ def can_join_norm_linear(product: PendingProduct, resid: torch.Tensor, w: torch.
     return (JOIN_NORM_LINEAR and resid.dtype == torch.float32 and resid.is_contiguous()
             and product.shape == (T, H) and w.dim() == 2 and w.shape[1] == H
             and w.dtype == torch.bfloat16 and w.stride(1) == 1 and w.stride(0) % 8 == 0
-            and w.data_ptr() % 16 == 0 and _one_item_per_wave(H))
+            and w.data_ptr() % 16 == 0 and _one_item_per_wave(H) and T <= stream_rows(H)
+            # (17 to 32 rows: the scaled form takes up to 256 partial sums of squares a row)
+            and (T <= 16 or lib.load().rlis_gemm_bf16_stream_join_tiles(H, product.x.shape[1]) <= 256))
 
 
 def linear_join_norm(product: PendingProduct, resid: torch.Tensor, norm_weight: torch.Tensor,
@@ -437,7 +456,7 @@ def linear_join_norm(product: PendingProduct, resid: torch.Tensor, norm_weight: 
         raise KernelError("linear_join_norm: cannot read the device properties")
     xw = torch.empty((T, N), dtype=torch.bfloat16, device=x.device)
     stride = -(-tiles // 4) * 4
-    ss = torch.empty((16, stride), dtype=torch.float32, device=x.device)[:, :tiles]
+    ss = torch.empty((-(-T // 16) * 16, stride), dtype=torch.float32, device=x.device)[:, :tiles]
     lib.call("rlis_gemm_bf16_stream_join", x.data_ptr(), w.data_ptr(), T, N, K, x.stride(0),
              w.stride(0), resid.data_ptr(), resid.data_ptr(), norm_weight.data_ptr(),
              _dt(norm_weight), int(bool(round_sum)), xw.data_ptr(), ss.data_ptr(), stride,
@@ -479,7 +498,7 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
                and 0 < T and K == w_gate_up.shape[1] and K % 8 == 0
                and ldx % 8 == 0 and ldw % 8 == 0 and x.data_ptr() % 16 == 0
                and w_gate_up.data_ptr() % 16 == 0)
-    streamed = fusable and T <= STREAM_MAX_ROWS and _one_item_per_wave(K)
+    streamed = fusable and T <= stream_rows(K) and _one_item_per_wave(K)
     skinny = fusable and not streamed and T <= SKINNY_MAX_ROWS and \
         (BF16_GEMM == "own" or T <= STREAM_MAX_ROWS)
     if not (streamed or skinny):

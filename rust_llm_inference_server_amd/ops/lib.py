@@ -80,6 +80,8 @@ def load() -> ctypes.CDLL:
     lib.rlis_attn_register_unit.argtypes = [I, P, P]
     lib.rlis_norm_linear_max_k.restype = c_int
     lib.rlis_norm_linear_max_k.argtypes = []
+    lib.rlis_gemm_bf16_stream_max_rows.restype = c_int
+    lib.rlis_gemm_bf16_stream_max_rows.argtypes = [I]
     _LIB = lib
     library_workspace(torch.device("cuda", torch.cuda.current_device()))
     return lib

@@ -38,8 +38,7 @@ class RMSNorm(Norm):
 
     def fused_linear(self, stream: ResidualStream, w: torch.Tensor, out_dtype: torch.dtype,
                      gated: bool, rows: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
-        count = stream.x.shape[0] if rows is None else rows.numel()
-        if self.out_dtype != torch.bfloat16 or not ops.can_fuse_norm_linear(stream.x, w, count):
+        if self.out_dtype != torch.bfloat16:
             return None
         product = stream.pending
         if isinstance(product, ops.PendingProduct) and rows is None \
@@ -49,6 +48,9 @@ class RMSNorm(Norm):
             xw, ss = ops.linear_join_norm(product, stream.x, self.weight, stream.round_parts)
             stream.pending = None
             return ops.linear_scaled(xw, ss, self.eps, w, out_dtype, gated=gated)
+        count = stream.x.shape[0] if rows is None else rows.numel()
+        if not ops.can_fuse_norm_linear(stream.x, w, count):
+            return None
         y, total = ops.norm_linear(stream.x, stream.delta(), self.weight, self.eps, w, out_dtype,
                                    gated=gated, rows=rows, round_parts=stream.round_parts)
         if rows is None:

@@ -217,15 +217,112 @@ def test_linear_streaming_kernel(ops, out_dtype, T, N, K):
                                    rtol=2e-2)
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16], ids=["f32out", "bf16out"])
+@pytest.mark.parametrize("T,N,K", [(17, 2048, 2048), (32, 3072, 2048), (31, 2048, 1024), (32, 3072, 3072),
+                                   (24, 130, 256), (32, 331, 512), (28, 17, 1792), (20, 16, 768),
+                                   (32, 16384, 2048), (19, 1002, 2816), (32, 128256, 256)])
+def test_linear_streaming_kernel_for_17_to_32_rows(ops, out_dtype, T, N, K):
+    """The streaming kernel's form for 17 to 32 rows (two groups of 16 tokens in a wave's
+    registers; k up to 3072 in whole items of 256; two tiles ahead up to eight waves), plain
+    and gated, against float64 products of the same bf16-rounded operands: sizes that end inside
+    a group of tokens, inside a row tile, with fewer k items than a workgroup has waves; and the
+    same rows as the kernel for up to 16 rows gives them (the same sums in the same order)."""
+    assert ops.stream_rows(K) >= T
+    x, w = rnd(T, K, dtype=torch.bfloat16, seed=3), rnd(N, K, dtype=torch.bfloat16, seed=4, scale=0.05)
+    want = (x.double() @ w.double().t()).float()
+    got = ops.linear(x, w, out_dtype)
+    assert got.dtype == out_dtype and got.shape == (T, N)
+    scale = max(1.0, want.abs().max().item())
+    if out_dtype == torch.float32:
+        torch.testing.assert_close(got, want, atol=2e-5 * scale * math.sqrt(K / 64), rtol=1e-4)
+    else:
+        torch.testing.assert_close(got.float(), want, atol=scale / 128, rtol=1e-2)
+    few = ops.linear(x[:16], w, out_dtype)
+    assert torch.equal(got[:16], few)
+    old = ops.STREAM_WIDE_MAX_ROWS
+    try:
+        ops.STREAM_WIDE_MAX_ROWS = 0                       # the library's product instead
+        other = ops.linear(x, w, out_dtype)
+    finally:
+        ops.STREAM_WIDE_MAX_ROWS = old
+    torch.testing.assert_close(got.float(), other.float(), atol=scale / 64, rtol=2e-2)
+    if N % 2 == 0 and out_dtype == torch.bfloat16:
+        gated = ops.linear_swiglu(x, w)
+        g, u = want[:, :N // 2].double(), want[:, N // 2:].double()
+        want_g = (torch.nn.functional.silu(g) * u).float()
+        torch.testing.assert_close(gated.float(), want_g, atol=max(1.0, want_g.abs().max().item()) / 64,
+                                   rtol=2e-2)
+        assert torch.equal(gated[:16], ops.linear_swiglu(x[:16], w))
+
+
+@pytest.mark.parametrize("T,H,K,N", [(17, 2048, 2048, 4096), (32, 2048, 2048, 16384), (31, 256, 512, 72),
+                                     (32, 1024, 1024, 1002), (25, 768, 2048, 64), (32, 3072, 3072, 512),
+                                     (20, 2048, 2816, 3072), (32, 1536, 256, 520)])
+@pytest.mark.parametrize("norm_dtype", DTYPES, ids=["normw32", "normw16"])
+@pytest.mark.parametrize("round_sum", [True, False])
+def test_linear_join_norm_and_linear_scaled_for_17_to_32_rows(ops, T, H, K, N, norm_dtype, round_sum):
+    """The norm between two streaming products in two kernels, as above, with 17 to 32 rows:
+    against float64 formulas and against the norm kernel on the plain product's result."""
+    x = rnd(T, K, dtype=torch.bfloat16, seed=1)
+    w1 = rnd(H, K, dtype=torch.bfloat16, seed=2, scale=0.05)
+    w2 = rnd(N, H, dtype=torch.bfloat16, seed=3, scale=0.05)
+    resid = rnd(T, H, seed=4, scale=3.0)
+    nw = (rnd(H, seed=5).abs() + 0.5).to(norm_dtype)
+    eps = 1e-5
+    product = ops.pending_linear(x, w1, torch.bfloat16)
+    assert isinstance(product, ops.PendingProduct) and product.shape == (T, H)
+    assert ops.can_join_norm_linear(product, resid, w2)
+    delta = x.double() @ w1.double().t()
+    if round_sum:
+        delta = delta.float().to(torch.bfloat16).double()
+    s = resid.double() + delta
+    normed = s / torch.sqrt((s * s).mean(-1, keepdim=True) + eps) * nw.double()
+    want = normed @ w2.double().t()
+    mine = resid.clone()
+    xw, ss = ops.linear_join_norm(product, mine, nw, round_sum)
+    torch.testing.assert_close(mine.double(), s, atol=2e-2 if round_sum else 1e-3, rtol=1e-2)
+    if round_sum:                       # the plain product, rounded, added by the residual kernel
+        ref = resid.clone()
+        ops.add_residual(ref, product.run(), round_parts=True)
+        torch.testing.assert_close(mine, ref, atol=1e-6, rtol=1e-6)
+    assert xw.dtype == torch.bfloat16 and xw.shape == (T, H) and ss.shape[0] == -(-T // 16) * 16
+    torch.testing.assert_close(ss[:T].sum(1).double(), (mine.double() ** 2).sum(-1), rtol=1e-5, atol=1e-5)
+    assert torch.equal(xw, (mine * nw.float()).to(torch.bfloat16))
+    for out_dtype in (torch.float32, torch.bfloat16):
+        got = ops.linear_scaled(xw, ss, eps, w2, out_dtype)
+        assert got.dtype == out_dtype and got.shape == (T, N)
+        scale = max(1.0, want.abs().max().item())
+        torch.testing.assert_close(got.double(), want, atol=scale / 64, rtol=2e-2)
+    # the same rows as 16 rows by themselves give (the first product's sums in the same order;
+    # the second's scale from another order of the partial sums of squares)
+    few = resid[:16].clone()
+    xw16, ss16 = ops.linear_join_norm(ops.pending_linear(x[:16], w1, torch.bfloat16), few, nw, round_sum)
+    assert torch.equal(few, mine[:16]) and torch.equal(xw16, xw[:16])
+    torch.testing.assert_close(ops.linear_scaled(xw16, ss16, eps, w2, torch.float32),
+                               ops.linear_scaled(xw, ss, eps, w2, torch.float32)[:16], atol=1e-4, rtol=1e-5)
+    if N % 2 == 0:
+        got = ops.linear_scaled(xw, ss, eps, w2, torch.bfloat16, gated=True)
+        g, u = want[:, :N // 2], want[:, N // 2:]
+        want_g = torch.nn.functional.silu(g) * u
+        torch.testing.assert_close(got.double(), want_g, atol=max(1.0, want_g.abs().max().item()) / 32,
+                                   rtol=3e-2)
+    # a k that no wave holds 17 rows of, or more than 32 rows: the plain product comes back
+    assert isinstance(ops.pending_linear(rnd(T, 4096, dtype=torch.bfloat16), rnd(64, 4096, dtype=torch.bfloat16)),
+                      torch.Tensor)
+    assert isinstance(ops.pending_linear(rnd(33, K, dtype=torch.bfloat16), w1), torch.Tensor)
+
+
 @pytest.mark.parametrize("T,N,K", [(17, 2048, 2048), (64, 2048, 8192), (33, 3072, 2048), (24, 130, 96),
                                    (64, 331, 104), (48, 17, 14336), (19, 1001, 4608), (40, 16, 8),
                                    (64, 4096, 14336), (50, 3072, 3072), (64, 3072, 8192),
                                    (32, 4096, 14344), (48, 8192, 3000), (17, 6144, 1536)])
-def test_linear_split_k_kernel(ops, T, N, K):
+def test_linear_split_k_kernel(ops, monkeypatch, T, N, K):
     """The split-k kernel that 17 to 64 rows take where the result joins the residual stream:
     float32 partial sums per k slice against float64 products of the same bf16-rounded
     operands; sizes that end inside a slice, inside a block of weight rows and inside a token
-    group.  A row's sums are the same bits with 17 rows in the call as with 64."""
+    group.  A row's sums are the same bits with 17 rows in the call as with 64.  (With the
+    streaming kernel's form for 17 to 64 rows switched off, which takes the short k first.)"""
+    monkeypatch.setattr(ops, "STREAM_WIDE_MAX_ROWS", 0)
     x, w = rnd(T, K, dtype=torch.bfloat16, seed=3), rnd(N, K, dtype=torch.bfloat16, seed=4, scale=0.05)
     want = (x.double() @ w.double().t()).float()
     parts = ops.linear(x, w, partials=True)
@@ -252,10 +349,11 @@ def test_linear_split_k_kernel(ops, T, N, K):
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16], ids=["f32out", "bf16out"])
 @pytest.mark.parametrize("T,N,K", [(17, 3072, 2048), (64, 16384, 2048), (100, 2048, 8192), (575, 5120, 3072),
                                    (2048, 2048, 2048), (33, 331, 104), (300, 1001, 776), (65, 8, 8)])
-def test_library_product_called_directly(ops, out_dtype, T, N, K):
+def test_library_product_called_directly(ops, monkeypatch, out_dtype, T, N, K):
     """bfloat16 products beyond the hand-written kernels' row counts go to hipBLASLt through its
     own entry points: against float64 products of the same operands, against the same library
     through torch.matmul, strided operands, and twice (the second call takes the kept plan)."""
+    monkeypatch.setattr(ops, "STREAM_WIDE_MAX_ROWS", 0)   # 17 to 64 rows of a short k: the library's too
     from rust_llm_inference_server_amd.ops import lib
     assert lib.library_workspace(torch.device(DEV)) is not None, "hipBLASLt's entry points were not found"
     x, w = rnd(T, K, dtype=torch.bfloat16, seed=3), rnd(N, K, dtype=torch.bfloat16, seed=4, scale=0.05)
@@ -417,10 +515,13 @@ def test_linear_join_norm_and_linear_scaled(ops, T, H, K, N, norm_dtype, round_s
         want_g = torch.nn.functional.silu(g) * u
         torch.testing.assert_close(got.double(), want_g, atol=max(1.0, want_g.abs().max().item()) / 32,
                                    rtol=3e-2)
-    # more than one k slice, more than 16 rows, or float32: the plain product comes back
+    # more than one k slice, more than 32 rows (more than 16 of a long k), or float32: the plain
+    # product comes back
     assert isinstance(ops.pending_linear(rnd(T, 8448, dtype=torch.bfloat16), rnd(64, 8448, dtype=torch.bfloat16)),
                       torch.Tensor)
-    assert isinstance(ops.pending_linear(rnd(17, K, dtype=torch.bfloat16), w1), torch.Tensor)
+    assert isinstance(ops.pending_linear(rnd(33, K, dtype=torch.bfloat16), w1), torch.Tensor)
+    assert isinstance(ops.pending_linear(rnd(17, 8192, dtype=torch.bfloat16), rnd(64, 8192, dtype=torch.bfloat16)),
+                      torch.Tensor)
     assert isinstance(ops.pending_linear(rnd(T, K), rnd(H, K)), torch.Tensor)
 
 

@@ -5,8 +5,9 @@ requests, and the decode attention deals its partitions out by the size of the b
 through the engine (the reference's engine tests at their largest batch,
 crates/engine/tests/engine.rs:58-83, 157-210) and logits through the step function, against
 the plain implementation, in float32 and bfloat16, on tiny A (head size 16: vector-unit
-attention in both dtypes) and tiny D (head size 64: the matrix-core decode kernel with the
-rotation inside)."""
+attention in both dtypes), tiny D (head size 64: the matrix-core decode kernel with the
+rotation inside) and a configuration whose widths the streaming kernels take with 17 to 64
+rows as well."""
 import pytest
 import torch
 
@@ -21,16 +22,27 @@ pytestmark = pytest.mark.gpu
 
 TOL = {"float32": 1e-4, "bfloat16": 2e-2}          # the replay tests' gates
 
+# Widths in whole k items of 256 (hidden 256, feed-forward 512), which the streaming kernels take
+# with 17 to 64 rows too: the output and down projections then join the residual themselves and
+# the products behind the norms scale by the sums they hand over, as with up to 16 rows.
+TINY_W = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 256, "intermediate_size": 512,
+    "num_hidden_layers": 2, "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 64,
+    "vocab_size": 300, "rms_norm_eps": 1e-5, "rope_theta": 10000.0, "rope_scaling": None,
+    "max_position_embeddings": 128, "tie_word_embeddings": False,
+}
+CONFIGS = dict(TINY, w=TINY_W)
 
-@pytest.fixture(scope="module", params=["a", "d"])
+
+@pytest.fixture(scope="module", params=["a", "d", "w"])
 def case(request, tmp_path_factory):
     name = request.param
     out = {}
     for dtype, tdt in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
-        folder = make_model_folder(tmp_path_factory.mktemp(f"many_{name}_{dtype}"), TINY[name],
+        folder = make_model_folder(tmp_path_factory.mktemp(f"many_{name}_{dtype}"), CONFIGS[name],
                                    seed=13, dtype=tdt)
         out[dtype] = (folder, plain.read_weights(folder), plain.read_config(folder))
-    return name, TINY[name], out
+    return name, CONFIGS[name], out
 
 
 def load(folder, dtype, max_positions):
