@@ -78,7 +78,6 @@ __global__ __launch_bounds__(AHEAD == 2 ? 512 : (TG == 2 ? 768 : 512)) void gemm
   uint4 a0[TR / 2], a1[AHEAD == 2 ? TR / 2 : 1];
   int tile = blockIdx.x;
   RLIS_WIDE_LOAD_TILE(a0, tile);         // the first tile is on its way during the prologue
-  if constexpr (AHEAD == 2) RLIS_WIDE_LOAD_TILE(a1, tile + (int)gridDim.x);
   asm volatile("" ::: "memory");
 
   // The rows of x in operand layout: token 16 g + oi, k = kb + (4 j + og) * 8 .. + 8 for step
@@ -90,11 +89,17 @@ __global__ __launch_bounds__(AHEAD == 2 ? 512 : (TG == 2 ? 768 : 512)) void gemm
 #pragma unroll
     for (int j = 0; j < 8; ++j) b[g][j].v = __builtin_bit_cast(bf16x8, *(GlobalU4)(xb + j * 32));
   }
+  // The second tile follows the rows of x: the first products wait for the first tile and x,
+  // not for the second tile as well.
+  if constexpr (AHEAD == 2) {
+    asm volatile("" ::: "memory");
+    RLIS_WIDE_LOAD_TILE(a1, tile + (int)gridDim.x);
+  }
 
   // SCALED: the rows' scales come as partial sums of squares, scale_count a token.  A wave
   // takes the tokens wave, wave + nwaves, ... (at most kScaleTokens of them: a workgroup has
-  // four waves or more, nine or more with one tile ahead), a lane the parts lane, lane + 64, ...  The first kScaleParts parts a
-  // lane are asked for here, all at once and without a condition, and added up only when the
+  // four waves or more, nine or more with one tile ahead), a lane the parts lane, lane + 64,
+  // ...  The first kScaleParts parts a lane are asked for here, all at once and without a condition, and added up only when the
   // first tile is stored; the order of a sum depends on scale_count alone (at most 64
   // kScaleParts: the launch sees to that).
   constexpr int kScaleTokens = SCALED ? (AHEAD == 1 ? 2 : 4) * TG : 1, kScaleParts = SCALED ? 4 : 1;
