@@ -1156,8 +1156,8 @@ static int dispatch_stream(const char* name, const void* X, const void* W, void*
 RLIS_API int rlis_gemm_bf16_stream_slices(int K) { return stream_slices(K); }
 
 // The most rows of x that rlis_gemm_bf16_stream and its joining and scaled forms take for rows
-// of K: 16, or up to 64 where K is a whole number of items and short enough for the kernel that
-// keeps 32 or 64 rows in registers.
+// of K: 16, or 32 where K is a whole number of items and short enough for the kernel that keeps
+// 32 rows in registers.
 RLIS_API int rlis_gemm_bf16_stream_max_rows(int K) { return rlis_stream_wide_rows(K); }
 
 // The longest row that rlis_norm_linear_bf16 takes.

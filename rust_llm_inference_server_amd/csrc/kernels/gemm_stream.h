@@ -1,4 +1,4 @@
-// What the streaming products (gemm.hip: up to 16 rows; gemm_wide.hip: 17 to 64 rows) share.
+// What the streaming products (gemm.hip: up to 16 rows; gemm_wide.hip: 17 to 32 rows) share.
 #pragma once
 #include "common.h"
 
@@ -77,11 +77,11 @@ int rlis_stream_compute_units();
 // tile.  Ties go to the larger tile (fewer workgroups, fewer prologues).
 int rlis_stream_balanced_rows(int N, int slices, bool gated, int num_cus);
 
-// The most rows of x that the streaming products take for rows of K: 16, or up to 64 where the
-// kernel for 17 to 64 rows holds them (gemm_wide.hip).
+// The most rows of x that the streaming products take for rows of K: 16, or 32 where the kernel
+// for 17 to 32 rows holds them (gemm_wide.hip).
 int rlis_stream_wide_rows(int K);
 
-// 17 to 64 rows (gemm_wide.hip).  mode: kStreamPlain, kStreamScaled or kStreamJoin; the
+// 17 to 32 rows (gemm_wide.hip).  mode: kStreamPlain, kStreamScaled or kStreamJoin; the
 // arguments as the entry points of gemm.hip take them.
 int rlis_launch_stream_wide(const char* name, int mode, const void* X, const void* W, void* Y,
                             int y_dtype, int T, int N, int K, long long ldx, long long ldw,

@@ -1,4 +1,4 @@
-// The streaming product for 17 to 64 rows of x: y (T, N) = x W^T at the speed of the weight
+// The streaming product for 17 to 32 rows of x: y (T, N) = x W^T at the speed of the weight
 // stream, with the same forms as the kernel for up to 16 rows (gemm.hip): plain, gated (the
 // SwiGLU before the store), scaled (rows that come normed but for a scale, taken from partial
 // sums of squares) and joining (the product adds itself to the residual and leaves the rows
@@ -7,11 +7,11 @@
 // The cut is the same: tiles of 16, 12 or 8 weight rows, a wave per k item of 256, persistent
 // workgroups that walk over tiles with their rows of x in registers, weights loaded row by row
 // (512 contiguous bytes per half wave) one tile ahead and turned into operand layout through an
-// LDS tile private to the wave.  What differs is that a wave holds TG = 2 or 4 groups of 16
-// tokens: TG accumulators and 32 TG registers of x, which every weight fragment read from LDS
-// then serves.  That fits up to 12 waves (K = 3072) with two groups and up to 8 (K = 2048) with
-// four; K is a whole number of items, and one slice.  Rows of x past T take row T - 1 (their
-// results are not stored), so nothing is zeroed after a load.
+// LDS tile private to the wave.  What differs is that a wave holds TG = 2 groups of 16 tokens:
+// TG accumulators and 32 TG registers of x, which every weight fragment read from LDS then
+// serves.  That fits up to 12 waves (K = 3072); K is a whole number of items, and one slice.
+// Rows of x past T take row T - 1 (their results are not stored), so nothing is zeroed after a
+// load.  (The kernel is written for any TG; four groups are not offered, see launch_groups.)
 #include "gemm_stream.h"
 
 namespace {
@@ -259,7 +259,7 @@ int launch_tiles(const void* X, const void* W, void* Y, StreamShape sh, const St
     hipError_t e = hipFuncSetAttribute(
         (const void*)gemm_bf16_stream_wide_kernel<TC, GATED, TR, MODE, TG, AHEAD>,
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)(wide_max_waves(TG) * kPerWave + kScales));
-    RLIS_REQUIRE(e == hipSuccess, "gemm_bf16_stream (17 to 64 rows): cannot raise the LDS limit: %s",
+    RLIS_REQUIRE(e == hipSuccess, "gemm_bf16_stream (17 to 32 rows): cannot raise the LDS limit: %s",
                  hipGetErrorString(e));
     lds_raised = true;
   }
@@ -342,7 +342,7 @@ int rlis_launch_stream_wide(const char* name, int mode, const void* X, const voi
       rc = launch_groups<bf16_t, false, kStreamPlain>(X, W, Y, sh, nm, nwaves, num_cus, stream);
     else RLIS_REQUIRE(false, "%s: unknown output dtype %d", name, y_dtype);
   } else {
-    RLIS_REQUIRE(false, "%s: no such form for 17 to 64 rows", name);
+    RLIS_REQUIRE(false, "%s: no such form for 17 to 32 rows", name);
   }
   if (rc) return rc;
   RLIS_LAUNCH_CHECK(name);
