@@ -99,8 +99,8 @@ __global__ __launch_bounds__(AHEAD == 2 ? 512 : (TG == 2 ? 768 : 512)) void gemm
   // SCALED: the rows' scales come as partial sums of squares, scale_count a token.  A wave
   // takes the tokens wave, wave + nwaves, ... (at most kScaleTokens of them: a workgroup has
   // four waves or more, nine or more with one tile ahead), a lane the parts lane, lane + 64,
-  // ...  The first kScaleParts parts a lane are asked for here, all at once and without a condition, and added up only when the
-  // first tile is stored; the order of a sum depends on scale_count alone (at most 64
+  // ...  They are asked for here, all at once and without a condition, and added up only when
+  // the first tile is stored; the order of a sum depends on scale_count alone (at most 64
   // kScaleParts: the launch sees to that).
   constexpr int kScaleTokens = SCALED ? (AHEAD == 1 ? 2 : 4) * TG : 1, kScaleParts = SCALED ? 4 : 1;
   float scale_ahead[kScaleTokens][kScaleParts];
