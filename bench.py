@@ -9,7 +9,7 @@ the engine (schedule, forward from the paged cache, on-device greedy sampling, t
 back), bracketed by device synchronisation.  On the same line: a 2,048-token prefill with its
 fraction of the bf16 matrix peak, the decode step's achieved fraction of the HBM roofline
 (bytes that must be read: every weight once plus the live requests' cache), and under
-``points`` decode throughput at batch 1, 8 and 64 over 256 new tokens after 512-token prompts,
+``points`` decode throughput at batch 1, 8, 32 and 64 over 256 new tokens after 512-token prompts,
 whatever ``--steps`` says (each with its fraction of the HBM roofline, ``..._frac``, and the mean
 context of its timed steps, ``..._ctx``) and, while the time budget lasts (``--extra-seconds``;
 ``--skip-extra`` leaves them out), three more workloads, each in a fresh model:
@@ -182,7 +182,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--points-context", type=int, default=512,
-                    help="prompt length of the decode points at batch 1, 8 and 64")
+                    help="prompt length of the decode points at batch 1, 8, 32 and 64")
     ap.add_argument("--points-new-tokens", type=int, default=256,
                     help="timed decode steps of each of those points")
     ap.add_argument("--skip-points", action="store_true")
@@ -333,9 +333,9 @@ def main() -> int:
 
     points = {}
     if not args.skip_points:
-        # the metric's own workload: 512-token prompts, then 256 new tokens at batch 1, 8 and 64
+        # the metric's own workload: 512-token prompts, then 256 new tokens at batch 1, 8, 32 and 64
         # (after W untimed decode steps, so the timed steps' mean context is 640 + W)
-        for b in (1, 8, 64):
+        for b in (1, 8, 32, 64):
             v, ms, mean = decode_run(b, 0, args.points_new_tokens, W, prompt_len=args.points_context)
             frac = shape.decode_step_bytes(b, mean) / (ms * 1e-3) / 1e9 / HBM_GBPS
             name = f"decode_b{b}" if b != args.batch else f"decode_b{b}_p{args.points_context}"

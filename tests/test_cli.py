@@ -118,9 +118,9 @@ def test_bench_line_has_the_agreed_fields():
     assert set(rec["prefill"]) == {"value", "tokens", "ms", "frac"} and rec["prefill"]["tokens"] == 2048
     assert rec["roofline"]["bound"] == "hbm" and rec["roofline"]["peak"] == 8000.0
     assert abs(rec["roofline"]["frac"] - rec["roofline"]["achieved"] / 8000.0) < 1e-3
-    assert {"decode_b1", "decode_b64", "decode_b8_p512"} <= set(rec["points"])
+    assert {"decode_b1", "decode_b32", "decode_b64", "decode_b8_p512"} <= set(rec["points"])
     assert all(isinstance(v, (int, float)) for v in rec["points"].values())
-    for name in ("decode_b1", "decode_b64", "decode_b8_p512"):
+    for name in ("decode_b1", "decode_b32", "decode_b64", "decode_b8_p512"):
         assert 0 < rec["points"][name + "_frac"] < 1
         # the metric's own workload whatever --steps says: 256 new tokens after prompts of
         # 512, timed after the warm-up steps, so a mean context of 512 + 2 + 129
