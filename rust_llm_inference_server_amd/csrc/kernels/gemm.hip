@@ -651,7 +651,7 @@ __device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
 }
 
 template <typename TC, bool GATED, int TR /* weight rows per tile: 16, 12 or 8 */, int MODE,
-          int IPW /* k items per wave: 1 or 4 */>
+          int IPW /* k items per wave: 1 or 4 */, bool PACK = false /* see below */>
 __global__ __launch_bounds__(IPW == 1 ? 1024 : 512) void gemm_bf16_stream_kernel(const bf16_t* __restrict__ X,
                                                                 const bf16_t* __restrict__ W,
                                                                 TC* __restrict__ Y,
@@ -663,6 +663,13 @@ __global__ __launch_bounds__(IPW == 1 ? 1024 : 512) void gemm_bf16_stream_kernel
   static_assert(!(JOIN && GATED), "a product that joins the residual has no gate");
   static_assert(IPW == 1 || (IPW == 4 && TR == 8 && !GATED && (MODE == kStreamPlain || JOIN)),
                 "four items per wave: tiles of 8 rows of a plain or joining product");
+  // PACK (four items per wave, up to 8 tokens): a tile of 8 weight rows and 8 tokens fill half
+  // of a 16 x 16 product each, so two halves of k share one: lanes oi >= 8 hold, for weight row
+  // and token oi - 8, the k chunks four further on.  Rows and columns 0..7 of the result then
+  // carry one half of k and rows and columns 8..15 the other (the rest is not looked at), a
+  // product covers 64 k, and x takes half the loads and registers.
+  static_assert(!PACK || IPW > 1, "packing two halves of k is for several items per wave");
+  constexpr int NJ = PACK ? 4 : 8;                      // products per item
   constexpr int kTileBytes = NORM ? kStreamTileBytes : TR * kStreamItem * 2;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, nwaves = blockDim.x / 64;
   unsigned char* tile_s = stream_smem + wave * (IPW * kTileBytes);     // a tile per item
@@ -732,7 +739,7 @@ __global__ __launch_bounds__(IPW == 1 ? 1024 : 512) void gemm_bf16_stream_kernel
 
   // The rows of x in operand layout: token oi, k = kb + (4 j + og) * 8 .. + 8 for step j (of
   // item `it`, kStreamItem further on).
-  Frag8 b[IPW][8];
+  Frag8 b[IPW][NJ];
   float inv_rms = 1.f;                   // NORM: of token tid / 16, in the threads that store
   // SCALED: the scale comes as partial sums of squares, scale_count a token.  Thread (token
   // tid / 16, i = tid % 16) of the 256 storing threads takes parts 4 i .. 4 i + 3, + 64, ...
@@ -747,10 +754,15 @@ __global__ __launch_bounds__(IPW == 1 ? 1024 : 512) void gemm_bf16_stream_kernel
 #pragma unroll
     for (int it = 0; it < IPW; ++it) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
+      for (int j = 0; j < NJ; ++j) {
         const int k = kb + it * kStreamItem + (4 * j + og) * 8;
         const bool ok = item + it < nitems && oi < T && k < K;
-        if constexpr (IPW == 1) {
+        if constexpr (PACK) {
+          // token oi % 8, chunks 8 j + 4 (oi / 8) + og: one address for the four loads
+          GlobalBf16 xb = x_base + (long long)min(oi % 8, T - 1) * sh.ldx + kb + it * kStreamItem +
+                          (oi / 8) * 32 + og * 8;
+          b[it][j].v = __builtin_bit_cast(bf16x8, *(GlobalU4)(xb + j * 64));
+        } else if constexpr (IPW == 1) {
           const uint4 v = *(const uint4*)(X + (ok ? (long long)oi * sh.ldx + k : 0));
           b[it][j].u = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
         } else {
@@ -926,13 +938,15 @@ __global__ __launch_bounds__(IPW == 1 ? 1024 : 512) void gemm_bf16_stream_kernel
 #pragma unroll
       for (int it = 0; it < IPW; ++it) {
 #pragma unroll
-        for (int j0 = 0; j0 < 8; j0 += 4) {
+        for (int j0 = 0; j0 < NJ; j0 += 4) {
           Bits4 af[4];
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            // tile rows beyond TR repeat the first ones: their products are not stored
+            // tile rows beyond TR repeat the first ones: their products are not stored (PACK:
+            // they carry the chunks of the other half of k)
+            const int chunk = PACK ? 8 * (j0 + j) + 4 * (oi / 8) + og : 4 * (j0 + j) + og;
             af[j] = *(const Bits4*)(tile_s + it * kTileBytes + (oi % TR) * (kStreamItem * 2) +
-                                    (((4 * (j0 + j) + og) ^ (oi % TR)) * 16));
+                                    ((chunk ^ (oi % TR)) * 16));
           }
           // With two waves per SIMD nobody else fills the time a read from LDS takes: four are
           // asked for before the first of their products (the statement, which every read
@@ -990,7 +1004,10 @@ __global__ __launch_bounds__(IPW == 1 ? 1024 : 512) void gemm_bf16_stream_kernel
         float sq = 0.f;
         if (i < TR && t < T && n < N) {
           float sum = 0.f;
-          for (int w = 0; w < nwaves; ++w) sum += red_p[w * 256 + t * 16 + i];
+          for (int w = 0; w < nwaves; ++w) {
+            sum += red_p[w * 256 + t * 16 + i];
+            if constexpr (PACK) sum += red_p[w * 256 + (t + 8) * 16 + i + 8];
+          }
           sum *= inv_rms;
           if (nm.round_parts) sum = bf16_to_f32(f32_to_bf16(sum));
           const float total = join_resid + sum;
@@ -1007,7 +1024,10 @@ __global__ __launch_bounds__(IPW == 1 ? 1024 : 512) void gemm_bf16_stream_kernel
         const long long n = (long long)tile * TR + i;
         if (i < TR && t < T && n < N) {
           float sum = 0.f;
-          for (int w = 0; w < nwaves; ++w) sum += red_p[w * 256 + t * 16 + i];
+          for (int w = 0; w < nwaves; ++w) {
+            sum += red_p[w * 256 + t * 16 + i];
+            if constexpr (PACK) sum += red_p[w * 256 + (t + 8) * 16 + i + 8];
+          }
           st(y + n, sum * inv_rms);
         }
       }
@@ -1034,7 +1054,7 @@ static int stream_slices(int K) {
 // scaled form.
 constexpr int kStreamNormMaxK = kStreamMaxWaves * kStreamItem;
 
-template <typename TC, bool GATED, int TR, int MODE, int IPW = 1>
+template <typename TC, bool GATED, int TR, int MODE, int IPW = 1, bool PACK = false>
 static int launch_stream_tiles(const void* X, const void* W, void* Y, StreamShape sh,
                                const StreamNorm& nm, int nwaves, int num_cus,
                                hipStream_t stream) {
@@ -1042,7 +1062,7 @@ static int launch_stream_tiles(const void* X, const void* W, void* Y, StreamShap
   static bool lds_raised = false;
   if (!lds_raised) {
     hipError_t e = hipFuncSetAttribute(
-        (const void*)gemm_bf16_stream_kernel<TC, GATED, TR, MODE, IPW>,
+        (const void*)gemm_bf16_stream_kernel<TC, GATED, TR, MODE, IPW, PACK>,
         hipFuncAttributeMaxDynamicSharedMemorySize,
         (IPW == 1 ? kStreamMaxWaves : 2 * kStreamMaxWaves / IPW) * (kTileBytes + 2048));
     RLIS_REQUIRE(e == hipSuccess, "gemm_bf16_stream: cannot raise the LDS limit: %s",
@@ -1057,7 +1077,7 @@ static int launch_stream_tiles(const void* X, const void* W, void* Y, StreamShap
   long long groups = tiles;                                // workgroups per slice
   const long long cap = max(1, num_cus * per_cu / sh.num_slices);
   if (groups > cap) groups = cap;
-  gemm_bf16_stream_kernel<TC, GATED, TR, MODE, IPW>
+  gemm_bf16_stream_kernel<TC, GATED, TR, MODE, IPW, PACK>
       <<<(int)(groups * sh.num_slices), nwaves * 64, smem, stream>>>(
           (const bf16_t*)X, (const bf16_t*)W, (TC*)Y, sh, nm);
   return 0;
@@ -1110,9 +1130,13 @@ static int launch_stream(const void* X, const void* W, void* Y, int T, int N, in
   sh.num_slices = slices;
   sh.num_tiles = 0;
   if (ipw > 1) {
-    if constexpr (!GATED && (MODE == kStreamPlain || MODE == kStreamJoin))
+    if constexpr (!GATED && (MODE == kStreamPlain || MODE == kStreamJoin)) {
+      if (T <= 8)
+        return launch_stream_tiles<TC, false, 8, MODE, kStreamFour, true>(X, W, Y, sh, nm, nwaves,
+                                                                          num_cus, stream);
       return launch_stream_tiles<TC, false, 8, MODE, kStreamFour>(X, W, Y, sh, nm, nwaves, num_cus,
                                                                   stream);
+    }
     RLIS_REQUIRE(false, "gemm_bf16_stream: K=%d is too long for this form (at most %d)", K,
                  kStreamNormMaxK);
   }
