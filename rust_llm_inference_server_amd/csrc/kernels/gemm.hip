@@ -663,12 +663,14 @@ __global__ __launch_bounds__(IPW == 1 ? 1024 : 512) void gemm_bf16_stream_kernel
   static_assert(!(JOIN && GATED), "a product that joins the residual has no gate");
   static_assert(IPW == 1 || (IPW == 4 && TR == 8 && !GATED && (MODE == kStreamPlain || JOIN)),
                 "four items per wave: tiles of 8 rows of a plain or joining product");
-  // PACK (four items per wave, up to 8 tokens): a tile of 8 weight rows and 8 tokens fill half
+  // PACK (up to 8 tokens): a tile of 8 weight rows and 8 tokens fill half
   // of a 16 x 16 product each, so two halves of k share one: lanes oi >= 8 hold, for weight row
   // and token oi - 8, the k chunks four further on.  Rows and columns 0..7 of the result then
   // carry one half of k and rows and columns 8..15 the other (the rest is not looked at), a
   // product covers 64 k, and x takes half the loads and registers.
-  static_assert(!PACK || IPW > 1, "packing two halves of k is for several items per wave");
+  // (The launch sees to it that every wave then has whole items: nothing is zeroed.)
+  static_assert(!PACK || (TR == 8 && !GATED && (MODE == kStreamPlain || JOIN)),
+                "packing two halves of k: tiles of 8 rows of a plain or joining product");
   constexpr int NJ = PACK ? 4 : 8;                      // products per item
   constexpr int kTileBytes = NORM ? kStreamTileBytes : TR * kStreamItem * 2;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, nwaves = blockDim.x / 64;
@@ -1142,6 +1144,12 @@ static int launch_stream(const void* X, const void* W, void* Y, int T, int N, in
   }
   switch (stream_tile_rows(N, K, GATED, MODE == kStreamNorm, num_cus)) {
     case 8:
+      // up to 8 tokens over whole items, one for every wave: two halves of k share a product
+      if constexpr (!GATED && (MODE == kStreamPlain || MODE == kStreamJoin)) {
+        if (T <= 8 && K % kStreamItem == 0 && slices * nwaves == nitems)
+          return launch_stream_tiles<TC, false, 8, MODE, 1, true>(X, W, Y, sh, nm, nwaves, num_cus,
+                                                                  stream);
+      }
       return launch_stream_tiles<TC, GATED, 8, MODE>(X, W, Y, sh, nm, nwaves, num_cus, stream);
     case 12:
       return launch_stream_tiles<TC, GATED, 12, MODE>(X, W, Y, sh, nm, nwaves, num_cus, stream);
