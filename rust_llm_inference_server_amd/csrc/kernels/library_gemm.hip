@@ -115,8 +115,12 @@ static int lt_gemm(const void* X, const void* W, void* Y, int out_f32, int T, in
   RLIS_REQUIRE(he == hipSuccess, "lt_gemm: %s", hipGetErrorString(he));
   hipblasLtHandle_t handle = nullptr;
   LtPlan plan;
+  // One lock from the look-up to the launch: the device's handle is shared by all threads, and
+  // the library's launch path is not known to take two calls on one handle at once (two
+  // runners on two threads did get wrong products and a failed call that way).  The launch is
+  // asynchronous, so what is serialised is the host's part of it.
+  std::lock_guard<std::mutex> lock(lt_mutex);
   {
-    std::lock_guard<std::mutex> lock(lt_mutex);
     RLIS_REQUIRE(lt.lib != nullptr, "lt_gemm: the library has not been opened");
     auto h = lt_handles.find(device);
     if (h == lt_handles.end()) {

@@ -17,7 +17,7 @@ from __future__ import annotations
 
 import itertools
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional, Sequence, Tuple
+from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -70,6 +70,11 @@ class StepContext:
     host_new: List[int] = field(default_factory=list)
     host_state_slots: List[int] = field(default_factory=list)
     host_order: List[int] = field(default_factory=list)   # entry index of every sequence
+    # The one device buffer that all the arrays above are views of, and the same step over
+    # another buffer of that layout (for a captured step, whose kernels read a buffer that
+    # stays where it is).
+    buffer: Optional[torch.Tensor] = None
+    over: Optional[Callable[[torch.Tensor], "StepContext"]] = None
 
 
 class MetadataBuffer:
@@ -217,25 +222,34 @@ def build_step(entries: Sequence[StepEntry], cache, device: torch.device,
         o, c = layout[name]
         view_host[o:o + c] = arr
     dev = host[:at].to(device, non_blocking=True)
+    fixed = dict(num_tokens=T, num_seqs=S, num_logit_rows=R, max_context=max_context,
+                 max_new=max_new, all_decode=num_single == S, num_single=num_single,
+                 lengths=lengths, host_start_pos=start_pos.tolist(), host_new=new.tolist(),
+                 host_state_slots=host_view("state_slots").tolist(), host_order=order)
+    return _context_over(dev, layout, cache, widths, host_plans, fixed)
 
+
+def _context_over(dev: torch.Tensor, layout: Dict[str, Tuple[int, int]], cache,
+                  widths: Sequence[int], host_plans: Sequence[Tuple[Any, HostPlan]],
+                  fixed: Dict[str, Any]) -> StepContext:
+    """The step whose arrays are views of ``dev`` by ``layout`` (name -> (offset, count))."""
     def view(name):
         o, c = layout[name]
         return dev[o:o + c]
 
-    ng = cache.num_groups
+    S, ps = fixed["num_seqs"], cache.page_size
     groups = [GroupStep(page_size=ps, window=cache.groups[g].window,
                         block_tables=view(f"tables{g}").reshape(S, widths[g]),
-                        slots=view(f"slots{g}")) for g in range(ng)]
+                        slots=view(f"slots{g}")) for g in range(cache.num_groups)]
     plans = {key: StepPlan({name: view(plan_name(k, name)) for name in plan.arrays}, plan.values)
              for k, (key, plan) in enumerate(host_plans)}
     return StepContext(
-        num_tokens=T, num_seqs=S, ids=view("ids"), positions=view("positions"),
-        seq_of_token=view("seq_of_token"), cu_seqlens=view("cu"), start_pos=view("start_pos"),
-        ctx_lens=view("ctx_lens"), logit_rows=view("logit_rows"), num_logit_rows=R,
-        state_slots=view("state_slots"), groups=groups, max_context=max_context,
-        max_new=max_new, all_decode=num_single == S, num_single=num_single, plans=plans,
-        lengths=lengths, host_start_pos=start_pos.tolist(), host_new=new.tolist(),
-        host_state_slots=host_view("state_slots").tolist(), host_order=order)
+        ids=view("ids"), positions=view("positions"), seq_of_token=view("seq_of_token"),
+        cu_seqlens=view("cu"), start_pos=view("start_pos"), ctx_lens=view("ctx_lens"),
+        logit_rows=view("logit_rows"), state_slots=view("state_slots"), groups=groups,
+        plans=plans, buffer=dev,
+        over=lambda other: _context_over(other, layout, cache, widths, host_plans, fixed),
+        **fixed)
 
 
 def build_step_in_python(entries: Sequence[StepEntry], cache, device: torch.device,
@@ -334,20 +348,8 @@ def build_step_in_python(entries: Sequence[StepEntry], cache, device: torch.devi
     if device.type == "cuda":
         host = host.pin_memory()
     dev = host.to(device, non_blocking=True)
-
-    def view(name):
-        return meta.view(dev, name)
-
-    groups = [GroupStep(page_size=ps, window=cache.groups[g].window,
-                        block_tables=view(f"tables{g}").reshape(S, widths[g]),
-                        slots=view(f"slots{g}")) for g in range(ng)]
-    plans = {key: StepPlan({name: view(plan_name(k, name)) for name in plan.arrays}, plan.values)
-             for k, (key, plan) in enumerate(host_plans)}
-    return StepContext(
-        num_tokens=T, num_seqs=S, ids=view("ids"), positions=view("positions"),
-        seq_of_token=view("seq_of_token"), cu_seqlens=view("cu"), start_pos=view("start_pos"),
-        ctx_lens=view("ctx_lens"), logit_rows=view("logit_rows"), num_logit_rows=len(logit_rows),
-        state_slots=view("state_slots"), groups=groups, max_context=max(ctx_lens),
-        max_new=max(new), all_decode=num_single == S, num_single=num_single, plans=plans,
-        lengths=lengths, host_start_pos=start_pos, host_new=new, host_state_slots=state_slots,
-        host_order=order)
+    fixed = dict(num_tokens=T, num_seqs=S, num_logit_rows=len(logit_rows),
+                 max_context=max(ctx_lens), max_new=max(new), all_decode=num_single == S,
+                 num_single=num_single, lengths=lengths, host_start_pos=start_pos, host_new=new,
+                 host_state_slots=state_slots, host_order=order)
+    return _context_over(dev, dict(meta.offsets), cache, widths, host_plans, fixed)

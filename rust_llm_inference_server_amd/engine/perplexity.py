@@ -49,7 +49,8 @@ def perplexity(runner: ModelRunner, tokens: Sequence[int], bos: int, ctx: int,
         runner.reserve(seq_id, ctx)
         try:
             # Rows first .. ctx-2 predict tokens first+1 .. ctx-1; the last row has no target.
-            logits = runner.step([StepEntry(seq_id, chunk, list(range(first, ctx - 1)))])
+            logits = runner.step([StepEntry(seq_id, chunk, list(range(first, ctx - 1)))],
+                                 keep=False)          # scored before the next window runs
         finally:
             runner.free(seq_id)       # also when the step raises: the next call starts clean
         targets = torch.tensor(chunk[first + 1:], device=logits.device).reshape(-1, 1)

@@ -98,6 +98,10 @@ class ModelRunner:
         self.model = model
         self.use_graphs = use_graphs and model.device.type == "cuda" and model.graph_safe
         self._graphs: Dict[int, object] = {}
+        # other steps than pure decode steps are captured when their shape comes back
+        # (engine/graph.py::RepeatedSteps)
+        self.capture_repeated_steps = True
+        self._repeated = None
         self.device = model.device
         self.page_size = page_size
         self.max_num_seqs = max_num_seqs
@@ -175,7 +179,16 @@ class ModelRunner:
             self.pools.zero_states([slot for start, slot in zip(step.host_start_pos,
                                                                 step.host_state_slots)
                                     if start == 0])
-        logits = self.model.forward(step, self.pools)
+        logits = None
+        if self.use_graphs and self.capture_repeated_steps:
+            if self._repeated is None:
+                from .graph import RepeatedSteps
+                self._repeated = RepeatedSteps(self)
+            logits = self._repeated.run(step)
+            if logits is not None and keep:
+                logits = logits.clone()
+        if logits is None:
+            logits = self.model.forward(step, self.pools)
         for i, start in zip(step.host_order, step.host_start_pos):
             self.cache.advance(entries[i].seq_id, start + len(entries[i].tokens))
         return logits

@@ -4,7 +4,9 @@ There is no fallback: without a GPU, or without the library, every op raises.  T
 is built on first use when it is absent (``csrc/build.py``)."""
 from __future__ import annotations
 
+import contextlib
 import ctypes
+import threading
 from ctypes import c_char_p, c_float, c_int, c_longlong, c_void_p
 from typing import Optional
 
@@ -87,16 +89,20 @@ def load() -> ctypes.CDLL:
     return lib
 
 
+_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 # ---------------------------------------------------------------- the library's products
-# Workspace that hipBLASLt may use for a product, per device (what the tensor library grants it
-# on this family of chips).  Allocated when the kernels are loaded and at the first product on
-# any other device, never while a stream is capturing.  One per device, not per stream: library
-# products whose algorithm uses the workspace must not overlap in time on one device (an engine
-# runs its steps on one stream; the algorithms that the heuristics have picked for the shapes
-# met so far ask for none).
+# Workspace that hipBLASLt may use for a product (what the tensor library grants it on this
+# family of chips): one per device and stream, since products on two streams may run at the
+# same time (two runners on two threads, each on a stream of its own).  Allocated at the first
+# product on a stream, never while a stream is capturing: a capture runs on a stream of its own
+# for a graph that its owner replays on the owner's stream, so whoever captures names that
+# stream (``workspace_owner``), and the graph's products take its workspace.
 LT_WORKSPACE_BYTES = 76 << 20
 _LT_OPEN: Optional[bool] = None
-_LT_WORKSPACES: dict = {}
+_LT_WORKSPACES: dict = {}          # (device index, stream handle) -> uint8 tensor
+_LT_OWNER = threading.local()
 
 
 def _hipblaslt_path() -> str:
@@ -106,23 +112,42 @@ def _hipblaslt_path() -> str:
     return own if os.path.exists(own) else "libhipblaslt.so"
 
 
+@contextlib.contextmanager
+def workspace_owner(stream: "torch.cuda.Stream"):
+    """Inside the block, this thread's library products take the workspace of ``stream``
+    whichever stream is current (the warm-up and the capture of a graph that will be replayed
+    on ``stream``).  The workspace is made on entry, before anything captures."""
+    old = getattr(_LT_OWNER, "stream", None)
+    _LT_OWNER.stream = int(stream.cuda_stream)
+    try:
+        library_workspace(stream.device)
+        yield
+    finally:
+        _LT_OWNER.stream = old
+
+
 def library_workspace(device: torch.device) -> Optional[torch.Tensor]:
-    """The device's workspace for ``rlis_lt_gemm_bf16``, or None when the library's products
-    cannot be called directly (its entry points were not found, or the workspace would have
-    to be allocated under a capturing stream): the caller then goes through ``torch.matmul``,
-    which reaches the same library."""
+    """The workspace of the device's current stream (or of the stream that ``workspace_owner``
+    names) for ``rlis_lt_gemm_bf16``, or None when the library's products cannot be called
+    directly (its entry points were not found, or the workspace would have to be allocated
+    under a capturing stream): the caller then goes through ``torch.matmul``, which reaches the
+    same library."""
     global _LT_OPEN
     if _LT_OPEN is None:
         _LT_OPEN = load().rlis_lt_open(_hipblaslt_path().encode()) == 0
     if not _LT_OPEN:
         return None
     index = device.index if device.index is not None else torch.cuda.current_device()
-    ws = _LT_WORKSPACES.get(index)
+    owner = getattr(_LT_OWNER, "stream", None)
+    if owner is None:
+        owner = (_RAW_STREAM(index) if _RAW_STREAM is not None
+                 else torch.cuda.current_stream(index).cuda_stream)
+    ws = _LT_WORKSPACES.get((index, owner))
     if ws is None:
         if torch.cuda.is_current_stream_capturing():
             return None
         ws = torch.empty(LT_WORKSPACE_BYTES, dtype=torch.uint8, device=torch.device("cuda", index))
-        _LT_WORKSPACES[index] = ws
+        _LT_WORKSPACES[(index, owner)] = ws
     return ws
 
 
@@ -162,9 +187,6 @@ def call(name: str, *args) -> None:
     rc = getattr(lib, name)(*args)
     if rc != 0:
         raise KernelError(lib.rlis_last_error().decode("utf-8", "replace"))
-
-
-_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def stream_ptr() -> int:

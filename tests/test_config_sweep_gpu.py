@@ -128,3 +128,43 @@ def test_whole_llama_1b_shape(tmp_path):
             print(f"1b {dtype} {build.__name__}: worst |diff| {worst:.3e}, largest |logit| {spread:.2f}")
             del runner
             torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("tokens", [2048, 512, 100])
+def test_captured_prompt_steps_at_the_1b_layer_sizes(tokens, monkeypatch):
+    """Whole prompts of one length, one after the other, at the layer sizes of the 1B shape (two
+    layers, a small vocabulary): from the second on (here; later by default) the step is a
+    captured HIP graph.  At these
+    sizes the products are the library's (at 512 and 100 rows the down projection in slices of
+    k, with a norm that adds partial sums) and the attention takes tiles of 64 or 128 queries
+    with key runs; every replay, with other tokens on other pages and an eager step of another
+    shape in between, must give what the runner without captured steps gives, bit for bit."""
+    from rust_llm_inference_server_amd.config import preset_dict
+    from rust_llm_inference_server_amd.engine import ModelRunner, StepEntry, random_model
+    from rust_llm_inference_server_amd.engine.graph import RepeatedSteps
+    monkeypatch.setattr(RepeatedSteps, "CAPTURE_AT", 2)
+    cfg = preset_dict("llama-3.2-1b")
+    cfg.update(num_hidden_layers=2, vocab_size=1000, max_position_embeddings=4096)
+    model = random_model(cfg, seed=3, dtype="bfloat16", max_positions=4096)
+    g = torch.Generator().manual_seed(tokens)
+    runners = []
+    for captures in (False, True):
+        r = ModelRunner(model, num_pages=3 * (tokens // 16 + 2) + 2, page_size=16, max_num_seqs=4)
+        r.capture_repeated_steps = captures
+        runners.append(r)
+    for i in range(5):
+        prompt = torch.randint(0, 1000, (tokens,), generator=g).tolist()
+        other = torch.randint(0, 1000, (7 + i,), generator=g).tolist()
+        got = []
+        for r in runners:
+            r.reserve(10 + i, len(other))                       # an eager step of another shape
+            r.step([StepEntry(10 + i, other, [0])])
+            r.free(10 + i)
+            r.reserve(i, tokens)
+            got.append(r.step([StepEntry(i, prompt, [0, tokens // 2, tokens - 1])]))
+            torch.cuda.synchronize()
+            if i % 2:
+                r.free(i)                                        # the next prompt takes these pages
+        assert torch.equal(got[0], got[1]), f"prompt {i}"
+        assert torch.isfinite(got[0]).all() and got[0].abs().max() > 0
+    assert runners[1]._repeated.replays == 4 and runners[0]._repeated is None

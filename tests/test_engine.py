@@ -464,11 +464,11 @@ def test_perplexity_gives_its_pages_back_when_a_step_fails(backend, tiny_folders
     runner = ModelRunner(load(folder, backend, max_positions=128), num_pages=4, page_size=8, max_num_seqs=2)
     real, calls = runner.step, []
 
-    def failing(entries):
+    def failing(entries, **kw):
         calls.append(1)
         if len(calls) == 2:
             raise RuntimeError("the device said no")
-        return real(entries)
+        return real(entries, **kw)
 
     runner.step = failing
     with pytest.raises(RuntimeError, match="the device said no"):

@@ -439,7 +439,7 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
         assert runner.cache.num_free_slots() == 4
 
 
-def test_toy_mixer_with_state_through_captured_decode_steps(tmp_path):
+def test_toy_mixer_with_state_through_captured_decode_steps(tmp_path, monkeypatch):
     """The same toy mixer doing its single-token steps on the device alone, so that the model's
     decode steps are captured into HIP graphs: every way of cutting, then requests that start
     with single tokens on state slots that earlier requests left full.  The captured path must
@@ -498,6 +498,27 @@ def test_toy_mixer_with_state_through_captured_decode_steps(tmp_path):
             pos = t - (4 if i == 3 else 0)
             assert (logits[row] - ref[keys[i]][pos]).abs().max().item() < 2e-4, (keys[i], pos)
     assert {1 << 2} <= set(runner._graphs)
+    for i in range(4):
+        runner.free(100 + i)
+    # Prompt steps whose shape comes back are captured too.  Off the decode path this mixer
+    # works through the state slots in a host loop, so a captured step holds its slot for
+    # good: the slot is part of a step's shape, and a request on another slot (a bystander
+    # holds the first one meanwhile) is another shape with a capture of its own.  The slot
+    # of a request that starts is cleared outside the captured step.
+    from rust_llm_inference_server_amd.engine.graph import RepeatedSteps
+    monkeypatch.setattr(RepeatedSteps, "CAPTURE_AT", 2)
+    for r in range(8):
+        if r == 4:
+            runner.reserve(300, 3)
+            runner.step([StepEntry(300, reqs["r0"][:3], [])])
+        k = ("r2", "r4")[r % 2]
+        runner.reserve(200 + r, 20)
+        first = runner.step([StepEntry(200 + r, reqs[k][:9], [8])]).float().cpu()
+        second = runner.step([StepEntry(200 + r, reqs[k][9:20], [0, 10])]).float().cpu()
+        runner.free(200 + r)
+        for got_row, pos in ((first[0], 8), (second[0], 9), (second[1], 19)):
+            assert (got_row - ref[k][pos]).abs().max().item() < 2e-4, (r, k, pos)
+    assert len(runner._repeated.graphs) == 4 and runner._repeated.replays == 12
 
 
 # ------------------------- a toy mixer that caches one vector per position

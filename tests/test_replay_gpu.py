@@ -114,6 +114,67 @@ def test_captured_decode_steps_match_eager_ones(case, dtype):
             assert torch.equal(out_g[k], out_e[k]), f"step {k}"
 
 
+def rounds_of_one_schedule(vocab, rounds, page):
+    """The same schedule of steps ``rounds`` times over (a portion of a prompt alone; two
+    portions side by side; a single token beside a portion), each round with tokens of its own
+    and, since a bystander of growing length holds pages meanwhile, on pages of its own."""
+    g = torch.Generator().manual_seed(11)
+    steps = []
+    for r in range(rounds):
+        a, b, c = (torch.randint(0, vocab, (n,), generator=g).tolist() for n in (42, 23, 9))
+        z = torch.randint(0, vocab, (1 + r * page,), generator=g).tolist()
+        n = len(steps)
+        steps += [
+            {"step": n, "entries": [{"id": f"z{r}", "tokens": z, "want": []}], "end": []},
+            {"step": n + 1, "entries": [{"id": f"a{r}", "tokens": a[:17], "want": [16]}], "end": []},
+            {"step": n + 2, "entries": [{"id": f"a{r}", "tokens": a[17:41], "want": [0, 23]},
+                                        {"id": f"b{r}", "tokens": b, "want": [22]}], "end": []},
+            {"step": n + 3, "entries": [{"id": f"a{r}", "tokens": a[41:], "want": [0]},
+                                        {"id": f"c{r}", "tokens": c, "want": [3, 8]}],
+             "end": [f"a{r}", f"b{r}", f"c{r}", f"z{r}"]},
+        ]
+    return steps
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_whose_shape_comes_back_are_captured(case, dtype, monkeypatch):
+    """A step that is no pure decode step is captured into a HIP graph when its shape (every
+    sequence's cached and new positions, the number of wanted rows) has come back often enough,
+    here the second time it is seen, and replayed from then on with the new step's metadata.  Five rounds of one schedule, each with
+    other tokens on other pages, with eager steps and host synchronisation between the replays:
+    every step must give what a runner without captured steps gives, bit for bit."""
+    from rust_llm_inference_server_amd.engine.graph import RepeatedSteps
+    assert RepeatedSteps.CAPTURE_AT > 2
+    monkeypatch.setattr(RepeatedSteps, "CAPTURE_AT", 2)
+    name, cfg, per_dtype = case
+    folder, _, _ = per_dtype[dtype]
+    page = 8 if name == "b" else 16
+    rounds = 5
+    steps = rounds_of_one_schedule(cfg["vocab_size"], rounds, page)
+    max_tokens = 4 * 64 + rounds * page + 64
+    eager = make_runner(folder, dtype, max_tokens, page)
+    eager.capture_repeated_steps = False
+    graphed = make_runner(folder, dtype, max_tokens, page)
+    out_e = traces.replay_in_process(eager, steps)
+    out_g = traces.replay_in_process(graphed, steps)
+    assert eager._repeated is None
+    # three shapes come back (the bystander's never does): captured in the second round,
+    # replayed in that one and in the three after it
+    assert len(graphed._repeated.graphs) == 3 and graphed._repeated.replays == 3 * (rounds - 1)
+    assert sorted(out_e) == sorted(out_g) and len(out_g) == 3 * rounds
+    for k in out_e:
+        assert torch.equal(out_g[k], out_e[k]), f"step {k}"
+    assert graphed.cache.num_free_pages(0) == graphed.cache.num_pages(0)
+    assert int(graphed.pools.counters.abs().sum()) == 0
+    # a fifth shape pushes the least recently used one out
+    graphed._repeated.limit = 3
+    extra = [{"step": 100 + i, "entries": [{"id": f"x{i}", "tokens": [1, 2, 3], "want": [2]}],
+              "end": [f"x{i}"]} for i in range(3)]
+    out_x = traces.replay_in_process(graphed, extra)
+    assert len(graphed._repeated.graphs) == 3
+    assert torch.equal(out_x[100], out_x[101]) and torch.equal(out_x[100], out_x[102])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_chained_steps_sample_what_fed_steps_sample(case, dtype):
     """``step_chained`` runs the same requests once more on the tokens that the sampling kernel
@@ -340,7 +401,9 @@ def test_two_runners_decode_on_two_streams_at_once(tmp_path):
     several partitions at the same time.  The decode attention merges a sequence's partitions
     inside the kernel and counts the workgroups' arrivals in memory that each runner owns, so
     neither counts into the other's: both give, step for step and bit for bit, what they give
-    one after the other, and both leave their counters at zero."""
+    one after the other, and both leave their counters at zero.  Their prompts run at the same
+    time as well, through the library's products: each stream has a workspace of its own there,
+    and the calls on the device's one handle take turns."""
     import threading
     from rust_llm_inference_server_amd.engine import ModelRunner, StepEntry, load_model
     folder = make_model_folder(tmp_path / "long", LONG, seed=6, dtype=torch.bfloat16)
@@ -354,12 +417,14 @@ def test_two_runners_decode_on_two_streams_at_once(tmp_path):
             runner = ModelRunner(model, num_pages=3 * 200, page_size=16, max_num_seqs=4,
                                  use_graphs=False)
             keys = sorted(reqs[which])
+            if barrier is not None:
+                barrier.wait(timeout=60)         # the prompts run at the same time too
             for i, k in enumerate(keys):
                 runner.reserve(i, len(reqs[which][k]))
                 runner.step([StepEntry(i, reqs[which][k][:-steps], [])])
             stream.synchronize()
             if barrier is not None:
-                barrier.wait()
+                barrier.wait(timeout=60)
             rows = []
             for t in range(steps):
                 logits = runner.step([StepEntry(i, [reqs[which][k][len(reqs[which][k]) - steps + t]], [0])
