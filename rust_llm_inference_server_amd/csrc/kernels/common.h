@@ -110,6 +110,24 @@ void rlis_set_error(const char* fmt, ...);
     }                                      \
   } while (0)
 
+// A kernel's limit of dynamic LDS is raised once on every device it runs on (function
+// attributes are the device's): `LdsGrant` remembers where, `grant_lds` raises it for the
+// current device when it has not been yet.
+struct LdsGrant {
+  static constexpr int kDevices = 64;
+  bool done[kDevices] = {};
+};
+inline hipError_t grant_lds(LdsGrant& grant, const void* kernel, int bytes) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const bool known = dev >= 0 && dev < LdsGrant::kDevices;
+  if (known && grant.done[dev]) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess && known) grant.done[dev] = true;
+  return e;
+}
+
 #define RLIS_LAUNCH_CHECK(name)                                              \
   do {                                                                       \
     hipError_t e_ = hipGetLastError();                                       \

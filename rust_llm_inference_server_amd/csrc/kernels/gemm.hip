@@ -586,14 +586,12 @@ RLIS_API int rlis_gemm_bf16_splitk(const void* X, const void* W, void* Y, int T,
   const size_t smem = (size_t)nt * 16 * (ks + kSplitPad) * sizeof(bf16_t);
 #define GO(KS, NT, WALK)                                                                    \
   {                                                                                         \
-    static bool raised = false;                                                             \
-    if (!raised && smem > 48 * 1024) {                                                      \
-      hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_splitk_kernel<KS, NT, WALK>, \
-                                         hipFuncAttributeMaxDynamicSharedMemorySize,        \
-                                         (int)smem);                                        \
+    static LdsGrant raised;                                                                 \
+    if (smem > 48 * 1024) {                                                                 \
+      hipError_t e = grant_lds(raised, (const void*)gemm_bf16_splitk_kernel<KS, NT, WALK>,  \
+                               (int)smem);                                                  \
       RLIS_REQUIRE(e == hipSuccess, "gemm_bf16_splitk: cannot raise the LDS limit: %s",     \
                    hipGetErrorString(e));                                                   \
-      raised = true;                                                                        \
     }                                                                                       \
     gemm_bf16_splitk_kernel<KS, NT, WALK><<<grid, 256, smem, stream>>>(                     \
         (const bf16_t*)X, (const bf16_t*)W, (float*)Y, T, N, K, ldx, ldw, part_stride,      \
@@ -1061,15 +1059,13 @@ static int launch_stream_tiles(const void* X, const void* W, void* Y, StreamShap
                                const StreamNorm& nm, int nwaves, int num_cus,
                                hipStream_t stream) {
   constexpr int kTileBytes = IPW * (MODE == kStreamNorm ? kStreamTileBytes : TR * kStreamItem * 2);
-  static bool lds_raised = false;
-  if (!lds_raised) {
-    hipError_t e = hipFuncSetAttribute(
-        (const void*)gemm_bf16_stream_kernel<TC, GATED, TR, MODE, IPW, PACK>,
-        hipFuncAttributeMaxDynamicSharedMemorySize,
+  static LdsGrant lds_raised;
+  {
+    hipError_t e = grant_lds(
+        lds_raised, (const void*)gemm_bf16_stream_kernel<TC, GATED, TR, MODE, IPW, PACK>,
         (IPW == 1 ? kStreamMaxWaves : 2 * kStreamMaxWaves / IPW) * (kTileBytes + 2048));
     RLIS_REQUIRE(e == hipSuccess, "gemm_bf16_stream: cannot raise the LDS limit: %s",
                  hipGetErrorString(e));
-    lds_raised = true;
   }
   const size_t smem = (size_t)nwaves * (kTileBytes + 2048);
   const int per_cu = max(1, (int)((160 * 1024) / smem));
@@ -1086,14 +1082,16 @@ static int launch_stream_tiles(const void* X, const void* W, void* Y, StreamShap
 }
 
 int rlis_stream_compute_units() {
-  static int num_cus = 0;
-  if (num_cus == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-      num_cus = prop.multiProcessorCount;
-  }
-  return num_cus;
+  constexpr int kDevices = 64;
+  static int num_cus[kDevices];                    // of every device asked about so far
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  const bool known = dev >= 0 && dev < kDevices;
+  if (known && num_cus[dev] > 0) return num_cus[dev];
+  int n = 0;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  if (known) num_cus[dev] = n;
+  return n;
 }
 
 int rlis_stream_balanced_rows(int N, int slices, bool gated, int num_cus) {

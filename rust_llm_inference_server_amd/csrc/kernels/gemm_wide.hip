@@ -254,14 +254,13 @@ int launch_tiles(const void* X, const void* W, void* Y, StreamShape sh, const St
                  int nwaves, int num_cus, hipStream_t stream) {
   constexpr size_t kPerWave = TR * kStreamItem * 2 + 2 * TG * 256 * sizeof(float);
   constexpr size_t kScales = TG * 16 * sizeof(float);
-  static bool lds_raised = false;
-  if (!lds_raised) {
-    hipError_t e = hipFuncSetAttribute(
-        (const void*)gemm_bf16_stream_wide_kernel<TC, GATED, TR, MODE, TG, AHEAD>,
-        hipFuncAttributeMaxDynamicSharedMemorySize, (int)(wide_max_waves(TG) * kPerWave + kScales));
+  static LdsGrant lds_raised;
+  {
+    hipError_t e = grant_lds(
+        lds_raised, (const void*)gemm_bf16_stream_wide_kernel<TC, GATED, TR, MODE, TG, AHEAD>,
+        (int)(wide_max_waves(TG) * kPerWave + kScales));
     RLIS_REQUIRE(e == hipSuccess, "gemm_bf16_stream (17 to 32 rows): cannot raise the LDS limit: %s",
                  hipGetErrorString(e));
-    lds_raised = true;
   }
   const size_t smem = nwaves * kPerWave + kScales;
   const int per_cu = max(1, (int)((160 * 1024) / smem));

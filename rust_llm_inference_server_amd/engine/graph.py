@@ -308,7 +308,7 @@ class RepeatedSteps:
     on an otherwise idle engine; a step that mixes decoding requests with a portion hardly
     ever meets its shape again and stays eager.  What a replay saves is the host's time for
     the launches where that exceeds the kernels' time (1B shape, 16 layers: a step of 128
-    tokens 2.6 -> 1.7 ms, of 512 tokens 2.6 -> 2.4, of 2,048 tokens 5.50 -> 5.44), and a
+    tokens 2.6 -> 1.7 ms, of 512 tokens 2.6 -> 2.4, of 2,048 tokens 5.6 -> 5.4), and a
     capture costs 30 to 60 ms, which is why a shape is not captured the first time it comes
     back.  A capture runs nothing, so the step it captures is run once, by its first replay.
     The least recently used of more than ``limit`` captured shapes is dropped with its memory;
