@@ -114,6 +114,10 @@ class Model:
         self.graph_safe = all(getattr(p, "graph_safe", False)
                               for p in (self.embedding, *self.layers, self.final_norm, self.head))
         self._plan_cache()
+        if device.type == "cuda":
+            # the library's products are tried out over the weights of one shape in turn
+            from .. import ops
+            ops.note_weights(self._tensors())
         # The per-step planners of the mixers, one per distinct key.
         self.step_planners: List[Any] = []
         seen = set()
@@ -122,6 +126,22 @@ class Model:
             if planner is not None and planner.key() not in seen:
                 seen.add(planner.key())
                 self.step_planners.append(planner)
+
+    def _tensors(self):
+        """Every tensor that a part of the model holds as an attribute (parts within parts
+        included)."""
+        from ..parts.base import Part
+        todo, seen = [self.embedding, *self.layers, self.final_norm, self.head], set()
+        while todo:
+            part = todo.pop()
+            if id(part) in seen:
+                continue
+            seen.add(id(part))
+            for value in vars(part).values():
+                if isinstance(value, torch.Tensor):
+                    yield value
+                elif isinstance(value, Part):
+                    todo.append(value)
 
     # ---------------------------------------------------------------- cache plan
     def _plan_cache(self) -> None:

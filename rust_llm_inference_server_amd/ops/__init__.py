@@ -6,8 +6,10 @@ the CPU; without the compiled library or without a GPU the first call raises.
 """
 from __future__ import annotations
 
+import ctypes
 import functools
 import math
+import weakref
 from typing import Optional, Tuple
 
 import torch
@@ -259,6 +261,62 @@ def _one_item_per_wave(K: int) -> bool:
     return K <= lib.load().rlis_norm_linear_max_k()
 
 
+# The library's products of 33 to 1,024 rows are tried out before a shape's first product: the
+# heuristics' first candidates are timed on the spot and the fastest is kept for the shape
+# (``rlis_lt_tune``; their order is erratic at these sizes, see library_gemm.hip), over the
+# weights of up to sixteen layers in turn, so that no candidate finds its weights in a cache
+# (timed on four weights of 31 MB, which the memory-side cache holds, the pick for the 3B
+# shape's q/k/v at 640 rows was 7 % slower in a step than the heuristics' first).  A
+# shape is tried out once, before anything has used it, and keeps its algorithm from then on: a
+# step computes the same bits whenever it runs.  Row counts beyond 64 are tried out when they
+# are a multiple of 32 (what a token budget makes of most steps); the others take the
+# heuristics' first algorithm, as every shape does under a capturing stream.
+LIBRARY_TUNE = True
+LIBRARY_TUNE_MAX_ROWS = 1024
+LIBRARY_TUNE_CANDIDATES = 12
+LIBRARY_TUNE_MARGIN = 0.05       # the first candidate stays unless another is this much faster
+LIBRARY_TUNE_BYTES = 512 << 20   # weights that the timed products of a candidate walk over
+_tried_out: set = set()
+_same_shape: dict = {}           # (device index, N, K, row stride) -> {address: weak reference}
+tune_log: list = []              # (T, N, K, slices, candidate taken, us of the first, us of it)
+
+
+def note_weights(tensors) -> None:
+    """Tells the tuner which weights a model holds: products are tried out over the weights of
+    one shape in turn (two-dimensional bfloat16 tensors; anything else is skipped)."""
+    for t in tensors:
+        if (isinstance(t, torch.Tensor) and t.dim() == 2 and t.dtype == torch.bfloat16
+                and t.is_cuda and t.stride(1) == 1):
+            key = (t.device.index, t.shape[0], t.shape[1], t.stride(0))
+            _same_shape.setdefault(key, {})[t.data_ptr()] = weakref.ref(t)
+
+
+def _try_out(x, w, y, out_f32, T, N, K, ldx, ldw, slices, ws, stream) -> None:
+    if not LIBRARY_TUNE or T > LIBRARY_TUNE_MAX_ROWS:
+        return
+    key = (x.device.index, T, N, K, ldx, ldw, bool(out_f32), slices)
+    if key in _tried_out:
+        return
+    _tried_out.add(key)
+    if (T > 64 and T % 32) or torch.cuda.is_current_stream_capturing():
+        return
+    # as many weights as make up LIBRARY_TUNE_BYTES (the memory-side cache is 256 MB), 4 to 16
+    most = max(4, min(16, -(-LIBRARY_TUNE_BYTES // (N * K * 2))))
+    held = [w]                                        # (strong references while they are used)
+    for ref in list(_same_shape.get((x.device.index, N, K, ldw), {}).values()):
+        t = ref()
+        if t is not None and t.data_ptr() != w.data_ptr() and len(held) < most:
+            held.append(t)
+    ptrs = (ctypes.c_void_p * len(held))(*[t.data_ptr() for t in held])
+    chosen = ctypes.c_int(-1)
+    us = (ctypes.c_float * 2)()
+    lib.call("rlis_lt_tune", x.data_ptr(), ptrs, len(held), y.data_ptr(), int(out_f32), T, N, K,
+             ldx, ldw, N, slices, T * N, ws.data_ptr(), ws.numel(), LIBRARY_TUNE_CANDIDATES,
+             2 if len(held) < 8 else 1, LIBRARY_TUNE_MARGIN, ctypes.byref(chosen), us, stream)
+    if chosen.value >= 0:
+        tune_log.append((T, N, K, slices, chosen.value, float(us[0]), float(us[1])))
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
            partials: bool = False) -> torch.Tensor:
     """``x @ w.T`` for ``x (T, K)`` and ``w (N, K)``, float32 accumulation.
@@ -300,11 +358,13 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         slices = library_slices(T, K) if partials and ws is not None else 1
         if slices > 1:
             y = torch.empty((slices, T, N), dtype=torch.float32, device=x.device)
+            _try_out(x, w, y, True, T, N, K, ldx, ldw, slices, ws, stream)
             lib.call("rlis_lt_gemm_bf16_slices", x.data_ptr(), w.data_ptr(), y.data_ptr(), T, N, K,
                      ldx, ldw, N, slices, T * N, ws.data_ptr(), ws.numel(), stream)
             return y
         if ws is not None and out_dtype in (torch.bfloat16, torch.float32):
             y = torch.empty((T, N), dtype=out_dtype, device=x.device)
+            _try_out(x, w, y, out_dtype == torch.float32, T, N, K, ldx, ldw, 1, ws, stream)
             lib.call("rlis_lt_gemm_bf16", x.data_ptr(), w.data_ptr(), y.data_ptr(),
                      int(out_dtype == torch.float32), T, N, K, ldx, ldw, N, ws.data_ptr(),
                      ws.numel(), stream)

@@ -82,6 +82,9 @@ def load() -> ctypes.CDLL:
     lib.rlis_attn_register_unit.argtypes = [I, P, P]
     lib.rlis_norm_linear_max_k.restype = c_int
     lib.rlis_norm_linear_max_k.argtypes = []
+    lib.rlis_lt_tune.restype = c_int
+    lib.rlis_lt_tune.argtypes = [P, P, I, P, I, I, I, I, L, L, L, I, L, P, ctypes.c_size_t, I, I, F,
+                                 P, P, P]
     lib.rlis_gemm_bf16_stream_max_rows.restype = c_int
     lib.rlis_gemm_bf16_stream_max_rows.argtypes = [I]
     _LIB = lib

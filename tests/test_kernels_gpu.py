@@ -380,6 +380,61 @@ def test_library_product_called_directly(ops, monkeypatch, out_dtype, T, N, K):
         ops.LIBRARY_GEMM_DIRECT = old
 
 
+def test_library_products_are_tried_out_before_their_first_use(ops, monkeypatch):
+    """A shape of the library's products (33 to 64 rows, or a multiple of 32 up to 1,024) is
+    tried out before its first product: the heuristics' first candidates are timed over the
+    weights of that shape in turn and the fastest is kept.  Once, and never under a capturing
+    stream: a shape keeps its algorithm, so a product gives the same bits every time; other row
+    counts, and everything with the switch off, take the heuristics' first choice untimed.
+    (Shapes that nothing else in the tests uses: a plan made earlier would not be tried out.)"""
+    monkeypatch.setattr(ops, "STREAM_WIDE_MAX_ROWS", 0)
+    N, K = 1192, 1096
+    ws = [rnd(N, K, dtype=torch.bfloat16, seed=20 + i, scale=0.05) for i in range(3)]
+    ops.note_weights(ws + [rnd(N, K, seed=9), rnd(8, dtype=torch.bfloat16, seed=9)])   # (skipped)
+    log = ops.tune_log
+
+    def product(T, out_dtype=torch.bfloat16, w=ws[0], **kw):
+        x = rnd(T, K, dtype=torch.bfloat16, seed=T)
+        got = ops.linear(x, w, out_dtype, **kw)
+        want = (x.double() @ w.double().t()).float()
+        scale = max(1.0, want.abs().max().item())
+        torch.testing.assert_close(got.float() if got.dim() == 2 else got.sum(0), want,
+                                   atol=8e-3 * scale * math.sqrt(K / 64), rtol=1e-2)
+        return got
+
+    before = len(log)
+    first = product(96)
+    assert len(log) == before + 1
+    T, n, k, slices, taken, us_first, us_taken = log[-1]
+    assert (T, n, k, slices) == (96, N, K, 1) and 0 <= taken < ops.LIBRARY_TUNE_CANDIDATES
+    assert 0 < us_taken <= us_first and (taken == 0 or us_taken < us_first * (1 - ops.LIBRARY_TUNE_MARGIN))
+    assert torch.equal(product(96), first) and len(log) == before + 1        # once
+    assert torch.equal(product(96, w=ws[1]), ops.linear(rnd(96, K, dtype=torch.bfloat16, seed=96), ws[1],
+                                                        torch.bfloat16)) and len(log) == before + 1
+    product(40)                                  # a decode batch of 33 to 64 requests
+    product(64, torch.float32)                   # ... another output type is another shape
+    assert len(log) == before + 3
+    product(100)                                 # beyond 64 rows: multiples of 32 only
+    product(1056)                                # and up to 1,024
+    assert len(log) == before + 3
+    monkeypatch.setattr(ops, "LIBRARY_TUNE", False)
+    product(128)
+    assert len(log) == before + 3
+    monkeypatch.setattr(ops, "LIBRARY_TUNE", True)
+    product(128)                                 # (has a plan by now: nothing is tried out)
+    assert len(log) == before + 3
+    # under a capturing stream nothing can be timed: the shape takes the heuristics' first
+    x = rnd(160, K, dtype=torch.bfloat16, seed=160)
+    from rust_llm_inference_server_amd.ops import lib
+    graph = torch.cuda.CUDAGraph()
+    with lib.workspace_owner(torch.cuda.current_stream()), torch.cuda.graph(graph):
+        captured = ops.linear(x, ws[2], torch.bfloat16)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert len(log) == before + 3
+    assert torch.equal(captured, ops.linear(x, ws[2], torch.bfloat16)) and len(log) == before + 3
+
+
 @pytest.mark.parametrize("T,N,K", [(100, 2048, 8192), (512, 3072, 8192), (300, 136, 14336), (1024, 264, 8192),
                                    (65, 8, 8192)])
 def test_library_product_in_slices_of_k(ops, T, N, K):
