@@ -21,6 +21,7 @@
 #include <dlfcn.h>
 #include <hipblaslt/hipblaslt.h>
 
+#include <algorithm>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -230,7 +231,7 @@ RLIS_API int rlis_lt_gemm_bf16_slices(const void* X, const void* W, float* Y, in
 // algorithms (at most 16, those whose workspace fits) each compute the product once untimed and
 // then `runs` times over every one of the `num_w` weights of that shape in turn (other layers'
 // weights, so that no candidate finds the weights in a cache that a step would not find them
-// in); the fastest becomes the shape's algorithm if it beats the heuristics' first by more than
+// in; 32 products at most); the fastest by the median of its products' times becomes the shape's algorithm if it beats the heuristics' first by more than
 // `margin` (a fraction), else the first does.  Y is written by every candidate.  Nothing
 // happens when the shape has a plan already (an algorithm in use is never changed) or the
 // stream is capturing (*chosen = -1).  *chosen: the index taken; us[0], us[1]: the times of
@@ -271,10 +272,20 @@ RLIS_API int rlis_lt_tune(const void* X, const void* const* Ws, int num_w, void*
   if (describe(handle, made, found, want, &count, out_f32, T, N, K, ldx, ldw, ldy, slices,
                y_stride, workspace_bytes))
     return 1;
-  hipEvent_t begin = nullptr, end = nullptr;
-  he = hipEventCreate(&begin);
-  if (he == hipSuccess) he = hipEventCreate(&end);
-  RLIS_REQUIRE(he == hipSuccess, "lt_tune: %s", hipGetErrorString(he));
+  // Every timed product stands between two events of its own, and a candidate's time is the
+  // median of its products': what passes between one product's events is the device's time for
+  // it, whereas a loop timed from end to end is bound by the host's launches where a product
+  // takes less than they do (and then says nothing about the candidates).
+  constexpr int kTimed = 32;
+  const int timed = runs * num_w < kTimed ? runs * num_w : kTimed;
+  hipEvent_t marks[2 * kTimed] = {};
+  for (int i = 0; i < 2 * timed; ++i) {
+    he = hipEventCreate(&marks[i]);
+    if (he != hipSuccess) {
+      for (int j = 0; j < i; ++j) (void)hipEventDestroy(marks[j]);
+      RLIS_REQUIRE(false, "lt_tune: %s", hipGetErrorString(he));
+    }
+  }
   const float one = 1.f, zero = 0.f;
   float best = 0.f, first = 0.f;
   int taken = 0;
@@ -286,27 +297,29 @@ RLIS_API int rlis_lt_tune(const void* X, const void* const* Ws, int num_w, void*
                        &found[c].algo, workspace, workspace_bytes, stream) == HIPBLAS_STATUS_SUCCESS;
     };
     bool ok = product(Ws[0]);
-    ok = ok && hipEventRecord(begin, stream) == hipSuccess;
-    for (int r = 0; ok && r < runs; ++r)
-      for (int i = 0; ok && i < num_w; ++i) ok = product(Ws[i]);
-    ok = ok && hipEventRecord(end, stream) == hipSuccess;
-    ok = ok && hipEventSynchronize(end) == hipSuccess;
-    float ms = 0.f;
-    ok = ok && hipEventElapsedTime(&ms, begin, end) == hipSuccess;
+    for (int i = 0; ok && i < timed; ++i) {
+      ok = hipEventRecord(marks[2 * i], stream) == hipSuccess && product(Ws[i % num_w]) &&
+           hipEventRecord(marks[2 * i + 1], stream) == hipSuccess;
+    }
+    ok = ok && hipEventSynchronize(marks[2 * timed - 1]) == hipSuccess;
+    float each[kTimed];
+    for (int i = 0; ok && i < timed; ++i)
+      ok = hipEventElapsedTime(&each[i], marks[2 * i], marks[2 * i + 1]) == hipSuccess;
     if (!ok) {
       (void)hipGetLastError();              // a candidate that cannot run is left out
+      (void)hipStreamSynchronize(stream);
       if (c == 0) break;                    // ... but without the first there is no yardstick
       continue;
     }
-    const float t = ms * 1e3f / (float)(runs * num_w);
+    std::sort(each, each + timed);
+    const float t = each[timed / 2] * 1e3f;
     if (c == 0) first = best = t;
     else if (t < best && t < first * (1.f - margin)) {
       best = t;
       taken = c;
     }
   }
-  (void)hipEventDestroy(begin);
-  (void)hipEventDestroy(end);
+  for (int i = 0; i < 2 * timed; ++i) (void)hipEventDestroy(marks[i]);
   RLIS_REQUIRE(first > 0.f, "lt_tune: the heuristics' first algorithm for T=%d N=%d K=%d did not run",
                T, N, K);
   made.algo = found[taken].algo;

@@ -17,7 +17,10 @@ Unused rows of a bucket are padding requests of context 1 that read and write a 
 beyond the manager's pages and a scratch state slot beyond its slots, so they touch nothing a
 live request owns.  Nothing in the graph depends on the host: what a mixer's planner sizes by
 the longest context is fixed per context bucket, and how a sequence's own work is cut follows
-from its own lengths on the device, so a replay computes bit for bit what the eager step does.
+from its own lengths on the device, so a replay computes bit for bit what the eager step does
+(to rounding where the library's products compute, bfloat16 at 33 to 64 rows: a captured step
+runs its bucket's rows, for which the library may take another algorithm than for the step's
+own count).
 Graphs hold no memset nodes (the kernels clear nothing) and are checked against the eager step
 in the tests, replay after replay with eager work in between."""
 from __future__ import annotations

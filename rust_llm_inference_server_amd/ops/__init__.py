@@ -274,7 +274,7 @@ def _one_item_per_wave(K: int) -> bool:
 LIBRARY_TUNE = True
 LIBRARY_TUNE_MAX_ROWS = 1024
 LIBRARY_TUNE_CANDIDATES = 12
-LIBRARY_TUNE_MARGIN = 0.05       # the first candidate stays unless another is this much faster
+LIBRARY_TUNE_MARGIN = 0.08       # the first candidate stays unless another is this much faster
 LIBRARY_TUNE_BYTES = 512 << 20   # weights that the timed products of a candidate walk over
 _tried_out: set = set()
 _same_shape: dict = {}           # (device index, N, K, row stride) -> {address: weak reference}

@@ -617,12 +617,16 @@ def test_linear_mixed_dtypes(ops):
 
 
 def test_linear_rows_do_not_depend_on_the_batch(ops):
-    """A row's product is the same bits whichever other rows share the call (same kernel)."""
-    for dtype in DTYPES:
-        x, w = rnd(40, 256, dtype=dtype, seed=1), rnd(300, 256, dtype=dtype, seed=2)
-        full = ops.linear(x, w, torch.float32)
-        part = ops.linear(x[5:23].contiguous(), w, torch.float32)
-        torch.testing.assert_close(part, full[5:23], atol=0, rtol=0)
+    """A row's product is the same bits whichever other rows share the call, within the row
+    counts that one of the engine's kernels takes (float32: any; bfloat16: up to 16 rows and 17
+    to 32 rows; beyond that the library computes, which promises no such thing)."""
+    for dtype, counts in ((torch.float32, (40, 16)), (torch.bfloat16, (30, 16))):
+        for rows in counts:
+            lo, hi = (5, 23) if rows > 16 else (3, 9)
+            x, w = rnd(rows, 256, dtype=dtype, seed=1), rnd(300, 256, dtype=dtype, seed=2)
+            full = ops.linear(x, w, torch.float32)
+            part = ops.linear(x[lo:hi].contiguous(), w, torch.float32)
+            torch.testing.assert_close(part, full[lo:hi], atol=0, rtol=0)
 
 
 # ---------------------------------------------------------- rotation + cache write

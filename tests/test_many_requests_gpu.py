@@ -135,16 +135,18 @@ def rows_trace(reqs, prompt_len, counts):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_logits_of_steps_with_17_33_and_64_rows(case, dtype):
     """64 requests with prompts of 1 to 12 tokens decode together, and the number of rows in
-    a step moves through 64, 17, 16, 33, 32, 65 (63 single tokens beside a two-token portion),
-    1, 64 ...: a request's consecutive tokens are computed by the kernels of each range in
+    a step moves through 16, 17, 32, 1, 24, ... 64, 33, 65 (63 single tokens beside a two-token
+    portion), 48, 64 ...: a request's consecutive tokens are computed by the kernels of each range in
     turn.  Every logit is the plain implementation's within the replay tests' gates; captured
-    steps give bit for bit what eager steps give, at the buckets of 32 and 64 too."""
+    steps give bit for bit what eager steps give while the engine's own kernels compute (all
+    of float32, and bfloat16 up to the first step that brings the library's products in), and
+    the same within the gate from there on."""
     from rust_llm_inference_server_amd.engine import ModelRunner
     name, cfg, per_dtype = case
     folder, w, c = per_dtype[dtype]
     g = torch.Generator().manual_seed(23)
     prompt_len = {f"r{i}": int(n) for i, n in enumerate(torch.randint(1, 13, (65,), generator=g))}
-    counts = [64, 17, 16, 33, 32, 65, 1, 64, 48, 17, 64, 66, 33, 16, 64]
+    counts = [16, 17, 32, 1, 24, 16, 32, 17, 64, 33, 65, 48, 64, 66, 33, 16, 64]
     reqs = {k: torch.randint(0, cfg["vocab_size"], (n + len(counts) + 2,), generator=g).tolist()
             for k, n in prompt_len.items()}
     reqs["r64"] = reqs["r64"][:10]
@@ -169,6 +171,20 @@ def test_logits_of_steps_with_17_33_and_64_rows(case, dtype):
             assert diff <= TOL[dtype], f"request {k} position {p}: |diff| {diff:.3e}"
             worst = max(worst, diff)
     assert sum(len(v) for v in got.values()) > 600
-    for k in outputs[False]:
-        assert torch.equal(outputs[True][k], outputs[False][k]), f"step {k} ({sizes[k]} rows)"
+    # A captured step runs its bucket's rows, the eager one the step's own count.  Where the
+    # engine's kernels compute, a row's bits do not depend on the count; the library's products
+    # (bfloat16 beyond the rows that the streaming kernels take: 32 for widths that are a
+    # multiple of 256, else 16) may take another algorithm for another count (each is tried out
+    # on its own) and then sum a row's k in another order.  From the first such step on the two
+    # runs' caches differ by rounding, and so does everything behind it.
+    own = 1 << 30 if dtype == "float32" else (32 if name == "w" else 16)
+    single = [all(len(e["tokens"]) == 1 for e in s["entries"]) for s in steps]
+    exact = True
+    for k in sorted(outputs[False]):
+        exact = exact and not (single[k] and own < sizes[k] <= 64)
+        if exact:
+            assert torch.equal(outputs[True][k], outputs[False][k]), f"step {k} ({sizes[k]} rows)"
+        else:
+            assert (outputs[True][k] - outputs[False][k]).abs().max().item() <= TOL[dtype], \
+                f"step {k} ({sizes[k]} rows)"
     print(f"{name} {dtype}: worst |diff| {worst:.3e} over {sum(len(v) for v in got.values())} rows")
