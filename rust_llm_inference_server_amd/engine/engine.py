@@ -102,6 +102,10 @@ class Engine:
             model = load_model(model, dtype, max_positions=cfg.max_seq_len)
         self.model = model
         budget = max(cfg.max_batched_tokens, cfg.max_num_seqs)
+        if model.device.type == "cuda":
+            # steps that fill the budget are the common ones: their products are tried out
+            from .. import ops
+            ops.LIBRARY_TUNE_ROWS.add(budget)
         if cfg.num_pages is not None:
             pools = [cfg.num_pages] * max(1, len(model.cache_groups))
         else:

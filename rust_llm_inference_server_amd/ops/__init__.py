@@ -269,12 +269,14 @@ def _one_item_per_wave(K: int) -> bool:
 # shape's q/k/v at 640 rows was 7 % slower in a step than the heuristics' first).  A
 # shape is tried out once, before anything has used it, and keeps its algorithm from then on: a
 # step computes the same bits whenever it runs.  Row counts beyond 64 are tried out when they
-# are a multiple of 32 (what a token budget makes of most steps); the others take the
-# heuristics' first algorithm, as every shape does under a capturing stream.
+# are a multiple of 32 (what a token budget makes of most steps) or named in
+# ``LIBRARY_TUNE_ROWS`` (an engine names its token budget); the others take the heuristics'
+# first algorithm, as every shape does under a capturing stream.
 LIBRARY_TUNE = True
 LIBRARY_TUNE_MAX_ROWS = 1024
 LIBRARY_TUNE_CANDIDATES = 12
 LIBRARY_TUNE_MARGIN = 0.08       # the first candidate stays unless another is this much faster
+LIBRARY_TUNE_ROWS: set = set()   # further row counts to try out (an engine's token budget)
 LIBRARY_TUNE_BYTES = 512 << 20   # weights that the timed products of a candidate walk over
 _tried_out: set = set()
 _same_shape: dict = {}           # (device index, N, K, row stride) -> {address: weak reference}
@@ -298,7 +300,7 @@ def _try_out(x, w, y, out_f32, T, N, K, ldx, ldw, slices, ws, stream) -> None:
     if key in _tried_out:
         return
     _tried_out.add(key)
-    if (T > 64 and T % 32) or torch.cuda.is_current_stream_capturing():
+    if (T > 64 and T % 32 and T not in LIBRARY_TUNE_ROWS) or torch.cuda.is_current_stream_capturing():
         return
     # as many weights as make up LIBRARY_TUNE_BYTES (the memory-side cache is 256 MB), 4 to 16
     most = max(4, min(16, -(-LIBRARY_TUNE_BYTES // (N * K * 2))))

@@ -417,6 +417,11 @@ def test_library_products_are_tried_out_before_their_first_use(ops, monkeypatch)
     product(100)                                 # beyond 64 rows: multiples of 32 only
     product(1056)                                # and up to 1,024
     assert len(log) == before + 3
+    monkeypatch.setattr(ops, "LIBRARY_TUNE_ROWS", {200})      # ... or named (an engine's budget)
+    product(200)
+    monkeypatch.setattr(ops, "LIBRARY_TUNE_ROWS", set())
+    assert len(log) == before + 4 and log[-1][0] == 200
+    before += 1
     monkeypatch.setattr(ops, "LIBRARY_TUNE", False)
     product(128)
     assert len(log) == before + 3
