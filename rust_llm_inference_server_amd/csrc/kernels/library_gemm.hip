@@ -21,6 +21,8 @@
 #include <dlfcn.h>
 #include <hipblaslt/hipblaslt.h>
 
+#include <string.h>
+
 #include <algorithm>
 #include <map>
 #include <mutex>
@@ -328,5 +330,54 @@ RLIS_API int rlis_lt_tune(const void* X, const void* const* Ws, int num_w, void*
   *chosen = taken;
   us[0] = first;
   us[1] = best;
+  return 0;
+}
+
+// Gives the shape of T rows the algorithm that the shape of T_like rows has (the same N, K and
+// kinds of operands; x rows ldx_like apart there): among the heuristics' first sixteen
+// candidates for T, the one that names the same kernel, if there is one; else the heuristics'
+// first.  For row counts next to one that has been tried out: the same kernel does as well
+// there, and nothing is timed.  Nothing happens when T has a plan already (*taken = -2);
+// *taken = -1: T_like has no plan or none of T's candidates is its algorithm (T then takes the
+// heuristics' first), else the candidate's index.
+RLIS_API int rlis_lt_adopt(int T, int T_like, int out_f32, int N, int K, long long ldx,
+                           long long ldx_like, long long ldw, long long ldy, int slices,
+                           long long y_stride, size_t workspace_bytes, int* taken) {
+  constexpr int kMost = 16;
+  RLIS_REQUIRE(T > 0 && T_like > 0 && N > 0 && K > 0 && ldx >= K && ldx_like >= K && ldw >= K &&
+                   ldy >= N && slices >= 1 && K % slices == 0 && taken,
+               "lt_adopt: bad arguments T=%d like %d N=%d K=%d", T, T_like, N, K);
+  *taken = -2;
+  const int full_k = K;
+  K /= slices;
+  int device = 0;
+  hipError_t he = hipGetDevice(&device);
+  RLIS_REQUIRE(he == hipSuccess, "lt_adopt: %s", hipGetErrorString(he));
+  std::lock_guard<std::mutex> lock(lt_mutex);
+  RLIS_REQUIRE(lt.lib != nullptr, "lt_adopt: the library has not been opened");
+  hipblasLtHandle_t handle = nullptr;
+  if (handle_of(device, &handle)) return 1;
+  const LtKey key(device, T, N, full_k, ldx, ldw, ldy, out_f32 ? 1 : 0, workspace_bytes, slices);
+  if (lt_plans.count(key)) return 0;
+  const LtKey like(device, T_like, N, full_k, ldx_like, ldw, ldy, out_f32 ? 1 : 0, workspace_bytes,
+                   slices);
+  auto model = lt_plans.find(like);
+  LtPlan made;
+  hipblasLtMatmulHeuristicResult_t found[kMost];
+  int count = 0;
+  if (describe(handle, made, found, kMost, &count, out_f32, T, N, K, ldx, ldw, ldy, slices,
+               y_stride, workspace_bytes))
+    return 1;
+  int pick = -1;
+  if (model != lt_plans.end()) {
+    for (int c = 0; c < count && pick < 0; ++c)
+      if (found[c].state == HIPBLAS_STATUS_SUCCESS && found[c].workspaceSize <= workspace_bytes &&
+          memcmp(found[c].algo.data, model->second.algo.data, sizeof(found[c].algo.data)) == 0)
+        pick = c;
+  }
+  made.algo = found[pick < 0 ? 0 : pick].algo;
+  made.workspace = found[pick < 0 ? 0 : pick].workspaceSize;
+  lt_plans.emplace(key, made);
+  *taken = pick;
   return 0;
 }

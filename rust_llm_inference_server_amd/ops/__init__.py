@@ -270,8 +270,9 @@ def _one_item_per_wave(K: int) -> bool:
 # shape is tried out once, before anything has used it, and keeps its algorithm from then on: a
 # step computes the same bits whenever it runs.  Row counts beyond 64 are tried out when they
 # are a multiple of 32 (what a token budget makes of most steps) or named in
-# ``LIBRARY_TUNE_ROWS`` (an engine names its token budget); the others take the heuristics'
-# first algorithm, as every shape does under a capturing stream.
+# ``LIBRARY_TUNE_ROWS`` (an engine names its token budget); the others take the algorithm of
+# the next multiple of 32 (``rlis_lt_adopt``: the candidate of their own that names the same
+# kernel, untimed), and under a capturing stream every new shape takes the heuristics' first.
 LIBRARY_TUNE = True
 LIBRARY_TUNE_MAX_ROWS = 1024
 LIBRARY_TUNE_CANDIDATES = 12
@@ -281,6 +282,7 @@ LIBRARY_TUNE_BYTES = 512 << 20   # weights that the timed products of a candidat
 _tried_out: set = set()
 _same_shape: dict = {}           # (device index, N, K, row stride) -> {address: weak reference}
 tune_log: list = []              # (T, N, K, slices, candidate taken, us of the first, us of it)
+adopt_log: list = []             # (T, rows it follows, N, K, slices, candidate taken or -1)
 
 
 def note_weights(tensors) -> None:
@@ -293,14 +295,32 @@ def note_weights(tensors) -> None:
             _same_shape.setdefault(key, {})[t.data_ptr()] = weakref.ref(t)
 
 
-def _try_out(x, w, y, out_f32, T, N, K, ldx, ldw, slices, ws, stream) -> None:
+def _try_out(x, w, y, out_f32, T, N, K, ldx, ldw, slices, ws, stream, partial=False) -> None:
     if not LIBRARY_TUNE or T > LIBRARY_TUNE_MAX_ROWS:
         return
     key = (x.device.index, T, N, K, ldx, ldw, bool(out_f32), slices)
     if key in _tried_out:
         return
     _tried_out.add(key)
-    if (T > 64 and T % 32 and T not in LIBRARY_TUNE_ROWS) or torch.cuda.is_current_stream_capturing():
+    if torch.cuda.is_current_stream_capturing():
+        return
+    if T > 64 and T % 32 and T not in LIBRARY_TUNE_ROWS:
+        # A row count between two that are tried out takes the algorithm of the next one up
+        # (tried out now, on rows of nothing, when it has not been yet): the same kernel does
+        # as well for a few rows fewer, and nothing more is timed.
+        like = -(-T // 32) * 32
+        like_slices = library_slices(like, K) if partial else 1
+        if like > LIBRARY_TUNE_MAX_ROWS or like_slices != slices:
+            return
+        if (x.device.index, like, N, K, K, ldw, bool(out_f32), slices) not in _tried_out:
+            rows = torch.empty((like, K), dtype=torch.bfloat16, device=x.device)
+            out = torch.empty((slices, like, N) if partial and slices > 1 else (like, N),
+                              dtype=y.dtype, device=x.device)
+            _try_out(rows, w, out, out_f32, like, N, K, K, ldw, slices, ws, stream, partial)
+        taken = ctypes.c_int(-1)
+        lib.call("rlis_lt_adopt", T, like, int(out_f32), N, K, ldx, K, ldw, N, slices, T * N,
+                 ws.numel(), ctypes.byref(taken))
+        adopt_log.append((T, like, N, K, slices, taken.value))
         return
     # as many weights as make up LIBRARY_TUNE_BYTES (the memory-side cache is 256 MB), 4 to 16
     most = max(4, min(16, -(-LIBRARY_TUNE_BYTES // (N * K * 2))))
@@ -360,7 +380,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         slices = library_slices(T, K) if partials and ws is not None else 1
         if slices > 1:
             y = torch.empty((slices, T, N), dtype=torch.float32, device=x.device)
-            _try_out(x, w, y, True, T, N, K, ldx, ldw, slices, ws, stream)
+            _try_out(x, w, y, True, T, N, K, ldx, ldw, slices, ws, stream, partial=True)
             lib.call("rlis_lt_gemm_bf16_slices", x.data_ptr(), w.data_ptr(), y.data_ptr(), T, N, K,
                      ldx, ldw, N, slices, T * N, ws.data_ptr(), ws.numel(), stream)
             return y

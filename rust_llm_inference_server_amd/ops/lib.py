@@ -85,6 +85,8 @@ def load() -> ctypes.CDLL:
     lib.rlis_lt_tune.restype = c_int
     lib.rlis_lt_tune.argtypes = [P, P, I, P, I, I, I, I, L, L, L, I, L, P, ctypes.c_size_t, I, I, F,
                                  P, P, P]
+    lib.rlis_lt_adopt.restype = c_int
+    lib.rlis_lt_adopt.argtypes = [I, I, I, I, I, L, L, L, L, I, L, ctypes.c_size_t, P]
     lib.rlis_gemm_bf16_stream_max_rows.restype = c_int
     lib.rlis_gemm_bf16_stream_max_rows.argtypes = [I]
     _LIB = lib

@@ -414,20 +414,29 @@ def test_library_products_are_tried_out_before_their_first_use(ops, monkeypatch)
     product(40)                                  # a decode batch of 33 to 64 requests
     product(64, torch.float32)                   # ... another output type is another shape
     assert len(log) == before + 3
-    product(100)                                 # beyond 64 rows: multiples of 32 only
-    product(1056)                                # and up to 1,024
-    assert len(log) == before + 3
-    monkeypatch.setattr(ops, "LIBRARY_TUNE_ROWS", {200})      # ... or named (an engine's budget)
+    # beyond 64 rows multiples of 32 are tried out; a count in between takes the algorithm of
+    # the next multiple (which is tried out for it, on rows of nothing), untimed
+    adopted = len(ops.adopt_log)
+    product(100)
+    assert len(log) == before + 4 and log[-1][0] == 128
+    assert len(ops.adopt_log) == adopted + 1 and ops.adopt_log[-1][:5] == (100, 128, N, K, 1)
+    assert -1 <= ops.adopt_log[-1][5] < 16
+    product(128)                                 # (has its plan from that)
+    product(101)
+    assert len(log) == before + 4 and len(ops.adopt_log) == adopted + 2
+    product(1056)                                # nothing beyond 1,024 rows
+    assert len(log) == before + 4 and len(ops.adopt_log) == adopted + 2
+    monkeypatch.setattr(ops, "LIBRARY_TUNE_ROWS", {200})      # a named count (an engine's budget)
     product(200)
     monkeypatch.setattr(ops, "LIBRARY_TUNE_ROWS", set())
-    assert len(log) == before + 4 and log[-1][0] == 200
-    before += 1
+    assert len(log) == before + 5 and log[-1][0] == 200 and len(ops.adopt_log) == adopted + 2
     monkeypatch.setattr(ops, "LIBRARY_TUNE", False)
-    product(128)
-    assert len(log) == before + 3
+    product(256)
+    assert len(log) == before + 5
     monkeypatch.setattr(ops, "LIBRARY_TUNE", True)
-    product(128)                                 # (has a plan by now: nothing is tried out)
-    assert len(log) == before + 3
+    product(256)                                 # (has a plan by now: nothing is tried out)
+    assert len(log) == before + 5 and len(ops.adopt_log) == adopted + 2
+    before += 2
     # under a capturing stream nothing can be timed: the shape takes the heuristics' first
     x = rnd(160, K, dtype=torch.bfloat16, seed=160)
     from rust_llm_inference_server_amd.ops import lib
