@@ -111,8 +111,11 @@ def _compute_units(device: torch.device) -> int:
 # partial sums) at the row counts of a budgeted step: the library's kernels for one such
 # product are few workgroups with long loops over k; as one batched call over slices of k they
 # are more and shorter (3B shape, down projection at 512 rows: 51 -> 36 us, against which the
-# consumer reads 25 MB more).  Rows and k from which on, rows up to which, and the slices' k
-# (the shorter up to LIBRARY_SLICES_FINE_ROWS rows).
+# consumer reads 25 MB more).  Rows and k from which on, rows up to which; eight slices up to
+# LIBRARY_SLICES_FINE_ROWS rows and four beyond (with the norm behind it and the library's
+# candidates tried out, k = 8,192 at 128 / 512 rows: one product 33 / 52 us, four slices 25 /
+# 40, eight 24.5 / 43; k = 14,336: one 57 / 97, four 40 / 72, seven 48 / 90, eight 38 / 76,
+# fourteen 46 / 99), fewer where k does not divide into slices whose rows stay 16-byte aligned.
 LIBRARY_SLICES_MIN_ROWS = 65
 LIBRARY_SLICES_MAX_ROWS = 1024
 LIBRARY_SLICES_MIN_K = 8192
@@ -124,8 +127,10 @@ def library_slices(T: int, K: int) -> int:
     partial sums (1: one product).  It follows from the row count and k alone."""
     if not (LIBRARY_SLICES_MIN_ROWS <= T <= LIBRARY_SLICES_MAX_ROWS) or K < LIBRARY_SLICES_MIN_K:
         return 1
-    step = 1024 if T <= LIBRARY_SLICES_FINE_ROWS else 2048
-    return K // step if K % step == 0 else 1
+    for slices in ((8, 4, 2) if T <= LIBRARY_SLICES_FINE_ROWS else (4, 2)):
+        if K % (slices * 8) == 0:
+            return slices
+    return 1
 
 
 def _dt(t: torch.Tensor) -> int:

@@ -461,7 +461,8 @@ def test_library_product_in_slices_of_k(ops, T, N, K):
     assert ops.library_slices(64, 8192) == 1 and ops.library_slices(2048, 8192) == 1
     assert ops.library_slices(512, 4096) == 1 and ops.library_slices(512, 8192 + 8) == 1
     assert ops.library_slices(512, 8192) == 4 and ops.library_slices(256, 8192) == 8
-    assert ops.library_slices(300, 14336) == 7 and ops.library_slices(100, 14336) == 14
+    assert ops.library_slices(300, 14336) == 4 and ops.library_slices(100, 14336) == 8
+    assert ops.library_slices(300, 8192 + 16) == 2 and ops.library_slices(100, 8192 + 32) == 4
     slices = ops.library_slices(T, K)
     assert slices > 1
     wide_x = rnd(T, K + 24, dtype=torch.bfloat16, seed=5)
