@@ -115,11 +115,14 @@ def _compute_units(device: torch.device) -> int:
 # LIBRARY_SLICES_FINE_ROWS rows and four beyond (with the norm behind it and the library's
 # candidates tried out, k = 8,192 at 128 / 512 rows: one product 33 / 52 us, four slices 25 /
 # 40, eight 24.5 / 43; k = 14,336: one 57 / 97, four 40 / 72, seven 48 / 90, eight 38 / 76,
-# fourteen 46 / 99), fewer where k does not divide into slices whose rows stay 16-byte aligned.
+# fourteen 46 / 99), two from LIBRARY_SLICES_MID_ROWS rows on (at 2,048 rows k = 8,192 of the
+# 1B shape 88.6 -> 84.2 us, k = 14,336 239 -> 227; four slices lose there), fewer where k does
+# not divide into slices whose rows stay 16-byte aligned.
 LIBRARY_SLICES_MIN_ROWS = 65
-LIBRARY_SLICES_MAX_ROWS = 1024
+LIBRARY_SLICES_MAX_ROWS = 2048
 LIBRARY_SLICES_MIN_K = 8192
 LIBRARY_SLICES_FINE_ROWS = 256
+LIBRARY_SLICES_MID_ROWS = 1024
 
 
 def library_slices(T: int, K: int) -> int:
@@ -127,7 +130,9 @@ def library_slices(T: int, K: int) -> int:
     partial sums (1: one product).  It follows from the row count and k alone."""
     if not (LIBRARY_SLICES_MIN_ROWS <= T <= LIBRARY_SLICES_MAX_ROWS) or K < LIBRARY_SLICES_MIN_K:
         return 1
-    for slices in ((8, 4, 2) if T <= LIBRARY_SLICES_FINE_ROWS else (4, 2)):
+    counts = ((8, 4, 2) if T <= LIBRARY_SLICES_FINE_ROWS else
+              (4, 2) if T <= LIBRARY_SLICES_MID_ROWS else (2,))
+    for slices in counts:
         if K % (slices * 8) == 0:
             return slices
     return 1
@@ -301,8 +306,8 @@ def note_weights(tensors) -> None:
 
 
 def _try_out(x, w, y, out_f32, T, N, K, ldx, ldw, slices, ws, stream, partial=False) -> None:
-    if not LIBRARY_TUNE or T > LIBRARY_TUNE_MAX_ROWS:
-        return
+    if not LIBRARY_TUNE or T > (LIBRARY_SLICES_MAX_ROWS if slices > 1 else LIBRARY_TUNE_MAX_ROWS):
+        return                  # (in slices of k the heuristics' first is not the best at 2,048 rows either)
     key = (x.device.index, T, N, K, ldx, ldw, bool(out_f32), slices)
     if key in _tried_out:
         return
@@ -315,7 +320,7 @@ def _try_out(x, w, y, out_f32, T, N, K, ldx, ldw, slices, ws, stream, partial=Fa
         # as well for a few rows fewer, and nothing more is timed.
         like = -(-T // 32) * 32
         like_slices = library_slices(like, K) if partial else 1
-        if like > LIBRARY_TUNE_MAX_ROWS or like_slices != slices:
+        if like > (LIBRARY_SLICES_MAX_ROWS if slices > 1 else LIBRARY_TUNE_MAX_ROWS) or like_slices != slices:
             return
         if (x.device.index, like, N, K, K, ldw, bool(out_f32), slices) not in _tried_out:
             rows = torch.empty((like, K), dtype=torch.bfloat16, device=x.device)

@@ -458,7 +458,8 @@ def test_library_product_in_slices_of_k(ops, T, N, K):
     the operands inside wider arrays, twice (the kept plan); and the rule for the slices."""
     from rust_llm_inference_server_amd.ops import lib
     assert lib.library_workspace(torch.device(DEV)) is not None, "hipBLASLt's entry points were not found"
-    assert ops.library_slices(64, 8192) == 1 and ops.library_slices(2048, 8192) == 1
+    assert ops.library_slices(64, 8192) == 1 and ops.library_slices(2048, 8192) == 2
+    assert ops.library_slices(1025, 14336) == 2 and ops.library_slices(2049, 8192) == 1
     assert ops.library_slices(512, 4096) == 1 and ops.library_slices(512, 8192 + 8) == 1
     assert ops.library_slices(512, 8192) == 4 and ops.library_slices(256, 8192) == 8
     assert ops.library_slices(300, 14336) == 4 and ops.library_slices(100, 14336) == 8
