@@ -9,14 +9,14 @@ typedef int (*PrefillUnit)(const void* q, long long q_stride, void* out, long lo
                            const int* tile_map, int num_tiles, int nh, int nkv, int d,
                            int page_shift, int window, float scale, int tile_queries, int splits,
                            int row0, float* part_ml, float* part_acc, const float* cos,
-                           const float* sin, int rot, hipStream_t stream);
+                           const float* sin, int rot, const float* slopes, hipStream_t stream);
 typedef int (*DecodeUnit)(const void* q, long long q_stride, void* out, long long out_stride,
                           float* part_ml, float* part_acc, const void* k_pages,
                           const void* v_pages, const int* block_tables, int max_pages,
                           const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift,
                           int window, float scale, int splits, int part_keys, int max_parts,
                           int merge_inside, int groups, int cap, const DecodeRope* rope,
-                          const DecodeMerge* merge, hipStream_t stream);
+                          const DecodeMerge* merge, const float* slopes, hipStream_t stream);
 
 // The units (attention_mfma.hip compiled for a padded head size of 32, 64, ... 256) are
 // libraries of their own, built and loaded when a model needs them and registered here.
@@ -70,6 +70,9 @@ int rlis_launch_attn_reduce_bf16(void* out, long long out_stride, const float* p
 // cos == null: q is rotated already.  Otherwise cos/sin are float32 (max positions, rot / 2)
 // with rot = d = 64, 128 or 256, and the kernel turns each query by its position (start_pos of
 // its sequence plus its index among the new tokens) as it loads it; q itself stays as it is.
+//
+// slopes != null: nh float32 values, one per query head; slopes[head] * (key position - query
+// position) is added to every score in float32 before the softmax.
 RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out,
                                     long long out_stride, const void* k_pages,
                                     const void* v_pages, const int* block_tables, int max_pages,
@@ -78,7 +81,7 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
                                     int page_size, int window, float scale, int tile_queries,
                                     int splits, int row0, float* part_ml,
                                     float* part_acc, const float* cos, const float* sin,
-                                    int rot, hipStream_t stream) {
+                                    int rot, const float* slopes, hipStream_t stream) {
   // unit_map lists tiles of tile_queries new tokens: 64 (0 means that too) or 128.
   if (tile_queries == 0) tile_queries = 64;
   RLIS_REQUIRE(tile_queries == 64 || tile_queries == 128,
@@ -108,7 +111,7 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
       "attn_prefill_mfma",
       unit(q, q_stride, out, out_stride, k_pages, v_pages, block_tables, max_pages, cu_seqlens,
            start_pos, unit_map, num_tiles, nh, nkv, d, page_shift, window, scale, tile_queries,
-           splits, row0, part_ml, part_acc, cos, sin, rot, stream),
+           splits, row0, part_ml, part_acc, cos, sin, rot, slopes, stream),
       d);
 }
 
@@ -137,6 +140,8 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
 // order in which they are merged stay what part_keys makes them, so the floats are the same
 // whoever computes them; fewer workgroups pay fewer start-ups and hand-overs, which a batch
 // that fills the chip anyway does not need.
+//
+// slopes as in rlis_attn_prefill_mfma (the query's position is the last of its context).
 RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
                                    long long out_stride, float* part_ml, float* part_acc,
                                    void* k_pages, void* v_pages,
@@ -146,7 +151,8 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
                                    unsigned* arrivals, int arrival_slots, int groups, int cap,
                                    const float* cos, const float* sin,
                                    int rot, const int* positions, const int* slots,
-                                   long long k_off, long long v_off, hipStream_t stream) {
+                                   long long k_off, long long v_off, const float* slopes,
+                                   hipStream_t stream) {
   DecodeRope rope;
   rope.cos = positions ? cos : nullptr;
   rope.sin = positions ? sin : nullptr;
@@ -199,7 +205,7 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
       "attn_decode_mfma",
       unit(q, q_stride, out, out_stride, part_ml, part_acc, k_pages, v_pages, block_tables,
            max_pages, ctx_lens, S, nh, nkv, d, page_shift, window, scale, splits, part_keys,
-           max_parts, inside, groups, cap, &rope, &merge, stream),
+           max_parts, inside, groups, cap, &rope, &merge, slopes, stream),
       d);
   if (rc) return rc;
   if (splits > 1 && S > 0 && !inside)

@@ -91,7 +91,10 @@ __host__ __device__ constexpr int tile_bufs(int QB) {
 
 // Up to three waves per SIMD (two with two query blocks): the staging registers must not be
 // traded for another.
-template <int QB>
+// BIAS: a bias on the scores, slopes[head] * (key position - query position) added in float32
+// before the softmax (the reference has none; a position encoding of another kind has).  A form
+// of its own, so that the usual one pays nothing for it.
+template <int QB, bool BIAS = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 && D <= 64) ? 4 : 1, QB == 1 ? (D <= 64 ? 4 : 3) : (D <= 64 ? 3 : 2)))) void KERNEL_NAME(
     const bf16_t* __restrict__ q, long long q_stride, bf16_t* __restrict__ out,
     long long out_stride, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
@@ -99,7 +102,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
     const int* __restrict__ start_pos, const int* __restrict__ unit_map, int nh, int nkv, int d,
     int page_shift, float scale, int window, int num_tiles, int tiles_per_round, int part_stride,
     int row0, float* __restrict__ part_ml, float* __restrict__ part_acc,
-    const float* __restrict__ cos_t, const float* __restrict__ sin_t) {
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const float* __restrict__ slopes) {
   constexpr int BN = tile_keys(QB);
   // V^T tile rows: 64 keys padded to a stride of 32 bytes mod 64; 32 keys unpadded, with the
   // 16-byte piece index XORed with (-(row / 4)) & 3, which frees reads and stores of conflicts.
@@ -286,6 +290,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
   }
 
   const float scale2 = scale * 1.4426950408889634f;      // scores in the base-2 domain
+  // With a bias the scores are brought to the base-2 domain as soon as they are formed
+  // (score * scale2 + slope2 * distance), and maximum and exponent take them as they are.
+  const float slope2 = BIAS ? slopes[h] * 1.4426950408889634f : 0.f;
+  const float in_exp = BIAS ? 1.f : scale2;
   if (kt0 < khi) {           // else this run has no keys (only with splits)
   RLIS_LOAD_PAGES(kt0, page_ka, page_va);
   RLIS_LOAD_PAGES(kt0 + BN, page_kb, page_vb);
@@ -343,6 +351,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
             s[b][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[b][ks].v, s[b][nb], 0, 0, 0);
         }
       }
+      if constexpr (BIAS) {
+#pragma unroll
+        for (int b = 0; b < QB; ++b)
+#pragma unroll
+          for (int nb = 0; nb < BN / 16; ++nb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int kpos = k0 + (nb / 2) * 32 + lq * 8 + 2 * r + (nb % 2);
+              s[b][nb][r] = fmaf(s[b][nb][r], scale2, slope2 * (float)(kpos - my_qpos[b]));
+            }
+      }
       // ---- scale, mask (only where a tile meets the diagonal, the window or the end) -----
       const bool plain_tile = (k0 + BN - 1 <= P + wave_q_first) &&
                               (window <= 0 || k0 > P + wave_q_first + 16 * QB - 1 - window);
@@ -371,7 +390,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
             }
         }
         mx = xor32_max(xor16_max(mx));
-        const float m_new = fmaxf(m_run[b], mx * scale2);          // -inf stays -inf
+        const float m_new = fmaxf(m_run[b], mx * in_exp);          // -inf stays -inf
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;   // a query with no key yet
         corr[b] = __builtin_amdgcn_exp2f(m_run[b] - m_safe);       // 0 when m_run is -inf
         float sum = 0.f;
@@ -379,7 +398,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
         for (int nb = 0; nb < BN / 16; ++nb)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const float p = __builtin_amdgcn_exp2f(fmaf(s[b][nb][r], scale2, -m_safe));  // exp2(-inf) = 0
+            const float p = __builtin_amdgcn_exp2f(fmaf(s[b][nb][r], in_exp, -m_safe));  // exp2(-inf) = 0
             s[b][nb][r] = p;
             sum += p;
           }
@@ -508,7 +527,7 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
     const int* start_pos, const int* tile_map, int num_tiles, int nh, int nkv, int d,
     int page_shift, int window, float scale, int tile_queries, int splits, int row0,
     float* part_ml, float* part_acc, const float* cos, const float* sin, int rot,
-    hipStream_t stream) {
+    const float* slopes, hipStream_t stream) {
   if (num_tiles == 0) return 0;
   // rotation inside the kernel needs head_dim = rotated width = 64, 128 or 256
   if (cos && !(sin && D % 64 == 0 && rot == D && d == D)) return kUnitBadRotation;
@@ -516,18 +535,20 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
   if (blocks >= (1ll << 31)) return kUnitTooManyTiles;
   // 256 compute units: a round is the units whose blocks fill them once.
   const int tiles_per_round = (nh <= 256 && 256 % nh == 0) ? 256 / nh : 0;
-  if (tile_queries == 2 * BM)
-    KERNEL_NAME<2><<<(int)blocks, 256, 0, stream>>>(
-        (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,
-        (const bf16_t*)v_pages, block_tables, max_pages, cu_seqlens, start_pos, tile_map, nh, nkv,
-        d, page_shift, scale, window, num_tiles, tiles_per_round, splits, row0, part_ml, part_acc, cos,
-        sin);
-  else
-    KERNEL_NAME<1><<<(int)blocks, 256, 0, stream>>>(
-        (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,
-        (const bf16_t*)v_pages, block_tables, max_pages, cu_seqlens, start_pos, tile_map, nh, nkv,
-        d, page_shift, scale, window, num_tiles, tiles_per_round, splits, row0, part_ml, part_acc, cos,
-        sin);
+#define RLIS_PREFILL_LAUNCH(QB, BIAS)                                                            \
+  KERNEL_NAME<QB, BIAS><<<(int)blocks, 256, 0, stream>>>(                                        \
+      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,              \
+      (const bf16_t*)v_pages, block_tables, max_pages, cu_seqlens, start_pos, tile_map, nh, nkv, \
+      d, page_shift, scale, window, num_tiles, tiles_per_round, splits, row0, part_ml, part_acc, \
+      cos, sin, slopes)
+  if (tile_queries == 2 * BM) {
+    if (slopes) RLIS_PREFILL_LAUNCH(2, true);
+    else RLIS_PREFILL_LAUNCH(2, false);
+  } else {
+    if (slopes) RLIS_PREFILL_LAUNCH(1, true);
+    else RLIS_PREFILL_LAUNCH(1, false);
+  }
+#undef RLIS_PREFILL_LAUNCH
   RLIS_UNIT_LAUNCH_CHECK();
   return 0;
 }
@@ -614,7 +635,9 @@ __device__ __forceinline__ float load_shared_result(const float* p) {
 // instructions (30 fewer registers at head size 128, a tenth fewer instructions in the chunk
 // loop), and no key is masked for lying in front of a window.
 constexpr int kExactPageShift = 4;
-template <bool WALKS, bool EXACT>
+// BIAS: slopes[head] * (key position - the token's position) is added to every score, as in
+// the prefill kernel (a form of its own, in the general shape of the kernel only).
+template <bool WALKS, bool EXACT, bool BIAS = false>
 __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNEL_NAME(
     const bf16_t* __restrict__ q, long long q_stride, bf16_t* __restrict__ out,
     long long out_stride, float* __restrict__ part_ml, float* __restrict__ part_acc,
@@ -622,7 +645,7 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ ctx_lens,
     int nh, int nkv, int d, int page_shift, float scale, int window, int splits, int part_keys,
     int max_parts, int merge_inside, int groups, int cap, const DecodeRope rope,
-    const DecodeMerge merge) {
+    const DecodeMerge merge, const float* __restrict__ slopes) {
   if constexpr (EXACT) {
     d = D;
     page_shift = kExactPageShift;
@@ -800,6 +823,9 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
 #pragma unroll
   for (int db = 0; db < D / 16; ++db) o_acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
   const float scale2 = scale * 1.4426950408889634f;
+  // (with a bias the scores go to the base-2 domain as they are formed, see the prefill kernel)
+  const float slope2 = BIAS ? slopes[kvh * g + min(l16, g - 1)] * 1.4426950408889634f : 0.f;
+  const float in_exp = BIAS ? 1.f : scale2;
 
   auto compute = [&](int c0, const Frag8 (&kf)[2][D / 32], const Frag8 (&vf)[D / 16])
                      __attribute__((always_inline)) {
@@ -817,12 +843,13 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int key = c0 + nb * 16 + lq * 4 + r;
+        if constexpr (BIAS) s[nb][r] = fmaf(s[nb][r], scale2, slope2 * (float)(key - (ctx - 1)));
         const float sv = (key >= lo && key < kend) ? s[nb][r] : -INFINITY;
         s[nb][r] = sv;
         mx = fmaxf(mx, sv);
       }
     mx = xor32_max(xor16_max(mx));
-    const float m_new = fmaxf(m_run, mx * scale2);    // scale2 > 0; -inf stays -inf
+    const float m_new = fmaxf(m_run, mx * in_exp);    // in_exp > 0; -inf stays -inf
     const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
     const float corr = __builtin_amdgcn_exp2f(m_run - m_safe);
     float sum = 0.f;
@@ -831,7 +858,7 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
     for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float p = __builtin_amdgcn_exp2f(fmaf(s[nb][r], scale2, -m_safe));
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[nb][r], in_exp, -m_safe));
         sum += p;
         pf[nb * 4 + r] = (__bf16)p;
       }
@@ -1054,7 +1081,7 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
     float* part_acc, const void* k_pages, const void* v_pages, const int* block_tables,
     int max_pages, const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift, int window,
     float scale, int splits, int part_keys, int max_parts, int merge_inside, int groups, int cap,
-    const DecodeRope* rope, const DecodeMerge* merge, hipStream_t stream) {
+    const DecodeRope* rope, const DecodeMerge* merge, const float* slopes, hipStream_t stream) {
   if (S == 0) return 0;
   if (part_keys % (32 * kDecodeWaves) != 0 || part_keys <= 0) return kUnitBadPartition;
   if (merge_inside && (!merge->arrivals || (long long)S * nkv > merge->slots))
@@ -1076,7 +1103,8 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
     if (e != hipSuccess) return kUnitLaunchFailed + (int)e;
     if (dev < 0 || dev >= kDevices || !granted[dev]) {
       const void* forms[] = {reinterpret_cast<const void*>(&DECODE_KERNEL_NAME<true, false>),
-                             reinterpret_cast<const void*>(&DECODE_KERNEL_NAME<true, true>)};
+                             reinterpret_cast<const void*>(&DECODE_KERNEL_NAME<true, true>),
+                             reinterpret_cast<const void*>(&DECODE_KERNEL_NAME<true, false, true>)};
       for (const void* form : forms) {
         e = hipFuncSetAttribute(form, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWalkBytes);
         if (e != hipSuccess) return kUnitLaunchFailed + (int)e;
@@ -1091,17 +1119,19 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
   const int by_cap = (splits + cap - 1) / cap;
   dim3 grid(nkv, S, cap > 1 ? (groups > by_cap ? (groups < splits ? groups : splits) : by_cap)
                             : splits);
-#define RLIS_DEC_LAUNCH(WALKS, EXACT)                                                             \
-  DECODE_KERNEL_NAME<WALKS, EXACT><<<grid, 64 * kDecodeWaves, smem, stream>>>(                   \
+#define RLIS_DEC_LAUNCH(WALKS, EXACT, BIAS)                                                       \
+  DECODE_KERNEL_NAME<WALKS, EXACT, BIAS><<<grid, 64 * kDecodeWaves, smem, stream>>>(             \
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, part_ml, part_acc,                   \
       (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, max_pages, ctx_lens, nh, nkv, \
       d, page_shift, scale, window, splits, part_keys, max_parts, merge_inside, groups, cap,   \
-      *rope, *merge)
+      *rope, *merge, slopes)
   const bool exact = d == D && page_shift == kExactPageShift && window <= 0;
-  if (cap > 1 && exact) RLIS_DEC_LAUNCH(true, true);
-  else if (cap > 1) RLIS_DEC_LAUNCH(true, false);
-  else if (exact) RLIS_DEC_LAUNCH(false, true);
-  else RLIS_DEC_LAUNCH(false, false);
+  if (slopes && cap > 1) RLIS_DEC_LAUNCH(true, false, true);
+  else if (slopes) RLIS_DEC_LAUNCH(false, false, true);
+  else if (cap > 1 && exact) RLIS_DEC_LAUNCH(true, true, false);
+  else if (cap > 1) RLIS_DEC_LAUNCH(true, false, false);
+  else if (exact) RLIS_DEC_LAUNCH(false, true, false);
+  else RLIS_DEC_LAUNCH(false, false, false);
 #undef RLIS_DEC_LAUNCH
   RLIS_UNIT_LAUNCH_CHECK();
   return 0;

@@ -683,25 +683,26 @@ def _prefill_mfma_ok(qkv: torch.Tensor, d: int, page_size: int) -> bool:
 def attention_planner(num_heads: int, num_kv_heads: int, head_dim: int,
                       dtype: torch.dtype, biased: bool = False) -> AttentionPlanner:
     """The planner a mixer that calls ``paged_attention`` / ``rope_attention`` names as its
-    ``step_planner()``; ``biased``: it will pass ``bias_slopes`` (no matrix-core kernels then)."""
+    ``step_planner()``; ``biased``: it will pass ``bias_slopes`` (the matrix-core kernels take
+    them too, so the plan is the same)."""
     return AttentionPlanner(num_heads, num_kv_heads, head_dim,
-                            matrix=dtype == torch.bfloat16 and not biased,
+                            matrix=dtype == torch.bfloat16,
                             singles_apart=SPLIT_MIXED_ATTENTION and DECODE_ATTENTION != "vector")
 
 
 def _attention_kernel(qkv: torch.Tensor, nh: int, nkv: int, d: int, page_size: int, step,
                       force: Optional[str], biased: bool = False):
-    """(kind, matrix_decode): which attention kernel a batch takes.  A bias on the scores is
-    taken by the vector-unit kernels only (the generic one and the vector decode kernel)."""
+    """(kind, matrix_decode): which attention kernel a batch takes.  A bias on the scores
+    changes nothing here: every kernel takes one."""
     kind = force or FORCE_ATTENTION
     if kind is None:
         if step.all_decode and d % 8 == 0 and d <= 256 and (nh // nkv) * d <= 2048:
             kind = "decode"
-        elif _prefill_mfma_ok(qkv, d, page_size) and not step.all_decode and not biased:
+        elif _prefill_mfma_ok(qkv, d, page_size) and not step.all_decode:
             kind = "prefill"
         else:
             kind = "generic"
-    mfma = kind == "decode" and not biased and _decode_mfma_ok(qkv, nh, nkv, d, page_size)
+    mfma = kind == "decode" and _decode_mfma_ok(qkv, nh, nkv, d, page_size)
     return kind, mfma
 
 
@@ -748,6 +749,7 @@ def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
             raise KernelError("rope_attention: a cache write needs slots")
         return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
                                scale, window, plan=plan, counters=counters,
+                               bias_slopes=bias_slopes,
                                rope=(cos, sin, positions, slots if write_kv else None))
     if (kind == "prefill" and cos is not None and fusable and FUSE_ROPE_PREFILL and whole_rows
             and (_decode_mfma_ok(qkv, nh, nkv, d, page_size)
@@ -756,7 +758,7 @@ def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
                       write_kv=write_kv, rotate_q=False)
         return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
                                scale, window, plan=plan, counters=counters,
-                               rope=(cos, sin, positions, None))
+                               bias_slopes=bias_slopes, rope=(cos, sin, positions, None))
     rope_kv_write(qkv, nh, nkv, d, cos, sin, positions, slots, k_pages, v_pages, page_size,
                   write_kv=write_kv, interleaved=interleaved)
     return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
@@ -782,7 +784,7 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     keys are cut (decode partitions, tile form, key runs) follows from its own lengths alone.
     ``bias_slopes`` (float32, one per query head; the reference has no such thing): the score of
     key position ``u`` for a query at position ``p`` gets ``slope * (u - p)`` added before the
-    softmax; the vector-unit kernels take it, so such a batch goes to them.
+    softmax; every kernel takes it (the matrix-core ones in a form of their own).
     ``force`` names one of 'generic', 'decode', 'prefill' for tests.  ``rope`` (from
     ``rope_attention`` only): ``(cos, sin, positions, slots)`` for the matrix-core decode kernel
     to rotate and store the step's tokens itself; with portions of prompts in the batch
@@ -826,8 +828,6 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                                           and rope[0] is not None)):
         raise KernelError("attention: only the matrix-core kernels rotate, and only the decode "
                           "kernel stores")
-    if slopes_ptr is not None and kind == "prefill":
-        raise KernelError("attention: the matrix-core prefill kernel takes no bias on the scores")
     if kind == "generic":
         lib.call("rlis_attn_generic", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(), nh * d,
                  k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,
@@ -837,8 +837,7 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     if kind not in ("decode", "prefill"):
         raise KernelError(f"attention: unknown kernel '{kind}'")
     if plan is None or force == "prefill":
-        planner = AttentionPlanner(nh, nkv, d,
-                                   matrix=qkv.dtype == torch.bfloat16 and slopes_ptr is None,
+        planner = AttentionPlanner(nh, nkv, d, matrix=qkv.dtype == torch.bfloat16,
                                    singles_apart=force is None and SPLIT_MIXED_ATTENTION
                                    and DECODE_ATTENTION != "vector")
         plan = _plan_now(step, planner, qkv.device)
@@ -880,7 +879,7 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                      block_tables.data_ptr(), max_pages, _i32(step.ctx_lens, "ctx_lens", S), S,
                      nh, nkv, d, page_size, win, float(scale), depth, ap.DECODE_PART_KEYS,
                      ap.DECODE_MAX_PARTS, arrivals_p, arrival_slots, groups, cap, cos_p, sin_p,
-                     rot, pos_p, slots_p, nh * d, (nh + nkv) * d, stream)
+                     rot, pos_p, slots_p, nh * d, (nh + nkv) * d, slopes_ptr, stream)
         else:
             lib.call("rlis_attn_decode", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(),
                      nh * d, ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
@@ -935,7 +934,7 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                  _i32(step.cu_seqlens, "cu_seqlens", step.num_seqs + 1),
                  _i32(step.start_pos, "start_pos", step.num_seqs),
                  _i32(plan[name], name, 4 * n), n, nh, nkv, d, page_size, win, float(scale), tile,
-                 max_runs, row0, ml_ptr, acc_ptr, cos_p, sin_p, rot, stream)
+                 max_runs, row0, ml_ptr, acc_ptr, cos_p, sin_p, rot, slopes_ptr, stream)
     if not launched and T > row0:
         raise KernelError("attention: the plan holds no tiles for the step's portions")
     if launched and max_runs > 1:

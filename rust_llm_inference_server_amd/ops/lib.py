@@ -35,9 +35,9 @@ _SIGNATURES = {
     "rlis_attn_generic": [P, I, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P, P],
     "rlis_attn_decode": [P, I, L, P, L, P, P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, I, I, P, P],
     "rlis_attn_decode_mfma": [P, L, P, L, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, I, I, P, I, I, I,
-                              P, P, I, P, P, L, L, P],
+                              P, P, I, P, P, L, L, P, P],
     "rlis_attn_prefill_mfma": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, I, P, P,
-                               P, P, I, P],
+                               P, P, I, P, P],
     "rlis_attn_reduce_rows": [P, L, P, P, P, P, I, I, I, I, I, P],
     "rlis_sample_rows": [P, L, I, I, P, P, P, I, P, P, P],
     "rlis_fill_normal_device": [P, I, L, ctypes.c_ulonglong, ctypes.c_ulonglong, ctypes.c_double,

@@ -1272,9 +1272,11 @@ def test_attention_window_edge(ops, dtype, kind, window, decode_kind):
 def test_attention_with_a_bias_on_the_scores(ops, dtype, nh, nkv, d, ps):
     """slope[h] * (key position - query position) added to the scores before the softmax (a
     position encoding that works on the scores; the reference has none): portions beside single
-    tokens through the generic kernel, single tokens through the vector decode kernel, with and
-    without a window, against the plain attention with the bias as an additive mask.  A slope
-    so steep that only the query's own position counts returns that position's value."""
+    tokens and single tokens alone, with and without a window, through the kernels that the
+    batch takes by itself (bfloat16: the matrix-core kernels' forms with a bias, over several
+    decode partitions and key runs too; float32: the vector-unit kernels) and through the
+    generic kernel, against the plain attention with the bias as an additive mask.  A slope so
+    steep that only the query's own position counts returns that position's value."""
     scale = 1.0 / math.sqrt(d)
     slopes = torch.tensor([0.5 ** (1 + h % 5) for h in range(nh)], dtype=torch.float32)
 
@@ -1292,13 +1294,16 @@ def test_attention_with_a_bias_on_the_scores(ops, dtype, nh, nkv, d, ps):
             outs.append(o.transpose(0, 1).reshape(n, nh * d))
         return torch.cat(outs)
 
-    for cached, new in (([0, 5, 40, 130, 17], [33, 1, 70, 2, 64]), ([4, 99, 0, 640], [1, 1, 1, 1])):
+    for cached, new in (([0, 5, 40, 130, 17], [33, 1, 70, 2, 64]), ([4, 99, 0, 640], [1, 1, 1, 1]),
+                        ([1, 1100], [1, 1]), ([1200, 2], [1, 130])):
         for window in (None, 50):
             qkv, kp, vp, bt, step, ks, vs, cu = paged_case(cached, new, nh, nkv, d, ps, dtype, seed=nh + 9)
-            got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window,
-                                      bias_slopes=slopes.to(DEV))
             want = reference(qkv, ks, vs, cu, cached, new, slopes, window)
-            torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
+            with attention_constants(DECODE_PART_KEYS=256, **key_runs(3)):
+                for force in (None, "generic"):
+                    got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window,
+                                              bias_slopes=slopes.to(DEV), force=force)
+                    torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
             plainly = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, window)
             assert (got.float() - plainly.float()).abs().max().item() > 1e-2       # the bias matters
     steep = torch.full((nh,), 1000.0, dtype=torch.float32, device=DEV)
@@ -1308,10 +1313,14 @@ def test_attention_with_a_bias_on_the_scores(ops, dtype, nh, nkv, d, ps):
         for h in range(nh):
             torch.testing.assert_close(got[s, h * d:(h + 1) * d].float().cpu(), vs[s][last, h // (nh // nkv)],
                                        **tol(dtype, 1e-5, 1e-2))
-    qkv, kp, vp, bt, step, *_ = paged_case([0], [40], 4, 2, 32, 8, torch.bfloat16)
-    with pytest.raises(ops.KernelError, match="no bias"):
-        ops.paged_attention(qkv, 4, 2, 32, kp, vp, 8, bt, step, 1.0, None, force="prefill",
-                            bias_slopes=torch.ones(4, device=DEV))
+    if dtype == torch.bfloat16:
+        # tiles of 128 queries (two query blocks a wave) take the bias too
+        qkv, kp, vp, bt, step, ks, vs, cu = paged_case([20], [300], nh, nkv, d, ps, dtype, seed=5)
+        want = reference(qkv, ks, vs, cu, [20], [300], slopes, None)
+        with attention_constants(PREFILL_WIDE_MIN_GROUPS=0):
+            got = ops.paged_attention(qkv, nh, nkv, d, kp, vp, ps, bt, step, scale, None,
+                                      bias_slopes=slopes.to(DEV), force="prefill")
+        torch.testing.assert_close(got.float().cpu(), want, **tol(dtype, 2e-5, 2e-2))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
