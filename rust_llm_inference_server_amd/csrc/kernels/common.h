@@ -30,6 +30,8 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
 
 __device__ __forceinline__ float ld(const float* p) { return *p; }
 __device__ __forceinline__ float ld(const bf16_t* p) { return bf16_to_f32(*p); }
+__device__ __forceinline__ float widen(float v) { return v; }
+__device__ __forceinline__ float widen(bf16_t v) { return bf16_to_f32(v); }
 __device__ __forceinline__ void st(float* p, float v) { *p = v; }
 __device__ __forceinline__ void st(bf16_t* p, float v) { *p = f32_to_bf16(v); }
 

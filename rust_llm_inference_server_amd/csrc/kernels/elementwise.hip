@@ -237,8 +237,9 @@ static bool launch_add_rmsnorm_bf16x8(float* resid, const void* delta, const voi
 // leave for their consumer), rows of a multiple of 4 and at most NT * 4 * CH elements: four
 // elements per thread and chunk, 16-byte accesses.  Such stacks come with few rows (64 at most)
 // and up to dozens of parts, so a row gets a wide workgroup (NT threads, as many as the row has
-// groups of four, up to 1024) and every thread keeps four parts of all its chunks in flight;
-// the parts are added in order and their sum rounded to bfloat16 when round_parts is set.
+// groups of four, up to 1024) and every thread keeps eight parts of its chunk in flight (four
+// of each where it has several chunks); the parts are added in order and their sum rounded to
+// bfloat16 when round_parts is set.
 template <typename TW, typename TO, int CH, int NT>
 __global__ __launch_bounds__(NT) void add_rmsnorm_stack_kernel(
     float* __restrict__ resid, const float* __restrict__ delta, const TW* __restrict__ weight,
@@ -253,34 +254,39 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_stack_kernel(
   int col[CH];
   bool live[CH];
   float4 xr[CH], s[CH];
+  // The norm's weight is asked for with the first loads, long before it is needed.
+  TW wt[CH][4];
 #pragma unroll
   for (int ch = 0; ch < CH; ++ch) {
     const int j = (threadIdx.x + ch * NT) * 4;
     live[ch] = j < H;
     col[ch] = live[ch] ? j : 0;
     xr[ch] = *(const float4*)(x + col[ch]);
-    s[ch] = *(const float4*)(d + col[ch]);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) wt[ch][e] = weight[col[ch] + e];
   }
-  int p = 1;
-  for (; p + 3 < parts; p += 4) {
-    float4 a[CH][4];
+  // The parts in batches of AHEAD, every batch's loads issued together and none under a
+  // condition (a part past the last reads the last again and adds nothing): a stack of eight
+  // parts is one trip to memory, and no part waits for the one before it.  They are added in
+  // order, the first one as it is.
+  constexpr int AHEAD = CH == 1 ? 8 : 4;
+  for (int p = 0; p < parts; p += AHEAD) {
+    float4 a[CH][AHEAD];
 #pragma unroll
     for (int ch = 0; ch < CH; ++ch)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) a[ch][q] = *(const float4*)(d + (p + q) * part_stride + col[ch]);
+      for (int q = 0; q < AHEAD; ++q)
+        a[ch][q] = *(const float4*)(d + (long long)min(p + q, parts - 1) * part_stride + col[ch]);
 #pragma unroll
     for (int ch = 0; ch < CH; ++ch)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        s[ch].x += a[ch][q].x; s[ch].y += a[ch][q].y; s[ch].z += a[ch][q].z; s[ch].w += a[ch][q].w;
+      for (int q = 0; q < AHEAD; ++q) {
+        if (p == 0 && q == 0) {
+          s[ch] = a[ch][0];
+        } else if (p + q < parts) {
+          s[ch].x += a[ch][q].x; s[ch].y += a[ch][q].y; s[ch].z += a[ch][q].z; s[ch].w += a[ch][q].w;
+        }
       }
-  }
-  for (; p < parts; ++p) {
-#pragma unroll
-    for (int ch = 0; ch < CH; ++ch) {
-      const float4 a = *(const float4*)(d + p * part_stride + col[ch]);
-      s[ch].x += a.x; s[ch].y += a.y; s[ch].z += a.z; s[ch].w += a.w;
-    }
   }
   float v[CH][4];
   float ss = 0.f;
@@ -307,7 +313,7 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_stack_kernel(
     if (live[ch]) {
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        st(o + col[ch] + e, v[ch][e] * inv * ld(weight + col[ch] + e));
+        st(o + col[ch] + e, v[ch][e] * inv * widen(wt[ch][e]));
     }
   }
 }
