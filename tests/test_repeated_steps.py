@@ -109,3 +109,20 @@ def test_a_shape_whose_capture_is_refused_stays_eager():
     for i in range(3 * RepeatedSteps.CAPTURE_AT):
         assert rs.run(step) is None
     assert len(tried) == 1 and not rs.graphs and runner is not None
+
+
+def test_the_rule_for_slices_of_k_follows_from_rows_and_k_alone():
+    """How the library's product over a long k is cut into slices when its consumer takes partial
+    sums (ops.library_slices): eight slices up to 256 rows, four up to 1,024, two up to 2,048,
+    fewer where k does not divide into slices of whole 16-byte pieces; one product below 65
+    rows, beyond 2,048 and for a short k."""
+    from rust_llm_inference_server_amd import ops
+    cut = ops.library_slices
+    assert [cut(t, 8192) for t in (64, 65, 256, 257, 1024, 1025, 2048, 2049)] == [1, 8, 8, 4, 4, 2, 2, 1]
+    assert [cut(t, 14336) for t in (100, 300, 1500)] == [8, 4, 2]
+    assert cut(512, 4096) == 1 and cut(512, 8192 + 8) == 1
+    assert cut(100, 8192 + 32) == 4 and cut(100, 8192 + 16) == 2 and cut(300, 8192 + 16) == 2
+    for t in (65, 200, 512, 2000):
+        for k in (8192, 8200, 8208, 11008, 14336, 28672):
+            n = cut(t, k)
+            assert k % n == 0 and (k // n) % 8 == 0
